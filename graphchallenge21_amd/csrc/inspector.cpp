@@ -1,0 +1,280 @@
+#include "inspector.hpp"
+
+#include <algorithm>
+#include <array>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+
+namespace spdnn {
+
+std::string normalize_csr(int N, const int32_t* rowptr, const int32_t* col, const float* val,
+                          std::vector<int32_t>& orp, std::vector<int32_t>& oc, std::vector<float>& ov) {
+    if (!rowptr || rowptr[0] != 0) return "rowptr[0] must be 0";
+    for (int j = 0; j < N; ++j)
+        if (rowptr[j + 1] < rowptr[j]) return "rowptr must be non-decreasing";
+    const int64_t nnz = rowptr[N];
+    if (nnz > 0 && (!col || !val)) return "col/val missing";
+    orp.assign(rowptr, rowptr + N + 1);
+    oc.resize((size_t)nnz);
+    ov.resize((size_t)nnz);
+    std::vector<int32_t> order;
+    for (int j = 0; j < N; ++j) {
+        const int b = rowptr[j], e = rowptr[j + 1];
+        bool sorted = true;
+        for (int k = b; k < e; ++k) {
+            if (col[k] < 0 || col[k] >= N) return "column index out of range";
+            if (!std::isfinite(val[k])) return "non-finite weight";
+            if (k > b && col[k] < col[k - 1]) sorted = false;
+        }
+        if (sorted) {
+            std::copy(col + b, col + e, oc.begin() + b);
+            std::copy(val + b, val + e, ov.begin() + b);
+        } else {
+            order.resize((size_t)(e - b));
+            std::iota(order.begin(), order.end(), b);
+            std::stable_sort(order.begin(), order.end(), [&](int32_t x, int32_t y) { return col[x] < col[y]; });
+            for (int k = b; k < e; ++k) { oc[k] = col[order[k - b]]; ov[k] = val[order[k - b]]; }
+        }
+    }
+    return std::string();
+}
+
+namespace {
+
+// number of common elements of two ascending lists of length K; the common elements go to `common`
+// (at most cap of them are stored)
+inline int intersect_sorted(const int32_t* a, const int32_t* b, int K, int32_t* common, int cap) {
+    int i = 0, j = 0, n = 0;
+    while (i < K && j < K) {
+        if (a[i] < b[j]) ++i;
+        else if (a[i] > b[j]) ++j;
+        else { if (n < cap) common[n] = a[i]; ++n; ++i; ++j; }
+    }
+    return n;
+}
+
+inline bool exact_weight(float w) {
+    if (w == 0.0f) return true;
+    int e = 0;
+    const float m = std::frexp(std::fabs(w), &e);  // |w| = m * 2^e, m in [0.5, 1)
+    return m == 0.5f && e >= -23 && e <= 25;
+}
+
+}  // namespace
+
+bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                   std::vector<int32_t>& in_pos, std::vector<int32_t>& out_at) {
+    if (K < 2 || N < 4 * K) return false;
+    // outputs of every input, ascending (counting pass over the rows in ascending output order)
+    std::vector<int32_t> outs((size_t)N * K);
+    std::vector<int32_t> fill((size_t)N, 0);
+    for (int j = 0; j < N; ++j) {
+        if (rowptr[j + 1] - rowptr[j] != K) return false;
+        for (int e = rowptr[j]; e < rowptr[j + 1]; ++e) {
+            const int i = col[e];
+            if (fill[i] >= K) return false;
+            outs[(size_t)i * K + fill[i]++] = j;
+        }
+    }
+    for (int i = 0; i < N; ++i) if (fill[i] != K) return false;
+    auto In = [&](int j) { return col.data() + rowptr[j]; };
+    auto Out = [&](int i) { return outs.data() + (size_t)i * K; };
+    int32_t tmp[4];
+
+    // --- bootstrap: the 2K-1 inputs around input 0, ordered by how many outputs they share with it
+    const int a0 = 0;
+    std::vector<int32_t> cnt((size_t)N, 0);
+    std::vector<int32_t> touched;
+    for (int t = 0; t < K; ++t) {
+        const int32_t* in = In(Out(a0)[t]);
+        for (int k = 0; k < K; ++k) if (cnt[in[k]]++ == 0) touched.push_back(in[k]);
+    }
+    if (cnt[a0] != K || (int)touched.size() != 2 * K - 1) return false;
+    std::vector<std::array<int32_t, 2>> by((size_t)K, std::array<int32_t, 2>{-1, -1});
+    for (int32_t i : touched) {
+        if (i == a0) continue;
+        const int d = K - cnt[i];
+        if (d < 1 || d > K - 1) return false;
+        if (by[d][0] < 0) by[d][0] = i;
+        else if (by[d][1] < 0) by[d][1] = i;
+        else return false;
+    }
+    std::vector<int32_t> plus((size_t)K), minus((size_t)K);
+    plus[0] = minus[0] = a0;
+    for (int d = 1; d < K; ++d) {
+        if (by[d][0] < 0 || by[d][1] < 0) return false;
+        if (d == 1) { plus[1] = by[1][0]; minus[1] = by[1][1]; continue; }
+        const int32_t c = by[d][0];
+        if (intersect_sorted(Out(c), Out(plus[d - 1]), K, tmp, 0) == K - 1) { plus[d] = c; minus[d] = by[d][1]; }
+        else { plus[d] = by[d][1]; minus[d] = c; }
+        if (intersect_sorted(Out(plus[d]), Out(plus[d - 1]), K, tmp, 0) != K - 1) return false;
+        if (intersect_sorted(Out(minus[d]), Out(minus[d - 1]), K, tmp, 0) != K - 1) return false;
+    }
+
+    // --- walk the band: positions 0..K-1 hold minus[K-1..1], a0; the output whose window is
+    //     exactly those inputs sits at position K-1
+    std::vector<int32_t> in_ext((size_t)N + 2 * K, -1), out_ext((size_t)N + 2 * K, -1);
+    for (int d = 1; d < K; ++d) in_ext[K - 1 - d] = minus[d];
+    in_ext[K - 1] = a0;
+    {
+        int found = -1, nfound = 0;
+        const int32_t* oa = Out(a0);
+        const int32_t* ob = Out(plus[1]);
+        for (int t = 0; t < K; ++t)
+            if (!std::binary_search(ob, ob + K, oa[t])) { found = oa[t]; ++nfound; }
+        if (nfound != 1) return false;
+        out_ext[K - 1] = found;
+    }
+    std::vector<uint8_t> mark((size_t)N, 0);
+    for (int p = 0; p < K; ++p) mark[in_ext[p]] = 1;
+    {
+        const int32_t* in = In(out_ext[K - 1]);
+        for (int k = 0; k < K; ++k) if (!mark[in[k]]) return false;
+    }
+    for (int v = K - 1; v < N + K - 1; ++v) {
+        const int32_t a_hi = in_ext[v], a_lo2 = in_ext[v - K + 2];
+        // outputs v and v+1 are the only ones reading both the newest and the second-oldest input
+        int32_t next;
+        if (a_hi == a_lo2) {  // K == 2
+            const int32_t* o = Out(a_hi);
+            if (o[0] == out_ext[v]) next = o[1];
+            else if (o[1] == out_ext[v]) next = o[0];
+            else return false;
+        } else {
+            if (intersect_sorted(Out(a_hi), Out(a_lo2), K, tmp, 4) != 2) return false;
+            if (tmp[0] == out_ext[v]) next = tmp[1];
+            else if (tmp[1] == out_ext[v]) next = tmp[0];
+            else return false;
+        }
+        int32_t newi = -1;
+        const int32_t* in = In(next);
+        for (int k = 0; k < K; ++k)
+            if (!mark[in[k]]) { if (newi >= 0) return false; newi = in[k]; }
+        if (newi < 0) return false;
+        mark[in_ext[v - K + 1]] = 0;
+        mark[newi] = 1;
+        in_ext[v + 1] = newi;
+        out_ext[v + 1] = next;
+    }
+    // the walk went once around: it must close on itself
+    for (int p = N; p < N + K; ++p) if (in_ext[p] != in_ext[p - N]) return false;
+    if (out_ext[N + K - 1] != out_ext[K - 1]) return false;
+
+    in_pos.assign((size_t)N, -1);
+    out_at.assign((size_t)N, -1);
+    for (int p = 0; p < N; ++p) {
+        if (in_pos[in_ext[p]] >= 0) return false;
+        in_pos[in_ext[p]] = p;
+    }
+    std::vector<uint8_t> seen((size_t)N, 0);
+    for (int v = K - 1; v < N + K - 1; ++v) {
+        const int j = out_ext[v];
+        if (seen[j]) return false;
+        seen[j] = 1;
+        out_at[v % N] = j;
+    }
+    // final check, independent of the walk: every output reads exactly the window behind it
+    for (int v = 0; v < N; ++v) {
+        const int32_t* in = In(out_at[v]);
+        for (int k = 0; k < K; ++k) {
+            int d = v - in_pos[in[k]];
+            if (d < 0) d += N;
+            if (d >= K) return false;
+        }
+    }
+    return true;
+}
+
+void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                   const std::vector<float>& val, int force_kernel, LayerPlan& plan) {
+    const int64_t nnz = rowptr[N];
+    int kmax = 0;
+    bool rows_regular = true, dup = false;
+    for (int j = 0; j < N; ++j) {
+        const int len = rowptr[j + 1] - rowptr[j];
+        kmax = std::max(kmax, len);
+        for (int e = rowptr[j] + 1; e < rowptr[j + 1]; ++e) if (col[e] == col[e - 1]) dup = true;
+    }
+    for (int j = 0; j < N; ++j) if (rowptr[j + 1] - rowptr[j] != kmax) rows_regular = false;
+    bool cols_regular = rows_regular;
+    if (rows_regular) {
+        std::vector<int32_t> cc((size_t)N, 0);
+        for (int64_t e = 0; e < nnz; ++e) cc[col[e]]++;
+        for (int i = 0; i < N; ++i) if (cc[i] != kmax) { cols_regular = false; break; }
+    }
+    bool uniform = nnz > 0, exact = true;
+    for (int64_t e = 0; e < nnz; ++e) {
+        if (val[e] != val[0]) uniform = false;
+        if (!exact_weight(val[e])) exact = false;
+    }
+
+    plan.kmax = kmax;
+    plan.info = spdnn_layer_plan{};
+    plan.info.max_row_nnz = kmax;
+    plan.info.regular = (rows_regular && cols_regular && !dup) ? 1 : 0;
+    plan.info.uniform_value = uniform ? 1 : 0;
+    plan.info.value = uniform ? val[0] : 0.0f;
+    plan.info.exact_products = exact ? 1 : 0;
+    plan.info.band_halo = -1;
+    plan.info.nnz = nnz;
+
+    bool band = false;
+    const int K = kmax;
+    if (force_kernel != SPDNN_KERNEL_GATHER && plan.info.regular && K >= 4 && K <= 32 && (K % 4) == 0 &&
+        (N % 256) == 0 && N >= 4 * K) {
+        band = discover_band(N, K, rowptr, col, plan.in_pos, plan.out_at);
+    }
+
+    if (band) {
+        plan.kernel = SPDNN_KERNEL_BAND;
+        plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
+        plan.info.band_halo = K - 1;
+        plan.sel.resize((size_t)N * K);
+        if (plan.wmode != 0) plan.wv.resize((size_t)N * K); else plan.wv.clear();
+        for (int v = 0; v < N; ++v) {
+            const int j = plan.out_at[v];
+            for (int k = 0; k < K; ++k) {
+                const int e = rowptr[j] + k;  // ascending input index = accumulation order
+                plan.sel[(size_t)v * K + k] = (uint8_t)(plan.in_pos[col[e]] & 255);
+                if (plan.wmode != 0) plan.wv[(size_t)v * K + k] = val[e];
+            }
+        }
+        plan.ell_col.clear();
+        plan.rowlen.clear();
+    } else {
+        plan.kernel = SPDNN_KERNEL_GATHER;
+        plan.wmode = exact ? 1 : 2;
+        plan.in_pos.resize((size_t)N);
+        plan.out_at.resize((size_t)N);
+        std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
+        std::iota(plan.out_at.begin(), plan.out_at.end(), 0);
+        const int kw = std::max(kmax, 1);
+        plan.ell_col.assign((size_t)N * kw, 0);
+        plan.wv.assign((size_t)N * kw, 0.0f);
+        plan.rowlen.resize((size_t)N);
+        for (int j = 0; j < N; ++j) {
+            const int len = rowptr[j + 1] - rowptr[j];
+            plan.rowlen[j] = len;
+            for (int k = 0; k < len; ++k) {
+                plan.ell_col[(size_t)j * kw + k] = col[rowptr[j] + k];
+                plan.wv[(size_t)j * kw + k] = val[rowptr[j] + k];
+            }
+        }
+        plan.kmax = kw;
+        plan.sel.clear();
+    }
+    plan.info.kernel = plan.kernel;
+    plan.info.plan_bytes = (int64_t)(plan.sel.size() + 4 * (plan.ell_col.size() + plan.rowlen.size() +
+                                                              plan.wv.size() + 2 * (size_t)N));
+    plan.dst.clear();
+    plan.set = true;
+}
+
+void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos) {
+    const size_t N = cur.out_at.size();
+    cur.dst.resize(N);
+    for (size_t s = 0; s < N; ++s) cur.dst[s] = next_in_pos ? (*next_in_pos)[cur.out_at[s]] : cur.out_at[s];
+}
+
+}  // namespace spdnn

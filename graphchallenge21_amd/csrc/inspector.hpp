@@ -1,0 +1,53 @@
+// Host inspector: turns one layer's CSR into the arrays the kernels stream.
+//
+// Plays the role of the reference's src/inspector (BlockContainer + MaxInReuseBSchedule,
+// called from src/network.cpp:105-120), re-designed: instead of searching for dense rectangles
+// in a hash-reordered matrix it classifies the layer, looks for a relabelling of inputs and
+// outputs under which the layer is a circulant band, and emits either a BAND plan (ring
+// selectors in accumulation order) or a general GATHER plan.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../include/spdnn.h"
+
+namespace spdnn {
+
+struct LayerPlan {
+    bool set = false;
+    spdnn_layer_plan info{};
+    int kernel = SPDNN_KERNEL_GATHER;
+    int wmode = 2;                  // 0 uniform exact value, 1 exact products, 2 multiply then add
+    int kmax = 0;
+    // physical column of every input neuron in the buffer this layer reads
+    std::vector<int32_t> in_pos;
+    // neuron computed at every schedule slot (BAND: band position; GATHER: the neuron itself)
+    std::vector<int32_t> out_at;
+    std::vector<uint8_t> sel;       // BAND: [N][K] input position mod 256, accumulation order
+    std::vector<int32_t> ell_col;   // GATHER: [N][kmax] physical input column, accumulation order
+    std::vector<int32_t> rowlen;    // GATHER: [N]
+    std::vector<float> wv;          // [N][kmax] weights in accumulation order (empty when wmode 0)
+    std::vector<int32_t> dst;       // [N] physical column of slot's output in the next buffer
+};
+
+// Sorts every row of the CSR by input index (stable) and validates it.  Returns an empty
+// string on success, an error text otherwise.
+std::string normalize_csr(int N, const int32_t* rowptr, const int32_t* col, const float* val,
+                          std::vector<int32_t>& out_rowptr, std::vector<int32_t>& out_col,
+                          std::vector<float>& out_val);
+
+// Looks for a relabelling under which output v reads inputs v-K+1..v (mod N).  rowptr/col must
+// be normalized, every row and column holding exactly K entries.  On success in_pos[i] is the
+// band position of input i and out_at[v] the output neuron at position v.
+bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                   std::vector<int32_t>& in_pos, std::vector<int32_t>& out_at);
+
+// Full per-layer inspection (everything except dst, which needs the next layer's labelling).
+void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                   const std::vector<float>& val, int force_kernel, LayerPlan& plan);
+
+// dst[slot] = physical column (in the next buffer) of the neuron computed at `slot`.
+void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos);
+
+}  // namespace spdnn

@@ -1,0 +1,656 @@
+// gfx950 (CDNA4, MI355X) kernels of the Sparse DNN inference path.  wave64 only.
+//
+// All layer kernels share one scheme: a wavefront works on one row block (64*RL feature rows,
+// lane i holds rows i*RL..i*RL+RL-1 in registers) and on a run of output neurons; the input
+// index and the weight of every multiply-add are wave-uniform and live in scalar registers, so
+// the vector ALUs issue nothing but the multiply-adds, the LDS address add and the epilogue.
+// Every output keeps ONE accumulator per row and adds its inputs in ascending input index -
+// the order of the reference's CPU checker (src/utils/cpu_spmm.h:14-35) - so results are
+// bit-identical to it; no reduction tree over the 32 terms anywhere.
+//
+// Epilogue (fused into every layer kernel, reference all_network.cu:55-60):
+//     y = clamp(acc + bias, 0, 32);  store;  row is active iff some y != 0.
+#include "kernels.hpp"
+
+#include <algorithm>
+#include <climits>
+
+namespace spdnn {
+
+namespace {
+
+template <int RL> struct VecOf;
+template <> struct VecOf<1> { using type = float; };
+template <> struct VecOf<2> { using type = float2; };
+template <> struct VecOf<4> { using type = float4; };
+
+template <int RL> __device__ __forceinline__ void vec_to_arr(const typename VecOf<RL>::type& v, float* a);
+template <> __device__ __forceinline__ void vec_to_arr<1>(const float& v, float* a) { a[0] = v; }
+template <> __device__ __forceinline__ void vec_to_arr<2>(const float2& v, float* a) { a[0] = v.x; a[1] = v.y; }
+template <> __device__ __forceinline__ void vec_to_arr<4>(const float4& v, float* a) {
+    a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
+}
+template <int RL> __device__ __forceinline__ typename VecOf<RL>::type arr_to_vec(const float* a);
+template <> __device__ __forceinline__ float arr_to_vec<1>(const float* a) { return a[0]; }
+template <> __device__ __forceinline__ float2 arr_to_vec<2>(const float* a) { return make_float2(a[0], a[1]); }
+template <> __device__ __forceinline__ float4 arr_to_vec<4>(const float* a) {
+    return make_float4(a[0], a[1], a[2], a[3]);
+}
+
+// One multiply-add of the accumulation chain.
+//   WMODE 0/1: the product is exact (weight is 0 or a power of two), so a fused multiply-add
+//              rounds exactly like the reference's multiply followed by add.
+//   WMODE 2:   general weights: rounded multiply, then rounded add, as the CPU reference does.
+template <int WMODE> __device__ __forceinline__ float mac(float acc, float x, float w) {
+    if (WMODE == 2) return __fadd_rn(acc, __fmul_rn(x, w));
+    return __builtin_fmaf(x, w, acc);
+}
+
+__device__ __forceinline__ float relu_clamp(float y, float clampv) {
+    // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
+    return __builtin_amdgcn_fmed3f(y, 0.0f, clampv);
+}
+
+// ------------------------------------------------------------------------------------------
+// BAND kernel ("row-succ" / tiled variant).
+//
+// The inspector has relabelled the layer so that the output at band position v reads the K
+// input columns at positions v-K+1 .. v (mod N).  A workgroup takes one row block and one
+// segment [vb, ve) of band positions and walks it in chunks of T = NW*OPW outputs.  The input
+// columns live in an LDS ring of RING column slots (slot = position mod RING, RING | N): while
+// the waves compute chunk c from the ring, the T columns of chunk c+1 are already in flight
+// from HBM into registers and are dropped into the ring afterwards, so every input column is
+// read from HBM once per segment (plus K-1 halo columns at the segment start) and the loads
+// overlap the arithmetic.  Needs 2*T + K - 1 <= RING.
+//
+// Per output the scalar unit streams 32 one-byte ring selectors (already in accumulation order)
+// and, unless the layer has one exact value, 32 weights; the output column is written to the
+// physical column the NEXT layer wants it in (dst), RB*4 contiguous bytes.
+// ------------------------------------------------------------------------------------------
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+__global__ __launch_bounds__(NW * 64) void band_walk_kernel(
+    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
+    const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
+    int N, int Krt, int seglen, int stamp, float wu, float bias, float clampv) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    using V = typename VecOf<RL>::type;
+    constexpr int T = NW * OPW;
+    constexpr int RB = 64 * RL;
+    constexpr int COLB = RB * 4;
+    static_assert(2 * T + 31 <= RING, "ring too small for 32 entries per output");
+    static_assert((RING & (RING - 1)) == 0 && RING <= 256, "ring must be a power of two <= 256");
+    static_assert(KT == 0 || KT == 32, "KT is 32 (unrolled) or 0 (run-time row length)");
+
+    const int K = KT ? KT : Krt;
+    const int K4 = K >> 2;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rb = blockIdx.x;
+    const int vb = blockIdx.y * seglen;
+    const int ve = min(N, vb + seglen);
+    const size_t blk = (size_t)rb * (size_t)N * RB;
+    const float* __restrict__ yin = yin_all + blk;
+    float* __restrict__ yout = yout_all + blk;
+    const int loff = lane * RL;
+    const unsigned char* lane_smem = smem + loff * 4;
+
+    // prologue: halo (K-1 columns before the segment, wrapping below 0) + first chunk
+    for (int c = wave; c < K - 1 + T; c += NW) {
+        const int p = vb - (K - 1) + c;
+        if (p < ve) {
+            const int g = p < 0 ? p + N : p;
+            V x = *reinterpret_cast<const V*>(yin + (size_t)g * RB + loff);
+            *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = x;
+        }
+    }
+    __syncthreads();
+
+    float nz[RL];
+#pragma unroll
+    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+
+    for (int cb = vb; cb < ve; cb += T) {
+        // columns of the next chunk: issue the HBM loads now, park them in registers (past the
+        // segment end the last column is loaded again and never stored)
+        float pf[OPW][RL];
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+            const int p = min(cb + T + wave + i * NW, ve - 1);
+            vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
+        }
+
+        int v[OPW];
+        float acc[OPW][RL];
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+            v[i] = min(cb + wave + i * NW, ve - 1);
+#pragma unroll
+            for (int q = 0; q < RL; ++q) acc[i][q] = 0.0f;
+        }
+
+        if (KT == 32) {
+            // all 32 one-byte selectors of every output sit in scalar registers up front
+            uint4 sa[OPW], sb[OPW];
+            float4 w_cur[OPW];
+#pragma unroll
+            for (int i = 0; i < OPW; ++i) {
+                const uint4* sp = reinterpret_cast<const uint4*>(sel + (size_t)v[i] * 8);
+                sa[i] = sp[0];
+                sb[i] = sp[1];
+                if (WMODE) w_cur[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * 32)[0];
+            }
+#pragma unroll
+            for (int m4 = 0; m4 < 8; ++m4) {
+                float4 w_nxt[OPW];
+                if (WMODE && m4 < 7) {
+#pragma unroll
+                    for (int i = 0; i < OPW; ++i)
+                        w_nxt[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * 32)[m4 + 1];
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+#pragma unroll
+                    for (int i = 0; i < OPW; ++i) {
+                        const uint4 sq = m4 < 4 ? sa[i] : sb[i];
+                        const uint32_t sw = (m4 & 3) == 0 ? sq.x : (m4 & 3) == 1 ? sq.y : (m4 & 3) == 2 ? sq.z : sq.w;
+                        const uint32_t slot = (sw >> (8 * b)) & (RING - 1);
+                        V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
+                        float x[RL];
+                        vec_to_arr<RL>(xv, x);
+                        float w = wu;
+                        if (WMODE) w = b == 0 ? w_cur[i].x : b == 1 ? w_cur[i].y : b == 2 ? w_cur[i].z : w_cur[i].w;
+#pragma unroll
+                        for (int q = 0; q < RL; ++q) acc[i][q] = mac<WMODE>(acc[i][q], x[q], w);
+                    }
+                }
+                if (WMODE && m4 < 7) {
+#pragma unroll
+                    for (int i = 0; i < OPW; ++i) w_cur[i] = w_nxt[i];
+                }
+                // pin this trip's arithmetic before the next trip's LDS reads: without it the
+                // compiler issues all 32 reads of every output first and spills the results
+#pragma unroll
+                for (int i = 0; i < OPW; ++i)
+#pragma unroll
+                    for (int q = 0; q < RL; ++q) asm volatile("" : "+v"(acc[i][q]) : : "memory");
+            }
+        } else {
+            const uint32_t* sp[OPW];
+            const float4* wp[OPW];
+            uint32_t s_cur[OPW];
+            float4 w_cur[OPW];
+#pragma unroll
+            for (int i = 0; i < OPW; ++i) {
+                sp[i] = sel + (size_t)v[i] * K4;
+                s_cur[i] = sp[i][0];
+                if (WMODE) {
+                    wp[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * K);
+                    w_cur[i] = wp[i][0];
+                }
+            }
+            // 4 entries of every output per trip; the selectors (and weights) of the next trip
+            // are requested from the scalar cache before this trip's arithmetic starts
+#pragma unroll 1
+            for (int m4 = 0; m4 < K4; ++m4) {
+                uint32_t s_nxt[OPW];
+                float4 w_nxt[OPW];
+                const int mn = min(m4 + 1, K4 - 1);
+#pragma unroll
+                for (int i = 0; i < OPW; ++i) {
+                    s_nxt[i] = sp[i][mn];
+                    if (WMODE) w_nxt[i] = wp[i][mn];
+                }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) {
+#pragma unroll
+                    for (int i = 0; i < OPW; ++i) {
+                        const uint32_t slot = (s_cur[i] >> (8 * b)) & (RING - 1);
+                        V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
+                        float x[RL];
+                        vec_to_arr<RL>(xv, x);
+                        float w = wu;
+                        if (WMODE) w = b == 0 ? w_cur[i].x : b == 1 ? w_cur[i].y : b == 2 ? w_cur[i].z : w_cur[i].w;
+#pragma unroll
+                        for (int q = 0; q < RL; ++q) acc[i][q] = mac<WMODE>(acc[i][q], x[q], w);
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < OPW; ++i) {
+                    s_cur[i] = s_nxt[i];
+                    if (WMODE) w_cur[i] = w_nxt[i];
+                }
+            }
+        }
+
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+            if (cb + wave + i * NW < ve) {
+                float y[RL];
+#pragma unroll
+                for (int q = 0; q < RL; ++q) {
+                    y[q] = relu_clamp(acc[i][q] + bias, clampv);
+                    nz[q] = fmaxf(nz[q], y[q]);
+                }
+                const int d = dst[v[i]];
+                *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
+            }
+        }
+
+        // the parked columns go into ring slots no wave reads during this chunk
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+            const int p = cb + T + wave + i * NW;
+            if (p < ve) *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(pf[i]);
+        }
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int q = 0; q < RL; ++q)
+        if (nz[q] > 0.0f) active[(size_t)rb * RB + loff + q] = stamp;
+}
+
+// ------------------------------------------------------------------------------------------
+// GATHER kernel (general CSR / ELL): any sparsity pattern, any row length.  Each wave takes
+// OPG consecutive outputs of one row block and reads every input column straight from
+// global memory (L2), RB*4 contiguous bytes per read.  No reuse beyond the caches: this is the
+// fallback for layers the inspector cannot relabel into a band.
+// ------------------------------------------------------------------------------------------
+template <int RL, int WMODE>
+__global__ __launch_bounds__(256) void gather_kernel(
+    const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ cols,
+    const int32_t* __restrict__ rowlen, const float* __restrict__ wv, const int32_t* __restrict__ dst,
+    int32_t* __restrict__ active, int N, int kmax, int opg, int stamp, float bias, float clampv) {
+    using V = typename VecOf<RL>::type;
+    constexpr int RB = 64 * RL;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rb = blockIdx.x;
+    const size_t blk = (size_t)rb * (size_t)N * RB;
+    const float* __restrict__ yin = yin_all + blk;
+    float* __restrict__ yout = yout_all + blk;
+    const int loff = lane * RL;
+    const int j0 = (blockIdx.y * 4 + wave) * opg;
+    const int j1 = min(N, j0 + opg);
+
+    float nz[RL];
+#pragma unroll
+    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+
+    for (int j = j0; j < j1; ++j) {
+        const int cnt = rowlen[j];
+        const int32_t* cp = cols + (size_t)j * kmax;
+        const float* wp = wv + (size_t)j * kmax;
+        float acc[RL];
+#pragma unroll
+        for (int q = 0; q < RL; ++q) acc[q] = 0.0f;
+        for (int m = 0; m < cnt; ++m) {
+            const int c = cp[m];
+            const float w = wp[m];
+            V xv = *reinterpret_cast<const V*>(yin + (size_t)c * RB + loff);
+            float x[RL];
+            vec_to_arr<RL>(xv, x);
+#pragma unroll
+            for (int q = 0; q < RL; ++q) acc[q] = mac<WMODE>(acc[q], x[q], w);
+        }
+        float y[RL];
+#pragma unroll
+        for (int q = 0; q < RL; ++q) {
+            y[q] = relu_clamp(acc[q] + bias, clampv);
+            nz[q] = fmaxf(nz[q], y[q]);
+        }
+        *reinterpret_cast<V*>(yout + (size_t)dst[j] * RB + loff) = arr_to_vec<RL>(y);
+    }
+#pragma unroll
+    for (int q = 0; q < RL; ++q)
+        if (nz[q] > 0.0f) active[(size_t)rb * RB + loff + q] = stamp;
+}
+
+// ------------------------------------------------------------------------------------------
+// Active-row scan (one workgroup): wave64 ballot + popcount prefix inside a wave, an LDS scan
+// over the 16 wave totals, a running base across 1024-row chunks.  Stable: survivors keep
+// their order, as the reference's host loop does (all_network.cu:455-463).
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void scan_active_kernel(
+    const int32_t* __restrict__ active, const int32_t* __restrict__ gid, int rows, int stamp,
+    int32_t* __restrict__ count, int32_t* __restrict__ alive_src, int32_t* __restrict__ alive_gid) {
+    __shared__ int wave_tot[16];
+    __shared__ int base_s;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0) base_s = 0;
+    __syncthreads();
+    for (int r0 = 0; r0 < rows; r0 += 1024) {
+        const int r = r0 + threadIdx.x;
+        int g = -1;
+        bool alive = false;
+        if (r < rows) {
+            g = gid[r];
+            alive = (active[r] == stamp) && (g >= 0);
+        }
+        const unsigned long long mask = __ballot(alive);
+        const int before = __popcll(mask & ((1ull << lane) - 1ull));
+        if (lane == 0) wave_tot[wave] = __popcll(mask);
+        __syncthreads();
+        int wbase = 0;
+        for (int w = 0; w < wave; ++w) wbase += wave_tot[w];
+        const int base = base_s;
+        if (alive) {
+            const int k = base + wbase + before;
+            alive_src[k] = r;
+            alive_gid[k] = g;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int t = 0;
+            for (int w = 0; w < 16; ++w) t += wave_tot[w];
+            base_s = base + t;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) count[0] = base_s;
+}
+
+// Repack survivors into dense row blocks.  Thread = destination row slot; loops over a chunk of
+// columns.  Reads are 4-byte gathers (one per surviving row and column), writes are coalesced.
+template <int RL>
+__global__ __launch_bounds__(64 * RL) void repack_kernel(
+    const float* __restrict__ src, float* __restrict__ dstb, const int32_t* __restrict__ count,
+    const int32_t* __restrict__ alive_src, const int32_t* __restrict__ alive_gid,
+    int32_t* __restrict__ gid_out, int N, int cols_per_wg) {
+    constexpr int RB = 64 * RL;
+    const int nb = blockIdx.y;
+    const int slot = nb * RB + threadIdx.x;
+    const int cnt = count[0];
+    const bool live = slot < cnt;
+    const int srow = live ? alive_src[slot] : 0;
+    const size_t sbase = (size_t)(srow / RB) * (size_t)N * RB + (size_t)(srow % RB);
+    const size_t dbase = (size_t)nb * (size_t)N * RB + threadIdx.x;
+    const int c0 = blockIdx.x * cols_per_wg;
+    const int c1 = min(N, c0 + cols_per_wg);
+    for (int c = c0; c < c1; ++c) {
+        const float x = live ? src[sbase + (size_t)c * RB] : 0.0f;
+        dstb[dbase + (size_t)c * RB] = x;
+    }
+    if (blockIdx.x == 0) gid_out[slot] = live ? alive_gid[slot] : -1;
+}
+
+// ------------------------------------------------------------------------------------------
+// Features
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t sm64(uint64_t x) {
+    uint64_t z = x + 0x9E3779B97F4A7C15ULL;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    return z ^ (z >> 31);
+}
+
+// Seeded Bernoulli rows: element (row, c) = hi32(sm64(rk(row) + c)) < thr(row) ? 1 : 0, where
+// rk and thr depend on the seed and the row only.  Thread = row; a workgroup covers one row
+// block and a chunk of physical columns.
+template <int RL>
+__global__ __launch_bounds__(64 * RL) void synth_features_kernel(
+    float* __restrict__ y, const int32_t* __restrict__ col_of_phys, int N, int batch, int cols_per_wg,
+    uint64_t kf, uint64_t lo, uint64_t span) {
+    constexpr int RB = 64 * RL;
+    const int rb = blockIdx.y;
+    const long long row = (long long)rb * RB + threadIdx.x;
+    const bool real = row < batch;
+    const uint64_t rk = sm64(kf + (uint64_t)row);
+    const uint64_t a = sm64(rk + 0xFFFFFFFF00000000ULL) >> 32;
+    uint64_t thr = lo + ((a * span) >> 32);
+    if (thr > 0xFFFFFFFFULL) thr = 0xFFFFFFFFULL;
+    const int c0 = blockIdx.x * cols_per_wg;
+    const int c1 = min(N, c0 + cols_per_wg);
+    const size_t base = (size_t)rb * (size_t)N * RB + threadIdx.x;
+    for (int pc = c0; pc < c1; ++pc) {
+        const int n = col_of_phys[pc];
+        const uint32_t e = (uint32_t)(sm64(rk + (uint64_t)n) >> 32);
+        y[base + (size_t)pc * RB] = (real && e < (uint32_t)thr) ? 1.0f : 0.0f;
+    }
+}
+
+// Row-major chunk -> row-block layout, 32 columns x RB rows per workgroup through an LDS tile.
+template <int RL>
+__global__ __launch_bounds__(256) void pack_rows_kernel(
+    const float* __restrict__ rowmajor, float* __restrict__ y, const int32_t* __restrict__ phys_of_col,
+    int N, long long row0, int nrows, int32_t* __restrict__ nonfinite) {
+    constexpr int RB = 64 * RL;
+    __shared__ float tile[RB][33];
+    const int n0 = blockIdx.x * 32;
+    const int lb = blockIdx.y;  // row block inside the chunk
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    bool bad = false;
+    for (int rr = ty; rr < RB; rr += 8) {
+        const int lr = lb * RB + rr;
+        float x = 0.0f;
+        if (lr < nrows && n0 + tx < N) x = rowmajor[(size_t)lr * N + n0 + tx];
+        if (!(fabsf(x) <= 3.4028234e38f)) bad = true;
+        tile[rr][tx] = x;
+    }
+    if (bad) nonfinite[0] = 1;
+    __syncthreads();
+    const size_t blk = ((size_t)(row0 / RB) + lb) * (size_t)N * RB;
+    for (int idx = threadIdx.x; idx < 32 * RB; idx += 256) {
+        const int c = idx / RB, r = idx % RB;
+        if (n0 + c < N) y[blk + (size_t)phys_of_col[n0 + c] * RB + r] = tile[r][c];
+    }
+}
+
+__global__ void unpack_rows_kernel(const float* __restrict__ y, const int32_t* __restrict__ phys_of_col,
+                                   const int32_t* __restrict__ phys_rows, int N, int RB,
+                                   float* __restrict__ rowmajor) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    const int pr = phys_rows[blockIdx.y];
+    float x = 0.0f;
+    if (pr >= 0) {
+        const int pc = phys_of_col ? phys_of_col[n] : n;
+        x = y[((size_t)(pr / RB) * (size_t)N + (size_t)pc) * RB + (pr % RB)];
+    }
+    rowmajor[(size_t)blockIdx.y * N + n] = x;
+}
+
+__global__ void fill_i32_kernel(int32_t* p, long long n, int32_t v) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+__global__ void iota_gid_kernel(int32_t* gid, int rows, int batch) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < rows) gid[i] = i < batch ? i : -1;
+}
+
+__global__ __launch_bounds__(256) void copy_f4_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
+                                                      long long n4) {
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) dst[i] = src[i];
+}
+
+// Segment length for the band walk: a multiple of the chunk T.  More segments fill the 256 CUs
+// more evenly (one workgroup per CU at a time: the ring takes most of the LDS), fewer segments
+// load fewer halo columns; score both and take the best.
+int choose_seglen(int N, int K, int T, int nblk, int n_cu) {
+    const int nchunks = (N + T - 1) / T;
+    int best_len = nchunks * T;
+    double best = -1.0;
+    for (int cps = nchunks; cps >= 1; --cps) {  // chunks per segment
+        const int nseg = (nchunks + cps - 1) / cps;
+        if (nseg > 65535) break;
+        const long long wgs = (long long)nblk * nseg;
+        const long long rounds = (wgs + n_cu - 1) / n_cu;
+        const double fill = (double)wgs / (double)(rounds * n_cu);
+        const double halo = 1.0 / (1.0 + 0.25 * (double)(K - 1) / (double)(cps * T));
+        // a round costs cps chunks (+ prologue); prefer fuller rounds, then fewer halos
+        const double score = fill * halo;
+        if (score > best + 1e-9) { best = score; best_len = cps * T; }
+    }
+    return best_len;
+}
+
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
+    constexpr int T = NW * OPW;
+    constexpr size_t lds = (size_t)RING * 64 * RL * 4;
+    auto kern = band_walk_kernel<RL, NW, OPW, RING, WMODE, KT>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    const int seglen = choose_seglen(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256);
+    const int nseg = (a.N + seglen - 1) / seglen;
+    dim3 grid(a.nblk, nseg), block(NW * 64);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.N, a.K,
+                       seglen, a.stamp, a.wu, a.bias, a.clampv);
+    return hipGetLastError();
+}
+
+template <int RL, int NW, int OPW, int RING>
+hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
+    if (a.K == 32) {
+        switch (a.wmode) {
+            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 32>(a, s);
+            case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 32>(a, s);
+            default: return launch_band_inst<RL, NW, OPW, RING, 2, 32>(a, s);
+        }
+    }
+    switch (a.wmode) {
+        case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 0>(a, s);
+        case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 0>(a, s);
+        default: return launch_band_inst<RL, NW, OPW, RING, 2, 0>(a, s);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
+    // host-side shape checks: what the kernel and its grid assume
+    if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
+        !a.yin || !a.yout || !a.sel || !a.dst || !a.active || (a.wmode != 0 && !a.wv))
+        return hipErrorInvalidValue;
+    switch (a.rl) {
+        case 4: return launch_band_rl<4, 16, 3, 128>(a, s);
+        case 2: return launch_band_rl<2, 16, 7, 256>(a, s);
+        case 1: return launch_band_rl<1, 16, 7, 256>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
+    if (a.N <= 0 || a.kmax < 0 || a.nblk <= 0 || !a.yin || !a.yout || !a.cols || !a.rowlen || !a.wv ||
+        !a.dst || !a.active)
+        return hipErrorInvalidValue;
+    const int opg = 8;
+    dim3 grid(a.nblk, (a.N + 4 * opg - 1) / (4 * opg)), block(256);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+#define SPDNN_GATHER(RLv, WM)                                                                         \
+    hipLaunchKernelGGL((gather_kernel<RLv, WM>), grid, block, 0, s, a.yin, a.yout, a.cols, a.rowlen,  \
+                       a.wv, a.dst, a.active, a.N, a.kmax, opg, a.stamp, a.bias, a.clampv)
+    const bool exact = a.wmode != 2;
+    switch (a.rl) {
+        case 4: if (exact) SPDNN_GATHER(4, 1); else SPDNN_GATHER(4, 2); break;
+        case 2: if (exact) SPDNN_GATHER(2, 1); else SPDNN_GATHER(2, 2); break;
+        case 1: if (exact) SPDNN_GATHER(1, 1); else SPDNN_GATHER(1, 2); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef SPDNN_GATHER
+    return hipGetLastError();
+}
+
+hipError_t launch_scan_active(const int32_t* active, const int32_t* gid, int rows, int stamp, int32_t* count,
+                              int32_t* alive_src, int32_t* alive_gid, hipStream_t s) {
+    if (rows < 0 || !active || !gid || !count || !alive_src || !alive_gid) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(scan_active_kernel, dim3(1), dim3(1024), 0, s, active, gid, rows, stamp, count,
+                       alive_src, alive_gid);
+    return hipGetLastError();
+}
+
+hipError_t launch_repack(const float* src, float* dst, const int32_t* count, const int32_t* alive_src,
+                         const int32_t* alive_gid, int32_t* gid_out, int N, int rl, int dst_blocks,
+                         hipStream_t s) {
+    if (dst_blocks <= 0 || dst_blocks > 65535 || N <= 0) return hipErrorInvalidValue;
+    const int cpw = 64;
+    dim3 grid((N + cpw - 1) / cpw, dst_blocks);
+    switch (rl) {
+        case 4: hipLaunchKernelGGL(repack_kernel<4>, grid, dim3(256), 0, s, src, dst, count, alive_src, alive_gid, gid_out, N, cpw); break;
+        case 2: hipLaunchKernelGGL(repack_kernel<2>, grid, dim3(128), 0, s, src, dst, count, alive_src, alive_gid, gid_out, N, cpw); break;
+        case 1: hipLaunchKernelGGL(repack_kernel<1>, grid, dim3(64), 0, s, src, dst, count, alive_src, alive_gid, gid_out, N, cpw); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_synth_features(float* y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
+                                 uint64_t seed, float dmin, float dmax, hipStream_t s) {
+    if (nblk <= 0 || nblk > 65535 || N <= 0) return hipErrorInvalidValue;
+    // host side of the generator definition: keys and the density range as 32.32 fixed point
+    auto h = [](uint64_t x) {
+        uint64_t z = x + 0x9E3779B97F4A7C15ULL;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+        return z ^ (z >> 31);
+    };
+    const uint64_t kf = h(seed ^ 0x46454154ULL);
+    const uint64_t lo = (uint64_t)((double)dmin * 4294967296.0);
+    const uint64_t span = (uint64_t)(((double)dmax - (double)dmin) * 4294967296.0);
+    const int cpw = 64;
+    dim3 grid((N + cpw - 1) / cpw, nblk);
+    switch (rl) {
+        case 4: hipLaunchKernelGGL(synth_features_kernel<4>, grid, dim3(256), 0, s, y, col_of_phys, N, batch, cpw, kf, lo, span); break;
+        case 2: hipLaunchKernelGGL(synth_features_kernel<2>, grid, dim3(128), 0, s, y, col_of_phys, N, batch, cpw, kf, lo, span); break;
+        case 1: hipLaunchKernelGGL(synth_features_kernel<1>, grid, dim3(64), 0, s, y, col_of_phys, N, batch, cpw, kf, lo, span); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys_of_col, int N, int64_t row0,
+                            int nrows, int rl, int32_t* nonfinite, hipStream_t s) {
+    const int RB = 64 * rl;
+    if (nrows <= 0 || N <= 0 || (row0 % RB) != 0) return hipErrorInvalidValue;
+    const int nb = (nrows + RB - 1) / RB;
+    if (nb > 65535) return hipErrorInvalidValue;
+    dim3 grid((N + 31) / 32, nb);
+    switch (rl) {
+        case 4: hipLaunchKernelGGL(pack_rows_kernel<4>, grid, dim3(256), 0, s, rowmajor, y, phys_of_col, N, (long long)row0, nrows, nonfinite); break;
+        case 2: hipLaunchKernelGGL(pack_rows_kernel<2>, grid, dim3(256), 0, s, rowmajor, y, phys_of_col, N, (long long)row0, nrows, nonfinite); break;
+        case 1: hipLaunchKernelGGL(pack_rows_kernel<1>, grid, dim3(256), 0, s, rowmajor, y, phys_of_col, N, (long long)row0, nrows, nonfinite); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows, int nreq,
+                              int N, int rl, float* rowmajor, hipStream_t s) {
+    if (nreq <= 0 || nreq > 65535 || N <= 0) return hipErrorInvalidValue;
+    dim3 grid((N + 255) / 256, nreq);
+    hipLaunchKernelGGL(unpack_rows_kernel, grid, dim3(256), 0, s, y, phys_of_col, phys_rows, N, 64 * rl, rowmajor);
+    return hipGetLastError();
+}
+
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s) {
+    if (n <= 0) return hipSuccess;
+    const int blocks = (int)std::min<int64_t>((n + 255) / 256, 4096);
+    hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, s, p, (long long)n, v);
+    return hipGetLastError();
+}
+
+hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s) {
+    if (rows <= 0) return hipSuccess;
+    hipLaunchKernelGGL(iota_gid_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, gid, rows, batch);
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s) {
+    if (n_floats <= 0 || (n_floats % 4) != 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(copy_f4_kernel, dim3(256 * 16), dim3(256), 0, s, reinterpret_cast<const float4*>(src),
+                       reinterpret_cast<float4*>(dst), (long long)(n_floats / 4));
+    return hipGetLastError();
+}
+
+}  // namespace spdnn

@@ -1,0 +1,77 @@
+// Launch wrappers of the gfx950 kernels (kernels.hip).  Everything here takes device pointers.
+//
+// Feature layout in HBM ("row-block layout"): rows are grouped in blocks of RB = 64*RL rows
+// (RL = rows per lane, 1, 2 or 4); inside a block the matrix is column-major:
+//
+//     Y[(block * N + column) * RB + row_in_block]        (fp32)
+//
+// so one neuron column of one row block is RB*4 contiguous bytes (256 B .. 1 KiB), the unit
+// every kernel loads, stores, gathers and scatters.  A wavefront owns one row block; lane i
+// holds rows i*RL .. i*RL+RL-1, indices and weights are wave-uniform scalars.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace spdnn {
+
+struct BandLaunch {
+    const float* yin;        // input buffer (row-block layout, labelled by the layer's band order)
+    float* yout;             // output buffer (labelled for the next layer through dst)
+    const uint32_t* sel;     // [N][K/4] packed ring selectors in accumulation order
+    const float* wv;         // [N][K] weights in accumulation order, or nullptr (uniform exact value)
+    const int32_t* dst;      // [N] physical output column per band position
+    int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
+    int N, K, nblk, stamp, rl;
+    int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
+    float wu, bias, clampv;
+    int n_cu;
+};
+
+struct GatherLaunch {
+    const float* yin;
+    float* yout;
+    const int32_t* cols;     // [N][kmax] physical input columns in accumulation order
+    const int32_t* rowlen;   // [N]
+    const float* wv;         // [N][kmax]
+    const int32_t* dst;      // [N]
+    int32_t* active;
+    int N, kmax, nblk, stamp, rl;
+    int wmode;               // 1 fma (exact products), 2 mul then add
+    float bias, clampv;
+};
+
+hipError_t launch_band(const BandLaunch& a, hipStream_t s);
+hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
+
+// Active-row scan: rows with active[row] == stamp and gid[row] >= 0 survive, in order.
+// Writes count[0] = number of survivors, alive_src[k] = physical row of survivor k,
+// alive_gid[k] = its global id.
+hipError_t launch_scan_active(const int32_t* active, const int32_t* gid, int rows, int stamp,
+                              int32_t* count, int32_t* alive_src, int32_t* alive_gid, hipStream_t s);
+
+// Repack: row slot k of the destination takes physical row alive_src[k] of the source for
+// k < count[0]; the remaining slots of the last block are zero-filled; gid_out likewise (-1).
+hipError_t launch_repack(const float* src, float* dst, const int32_t* count, const int32_t* alive_src,
+                         const int32_t* alive_gid, int32_t* gid_out, int N, int rl, int dst_blocks,
+                         hipStream_t s);
+
+// Seeded Bernoulli features written straight into the row-block layout; col_of_phys maps a
+// physical column to its neuron.
+hipError_t launch_synth_features(float* y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
+                                 uint64_t seed, float dmin, float dmax, hipStream_t s);
+
+// Row-major chunk [nrows][N] (nrows rows starting at row0, row0 a multiple of RB) into the
+// row-block layout with column labelling phys_of_col; rows >= batch are zero.  nonfinite[0] is
+// set to 1 if a value is NaN or infinite.
+hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys_of_col, int N,
+                            int64_t row0, int nrows, int rl, int32_t* nonfinite, hipStream_t s);
+
+// Row-block layout to row-major for a list of physical rows (-1 gives a zero row).
+hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows,
+                              int nreq, int N, int rl, float* rowmajor, hipStream_t s);
+
+hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
+hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s);
+hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s);
+
+}  // namespace spdnn

@@ -1,0 +1,822 @@
+// C ABI of the library (include/spdnn.h): host orchestration around the kernels.
+//
+// The layer loop mirrors test_benchmark_graph_challenge (reference
+// src/microbenchmark/all_network.cu:207-526) with these differences: weights arrive as CSR and
+// go through the inspector behind the boundary; the active-row scan and the repack run on the
+// device (the reference copies the flags to the host and scans them there,
+// all_network.cu:444-513); the input features are kept untouched so a run can be repeated.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <atomic>
+#include <cmath>
+#include <condition_variable>
+#include <cstdio>
+#include <cstring>
+#include <deque>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "../../include/spdnn.h"
+#include "inspector.hpp"
+#include "kernels.hpp"
+#include "synth.hpp"
+#include "tsv_io.hpp"
+
+using namespace spdnn;
+
+namespace {
+
+thread_local std::string g_err = "";
+
+int fail(int code, const std::string& msg) {
+    g_err = msg;
+    return code;
+}
+
+#define HIPCHK(expr)                                                                                 \
+    do {                                                                                             \
+        hipError_t e_ = (expr);                                                                      \
+        if (e_ != hipSuccess)                                                                        \
+            return fail(SPDNN_E_DEVICE, std::string(#expr) + ": " + hipGetErrorString(e_));         \
+    } while (0)
+
+// Small worker pool for the per-layer inspector jobs (bounded queue so that pending CSR copies
+// stay small).
+class JobPool {
+  public:
+    explicit JobPool(int nthreads) {
+        for (int i = 0; i < nthreads; ++i) workers_.emplace_back([this] { loop(); });
+    }
+    ~JobPool() {
+        {
+            std::unique_lock<std::mutex> lk(m_);
+            stop_ = true;
+        }
+        cv_job_.notify_all();
+        for (auto& t : workers_) t.join();
+    }
+    void submit(std::function<void()> f) {
+        std::unique_lock<std::mutex> lk(m_);
+        cv_room_.wait(lk, [this] { return q_.size() < 2 * workers_.size() + 2; });
+        q_.push_back(std::move(f));
+        ++pending_;
+        cv_job_.notify_one();
+    }
+    void wait_all() {
+        std::unique_lock<std::mutex> lk(m_);
+        cv_done_.wait(lk, [this] { return pending_ == 0; });
+    }
+
+  private:
+    void loop() {
+        for (;;) {
+            std::function<void()> f;
+            {
+                std::unique_lock<std::mutex> lk(m_);
+                cv_job_.wait(lk, [this] { return stop_ || !q_.empty(); });
+                if (q_.empty()) return;
+                f = std::move(q_.front());
+                q_.pop_front();
+                cv_room_.notify_one();
+            }
+            f();
+            {
+                std::unique_lock<std::mutex> lk(m_);
+                if (--pending_ == 0) cv_done_.notify_all();
+            }
+        }
+    }
+    std::vector<std::thread> workers_;
+    std::deque<std::function<void()>> q_;
+    std::mutex m_;
+    std::condition_variable cv_job_, cv_room_, cv_done_;
+    size_t pending_ = 0;
+    bool stop_ = false;
+};
+
+int host_threads() {
+    const char* e = getenv("SPDNN_HOST_THREADS");
+    int n = e ? atoi(e) : 0;
+    if (n <= 0) {
+        n = (int)std::thread::hardware_concurrency();
+        const char* omp = getenv("OMP_NUM_THREADS");
+        if (omp && atoi(omp) > 0) n = std::min(n > 0 ? n : 16, atoi(omp));
+    }
+    return std::max(1, std::min(n, 32));
+}
+
+struct DevLayer {
+    int32_t* in_pos = nullptr;
+    uint32_t* sel = nullptr;
+    int32_t* ell = nullptr;
+    int32_t* rowlen = nullptr;
+    float* wv = nullptr;
+    int32_t* dst = nullptr;
+};
+
+}  // namespace
+
+struct spdnn_net {
+    int N = 0, max_batch = 0, L = 0;
+    float bias = 0.0f, clampv = 32.0f;
+    int rl = 4, RB = 256;
+    int rows_cap = 0;
+    int force_kernel = SPDNN_KERNEL_AUTO;
+    std::vector<LayerPlan> layers;
+    std::unique_ptr<JobPool> pool;
+    std::mutex err_m;
+    std::string worker_err;
+    bool inspected = false;
+
+    // device
+    bool dev_ready = false, uploaded = false;
+    int n_cu = 256;
+    hipStream_t stream = nullptr;
+    void* arena = nullptr;
+    std::vector<DevLayer> dl;
+    float *F = nullptr, *A = nullptr, *C = nullptr;
+    int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
+    int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
+    int32_t* h_count = nullptr;  // pinned
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    std::vector<hipEvent_t> ev_layer;
+
+    // state
+    int batch = 0;
+    bool have_features = false;
+    float* cur = nullptr;
+    int cur_layer = 0;
+    int carried = 0;
+    int stamp = 0;
+    int64_t alive = 0;        // rows active after the last layer run
+    bool alive_list_valid = false;
+    bool gid_dirty = false;   // a repack permuted d_gid since it was last initialised
+    std::vector<char> pending; // layer has an inspection job in flight
+    std::vector<int64_t> counts;
+    std::vector<float> layer_ms;
+};
+
+namespace {
+
+int ensure_device(spdnn_net* n) {
+    if (n->dev_ready) return SPDNN_OK;
+    int cnt = 0;
+    hipError_t e = hipGetDeviceCount(&cnt);
+    if (e != hipSuccess || cnt < 1) return fail(SPDNN_E_DEVICE, "no HIP device available");
+    HIPCHK(hipSetDevice(0));
+    hipDeviceProp_t p;
+    HIPCHK(hipGetDeviceProperties(&p, 0));
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return fail(SPDNN_E_DEVICE, std::string("kernels are built for gfx950, device is ") + p.gcnArchName);
+    n->n_cu = p.multiProcessorCount;
+    HIPCHK(hipStreamCreate(&n->stream));
+    HIPCHK(hipEventCreate(&n->ev_start));
+    HIPCHK(hipEventCreate(&n->ev_stop));
+    const size_t rows = (size_t)n->rows_cap;
+    HIPCHK(hipMalloc(&n->d_active, rows * 4));
+    HIPCHK(hipMalloc(&n->d_gid, rows * 4));
+    HIPCHK(hipMalloc(&n->d_gid_tmp, rows * 4));
+    HIPCHK(hipMalloc(&n->d_alive_src, rows * 4));
+    HIPCHK(hipMalloc(&n->d_alive_gid, rows * 4));
+    HIPCHK(hipMalloc(&n->d_count, 64));
+    HIPCHK(hipMalloc(&n->d_nonfinite, 64));
+    HIPCHK(hipHostMalloc(&n->h_count, 64));
+    HIPCHK(hipMemset(n->d_active, 0, rows * 4));
+    n->dev_ready = true;
+    return SPDNN_OK;
+}
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int ensure_uploaded(spdnn_net* n) {
+    if (n->uploaded) return SPDNN_OK;
+    if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
+    int rc = ensure_device(n);
+    if (rc) return rc;
+    size_t total = 0;
+    for (const LayerPlan& p : n->layers) {
+        total += align256(p.in_pos.size() * 4) + align256(p.sel.size()) + align256(p.ell_col.size() * 4) +
+                 align256(p.rowlen.size() * 4) + align256(p.wv.size() * 4) + align256(p.dst.size() * 4);
+    }
+    HIPCHK(hipMalloc(&n->arena, std::max<size_t>(total, 256)));
+    n->dl.assign((size_t)n->L, DevLayer{});
+    char* base = (char*)n->arena;
+    size_t off = 0;
+    auto put = [&](const void* src, size_t bytes, void** dptr) -> hipError_t {
+        if (bytes == 0) { *dptr = nullptr; return hipSuccess; }
+        *dptr = base + off;
+        off += align256(bytes);
+        return hipMemcpy(*dptr, src, bytes, hipMemcpyHostToDevice);
+    };
+    for (int l = 0; l < n->L; ++l) {
+        const LayerPlan& p = n->layers[(size_t)l];
+        DevLayer& d = n->dl[(size_t)l];
+        HIPCHK(put(p.in_pos.data(), p.in_pos.size() * 4, (void**)&d.in_pos));
+        HIPCHK(put(p.sel.data(), p.sel.size(), (void**)&d.sel));
+        HIPCHK(put(p.ell_col.data(), p.ell_col.size() * 4, (void**)&d.ell));
+        HIPCHK(put(p.rowlen.data(), p.rowlen.size() * 4, (void**)&d.rowlen));
+        HIPCHK(put(p.wv.data(), p.wv.size() * 4, (void**)&d.wv));
+        HIPCHK(put(p.dst.data(), p.dst.size() * 4, (void**)&d.dst));
+    }
+    const size_t fbytes = (size_t)n->rows_cap * (size_t)n->N * 4;
+    HIPCHK(hipMalloc(&n->F, fbytes));
+    HIPCHK(hipMalloc(&n->A, fbytes));
+    HIPCHK(hipMalloc(&n->C, fbytes));
+    n->uploaded = true;
+    return SPDNN_OK;
+}
+
+void free_device(spdnn_net* n) {
+    if (n->arena) hipFree(n->arena);
+    if (n->F) hipFree(n->F);
+    if (n->A) hipFree(n->A);
+    if (n->C) hipFree(n->C);
+    n->arena = nullptr; n->F = n->A = n->C = nullptr;
+    n->uploaded = false;
+    n->have_features = false;
+}
+
+// physical-column labelling of the buffer that holds the state after `layers_done` layers
+const int32_t* labelling_dev(const spdnn_net* n, int layers_done) {
+    return layers_done < n->L ? n->dl[(size_t)layers_done].in_pos : nullptr;  // nullptr = identity
+}
+
+void reset_state(spdnn_net* n) {
+    if (n->gid_dirty) {
+        launch_iota_gid(n->d_gid, n->rows_cap, n->batch, n->stream);
+        n->gid_dirty = false;
+    }
+    n->cur = n->F;
+    n->cur_layer = 0;
+    n->carried = ((n->batch + n->RB - 1) / n->RB) * n->RB;
+    n->alive = n->batch;
+    n->alive_list_valid = false;
+}
+
+int submit_layer(spdnn_net* n, int layer, std::shared_ptr<std::vector<int32_t>> rp,
+                 std::shared_ptr<std::vector<int32_t>> col, std::shared_ptr<std::vector<float>> val) {
+    n->inspected = false;
+    const int force = n->force_kernel;
+    const int N = n->N;
+    LayerPlan* plan = &n->layers[(size_t)layer];
+    n->pool->submit([=] { inspect_layer(N, *rp, *col, *val, force, *plan); });
+    return SPDNN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int spdnn_version(void) { return 100; }
+
+const char* spdnn_last_error(void) { return g_err.c_str(); }
+
+int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp, spdnn_net** out) {
+    if (!out) return fail(SPDNN_E_ARG, "out is NULL");
+    *out = nullptr;
+    if (neuron < 1 || neuron > (1 << 24)) return fail(SPDNN_E_ARG, "neuron must be in [1, 2^24]");
+    if (max_batch < 1) return fail(SPDNN_E_ARG, "max_batch must be positive");
+    if (layers < 1) return fail(SPDNN_E_ARG, "layers must be positive");
+    if (!std::isfinite(bias) || !(clamp > 0.0f) || !std::isfinite(clamp))
+        return fail(SPDNN_E_ARG, "bias must be finite and clamp positive");
+    spdnn_net* n = new (std::nothrow) spdnn_net();
+    if (!n) return fail(SPDNN_E_NOMEM, "out of host memory");
+    n->N = neuron; n->max_batch = max_batch; n->L = layers; n->bias = bias; n->clampv = clamp;
+    int rl = 4;
+    if (const char* e = getenv("SPDNN_ROWS_PER_LANE")) rl = atoi(e);
+    if (rl != 1 && rl != 2 && rl != 4) { delete n; return fail(SPDNN_E_ARG, "SPDNN_ROWS_PER_LANE must be 1, 2 or 4"); }
+    n->rl = rl; n->RB = 64 * rl;
+    n->rows_cap = ((max_batch + n->RB - 1) / n->RB) * n->RB;
+    n->layers.resize((size_t)layers);
+    n->pending.assign((size_t)layers, 0);
+    n->counts.assign((size_t)layers, -1);
+    n->layer_ms.assign((size_t)layers, 0.0f);
+    n->pool.reset(new JobPool(host_threads()));
+    *out = n;
+    return SPDNN_OK;
+}
+
+int spdnn_destroy(spdnn_net* n) {
+    if (!n) return SPDNN_OK;
+    n->pool->wait_all();
+    n->pool.reset();
+    if (n->dev_ready) {
+        hipStreamSynchronize(n->stream);
+        free_device(n);
+        hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp); hipFree(n->d_alive_src);
+        hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
+        hipHostFree(n->h_count);
+        for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
+        hipEventDestroy(n->ev_start); hipEventDestroy(n->ev_stop);
+        hipStreamDestroy(n->stream);
+    }
+    delete n;
+    return SPDNN_OK;
+}
+
+int spdnn_reference_bias(int neuron, float* bias) {
+    if (!bias) return fail(SPDNN_E_ARG, "bias is NULL");
+    switch (neuron) {
+        case 1024: *bias = -0.3f; return SPDNN_OK;
+        case 4096: *bias = -0.35f; return SPDNN_OK;
+        case 16384: *bias = -0.4f; return SPDNN_OK;
+        case 65536: *bias = -0.45f; return SPDNN_OK;
+        default: return fail(SPDNN_E_ARG, "no reference bias for this neuron count");
+    }
+}
+
+int spdnn_set_force_kernel(spdnn_net* n, int kernel) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (kernel != SPDNN_KERNEL_AUTO && kernel != SPDNN_KERNEL_GATHER)
+        return fail(SPDNN_E_ARG, "only AUTO or GATHER can be forced");
+    for (const LayerPlan& p : n->layers)
+        if (p.set) return fail(SPDNN_E_STATE, "set the forced kernel before any layer");
+    n->force_kernel = kernel;
+    return SPDNN_OK;
+}
+
+int spdnn_set_layer_csr(spdnn_net* n, int layer, const int32_t* rowptr, const int32_t* col, const float* val) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    auto rp = std::make_shared<std::vector<int32_t>>();
+    auto cc = std::make_shared<std::vector<int32_t>>();
+    auto vv = std::make_shared<std::vector<float>>();
+    const std::string err = normalize_csr(n->N, rowptr, col, val, *rp, *cc, *vv);
+    if (!err.empty()) return fail(SPDNN_E_ARG, err);
+    if (n->pending[(size_t)layer]) {  // the layer is being replaced: never race with its earlier job
+        n->pool->wait_all();
+        std::fill(n->pending.begin(), n->pending.end(), 0);
+    }
+    n->pending[(size_t)layer] = 1;
+    return submit_layer(n, layer, rp, cc, vv);
+}
+
+int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
+    if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    std::vector<int32_t> rp, cc;
+    std::vector<float> vv;
+    std::string err;
+    if (!read_weight_tsv_csr(path, n->N, rp, cc, vv, err)) return fail(SPDNN_E_IO, err);
+    return spdnn_set_layer_csr(n, layer, rp.data(), cc.data(), vv.data());
+}
+
+int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap) {
+    if (!data_dir || !out || cap < 1) return fail(SPDNN_E_ARG, "NULL argument");
+    const int w = snprintf(out, (size_t)cap, "%s/neuron%d/n%d-l%d.tsv", data_dir, neuron, neuron, layer + 1);
+    if (w < 0 || w >= cap) return fail(SPDNN_E_ARG, "buffer too small");
+    return SPDNN_OK;
+}
+
+int spdnn_synth_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row, float value,
+                          int32_t* rowptr, int32_t* col, float* val) {
+    if (!rowptr || !col || !val) return fail(SPDNN_E_ARG, "NULL argument");
+    std::vector<int32_t> rp, cc;
+    std::vector<float> vv;
+    if (!synth_layer_csr(seed, layer, neuron, nnz_per_row, value, rp, cc, vv))
+        return fail(SPDNN_E_ARG, "bad generator arguments");
+    std::copy(rp.begin(), rp.end(), rowptr);
+    std::copy(cc.begin(), cc.end(), col);
+    std::copy(vv.begin(), vv.end(), val);
+    return SPDNN_OK;
+}
+
+int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nnz_per_row, float value) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
+    if (nnz_per_row < 1 || nnz_per_row > n->N || !std::isfinite(value))
+        return fail(SPDNN_E_ARG, "bad nnz_per_row or value");
+    n->pool->wait_all();
+    std::fill(n->pending.begin(), n->pending.end(), 0);
+    n->inspected = false;
+    const int N = n->N, force = n->force_kernel;
+    for (int l = first; l < first + count; ++l) {
+        n->pending[(size_t)l] = 1;
+        LayerPlan* plan = &n->layers[(size_t)l];
+        n->pool->submit([=] {
+            std::vector<int32_t> rp, cc;
+            std::vector<float> vv;
+            synth_layer_csr(seed, l, N, nnz_per_row, value, rp, cc, vv);
+            inspect_layer(N, rp, cc, vv, force, *plan);
+        });
+    }
+    return SPDNN_OK;
+}
+
+int spdnn_inspect(spdnn_net* n) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    n->pool->wait_all();
+    std::fill(n->pending.begin(), n->pending.end(), 0);
+    for (int l = 0; l < n->L; ++l)
+        if (!n->layers[(size_t)l].set) return fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
+    for (int l = 0; l < n->L; ++l) {
+        LayerPlan* cur = &n->layers[(size_t)l];
+        const std::vector<int32_t>* nxt = l + 1 < n->L ? &n->layers[(size_t)l + 1].in_pos : nullptr;
+        n->pool->submit([=] { link_layers(*cur, nxt); });
+    }
+    n->pool->wait_all();
+    if (n->uploaded) free_device(n);  // plans changed: upload again on next use
+    n->inspected = true;
+    return SPDNN_OK;
+}
+
+int spdnn_get_layer_plan(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
+    if (!n || !out) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    if (!n->layers[(size_t)layer].set) return fail(SPDNN_E_STATE, "layer has not been set");
+    *out = n->layers[(size_t)layer].info;
+    return SPDNN_OK;
+}
+
+int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    const LayerPlan& p = n->layers[(size_t)layer];
+    if (!p.set || p.kernel != SPDNN_KERNEL_BAND) return fail(SPDNN_E_STATE, "not a BAND layer");
+    if (in_pos) std::copy(p.in_pos.begin(), p.in_pos.end(), in_pos);
+    if (out_at) std::copy(p.out_at.begin(), p.out_at.end(), out_at);
+    if (sel) std::copy(p.sel.begin(), p.sel.end(), sel);
+    return SPDNN_OK;
+}
+
+int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
+    if (!n || !dst) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
+    const LayerPlan& p = n->layers[(size_t)layer];
+    std::copy(p.dst.begin(), p.dst.end(), dst);
+    return SPDNN_OK;
+}
+
+int spdnn_get_input_labelling(const spdnn_net* n, int layer, int32_t* phys_col) {
+    if (!n || !phys_col) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer > n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    if (layer == n->L) {
+        for (int i = 0; i < n->N; ++i) phys_col[i] = i;
+        return SPDNN_OK;
+    }
+    const LayerPlan& p = n->layers[(size_t)layer];
+    if (!p.set) return fail(SPDNN_E_STATE, "layer has not been set");
+    std::copy(p.in_pos.begin(), p.in_pos.end(), phys_col);
+    return SPDNN_OK;
+}
+
+int spdnn_hash_reorder(int v, int buckets, int domain, int* out) {
+    if (!out) return fail(SPDNN_E_ARG, "out is NULL");
+    if (buckets <= 0 || domain <= 0 || v < 0 || v >= domain) return fail(SPDNN_E_ARG, "ERROR: Hasing Function error!");
+    const int width = domain / buckets;
+    *out = v / buckets + (v % buckets) * width;
+    return SPDNN_OK;
+}
+
+// ---- features ----------------------------------------------------------------------------
+
+static int begin_features(spdnn_net* n, int batch) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
+    int rc = ensure_uploaded(n);
+    if (rc) return rc;
+    n->batch = batch;
+    n->have_features = false;
+    return SPDNN_OK;
+}
+
+int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
+    if (!rowmajor) return fail(SPDNN_E_ARG, "rowmajor is NULL");
+    int rc = begin_features(n, batch);
+    if (rc) return rc;
+    const int RB = n->RB, N = n->N;
+    // staging chunk: a whole number of row blocks, about 256 MiB
+    int64_t chunk_rows = std::max<int64_t>(RB, ((int64_t)(256 << 20) / ((int64_t)N * 4)) / RB * RB);
+    chunk_rows = std::min<int64_t>(chunk_rows, n->rows_cap);
+    float* stage = nullptr;
+    HIPCHK(hipMalloc(&stage, (size_t)chunk_rows * N * 4));
+    HIPCHK(hipMemsetAsync(n->d_nonfinite, 0, 4, n->stream));
+    const int padded = ((batch + RB - 1) / RB) * RB;
+    for (int64_t r0 = 0; r0 < padded; r0 += chunk_rows) {
+        const int64_t rows_here = std::min<int64_t>(chunk_rows, padded - r0);
+        const int64_t real = std::max<int64_t>(0, std::min<int64_t>(rows_here, batch - r0));
+        if (real > 0) {
+            hipError_t e = hipMemcpyAsync(stage, rowmajor + (size_t)r0 * N, (size_t)real * N * 4,
+                                          hipMemcpyHostToDevice, n->stream);
+            if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
+        }
+        // rows >= real inside the chunk are written as zero by the kernel (nrows = real)
+        hipError_t e = launch_pack_rows(stage, n->F, n->dl[0].in_pos, N, r0, (int)std::max<int64_t>(real, 1),
+                                        n->rl, n->d_nonfinite, n->stream);
+        if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
+        e = hipStreamSynchronize(n->stream);
+        if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
+    }
+    int32_t bad = 0;
+    hipError_t e = hipMemcpy(&bad, n->d_nonfinite, 4, hipMemcpyDeviceToHost);
+    hipFree(stage);
+    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    if (bad) return fail(SPDNN_E_ARG, "features contain NaN or infinity");
+    HIPCHK(launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream));
+    HIPCHK(hipStreamSynchronize(n->stream));
+    n->have_features = true;
+    reset_state(n);
+    return SPDNN_OK;
+}
+
+int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
+    if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
+    if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
+    std::vector<float> dense;
+    std::string err;
+    int64_t kept = 0;
+    if (!read_features_tsv_dense(path, n->N, batch, dense, &kept, err)) return fail(SPDNN_E_IO, err);
+    return spdnn_set_features_dense(n, dense.data(), batch);
+}
+
+int spdnn_synth_features(spdnn_net* n, uint64_t seed, int batch, float dmin, float dmax) {
+    if (!(dmin >= 0.0f) || !(dmax >= dmin) || !(dmax <= 1.0f)) return fail(SPDNN_E_ARG, "need 0 <= dmin <= dmax <= 1");
+    int rc = begin_features(n, batch);
+    if (rc) return rc;
+    // physical column -> neuron (inverse of layer 0's input labelling)
+    const std::vector<int32_t>& pos = n->layers[0].in_pos;
+    std::vector<int32_t> inv((size_t)n->N);
+    for (int i = 0; i < n->N; ++i) inv[(size_t)pos[(size_t)i]] = i;
+    int32_t* d_inv = nullptr;
+    HIPCHK(hipMalloc(&d_inv, (size_t)n->N * 4));
+    hipError_t e = hipMemcpy(d_inv, inv.data(), (size_t)n->N * 4, hipMemcpyHostToDevice);
+    const int nblk = (batch + n->RB - 1) / n->RB;
+    if (e == hipSuccess) e = launch_synth_features(n->F, d_inv, n->N, batch, nblk, n->rl, seed, dmin, dmax, n->stream);
+    if (e == hipSuccess) e = launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(n->stream);
+    hipFree(d_inv);
+    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    n->have_features = true;
+    reset_state(n);
+    return SPDNN_OK;
+}
+
+int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows, float dmin,
+                              float dmax, float* rowmajor) {
+    if (!rowmajor || neuron < 1 || nrows < 0) return fail(SPDNN_E_ARG, "bad argument");
+    synth_features_host(seed, neuron, row_begin, nrows, dmin, dmax, rowmajor);
+    return SPDNN_OK;
+}
+
+// ---- inference -----------------------------------------------------------------------------
+
+int spdnn_default_run_options(spdnn_run_options* o) {
+    if (!o) return fail(SPDNN_E_ARG, "opt is NULL");
+    memset(o, 0, sizeof(*o));
+    o->prune = 1;
+    o->first_layer = 0;
+    o->n_layers = -1;
+    o->compact_threshold = 0.75f;
+    return SPDNN_OK;
+}
+
+static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp) {
+    const LayerPlan& p = n->layers[(size_t)l];
+    const DevLayer& d = n->dl[(size_t)l];
+    if (p.kernel == SPDNN_KERNEL_BAND) {
+        BandLaunch a{};
+        a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
+        a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
+        a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
+        return launch_band(a, n->stream);
+    }
+    GatherLaunch g{};
+    g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
+    g.active = n->d_active; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
+    g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv;
+    return launch_gather(g, n->stream);
+}
+
+int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    spdnn_run_options opt;
+    if (opt_in) opt = *opt_in; else spdnn_default_run_options(&opt);
+    if (!n->inspected || !n->uploaded) return fail(SPDNN_E_STATE, "inspect the network and set features first");
+    if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
+    if (opt.first_layer < 0 || opt.first_layer >= n->L) return fail(SPDNN_E_ARG, "first_layer out of range");
+    const int nl = opt.n_layers < 0 ? n->L - opt.first_layer : opt.n_layers;
+    if (nl < 1 || opt.first_layer + nl > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
+    if (opt.prune && n->bias > 0.0f)
+        return fail(SPDNN_E_UNSUPPORTED, "pruning needs bias <= 0 (an all-zero row must stay zero)");
+    if (opt.first_layer == 0) reset_state(n);
+    else if (opt.first_layer != n->cur_layer) return fail(SPDNN_E_STATE, "first_layer does not continue the current state");
+    float thr = opt.compact_threshold > 0.0f ? opt.compact_threshold : 0.75f;
+    if (thr > 1.0f) thr = 1.0f;
+
+    if (opt.time_layers && n->ev_layer.size() < (size_t)(2 * n->L)) {
+        while (n->ev_layer.size() < (size_t)(2 * n->L)) {
+            hipEvent_t e;
+            HIPCHK(hipEventCreate(&e));
+            n->ev_layer.push_back(e);
+        }
+    }
+    const int first = opt.first_layer, last = first + nl - 1;
+    for (int l = first; l <= last; ++l) { n->counts[(size_t)l] = -1; n->layer_ms[(size_t)l] = 0.0f; }
+
+    spdnn_run_result r{};
+    int64_t entering = n->alive;  // rows entering the next layer (for the byte model)
+    std::vector<int> timed;
+    HIPCHK(hipEventRecord(n->ev_start, n->stream));
+    for (int l = first; l <= last; ++l) {
+        const LayerPlan& p = n->layers[(size_t)l];
+        r.edges += (double)n->batch * (double)p.info.nnz;
+        if (n->carried == 0) {  // every row died earlier: the remaining outputs are all zero
+            n->counts[(size_t)l] = 0;
+            n->cur_layer = l + 1;
+            continue;
+        }
+        float* out = (n->cur == n->A) ? n->C : n->A;
+        const int nblk = n->carried / n->RB;
+        const int stamp = ++n->stamp;
+        if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
+        HIPCHK(launch_layer(n, l, n->cur, out, nblk, stamp));
+        if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back(l); }
+        r.layers_run++;
+        r.alg_bytes += 8.0 * (double)(opt.prune ? entering : n->batch) * (double)n->N + 8.0 * (double)p.info.nnz +
+                       4.0 * (double)(n->N + 1);
+        n->cur = out;
+        n->cur_layer = l + 1;
+        const bool need_count = opt.prune || opt.collect_counts;
+        if (need_count || l == last) {
+            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, stamp, n->d_count, n->d_alive_src,
+                                      n->d_alive_gid, n->stream));
+            n->alive_list_valid = true;
+            HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
+            HIPCHK(hipStreamSynchronize(n->stream));
+            const int64_t cnt = n->h_count[0];
+            n->counts[(size_t)l] = cnt;
+            n->alive = cnt;
+            entering = cnt;
+            if (opt.prune) {
+                if (cnt == 0) {
+                    n->carried = 0;
+                } else if ((double)cnt <= (double)thr * (double)n->carried && l + 1 < n->L) {
+                    const int nb = (int)((cnt + n->RB - 1) / n->RB);
+                    if (nb * n->RB < n->carried) {
+                        float* dstbuf = (n->cur == n->A) ? n->C : n->A;
+                        HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid,
+                                             n->d_gid_tmp, n->N, n->rl, nb, n->stream));
+                        std::swap(n->d_gid, n->d_gid_tmp);
+                        n->gid_dirty = true;
+                        n->cur = dstbuf;
+                        n->carried = nb * n->RB;
+                        r.compactions++;
+                    }
+                }
+            }
+        }
+    }
+    HIPCHK(hipEventRecord(n->ev_stop, n->stream));
+    HIPCHK(hipStreamSynchronize(n->stream));
+    HIPCHK(hipEventElapsedTime(&r.ms_total, n->ev_start, n->ev_stop));
+    for (int l : timed) {
+        float ms = 0.0f;
+        HIPCHK(hipEventElapsedTime(&ms, n->ev_layer[(size_t)(2 * l)], n->ev_layer[(size_t)(2 * l + 1)]));
+        n->layer_ms[(size_t)l] = ms;
+        r.ms_kernels += ms;
+    }
+    if (n->carried == 0) { n->alive = 0; }
+    r.active_rows = n->alive;
+    r.carried_rows = n->carried;
+    if (res) *res = r;
+    return SPDNN_OK;
+}
+
+int spdnn_get_active_count(const spdnn_net* n, int layer, int64_t* count) {
+    if (!n || !count) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    if (n->counts[(size_t)layer] < 0) return fail(SPDNN_E_STATE, "no count recorded for this layer");
+    *count = n->counts[(size_t)layer];
+    return SPDNN_OK;
+}
+
+int spdnn_get_categories(spdnn_net* n, int32_t* ids, int64_t cap, int64_t* cnt) {
+    if (!n || !cnt) return fail(SPDNN_E_ARG, "NULL argument");
+    if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
+    if (n->cur_layer == 0) {  // nothing run yet: every row counts
+        *cnt = n->batch;
+        if (ids) {
+            if (cap < n->batch) return fail(SPDNN_E_ARG, "ids buffer too small");
+            for (int i = 0; i < n->batch; ++i) ids[i] = i;
+        }
+        return SPDNN_OK;
+    }
+    *cnt = n->alive;
+    if (!ids || n->alive == 0) return SPDNN_OK;
+    if (cap < n->alive) return fail(SPDNN_E_ARG, "ids buffer too small");
+    if (!n->alive_list_valid) return fail(SPDNN_E_STATE, "no active list available");
+    HIPCHK(hipMemcpy(ids, n->d_alive_gid, (size_t)n->alive * 4, hipMemcpyDeviceToHost));
+    return SPDNN_OK;
+}
+
+int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+    if (!n || !rows || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
+    if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
+    if (nrows < 0) return fail(SPDNN_E_ARG, "nrows negative");
+    if (nrows == 0) return SPDNN_OK;
+    // global id -> physical row of the current buffer
+    std::vector<int32_t> gid((size_t)std::max(n->carried, 1));
+    if (n->carried > 0) HIPCHK(hipMemcpy(gid.data(), n->d_gid, (size_t)n->carried * 4, hipMemcpyDeviceToHost));
+    std::vector<int32_t> where((size_t)n->batch, -1);
+    for (int r = 0; r < n->carried; ++r)
+        if (gid[(size_t)r] >= 0 && gid[(size_t)r] < n->batch) where[(size_t)gid[(size_t)r]] = r;
+    std::vector<int32_t> phys((size_t)nrows);
+    for (int i = 0; i < nrows; ++i) {
+        if (rows[i] < 0 || rows[i] >= n->batch) return fail(SPDNN_E_ARG, "row id out of range");
+        phys[(size_t)i] = where[(size_t)rows[i]];
+    }
+    const int chunk = 4096;
+    int32_t* d_phys = nullptr;
+    float* d_out = nullptr;
+    HIPCHK(hipMalloc(&d_phys, (size_t)chunk * 4));
+    hipError_t e = hipMalloc(&d_out, (size_t)chunk * (size_t)n->N * 4);
+    if (e != hipSuccess) { hipFree(d_phys); return fail(SPDNN_E_NOMEM, hipGetErrorString(e)); }
+    const int32_t* lab = labelling_dev(n, n->cur_layer);
+    for (int i0 = 0; i0 < nrows && e == hipSuccess; i0 += chunk) {
+        const int m = std::min(chunk, nrows - i0);
+        e = hipMemcpyAsync(d_phys, phys.data() + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream);
+        if (e == hipSuccess) e = launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, d_out, n->stream);
+        if (e == hipSuccess)
+            e = hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * n->N * 4, hipMemcpyDeviceToHost, n->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(n->stream);
+    }
+    hipFree(d_phys);
+    hipFree(d_out);
+    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    return SPDNN_OK;
+}
+
+int spdnn_get_layer_times(const spdnn_net* n, float* ms, int cnt) {
+    if (!n || !ms) return fail(SPDNN_E_ARG, "NULL argument");
+    if (cnt < 0 || cnt > n->L) return fail(SPDNN_E_ARG, "n out of range");
+    std::copy(n->layer_ms.begin(), n->layer_ms.begin() + cnt, ms);
+    return SPDNN_OK;
+}
+
+int spdnn_write_categories(spdnn_net* n, const char* path) {
+    if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
+    int64_t cnt = 0;
+    int rc = spdnn_get_categories(n, nullptr, 0, &cnt);
+    if (rc) return rc;
+    std::vector<int32_t> ids((size_t)std::max<int64_t>(cnt, 1));
+    rc = spdnn_get_categories(n, ids.data(), (int64_t)ids.size(), &cnt);
+    if (rc) return rc;
+    FILE* f = fopen(path, "w");
+    if (!f) return fail(SPDNN_E_IO, std::string("cannot write ") + path);
+    for (int64_t i = 0; i < cnt; ++i) fprintf(f, "%d\n", ids[(size_t)i] + 1);
+    fclose(f);
+    return SPDNN_OK;
+}
+
+// ---- device utilities ------------------------------------------------------------------------
+
+int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
+    if (!gbps || bytes < 1024 || reps < 1) return fail(SPDNN_E_ARG, "bad argument");
+    bytes &= ~(int64_t)1023;
+    float *a = nullptr, *b = nullptr;
+    hipEvent_t e0, e1;
+    HIPCHK(hipMalloc(&a, (size_t)bytes));
+    hipError_t e = hipMalloc(&b, (size_t)bytes);
+    if (e != hipSuccess) { hipFree(a); return fail(SPDNN_E_NOMEM, hipGetErrorString(e)); }
+    hipMemset(a, 0, (size_t)bytes);
+    hipEventCreate(&e0); hipEventCreate(&e1);
+    (void)launch_copy_f4(a, b, bytes / 4, nullptr);
+    hipEventRecord(e0, nullptr);
+    for (int i = 0; i < reps; ++i) (void)launch_copy_f4(a, b, bytes / 4, nullptr);
+    hipEventRecord(e1, nullptr);
+    e = hipEventSynchronize(e1);
+    float ms = 0.0f;
+    hipEventElapsedTime(&ms, e0, e1);
+    hipEventDestroy(e0); hipEventDestroy(e1);
+    hipFree(a); hipFree(b);
+    if (e != hipSuccess || ms <= 0.0f) return fail(SPDNN_E_DEVICE, "copy benchmark failed");
+    *gbps = 2.0 * (double)bytes * reps / (ms * 1e-3) / 1e9;
+    return SPDNN_OK;
+}
+
+int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
+    int cnt = 0;
+    if (hipGetDeviceCount(&cnt) != hipSuccess || cnt < 1) return fail(SPDNN_E_DEVICE, "no HIP device available");
+    hipDeviceProp_t p;
+    HIPCHK(hipGetDeviceProperties(&p, 0));
+    if (name && cap > 0) snprintf(name, (size_t)cap, "%s (%s)", p.name, p.gcnArchName);
+    if (compute_units) *compute_units = p.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = (int64_t)p.totalGlobalMem;
+    return SPDNN_OK;
+}
+
+int spdnn_device_synchronize(void) {
+    HIPCHK(hipDeviceSynchronize());
+    return SPDNN_OK;
+}
+
+}  // extern "C"

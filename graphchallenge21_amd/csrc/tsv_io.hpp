@@ -1,0 +1,26 @@
+// TSV loaders in the challenge's file formats, the host data layer of the reference driver
+// (COOMatrix(file, 1, false), src/utils/matrix.h:255-282; read_input, src/network.cpp:33-54),
+// re-done as a single pass over the file bytes instead of iostream extraction.
+#pragma once
+#include <cstdint>
+#include <string>
+#include <vector>
+
+namespace spdnn {
+
+struct Triple { int32_t a, b; float v; };
+
+// Reads whitespace-separated "int int float" triples.  Returns false and sets err on failure.
+bool read_triples(const std::string& path, std::vector<Triple>& out, std::string& err);
+
+// Weight file "in out value" (1-based) -> CSR of an N x N layer with row = output neuron,
+// col = input neuron, entries of a row in ascending input index (file order among duplicates).
+bool read_weight_tsv_csr(const std::string& path, int N, std::vector<int32_t>& rowptr,
+                         std::vector<int32_t>& col, std::vector<float>& val, std::string& err);
+
+// Feature file "row neuron value" (1-based) -> dense row-major batch x N; rows beyond batch are
+// skipped like the reference does.  *kept receives the number of entries stored.
+bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
+                             int64_t* kept, std::string& err);
+
+}  // namespace spdnn

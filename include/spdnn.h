@@ -1,0 +1,225 @@
+/*
+ * spdnn.h - C ABI of the MI355X (gfx950) Sparse DNN Graph Challenge inference library.
+ *
+ * The library computes the layer chain  Y_{l+1} = min(ReLU(Y_l * W_l + bias), 32)  on one GPU
+ * with hand-written HIP kernels.  It is the drop-in for the reference's single-GPU executor
+ *
+ *     void ftxj::test_benchmark_graph_challenge(input, weight, row_access, batch, neuron, bias, env)
+ *     (reference: src/microbenchmark/header.h:16-19, defined at
+ *      src/microbenchmark/all_network.cu:207-526, sole caller src/network.cpp:123)
+ *
+ * and for the host pieces that executor depends on (TSV loaders, reorder, inspector).  Where
+ * the reference passes STL containers holding inspector-specific streams, this ABI takes plain
+ * CSR per layer (row = OUTPUT neuron, col = INPUT neuron: the reference's in-memory convention,
+ * src/utils/matrix.h:272-278) and dense or generated features; reorder, layout and kernel
+ * selection happen behind the boundary.
+ *
+ * Conventions
+ *   - every function returns an int status (SPDNN_OK = 0); none of them calls exit().  The
+ *     reference's Safe_Call (src/gpu_lib/gpu_runtime.h:6-17) and launch checks
+ *     (all_network.cu:362-366) terminate the process instead.
+ *   - all pointers are HOST pointers unless a name ends in _dev; the library copies what it
+ *     needs before returning, the caller may free its buffers immediately.
+ *   - a handle is used by one host thread at a time.
+ *   - row ids ("global ids", categories) are 0-based positions in the feature matrix that was
+ *     handed over.
+ *   - feature values and weights must be finite; products are expected not to underflow.
+ */
+#ifndef SPDNN_H
+#define SPDNN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct spdnn_net spdnn_net;
+
+enum spdnn_status {
+    SPDNN_OK = 0,
+    SPDNN_E_ARG = 1,         /* invalid argument (bad size, index out of range, non-finite value) */
+    SPDNN_E_STATE = 2,       /* call made in the wrong order (e.g. run before inspect)           */
+    SPDNN_E_IO = 3,          /* file missing or malformed                                         */
+    SPDNN_E_DEVICE = 4,      /* HIP runtime error or no gfx950 device                             */
+    SPDNN_E_NOMEM = 5,       /* host or device allocation failed                                  */
+    SPDNN_E_UNSUPPORTED = 6  /* valid request the library cannot serve                            */
+};
+
+/* Kernel classes the inspector chooses from (per layer). */
+enum spdnn_kernel {
+    SPDNN_KERNEL_AUTO = 0,
+    SPDNN_KERNEL_GATHER = 1, /* general CSR/ELL gather, any sparsity pattern                      */
+    SPDNN_KERNEL_BAND = 2    /* row-succ / tiled: relabelled circulant band walked through an LDS ring */
+};
+
+typedef struct spdnn_layer_plan {
+    int32_t kernel;          /* spdnn_kernel chosen for the layer                                 */
+    int32_t max_row_nnz;     /* longest row                                                       */
+    int32_t regular;         /* 1: every row and every column holds exactly max_row_nnz entries   */
+    int32_t uniform_value;   /* 1: all values equal `value`                                       */
+    float   value;
+    int32_t exact_products;  /* 1: every value is 0 or +-2^e, so x*w is exact and fma == mul+add  */
+    int32_t band_halo;       /* BAND: extra input columns a tile needs (max_row_nnz-1); else -1   */
+    int64_t nnz;
+    int64_t plan_bytes;      /* device bytes held for this layer                                  */
+} spdnn_layer_plan;
+
+typedef struct spdnn_run_options {
+    int32_t prune;             /* 1: drop rows that are all zero between layers (requires bias <= 0) */
+    int32_t first_layer;       /* 0 starts from the features; >0 continues from the current state  */
+    int32_t n_layers;          /* number of layers to run, -1 = through the last                   */
+    int32_t collect_counts;    /* 1: record the active-row count after every layer                 */
+    int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
+    float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
+    int32_t reserved[4];
+} spdnn_run_options;
+
+typedef struct spdnn_run_result {
+    int32_t layers_run;      /* layers actually launched (fewer when every row died)              */
+    int32_t compactions;     /* number of row repacks                                             */
+    int64_t active_rows;     /* rows active after the last requested layer                        */
+    int64_t carried_rows;    /* rows physically carried at the end                                */
+    float   ms_total;        /* HIP-event time, first launch to last completion                   */
+    float   ms_kernels;      /* sum of per-layer kernel times (time_layers only, else 0)          */
+    double  alg_bytes;       /* sum over layers of 8*B_l*N + nnz_l*8 + 4*(N+1)                     */
+    double  edges;           /* batch * nnz summed over the layers requested                      */
+} spdnn_run_result;
+
+/* ---- life cycle ------------------------------------------------------------------------- */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int spdnn_version(void);
+
+/* Text of the most recent error on this thread (never NULL). */
+const char* spdnn_last_error(void);
+
+/* Creates a network of `layers` square layers of width `neuron`, for at most `max_batch`
+ * feature rows.  bias and clamp are the epilogue constants (reference: bias by neuron count,
+ * src/network.cpp:73-78; clamp 32, all_network.cu:8-10).  Touches no device. */
+int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp, spdnn_net** out);
+
+/* Releases host and device memory (the reference never frees, all_network.cu:240-303). */
+int spdnn_destroy(spdnn_net* net);
+
+/* Bias the reference driver selects for a neuron count (src/network.cpp:73-78): -0.3, -0.35,
+ * -0.4, -0.45 for 1024, 4096, 16384, 65536; returns SPDNN_E_ARG for other widths (the
+ * reference silently uses 0 there). */
+int spdnn_reference_bias(int neuron, float* bias);
+
+/* ---- weights ---------------------------------------------------------------------------- */
+
+/* Hands over layer `layer` as CSR with row = output neuron, col = input neuron, what
+ * COOMatrix(file,1,false) + CSRCSCMatrix hold in the reference (src/utils/matrix.h:255-282,
+ * :329-343).  Columns inside a row may come in any order; accumulation is always in ascending
+ * input index, the order of the reference's CPU checker (src/utils/cpu_spmm.h:14-35). */
+int spdnn_set_layer_csr(spdnn_net* net, int layer, const int32_t* rowptr, const int32_t* col, const float* val);
+
+/* Reads a weight TSV in the challenge format ("in out value", 1-based), the file format of
+ * COOMatrix(file, 1, false) (src/utils/matrix.h:255-282), and sets the layer. */
+int spdnn_load_layer_tsv(spdnn_net* net, int layer, const char* path);
+
+/* File name the reference driver uses for a layer: <dir>/neuron<N>/n<N>-l<layer+1>.tsv
+ * (get_weight_file_name, src/network.cpp:14-19). */
+int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap);
+
+/* Generates `count` synthetic layers [first, first+count) with the seeded permuted-stride
+ * generator: W_l[i, (pi_l(i) + o_l + k*s_l) mod N] = value for k = 0..nnz_per_row-1.  Runs on
+ * host threads and feeds the same path as spdnn_set_layer_csr. */
+int spdnn_synth_layers(spdnn_net* net, uint64_t seed, int first, int count, int nnz_per_row, float value);
+
+/* Host copy of one synthetic layer in CSR form (rowptr[N+1], col/val[N*nnz_per_row]). */
+int spdnn_synth_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row, float value,
+                          int32_t* rowptr, int32_t* col, float* val);
+
+/* ---- inspector -------------------------------------------------------------------------- */
+
+/* The per-layer inspector (classification, relabelling, kernel choice, plan emission; the role
+ * of BlockContainer + MaxInReuseBSchedule in src/network.cpp:105-120) runs on host worker
+ * threads as layers are handed over.  spdnn_inspect waits for it, checks that every layer is
+ * set and links consecutive layers (each layer stores its outputs in the column order the next
+ * one reads).  Host only; plans are uploaded on first device use. */
+int spdnn_inspect(spdnn_net* net);
+
+/* SPDNN_KERNEL_AUTO (default) lets the inspector choose per layer; SPDNN_KERNEL_GATHER makes it
+ * emit the general kernel for every layer.  Must be called before the first layer is set. */
+int spdnn_set_force_kernel(spdnn_net* net, int kernel);
+
+int spdnn_get_layer_plan(const spdnn_net* net, int layer, spdnn_layer_plan* out);
+
+/* Host view of a BAND plan, for verification: position of every input neuron along the band
+ * (in_pos[N]), the output neuron computed at every band position (out_at[N]), and per position
+ * the ring selectors of its inputs in accumulation order (sel[N*max_row_nnz], position mod 256).
+ * Any pointer may be NULL.  SPDNN_E_STATE if the layer is not a BAND layer. */
+int spdnn_get_band_plan(const spdnn_net* net, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel);
+
+/* Physical output column of every schedule slot of a layer (dst[N]); needs spdnn_inspect. */
+int spdnn_get_layer_dst(const spdnn_net* net, int layer, int32_t* dst);
+
+/* Physical column of every neuron in the buffer layer `layer` reads (layer == layers: the
+ * final output, always the identity). */
+int spdnn_get_input_labelling(const spdnn_net* net, int layer, int32_t* phys_col);
+
+/* HashReorder::reorder (src/reorder/hash.h:14-31): v -> v / buckets + (v % buckets) * (domain / buckets).
+ * Returns SPDNN_E_ARG where the reference prints an error and exits. */
+int spdnn_hash_reorder(int v, int buckets, int domain, int* out);
+
+/* ---- features --------------------------------------------------------------------------- */
+
+/* Dense row-major fp32 features, batch x neuron (what read_input + the flatten at
+ * all_network.cu:240-247 produce).  Requires spdnn_inspect. */
+int spdnn_set_features_dense(spdnn_net* net, const float* rowmajor, int batch);
+
+/* Sparse feature TSV in the challenge format ("row neuron value", 1-based; rows beyond batch
+ * are skipped): read_input, src/network.cpp:33-54. */
+int spdnn_load_features_tsv(spdnn_net* net, const char* path, int batch);
+
+/* Seeded Bernoulli rows generated on the device: row r has density uniform in [dmin, dmax],
+ * entries are 0.0f / 1.0f.  spdnn_synth_features_host produces the same values on the host. */
+int spdnn_synth_features(spdnn_net* net, uint64_t seed, int batch, float dmin, float dmax);
+int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows,
+                              float dmin, float dmax, float* rowmajor);
+
+/* ---- inference -------------------------------------------------------------------------- */
+
+int spdnn_default_run_options(spdnn_run_options* opt);
+
+/* Runs layers [first_layer, first_layer + n_layers): the layer loop of
+ * test_benchmark_graph_challenge (all_network.cu:333-519).  With prune the active-row scan and
+ * the repack run on the device; the host only reads the count. */
+int spdnn_run(spdnn_net* net, const spdnn_run_options* opt, spdnn_run_result* result);
+
+/* Active-row count recorded after layer `layer` of the last run (collect_counts or prune),
+ * the number the reference prints as "layer l, batch = n" (all_network.cu:508). */
+int spdnn_get_active_count(const spdnn_net* net, int layer, int64_t* count);
+
+/* Global ids (ascending) of the rows that are nonzero after the last layer run: the challenge's
+ * categories.  *n receives the count; ids may be NULL to query it. */
+int spdnn_get_categories(spdnn_net* net, int32_t* ids, int64_t cap, int64_t* n);
+
+/* Current activations of the given global rows, row-major nrows x neuron in natural neuron
+ * order (rows that were pruned are zero).  The reference copies the whole buffer back
+ * (all_network.cu:521). */
+int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
+
+/* Per-layer kernel milliseconds of the last run made with time_layers. */
+int spdnn_get_layer_times(const spdnn_net* net, float* ms, int n);
+
+/* Writes the categories as the challenge's truth-file format: one 1-based row id per line. */
+int spdnn_write_categories(spdnn_net* net, const char* path);
+
+/* ---- device utilities ------------------------------------------------------------------- */
+
+/* Measured device-to-device copy bandwidth (GB/s, read + write bytes over HIP-event time) of a
+ * plain float4 copy kernel over `bytes` bytes: the box's practical HBM peak. */
+int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps);
+
+/* Name and compute-unit count of device 0. */
+int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes);
+
+int spdnn_device_synchronize(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPDNN_H */

@@ -1,0 +1,314 @@
+/*
+ * CPU oracle for the Sparse DNN Graph Challenge inference path
+ *     Y_{l+1} = min(ReLU(Y_l * W_l + b), 32)
+ *
+ * TEST INFRASTRUCTURE ONLY: the shipped library never links, loads or calls this file.
+ * It exists so that tests, the smoke check and the benchmark's CPU-baseline leg have an
+ * independent statement of the reference's CPU results.
+ *
+ * Build: gcc -O2 -fopenmp -ffp-contract=off -fno-fast-math -shared -fPIC (see Makefile).
+ * -ffp-contract=off matters: the reference's CPU checkers are built by plain g++ for
+ * baseline x86-64, where `res += in * val` is a rounded multiply followed by a rounded
+ * add, never a fused multiply-add.
+ *
+ * Pinning status of each function (what independent evidence checks it) is listed in
+ * tests/test_oracle_*.py; in short
+ *   orc_read_weight_tsv / orc_coo_to_csr   pinned: reference loader built into oracle/_ref
+ *                                          dumps the same (row,col,val) stream
+ *   orc_hash_reorder                       pinned: oracle/_ref table + closed form + bijection
+ *   orc_layer                              pinned: oracle/_ref CpuSpmm / CpuSpmmFuse comparators,
+ *                                          dense brute force, permutation / all-ones closed forms
+ *   orc_relu_clamp                         pinned: special-value table
+ *   orc_compact                            pinned: invariants (stable order, row independence)
+ *   orc_gen_*                              the build's own definition (the reference has no
+ *                                          generator); pinned by structural invariants and
+ *                                          committed hashes of the generated buffers
+ *   orc_read_features_tsv                  pinned: hand-written TSV with known answer
+ */
+#include "spdnn_oracle.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------------------------
+ * Seeded synthetic inputs.
+ *
+ * The reference ships no generator (src/microbenchmark/random.h:5-13 is an empty stub)
+ * and reads downloaded TSV files instead, so the generator below is this build's own
+ * definition of "seeded permutation / offset / stride" and "Bernoulli rows":
+ *
+ *   sm64(x)          SplitMix64 output function applied to x + 0x9E3779B97F4A7C15
+ *   layer key        kl = sm64(sm64(seed ^ 0x4C41594552) + layer)
+ *   draw(n)          sm64(kl + n)
+ *   offset o         draw(0) mod N
+ *   stride s         draw(1) mod N, 0 -> 1, then incremented until gcd(s, N) = 1
+ *   permutation pi   Fisher-Yates, i = N-1 .. 1, j = (hi32(draw(2 + N-1-i)) * (i+1)) >> 32
+ *   W_l[i, (pi(i) + o + k*s) mod N] = value, k = 0 .. K-1   (input i feeds K outputs)
+ *
+ *   feature key      kf = sm64(seed ^ 0x46454154), row key rk = sm64(kf + row)
+ *   row density      thr = lo + ((hi32(sm64(rk + 0xFFFFFFFF00000000)) * span) >> 32) with
+ *                    lo = floor(dmin * 2^32), span = floor((dmax - dmin) * 2^32)
+ *   element (row,c)  1.0f if hi32(sm64(rk + c)) < thr else 0.0f
+ * ------------------------------------------------------------------------------------ */
+uint64_t orc_splitmix64(uint64_t x) {
+    uint64_t z = x + 0x9E3779B97F4A7C15ULL;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    return z ^ (z >> 31);
+}
+
+static int gcd_int(int a, int b) {
+    while (b) { int t = a % b; a = b; b = t; }
+    return a;
+}
+
+void orc_gen_layer_params(uint64_t seed, int layer, int neuron, int* perm, int* offset, int* stride) {
+    const uint64_t kl = orc_splitmix64(orc_splitmix64(seed ^ 0x4C41594552ULL) + (uint64_t)layer);
+    *offset = (int)(orc_splitmix64(kl + 0) % (uint64_t)neuron);
+    int s = (int)(orc_splitmix64(kl + 1) % (uint64_t)neuron);
+    if (s == 0) s = 1;
+    while (gcd_int(s, neuron) != 1) { s++; if (s >= neuron) s = 1; }
+    *stride = s;
+    for (int i = 0; i < neuron; ++i) perm[i] = i;
+    for (int i = neuron - 1; i >= 1; --i) {
+        uint64_t r = orc_splitmix64(kl + 2 + (uint64_t)(neuron - 1 - i)) >> 32;
+        int j = (int)((r * (uint64_t)(i + 1)) >> 32);
+        int t = perm[i]; perm[i] = perm[j]; perm[j] = t;
+    }
+}
+
+static int cmp_int(const void* a, const void* b) {
+    int x = *(const int*)a, y = *(const int*)b;
+    return (x > y) - (x < y);
+}
+
+/* CSR with row = output neuron, col = input neuron (ascending inside a row): the in-memory
+ * convention every reference driver uses (COOMatrix(file, 1, false), src/utils/matrix.h:272-278,
+ * then to_row_first_ordered, matrix.h:245-253). */
+int orc_gen_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row, float value,
+                      int* rowptr, int* col, float* val) {
+    if (neuron < 1 || nnz_per_row < 1 || nnz_per_row > neuron) return -1;
+    int* perm = (int*)malloc(sizeof(int) * (size_t)neuron);
+    int* inv = (int*)malloc(sizeof(int) * (size_t)neuron);
+    if (!perm || !inv) { free(perm); free(inv); return -2; }
+    int o, s;
+    orc_gen_layer_params(seed, layer, neuron, perm, &o, &s);
+    for (int i = 0; i < neuron; ++i) inv[perm[i]] = i;
+    for (int j = 0; j < neuron; ++j) {
+        int* c = col + (size_t)j * nnz_per_row;
+        rowptr[j] = j * nnz_per_row;
+        for (int k = 0; k < nnz_per_row; ++k) {
+            /* output j is fed by the input i with pi(i) + o + k*s = j (mod N) */
+            long long t = ((long long)j - o - (long long)k * s) % neuron;
+            if (t < 0) t += neuron;
+            c[k] = inv[t];
+        }
+        qsort(c, (size_t)nnz_per_row, sizeof(int), cmp_int);
+        for (int k = 0; k < nnz_per_row; ++k) val[(size_t)j * nnz_per_row + k] = value;
+    }
+    rowptr[neuron] = neuron * nnz_per_row;
+    free(perm); free(inv);
+    return 0;
+}
+
+uint32_t orc_feature_threshold(uint64_t seed, int64_t row, float dmin, float dmax) {
+    const uint64_t kf = orc_splitmix64(seed ^ 0x46454154ULL);
+    const uint64_t rk = orc_splitmix64(kf + (uint64_t)row);
+    const uint64_t lo = (uint64_t)((double)dmin * 4294967296.0);
+    const uint64_t span = (uint64_t)(((double)dmax - (double)dmin) * 4294967296.0);
+    const uint64_t a = orc_splitmix64(rk + 0xFFFFFFFF00000000ULL) >> 32;
+    uint64_t thr = lo + ((a * span) >> 32);
+    if (thr > 0xFFFFFFFFULL) thr = 0xFFFFFFFFULL;
+    return (uint32_t)thr;
+}
+
+void orc_gen_features(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows,
+                      float dmin, float dmax, float* out) {
+    const uint64_t kf = orc_splitmix64(seed ^ 0x46454154ULL);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < nrows; ++r) {
+        const int64_t row = row_begin + r;
+        const uint64_t rk = orc_splitmix64(kf + (uint64_t)row);
+        const uint32_t thr = orc_feature_threshold(seed, row, dmin, dmax);
+        float* o = out + (size_t)r * (size_t)neuron;
+        for (int c = 0; c < neuron; ++c) {
+            uint32_t e = (uint32_t)(orc_splitmix64(rk + (uint64_t)c) >> 32);
+            o[c] = e < thr ? 1.0f : 0.0f;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------------------
+ * Reference host data layer
+ * ------------------------------------------------------------------------------------ */
+
+/* HashReorder::hash, src/reorder/hash.h:14-22: v -> v / buckets + (v % buckets) * (N / buckets).
+ * Returns -1 where the reference prints an error and exits (v outside the domain). */
+int orc_hash_reorder(int v, int buckets, int max_domain) {
+    if (v >= max_domain || v < 0 || buckets <= 0) return -1;
+    int width = max_domain / buckets;
+    int c = v % buckets;
+    int r = v / buckets;
+    return r + c * width;
+}
+
+int64_t orc_count_tsv_triples(const char* path) {
+    FILE* f = fopen(path, "r");
+    if (!f) return -1;
+    int64_t n = 0;
+    int a, b; float v;
+    while (fscanf(f, "%d %d %f", &a, &b, &v) == 3) n++;
+    fclose(f);
+    return n;
+}
+
+/* COOMatrix(file, begin_idx, T=false), src/utils/matrix.h:255-282: a line "v u val" becomes the
+ * element {row = u - begin_idx, col = v - begin_idx, val}; i.e. the first number of the line is
+ * the INPUT neuron (stored as col), the second the OUTPUT neuron (stored as row).  Dimensions are
+ * the maxima seen.  Returns the number of elements, -1 if the file cannot be opened (the
+ * reference prints and exits, matrix.h:259-262), -2 if cap is too small. */
+int64_t orc_read_weight_tsv(const char* path, int begin_idx, int64_t cap,
+                            int* row, int* col, float* val, int* n_rows, int* n_cols) {
+    FILE* f = fopen(path, "r");
+    if (!f) return -1;
+    int64_t n = 0;
+    int v, u; float x;
+    int rmax = 0, cmax = 0;
+    while (fscanf(f, "%d %d %f", &v, &u, &x) == 3) {
+        if (n >= cap) { fclose(f); return -2; }
+        row[n] = u - begin_idx;
+        col[n] = v - begin_idx;
+        val[n] = x;
+        if (u + 1 - begin_idx > rmax) rmax = u + 1 - begin_idx;
+        if (v + 1 - begin_idx > cmax) cmax = v + 1 - begin_idx;
+        n++;
+    }
+    fclose(f);
+    if (n_rows) *n_rows = rmax;
+    if (n_cols) *n_cols = cmax;
+    return n;
+}
+
+typedef struct { int row, col; float val; int64_t seq; } coo_elm;
+
+static int cmp_elm(const void* a, const void* b) {
+    const coo_elm* x = (const coo_elm*)a; const coo_elm* y = (const coo_elm*)b;
+    if (x->row != y->row) return (x->row > y->row) - (x->row < y->row);
+    if (x->col != y->col) return (x->col > y->col) - (x->col < y->col);
+    return (x->seq > y->seq) - (x->seq < y->seq);
+}
+
+/* to_row_first_ordered (matrix.h:245-253) followed by the row-pointer construction of coo2csr
+ * (matrix.h:329-343).  Unlike coo2csr this one handles empty rows; the reference assumes there
+ * are none.  Ties (duplicate (row, col)) keep file order; the reference leaves them to an
+ * unstable std::sort. */
+int orc_coo_to_csr(int64_t nnz, int n_rows, const int* row, const int* col, const float* val,
+                   int* rowptr, int* csr_col, float* csr_val) {
+    coo_elm* e = (coo_elm*)malloc(sizeof(coo_elm) * (size_t)(nnz > 0 ? nnz : 1));
+    if (!e) return -2;
+    for (int64_t i = 0; i < nnz; ++i) {
+        if (row[i] < 0 || row[i] >= n_rows) { free(e); return -1; }
+        e[i].row = row[i]; e[i].col = col[i]; e[i].val = val[i]; e[i].seq = i;
+    }
+    qsort(e, (size_t)nnz, sizeof(coo_elm), cmp_elm);
+    for (int r = 0; r <= n_rows; ++r) rowptr[r] = 0;
+    for (int64_t i = 0; i < nnz; ++i) rowptr[e[i].row + 1]++;
+    for (int r = 0; r < n_rows; ++r) rowptr[r + 1] += rowptr[r];
+    for (int64_t i = 0; i < nnz; ++i) { csr_col[i] = e[i].col; csr_val[i] = e[i].val; }
+    free(e);
+    return 0;
+}
+
+/* read_input, src/network.cpp:33-54: lines "b n val" (1-based); rows beyond `batch` are
+ * skipped, everything else lands in dense[b-1][n-1].  Returns the number of entries kept,
+ * -1 if the file cannot be opened (the reference exits, network.cpp:37-40). */
+int64_t orc_read_features_tsv(const char* path, int neuron, int batch, float* dense) {
+    FILE* f = fopen(path, "r");
+    if (!f) return -1;
+    int b, n; float v;
+    int64_t kept = 0;
+    while (fscanf(f, "%d %d %f", &b, &n, &v) == 3) {
+        if (b <= batch && b >= 1 && n >= 1 && n <= neuron) {
+            dense[(size_t)(b - 1) * (size_t)neuron + (size_t)(n - 1)] = v;
+            kept++;
+        }
+    }
+    fclose(f);
+    return kept;
+}
+
+/* ------------------------------------------------------------------------------------
+ * Arithmetic
+ * ------------------------------------------------------------------------------------ */
+
+/* __ReLU, src/microbenchmark/all_network.cu:8-10: x<0 ? 0 : x>32 ? 32 : x (NaN and -0.0 pass
+ * through unchanged). */
+float orc_relu_clamp(float x) {
+    return x < 0.0f ? 0.0f : (x > 32.0f ? 32.0f : x);
+}
+
+static int g_threads = 0;
+void orc_set_threads(int n) { g_threads = n; }
+int orc_get_threads(void) {
+#ifdef _OPENMP
+    return g_threads > 0 ? g_threads : omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* One layer for `nrows` independent rows (row-major, `neuron` floats each).
+ *   accumulation  CpuSpmm::run_and_cmp with T=false, src/utils/cpu_spmm.h:14-35: walk the
+ *                 entries sorted by (row=output, col=input) and do res[b][row] += in[b][col]*val,
+ *                 starting from 0.0f - so each output adds its inputs in ascending input index.
+ *   epilogue      src/utils/cpu_spmm_fuse.h:46 / all_network.cu:57: bias is added once, after the
+ *                 sum, then clamped; the bias is a float here (the GPU kernels take float bias,
+ *                 all_network.cu:24; cpu_spmm_fuse.h:11 takes an int and so truncates -0.3 to 0,
+ *                 which the BASELINE configurations do not want).
+ *   active flag   all_network.cu:55-60: a row is active iff any of its outputs is nonzero
+ *                 (`if (C[..] = __ReLU(..)) active[row] = 1`; NaN counts, -0.0 does not). */
+void orc_layer(const float* yin, int64_t nrows, int neuron,
+               const int* rowptr, const int* col, const float* val,
+               float bias, float* yout, int* active) {
+#ifdef _OPENMP
+    const int nt = orc_get_threads();
+#endif
+#pragma omp parallel for schedule(dynamic, 4) num_threads(nt)
+    for (int64_t b = 0; b < nrows; ++b) {
+        const float* x = yin + (size_t)b * (size_t)neuron;
+        float* y = yout + (size_t)b * (size_t)neuron;
+        int any = 0;
+        for (int j = 0; j < neuron; ++j) {
+            float acc = 0.0f;
+            for (int e = rowptr[j]; e < rowptr[j + 1]; ++e) {
+                float p = x[col[e]] * val[e];
+                acc = acc + p;
+            }
+            float r = orc_relu_clamp(acc + bias);
+            y[j] = r;
+            if (r) any = 1;
+        }
+        if (active) active[b] = any;
+    }
+}
+
+/* Host compaction, all_network.cu:455-463: survivors keep their relative order.  The reference
+ * records only the slot in the previous compacted buffer (the global-id form is commented out at
+ * all_network.cu:459); here the global ids are carried along so categories can be reported. */
+int64_t orc_compact(const float* y, int64_t nrows, int neuron, const int* active,
+                    const int* gid_in, float* y_out, int* gid_out) {
+    int64_t n = 0;
+    for (int64_t k = 0; k < nrows; ++k) {
+        if (active[k]) {
+            if (y_out) memmove(y_out + (size_t)n * (size_t)neuron, y + (size_t)k * (size_t)neuron,
+                               sizeof(float) * (size_t)neuron);
+            if (gid_out) gid_out[n] = gid_in ? gid_in[k] : (int)k;
+            n++;
+        }
+    }
+    return n;
+}

@@ -1,0 +1,43 @@
+"""Shared helpers of the parity tests."""
+import numpy as np
+
+
+def random_csr(rng, n, row_nnz, values="pow2"):
+    """Random square layer in CSR (row = output neuron): row j holds row_nnz[j] distinct inputs."""
+    rowptr = np.zeros(n + 1, np.int32)
+    cols, vals = [], []
+    for j in range(n):
+        k = int(row_nnz[j]) if hasattr(row_nnz, "__len__") else int(row_nnz)
+        c = rng.choice(n, size=k, replace=False)
+        rng.shuffle(c)  # unsorted on purpose: the library must sort
+        cols.append(c)
+        if values == "pow2":
+            v = np.ldexp(1.0, rng.integers(-6, 1, size=k)) * rng.choice([-1.0, 1.0], size=k)
+        elif values == "uniform":
+            v = np.full(k, 0.0625)
+        else:
+            v = rng.uniform(-0.2, 0.3, size=k)
+        vals.append(v.astype(np.float32))
+        rowptr[j + 1] = rowptr[j] + k
+    col = np.concatenate(cols).astype(np.int32) if cols else np.zeros(0, np.int32)
+    val = np.concatenate(vals).astype(np.float32) if vals else np.zeros(0, np.float32)
+    return rowptr, col, val
+
+
+def sort_rows(csr):
+    """The same layer with every row sorted by input index (stable)."""
+    rowptr, col, val = csr
+    col2, val2 = col.copy(), val.copy()
+    for j in range(len(rowptr) - 1):
+        b, e = rowptr[j], rowptr[j + 1]
+        o = np.argsort(col[b:e], kind="stable")
+        col2[b:e] = col[b:e][o]
+        val2[b:e] = val[b:e][o]
+    return rowptr, col2, val2
+
+
+def same_floats(a, b):
+    """Bit-for-bit equality of fp32 arrays, except that +0.0 and -0.0 count as equal."""
+    a = np.asarray(a, np.float32)
+    b = np.asarray(b, np.float32)
+    return a.shape == b.shape and bool(np.all((a == b) | (np.isnan(a) & np.isnan(b))))

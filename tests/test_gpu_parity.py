@@ -1,0 +1,199 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle.
+
+Bar: active-row sets (categories) identical after every layer; fp32 activations bit-identical
+(the requirement is 1e-5 relative / 1e-6 absolute; accumulating in the reference's order makes
+equality attainable, so equality is what is asserted).
+"""
+import numpy as np
+import pytest
+
+from helpers import random_csr, same_floats, sort_rows
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6  # the stated tolerance; the tests assert the stricter bit equality
+
+
+def _layer_by_layer(gc, orc, net, layers, feats, prune):
+    """Runs one layer at a time and checks categories and activations after each."""
+    B = feats.shape[0]
+    ref = orc.infer(feats, layers, net.bias, prune=False, keep=set(range(len(layers))))
+    rows = np.arange(B, dtype=np.int32)
+    for l in range(len(layers)):
+        print("  layer", l, flush=True)
+        r = net.run(prune=prune, first_layer=l, n_layers=1, collect_counts=True)
+        want_ids = ref["active_ids"][l]
+        got_ids = net.categories()
+        assert np.array_equal(got_ids, want_ids), "categories differ after layer %d" % l
+        assert r.active_rows == len(want_ids)
+        assert net.active_count(l) == len(want_ids)
+        got = net.activations(rows)
+        want = ref["kept"][l][1]
+        assert same_floats(got, want), "activations differ after layer %d: max |d| = %g" % (
+            l, float(np.abs(got - want).max()))
+        assert np.allclose(got, want, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dmax", [0.25, 0.50])
+@pytest.mark.parametrize("prune", [True, False])
+def test_band_layer_by_layer(gc, orc, prune, dmax):
+    N, L, B = 1024, 8, 600
+    print("band N=%d L=%d B=%d prune=%s dmax=%g" % (N, L, B, prune, dmax), flush=True)
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
+    feats = orc.gen_features(0, N, 0, B, 0.10, dmax)
+    with gc.Network(N, B, L) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_BAND for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune)
+
+
+def test_device_features_match_host(gc, orc):
+    N, L, B = 1024, 2, 700
+    print("synth features N=%d B=%d" % (N, B), flush=True)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(3)
+        net.inspect()
+        net.synth_features(7, B, 0.10, 0.25)
+        got = net.activations(np.arange(B, dtype=np.int32))
+        want = orc.gen_features(7, N, 0, B, 0.10, 0.25)
+        assert np.array_equal(got, want)
+        assert np.array_equal(net.categories(), np.arange(B))
+
+
+@pytest.mark.parametrize("prune", [True, False])
+def test_full_chain_cfg0_shape(gc, orc, prune):
+    """N=1024, 120 layers, B=6000, bias -0.3: the reference's own CPU-runnable case."""
+    N, L, B = 1024, 120, 6000
+    print("cfg0 chain prune=%s" % prune, flush=True)
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
+    feats = orc.gen_features(0, N, 0, B)
+    ref = orc.infer(feats, layers[:12], -0.3, prune=True)   # every row is dead long before layer 12
+    assert len(ref["active_ids"][-1]) == 0
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, B)
+        r = net.run(prune=prune, collect_counts=True)
+        counts = [net.active_count(l) for l in range(L)]
+        assert counts[:12] == [len(a) for a in ref["active_ids"]]
+        assert counts[12:] == [0] * (L - 12)
+        assert r.active_rows == 0 and len(net.categories()) == 0
+        if prune:
+            assert r.layers_run < L and r.compactions >= 1
+        else:
+            assert r.layers_run == L
+
+
+def test_survivor_chain_with_compaction(gc, orc):
+    """Rows with density up to 0.5 survive and saturate: late-layer pruning and repacks."""
+    N, L, B = 1024, 24, 3000
+    print("survivor chain", flush=True)
+    layers = [orc.gen_layer_csr(5, l, N) for l in range(L)]
+    feats = orc.gen_features(5, N, 0, B, 0.10, 0.50)
+    ref = orc.infer(feats, layers, -0.3, prune=True)
+    assert 0 < len(ref["categories"]) < B
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(5)
+        net.inspect()
+        net.set_features_dense(feats)
+        for prune in (True, False):
+            r = net.run(prune=prune, collect_counts=True)
+            assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+            cats = net.categories()
+            assert np.array_equal(cats, ref["categories"])
+            got = net.activations(cats)
+            assert same_floats(got, ref["y"])
+            if prune:
+                assert r.compactions >= 1
+            # pruned rows read back as zero rows
+            dead = np.setdiff1d(np.arange(B), cats)[:50].astype(np.int32)
+            assert not net.activations(dead).any()
+
+
+@pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
+def test_gather_kernel_random_sparsity(gc, orc, values):
+    """Irregular rows (0..40 entries), unsorted columns: the general kernel."""
+    N, L, B = 512, 3, 300
+    print("gather values=%s" % values, flush=True)
+    rng = np.random.default_rng(11)
+    layers = [random_csr(rng, N, rng.integers(0, 41, size=N), values) for _ in range(L)]
+    feats = rng.uniform(0, 4, size=(B, N)).astype(np.float32) * (rng.random((B, N)) < 0.3)
+    feats = feats.astype(np.float32)
+    with gc.Network(N, B, L, bias=-0.05) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_GATHER for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, [sort_rows(c) for c in layers], feats, prune=True)
+
+
+@pytest.mark.parametrize("values", ["pow2", "general"])
+@pytest.mark.parametrize("K", [32, 16, 8])
+def test_band_kernel_weight_modes(gc, orc, values, K):
+    """Band structure with per-entry weights: exact products (fma) and general (mul then add)."""
+    N, L, B = 1024, 3, 260
+    print("band weights=%s K=%d" % (values, K), flush=True)
+    rng = np.random.default_rng(K)
+    layers = []
+    for l in range(L):
+        rowptr, col, val = orc.gen_layer_csr(21, l, N, K, 0.0625)
+        if values == "pow2":
+            val = (np.ldexp(1.0, rng.integers(-5, -1, size=len(val))) * rng.choice([-1.0, 1.0], size=len(val))).astype(np.float32)
+        else:
+            val = rng.uniform(-0.1, 0.2, size=len(val)).astype(np.float32)
+        layers.append((rowptr, col, val))
+    feats = rng.uniform(0, 2, size=(B, N)).astype(np.float32)
+    with gc.Network(N, B, L, bias=-0.1) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_BAND for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+
+
+def test_forced_gather_equals_band(gc, orc):
+    N, L, B = 1024, 5, 400
+    print("forced gather", flush=True)
+    layers = [orc.gen_layer_csr(2, l, N) for l in range(L)]
+    feats = orc.gen_features(2, N, 0, B, 0.10, 0.5)
+    with gc.Network(N, B, L, force_kernel=gc.KERNEL_GATHER) as net:
+        net.synth_layers(2)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_GATHER for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+
+
+@pytest.mark.parametrize("rl", [1, 2])
+def test_other_row_block_sizes(gc, orc, rl, monkeypatch):
+    """Row blocks of 64 and 128 rows (the default is 256)."""
+    monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
+    N, L, B = 1024, 4, 333
+    print("rows per lane", rl, flush=True)
+    layers = [orc.gen_layer_csr(9, l, N) for l in range(L)]
+    feats = orc.gen_features(9, N, 0, B, 0.10, 0.5)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(9)
+        net.inspect()
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+
+
+def test_wider_layers(gc, orc):
+    """N=4096 and N=16384 at a few layers, rows sampled."""
+    for N, bias in ((4096, -0.35), (16384, -0.4)):
+        L, B = 4, 520
+        print("wide N=%d" % N, flush=True)
+        layers = [orc.gen_layer_csr(1, l, N) for l in range(L)]
+        feats = orc.gen_features(1, N, 0, B, 0.10, 0.5)
+        with gc.Network(N, B, L) as net:
+            assert net.bias == pytest.approx(bias)
+            net.synth_layers(1)
+            net.inspect()
+            net.synth_features(1, B, 0.10, 0.5)
+            _layer_by_layer(gc, orc, net, layers, feats, prune=True)
