@@ -41,8 +41,13 @@ template <> __device__ __forceinline__ float4 arr_to_vec<4>(const float* a) {
 //   WMODE 0/1: the product is exact (weight is 0 or a power of two), so a fused multiply-add
 //              rounds exactly like the reference's multiply followed by add.
 //   WMODE 2:   general weights: rounded multiply, then rounded add, as the CPU reference does.
+__device__ __forceinline__ float mul_then_add(float acc, float x, float w) {
+#pragma clang fp contract(off)
+    const float p = x * w;
+    return acc + p;
+}
 template <int WMODE> __device__ __forceinline__ float mac(float acc, float x, float w) {
-    if (WMODE == 2) return __fadd_rn(acc, __fmul_rn(x, w));
+    if (WMODE == 2) return mul_then_add(acc, x, w);
     return __builtin_fmaf(x, w, acc);
 }
 
