@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Benchmark of the Sparse DNN inference hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg4] [--layers L]
+
+A step is one pass of the whole layer chain over the full batch (the headline configuration:
+N=65536, 1920 layers, batch 60000, bias -0.45, seed 0, synthetic weights and features generated
+by the library's seeded generator).  Reported on ONE JSON line:
+
+  value        edges/s = batch * N * 32 * layers / t of the SUSTAINED run: pruning off, every
+               layer processes the full batch, nothing skipped (with the literal inputs every row
+               dies within two layers, so the pruned run would be timing empty layers).
+  roofline     band-walk kernel: algorithmic bytes per launch (8*B*N + 8*nnz + 4*(N+1)) over the
+               average launch duration measured with HIP events on the library's stream, against
+               the 8 TB/s HBM peak.
+  cpu_baseline the CPU oracle (oracle/) timed on this box's host cores on a bounded row sample
+               of layer 0 of the same workload.
+  literal      the run as configured (pruning on): edges/s as defined, layers actually launched,
+               per-layer active rows; and the parity gate of a row sample against the oracle.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # name: (neuron, layers, batch, bias)
+    "cfg0": (1024, 120, 6000, -0.30),
+    "cfg1": (1024, 120, 60000, -0.30),
+    "cfg2": (4096, 480, 60000, -0.35),
+    "cfg3": (16384, 1920, 60000, -0.40),
+    "cfg4": (65536, 1920, 60000, -0.45),
+}
+HBM_PEAK_GBPS = 8000.0
+METRIC = "inference edges/sec at N=65536×1920 layers, batch 60000; % HBM roofline"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--config", default="cfg4", choices=sorted(CONFIGS))
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (quick runs)")
+    ap.add_argument("--batch", type=int, default=0, help="override the batch (quick runs)")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build is single-GPU (rows shard trivially, see DESIGN.md); run with --gpus 1")
+        return 2
+
+    import graphchallenge21_amd as gc
+
+    N, L, B, bias = CONFIGS[args.config]
+    if args.layers:
+        L = args.layers
+    if args.batch:
+        B = args.batch
+    seed = args.seed
+    dev_name, n_cu, hbm = gc.device_info()
+    log("device:", dev_name, "CUs", n_cu, "HBM GiB %.0f" % (hbm / 2**30))
+
+    t0 = time.time()
+    net = gc.Network(N, B, L, bias=bias)
+    net.synth_layers(seed)
+    net.inspect()
+    t_inspect = time.time() - t0
+    plans = [net.layer_plan(l) for l in range(L)]
+    n_band = sum(1 for p in plans if p.kernel == gc.KERNEL_BAND)
+    nnz_layer = plans[0].nnz
+    t0 = time.time()
+    net.synth_features(seed, B, 0.10, 0.25)
+    t_features = time.time() - t0
+    log("setup: inspector %.1f s (%d/%d layers BAND), plan upload + features %.1f s" % (t_inspect, n_band, L, t_features))
+
+    # ---- sustained run: the timed steps ---------------------------------------------------
+    for _ in range(args.warmup):
+        net.run(prune=False, time_layers=True)
+    gc.load_library().spdnn_device_synchronize()
+    layer_ms = []
+    t0 = time.perf_counter()
+    ms_events = 0.0
+    for _ in range(args.steps):
+        r = net.run(prune=False, time_layers=True)
+        ms_events += r.ms_total
+        layer_ms.append(net.layer_times().copy())
+    gc.load_library().spdnn_device_synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_per_step = wall_ms / args.steps
+    edges = float(B) * float(nnz_layer) * L
+    value = edges / (ms_per_step * 1e-3)
+    layer_ms = np.concatenate(layer_ms)
+    avg_launch_ms = float(layer_ms.mean())
+    alg_bytes_launch = 8.0 * B * N + 8.0 * nnz_layer + 4.0 * (N + 1)
+    achieved = alg_bytes_launch / (avg_launch_ms * 1e-3) / 1e9
+    sustained_final_active = int(r.active_rows)
+
+    # ---- layer 0 alone (live data), and the literal run -------------------------------------
+    r0 = net.run(prune=False, first_layer=0, n_layers=1, time_layers=True)
+    layer0_ms = float(net.layer_times()[0])
+    lit = net.run(prune=True, collect_counts=True)
+    lit_counts = []
+    for l in range(min(L, 8)):
+        lit_counts.append(int(net.active_count(l)))
+    lit_categories = int(lit.active_rows)
+
+    # ---- measured copy bandwidth --------------------------------------------------------------
+    copy_gbps = gc.measure_copy_bandwidth(1 << 32, 5)
+
+    # ---- CPU baseline + parity gate on a row sample ---------------------------------------------
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        from oracle import oracle as orc
+        cores = orc.get_threads()
+        rows = args.cpu_rows or max(256, min(B, int(7.0e10 * max(cores, 1) / 16 / (N * 32.0))) // 256 * 256)
+        rows = min(rows, B)
+        feats = orc.gen_features(seed, N, 0, rows, 0.10, 0.25)
+        csr0 = orc.gen_layer_csr(seed, 0, N)
+        t0 = time.perf_counter()
+        y1, act1 = orc.layer(feats, csr0, bias)
+        t_cpu = time.perf_counter() - t0
+        cpu = {"value": rows * float(nnz_layer) / t_cpu, "unit": "edges/s", "cores": cores, "kind": "port",
+               "sample": "layer 0 of the same workload on rows 0..%d (%.1f s)" % (rows - 1, t_cpu)}
+        # parity: first three layers of the sample rows, per-layer active ids and activations
+        ref_ids, ref_y = [], []
+        y, gid = feats, np.arange(rows, dtype=np.int32)
+        n_check = min(L, 3)
+        for l in range(n_check):
+            if l == 0:
+                yo, act = y1, act1
+            else:
+                yo, act = orc.layer(y, orc.gen_layer_csr(seed, l, N), bias)
+            ref_ids.append(gid[act != 0].copy())
+            ref_y.append((gid.copy(), yo))
+            y = yo
+        ok_ids, ok_y, max_abs = True, True, 0.0
+        sample = np.arange(rows, dtype=np.int32)
+        for l in range(n_check):
+            net.run(prune=True, first_layer=l, n_layers=1, collect_counts=True)
+            cats = net.categories()
+            ok_ids &= bool(np.array_equal(cats[cats < rows], ref_ids[l]))
+            got = net.activations(sample[: min(rows, 1024)])
+            want = ref_y[l][1][: min(rows, 1024)]
+            ok_y &= bool(np.array_equal(got, want))
+            max_abs = max(max_abs, float(np.abs(got - want).max()))
+        parity = {"rows": int(rows), "layers": n_check, "active_ids_equal": ok_ids,
+                  "activations_bit_equal": ok_y, "max_abs_diff": max_abs}
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "band_walk_traffic.json")
+    if os.path.exists(tpath) and args.config == "cfg4":
+        try:
+            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "edges/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "%s sustained: N=%d, %d layers, batch %d, bias %g, 32 nnz/row of 0.0625, "
+                        "pruning off (every layer at full batch), seed %d" % (args.config, N, L, B, bias, seed),
+            "neuron": N, "layers": L, "batch": B, "bias": bias, "seed": seed,
+            "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "mixed",
+            "final_active_rows": sustained_final_active,
+        },
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+                     "kernel": "band_walk_kernel", "alg_bytes_per_launch": alg_bytes_launch,
+                     "avg_launch_ms": avg_launch_ms, "launches_timed": int(layer_ms.size),
+                     "measured_copy_peak_gbps": copy_gbps,
+                     "frac_of_measured_copy": achieved / copy_gbps if copy_gbps else None},
+        "cpu_baseline": cpu,
+        "literal": {"workload": "same inputs, pruning on", "edges_per_s": edges / (lit.ms_total * 1e-3),
+                    "ms": lit.ms_total, "layers_launched": int(lit.layers_run), "compactions": int(lit.compactions),
+                    "active_rows_first_layers": lit_counts, "categories": lit_categories},
+        "layer0": {"ms": layer0_ms, "achieved_gbps": alg_bytes_launch / (layer0_ms * 1e-3) / 1e9,
+                   "edges_per_s": B * float(nnz_layer) / (layer0_ms * 1e-3)},
+        "parity": parity,
+        "setup_s": {"inspector": t_inspect, "upload_and_features": t_features},
+        "events_ms_per_step": ms_events / args.steps,
+    }
+    print(json.dumps(out))
+    net.close()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <climits>
+#include <cstdlib>
 
 namespace spdnn {
 
@@ -134,51 +135,73 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
         }
 
         if (KT == 32) {
-            // all 32 one-byte selectors of every output sit in scalar registers up front
+            // All 32 one-byte selectors of every output sit in scalar registers up front.  The
+            // 32 entries are processed in 16 stages of two; the LDS reads of stage s+1 are issued
+            // before the arithmetic of stage s, so a wave always has reads in flight while its
+            // multiply-adds issue.
             uint4 sa[OPW], sb[OPW];
-            float4 w_cur[OPW];
+            const float2* wp[OPW];
+            float2 w_cur[OPW];
 #pragma unroll
             for (int i = 0; i < OPW; ++i) {
                 const uint4* sp = reinterpret_cast<const uint4*>(sel + (size_t)v[i] * 8);
                 sa[i] = sp[0];
                 sb[i] = sp[1];
-                if (WMODE) w_cur[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * 32)[0];
-            }
-#pragma unroll
-            for (int m4 = 0; m4 < 8; ++m4) {
-                float4 w_nxt[OPW];
-                if (WMODE && m4 < 7) {
-#pragma unroll
-                    for (int i = 0; i < OPW; ++i)
-                        w_nxt[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * 32)[m4 + 1];
+                if (WMODE) {
+                    wp[i] = reinterpret_cast<const float2*>(wv + (size_t)v[i] * 32);
+                    w_cur[i] = wp[i][0];
                 }
+            }
+            float xbuf[2][2 * OPW][RL];
+#define SPDNN_SLOT(i, e)                                                                              \
+    ((((((e) >> 2) & 3) == 0 ? ((e) < 16 ? sa[i].x : sb[i].x)                                          \
+       : (((e) >> 2) & 3) == 1 ? ((e) < 16 ? sa[i].y : sb[i].y)                                        \
+       : (((e) >> 2) & 3) == 2 ? ((e) < 16 ? sa[i].z : sb[i].z)                                        \
+                               : ((e) < 16 ? sa[i].w : sb[i].w)) >> (8 * ((e) & 3))) & (RING - 1))
 #pragma unroll
-                for (int b = 0; b < 4; ++b) {
+            for (int j = 0; j < 2; ++j)
 #pragma unroll
-                    for (int i = 0; i < OPW; ++i) {
-                        const uint4 sq = m4 < 4 ? sa[i] : sb[i];
-                        const uint32_t sw = (m4 & 3) == 0 ? sq.x : (m4 & 3) == 1 ? sq.y : (m4 & 3) == 2 ? sq.z : sq.w;
-                        const uint32_t slot = (sw >> (8 * b)) & (RING - 1);
-                        V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
-                        float x[RL];
-                        vec_to_arr<RL>(xv, x);
-                        float w = wu;
-                        if (WMODE) w = b == 0 ? w_cur[i].x : b == 1 ? w_cur[i].y : b == 2 ? w_cur[i].z : w_cur[i].w;
+                for (int i = 0; i < OPW; ++i)
+                    vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, j) * COLB),
+                                   xbuf[0][j * OPW + i]);
 #pragma unroll
-                        for (int q = 0; q < RL; ++q) acc[i][q] = mac<WMODE>(acc[i][q], x[q], w);
+            for (int st = 0; st < 16; ++st) {
+                float2 w_nxt[OPW];
+                if (st < 15) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int i = 0; i < OPW; ++i)
+                            vec_to_arr<RL>(*reinterpret_cast<const V*>(
+                                               lane_smem + (size_t)SPDNN_SLOT(i, 2 * (st + 1) + j) * COLB),
+                                           xbuf[(st + 1) & 1][j * OPW + i]);
+                    if (WMODE) {
+#pragma unroll
+                        for (int i = 0; i < OPW; ++i) w_nxt[i] = wp[i][st + 1];
                     }
                 }
-                if (WMODE && m4 < 7) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int i = 0; i < OPW; ++i) {
+                        float w = wu;
+                        if (WMODE) w = j == 0 ? w_cur[i].x : w_cur[i].y;
+#pragma unroll
+                        for (int q = 0; q < RL; ++q)
+                            acc[i][q] = mac<WMODE>(acc[i][q], xbuf[st & 1][j * OPW + i][q], w);
+                    }
+                if (WMODE && st < 15) {
 #pragma unroll
                     for (int i = 0; i < OPW; ++i) w_cur[i] = w_nxt[i];
                 }
-                // pin this trip's arithmetic before the next trip's LDS reads: without it the
-                // compiler issues all 32 reads of every output first and spills the results
+                // pin this stage's arithmetic before the reads of the stage after next: without
+                // it the compiler issues all 32 reads of every output first and spills
 #pragma unroll
                 for (int i = 0; i < OPW; ++i)
 #pragma unroll
                     for (int q = 0; q < RL; ++q) asm volatile("" : "+v"(acc[i][q]) : : "memory");
             }
+#undef SPDNN_SLOT
         } else {
             const uint32_t* sp[OPW];
             const float4* wp[OPW];
@@ -533,13 +556,34 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
 
 }  // namespace
 
+// Tile shapes of the band walk for 256-row blocks, selectable with SPDNN_BAND_SHAPE (tuning knob,
+// default 1):
+//   0  16 waves x 3 outputs per chunk, 128-slot ring (128 KiB LDS, one workgroup per CU)
+//   1   8 waves x 2 outputs per chunk,  64-slot ring ( 64 KiB LDS, two workgroups per CU whose
+//      load / compute / barrier phases interleave)
+//   2   8 waves x 6 outputs per chunk, 128-slot ring (one workgroup per CU, more work per wave)
+static int band_shape() {
+    static int shape = -1;
+    if (shape < 0) {
+        const char* e = getenv("SPDNN_BAND_SHAPE");
+        shape = e ? atoi(e) : 1;
+        if (shape < 0 || shape > 2) shape = 1;
+    }
+    return shape;
+}
+
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     // host-side shape checks: what the kernel and its grid assume
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
         !a.yin || !a.yout || !a.sel || !a.dst || !a.active || (a.wmode != 0 && !a.wv))
         return hipErrorInvalidValue;
     switch (a.rl) {
-        case 4: return launch_band_rl<4, 16, 3, 128>(a, s);
+        case 4:
+            switch (band_shape()) {
+                case 1: { BandLaunch b = a; b.n_cu = 2 * (a.n_cu > 0 ? a.n_cu : 256); return launch_band_rl<4, 8, 2, 64>(b, s); }
+                case 2: return launch_band_rl<4, 8, 6, 128>(a, s);
+                default: return launch_band_rl<4, 16, 3, 128>(a, s);
+            }
         case 2: return launch_band_rl<2, 16, 7, 256>(a, s);
         case 1: return launch_band_rl<1, 16, 7, 256>(a, s);
         default: return hipErrorInvalidValue;
