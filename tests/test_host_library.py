@@ -1,0 +1,225 @@
+"""Host side of the C-ABI library, without a GPU: the library loads and exports every symbol
+the header declares, the inspector's plans reproduce the oracle when emulated on the CPU, the
+loaders and the error paths behave as documented."""
+import ctypes
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from helpers import random_csr, sort_rows
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLD = os.path.join(ROOT, "tests", "golden")
+
+
+def test_library_exports_every_declared_symbol(gc):
+    header = open(os.path.join(ROOT, "include", "spdnn.h")).read()
+    names = sorted(set(re.findall(r"\b(spdnn_[a-z0-9_]+)\s*\(", header)))
+    assert len(names) >= 30
+    lib = ctypes.CDLL(gc.lib_path())
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert gc.load_library().spdnn_version() >= 100
+
+
+def test_reference_tables(gc):
+    # bias by neuron count (reference src/network.cpp:73-78)
+    assert [gc.reference_bias(n) for n in (1024, 4096, 16384, 65536)] == pytest.approx([-0.3, -0.35, -0.4, -0.45])
+    with pytest.raises(gc.SpdnnError):
+        gc.reference_bias(1000)
+    # file names (reference src/network.cpp:14-19)
+    assert gc.weight_file_name("../data", 1024, 0) == "../data/neuron1024/n1024-l1.tsv"
+    assert gc.weight_file_name("/d", 65536, 1919) == "/d/neuron65536/n65536-l1920.tsv"
+    # HashReorder closed form (reference src/reorder/hash.h:14-22): bijection, reorder(65) = 17 at (64, 1024)
+    assert gc.hash_reorder(65, 64, 1024) == 17
+    assert sorted(gc.hash_reorder(v, 64, 1024) for v in range(1024)) == list(range(1024))
+    with pytest.raises(gc.SpdnnError):
+        gc.hash_reorder(1024, 64, 1024)
+
+
+def _emulate_band_layer(net, l, y_phys, value_of):
+    """CPU emulation of the band kernel from the plan arrays: ring selectors, accumulation in
+    plan order, output scattered through dst."""
+    n = net.neuron
+    in_pos, out_at, sel = net.band_plan(l)
+    dst = net.layer_dst(l)
+    k = sel.shape[1]
+    out = np.zeros_like(y_phys)
+    for v in range(n):
+        acc = np.zeros(y_phys.shape[0], np.float32)
+        window = [(v - d) % n for d in range(k)]
+        by_slot = {p % 256: p for p in window}
+        assert len(by_slot) == k
+        for m in range(k):
+            p = by_slot[int(sel[v, m])]
+            acc = acc + y_phys[:, p] * value_of(v, m)
+        y = acc + np.float32(net.bias)
+        out[:, dst[v]] = np.where(y < 0, np.float32(0), np.where(y > 32, np.float32(32), y))
+    return out
+
+
+def test_inspector_band_plan_reproduces_oracle(gc, orc):
+    n, L, b = 512, 3, 6
+    layers = [orc.gen_layer_csr(11, l, n) for l in range(L)]
+    with gc.Network(n, b, L, bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        for l in range(L):
+            p = net.layer_plan(l)
+            assert (p.kernel, p.max_row_nnz, p.regular, p.uniform_value, p.exact_products, p.band_halo, p.nnz) == \
+                   (gc.KERNEL_BAND, 32, 1, 1, 1, 31, 32 * n)
+            in_pos, out_at, sel = net.band_plan(l)
+            assert sorted(in_pos.tolist()) == list(range(n)) and sorted(out_at.tolist()) == list(range(n))
+            # every output reads exactly the window behind its band position
+            rowptr, col, _ = layers[l]
+            for v in (0, 1, 31, 32, n - 1):
+                want = {(v - d) % n for d in range(32)}
+                assert {int(in_pos[i]) for i in col[rowptr[out_at[v]]:rowptr[out_at[v] + 1]]} == want
+        assert np.array_equal(net.input_labelling(L), np.arange(n))
+        feats = orc.gen_features(11, n, 0, b, 0.1, 0.5)
+        y = np.zeros_like(feats)
+        y[:, net.input_labelling(0)] = feats
+        want = feats
+        for l in range(L):
+            y = _emulate_band_layer(net, l, y, lambda v, m: np.float32(0.0625))
+            want, _ = orc.layer(want, layers[l], -0.3)
+            assert np.array_equal(y[:, net.input_labelling(l + 1)], want)
+
+
+def test_inspector_falls_back_to_gather(gc, orc):
+    rng = np.random.default_rng(3)
+    n = 256
+    irregular = random_csr(rng, n, rng.integers(0, 20, size=n), "general")
+    # 8 entries per row AND per column but no band: output j reads inputs j, j+32, j+64, ... (mod n),
+    # i.e. 32 interleaved dense 8x8 blocks
+    cols = np.sort((np.arange(n)[:, None] + 32 * np.arange(8)[None, :]) % n, axis=1)
+    regular_random = (np.arange(0, 8 * n + 1, 8, dtype=np.int32), cols.reshape(-1).astype(np.int32),
+                      np.full(8 * n, 0.0625, np.float32))
+    band = orc.gen_layer_csr(2, 0, n, 8)
+    with gc.Network(n, 4, 4, bias=0.0) as net:
+        net.set_layer_csr(0, *irregular)
+        net.set_layer_csr(1, *regular_random)
+        net.set_layer_csr(2, *band)
+        net.set_layer_csr(3, band[0], band[1], np.linspace(0.1, 0.2, len(band[1])).astype(np.float32))
+        net.inspect()
+        p = [net.layer_plan(l) for l in range(4)]
+        assert [q.kernel for q in p] == [gc.KERNEL_GATHER, gc.KERNEL_GATHER, gc.KERNEL_BAND, gc.KERNEL_BAND]
+        assert (p[0].regular, p[0].exact_products) == (0, 0) and p[0].band_halo == -1
+        assert (p[1].regular, p[1].uniform_value, p[1].exact_products) == (1, 1, 1)
+        assert (p[2].max_row_nnz, p[2].band_halo) == (8, 7)
+        assert (p[3].uniform_value, p[3].exact_products) == (0, 0)
+        with pytest.raises(gc.SpdnnError) as e:
+            net.band_plan(0)
+        assert e.value.code == 2
+        # a gather layer reads its input in natural order; its outputs go where the next layer reads
+        assert np.array_equal(net.input_labelling(0), np.arange(n))
+        assert np.array_equal(net.layer_dst(1), net.input_labelling(2))
+        assert np.array_equal(net.layer_dst(3), np.arange(n)[net.band_plan(3)[1]])
+
+
+def test_forced_gather(gc, orc):
+    with gc.Network(256, 4, 2, bias=-0.3, force_kernel=gc.KERNEL_GATHER) as net:
+        net.synth_layers(0, nnz_per_row=8)
+        net.inspect()
+        assert [net.layer_plan(l).kernel for l in range(2)] == [gc.KERNEL_GATHER] * 2
+
+
+def test_tsv_layer_through_the_library(gc, orc, tmp_path):
+    """A layer written as a shuffled challenge-format TSV and loaded by the library gives the
+    same plan as the same layer handed over as CSR."""
+    n = 256
+    csr = orc.gen_layer_csr(6, 0, n, 8)
+    rowptr, col, val = csr
+    lines = ["%d\t%d\t%.9g\n" % (col[e] + 1, j + 1, val[e]) for j in range(n) for e in range(rowptr[j], rowptr[j + 1])]
+    np.random.default_rng(0).shuffle(lines)
+    p = tmp_path / "n256-l1.tsv"
+    p.write_text("".join(lines))
+    with gc.Network(n, 4, 1, bias=-0.3) as a, gc.Network(n, 4, 1, bias=-0.3) as b:
+        a.load_layer_tsv(0, str(p))
+        b.set_layer_csr(0, *csr)
+        a.inspect()
+        b.inspect()
+        for x, y in zip(a.band_plan(0), b.band_plan(0)):
+            assert np.array_equal(x, y)
+        with pytest.raises(gc.SpdnnError) as e:
+            a.load_layer_tsv(0, str(tmp_path / "missing.tsv"))
+        assert e.value.code == 3 and "does not exists" in e.value.message
+    # the committed fixture layers are plain (non-band) layers of width 64
+    with gc.Network(64, 12, 2, bias=-0.3) as net:
+        net.load_layer_tsv(0, os.path.join(GOLD, "tiny_n64-l1.tsv"))
+        net.load_layer_tsv(1, os.path.join(GOLD, "tiny_n64-l2.tsv"))
+        net.inspect()
+        assert net.layer_plan(0).nnz == 64 * 8
+
+
+def test_argument_and_state_errors(gc, orc):
+    E_ARG, E_STATE = 1, 2
+    with pytest.raises(gc.SpdnnError) as e:
+        gc.Network(0, 4, 1, bias=0.0)
+    assert e.value.code == E_ARG
+    with pytest.raises(gc.SpdnnError):
+        gc.Network(64, 0, 1, bias=0.0)
+    with pytest.raises(gc.SpdnnError):
+        gc.Network(64, 4, 1, bias=float("nan"))
+    n = 64
+    good = sort_rows(random_csr(np.random.default_rng(1), n, 4, "uniform"))
+    with gc.Network(n, 4, 2, bias=-0.1) as net:
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_layer_csr(2, *good)
+        assert e.value.code == E_ARG
+        bad_col = good[1].copy()
+        bad_col[5] = n
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_layer_csr(0, good[0], bad_col, good[2])
+        assert e.value.code == E_ARG and "out of range" in e.value.message
+        bad_val = good[2].copy()
+        bad_val[0] = np.inf
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_layer_csr(0, good[0], good[1], bad_val)
+        assert "non-finite" in e.value.message
+        bad_ptr = good[0].copy()
+        bad_ptr[3] = bad_ptr[2] - 1
+        with pytest.raises(gc.SpdnnError):
+            net.set_layer_csr(0, bad_ptr, good[1], good[2])
+        net.set_layer_csr(0, *good)
+        with pytest.raises(gc.SpdnnError) as e:
+            net.inspect()                           # layer 1 missing
+        assert e.value.code == E_STATE
+        with pytest.raises(gc.SpdnnError) as e:
+            net.run()                               # nothing inspected, no features
+        assert e.value.code == E_STATE
+        with pytest.raises(gc.SpdnnError) as e:
+            net.layer_plan(1)
+        assert e.value.code == E_STATE
+        net.set_layer_csr(1, *good)
+        net.inspect()
+        with pytest.raises(gc.SpdnnError) as e:
+            net.run()                               # still no features
+        assert e.value.code == E_STATE
+
+
+def test_replacing_a_layer(gc, orc):
+    n = 256
+    with gc.Network(n, 4, 1, bias=-0.3) as net:
+        net.set_layer_csr(0, *orc.gen_layer_csr(0, 0, n, 8))
+        net.set_layer_csr(0, *orc.gen_layer_csr(1, 0, n, 8))     # replaces the first hand-over
+        net.inspect()
+        other = gc.Network(n, 4, 1, bias=-0.3)
+        other.set_layer_csr(0, *orc.gen_layer_csr(1, 0, n, 8))
+        other.inspect()
+        assert np.array_equal(net.band_plan(0)[0], other.band_plan(0)[0])
+        other.close()
+
+
+def test_driver_usage_paths():
+    exe = os.path.join(ROOT, "graphchallenge21_amd", "spdnn_network")
+    if not os.path.exists(exe):
+        pytest.skip("driver not built")
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0 and "Usage: exe neuron batch layer" in r.stdout      # reference network.cpp:58-61
+    r = subprocess.run([exe, "1000", "10", "2"], capture_output=True, text=True)
+    assert r.returncode == 2 and "neuron must be one of" in r.stderr
