@@ -160,12 +160,11 @@ def main():
                   "activations_bit_equal": ok_y, "max_abs_diff": max_abs}
 
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "band_walk_traffic.json")
-    if os.path.exists(tpath) and args.config == "cfg4":
-        try:
-            traffic = json.load(open(tpath)).get("hbm_bytes_per_launch")
-        except Exception:
-            traffic = None
+    tpath = os.path.join(ROOT, "profiles", "band_walk_cfg4_hbm_traffic.txt")
+    if os.path.exists(tpath) and args.config == "cfg4" and B == 60000:
+        for line in open(tpath):
+            if line.startswith("hbm_bytes_per_launch"):
+                traffic = float(line.split("=")[1])
 
     out = {
         "metric": METRIC,

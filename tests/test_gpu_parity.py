@@ -197,3 +197,91 @@ def test_wider_layers(gc, orc):
             net.inspect()
             net.synth_features(1, B, 0.10, 0.5)
             _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+
+
+def test_committed_tsv_fixtures(gc, orc):
+    """Weights and features loaded from the challenge-format TSV fixtures by the library's own
+    loaders; expected values from tests/golden/tiny_expected.json (confirmed by the reference's
+    CPU comparators when the fixture was generated)."""
+    import json
+    import os
+    gold = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    exp = json.load(open(os.path.join(gold, "tiny_expected.json")))
+    N, B = 64, 12
+    print("tsv fixtures", flush=True)
+    for bias in (0.0, -1.0, -0.3):
+        e = exp["bias_%g" % bias]
+        with gc.Network(N, B, 2, bias=bias) as net:
+            net.load_layer_tsv(0, os.path.join(gold, "tiny_n64-l1.tsv"))
+            net.load_layer_tsv(1, os.path.join(gold, "tiny_n64-l2.tsv"))
+            net.inspect()
+            net.load_features_tsv(os.path.join(gold, "tiny_features-64.tsv"), B)
+            rows = np.arange(B, dtype=np.int32)
+            for l, key in ((0, "y_layer1_hex"), (1, "y_layer2_hex")):
+                net.run(prune=True, first_layer=l, n_layers=1)
+                assert net.categories().tolist() == e["active_ids"][l]
+                want = np.frombuffer(bytes.fromhex(e[key]), dtype="<f4").reshape(B, N)
+                assert same_floats(net.activations(rows), want)
+
+
+def test_positive_bias_and_error_paths(gc, orc):
+    """bias > 0: dead rows come back to life, so pruning is refused and the unpruned run must
+    still be exact (padding rows must never be reported)."""
+    N, L, B = 256, 3, 70
+    print("positive bias", flush=True)
+    layers = [orc.gen_layer_csr(8, l, N, 8, -0.0625) for l in range(L)]
+    feats = orc.gen_features(8, N, 0, B, 0.0, 0.3)
+    ref = orc.infer(feats, layers, 0.25, prune=False)
+    with gc.Network(N, B, L, bias=0.25) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_features_dense(np.full((B + 1, N), 1.0, np.float32))     # more rows than max_batch
+        assert e.value.code == 1
+        bad = feats.copy()
+        bad[5, 7] = np.nan
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_features_dense(bad)
+        assert e.value.code == 1 and "NaN" in e.value.message
+        net.set_features_dense(feats)
+        with pytest.raises(gc.SpdnnError) as e:
+            net.run(prune=True)
+        assert e.value.code == 6
+        r = net.run(prune=False, collect_counts=True)
+        assert np.array_equal(net.categories(), ref["categories"]) and r.active_rows == len(ref["categories"])
+        assert same_floats(net.activations(np.arange(B, dtype=np.int32)), ref["y"])
+
+
+def test_full_batch_properties_cfg1(gc, orc):
+    """N=1024, 120 layers, batch 60000 (the first full-GPU configuration), survivor densities so
+    that the late layers carry rows: size-independent properties plus an oracle sample."""
+    N, L, B = 1024, 120, 60000
+    print("cfg1 full batch", flush=True)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, B, 0.10, 0.50)
+        rp = net.run(prune=True, collect_counts=True)
+        counts_p = [net.active_count(l) for l in range(L)]
+        cats_p = net.categories()
+        sample = np.concatenate([cats_p[:40], cats_p[-40:]]).astype(np.int32)
+        y_p = net.activations(sample)
+        ru = net.run(prune=False, collect_counts=True)
+        counts_u = [net.active_count(l) for l in range(L)]
+        cats_u = net.categories()
+        y_u = net.activations(sample)
+    assert counts_p == counts_u and counts_p == sorted(counts_p, reverse=True)
+    assert 0 < counts_p[-1] < B and rp.compactions >= 1 and ru.compactions == 0
+    assert np.array_equal(cats_p, cats_u) and np.array_equal(cats_p, np.sort(cats_p))
+    assert same_floats(y_p, y_u)
+    # oracle on a row sample: rows are independent, so the sample's survivors must be exactly
+    # the categories that fall inside the sample
+    S = 1500
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
+    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.50), layers, -0.3, prune=True)
+    assert np.array_equal(cats_p[cats_p < S], ref["categories"])
+    k = int((sample < S).sum())
+    if k:
+        pos = np.searchsorted(ref["gid"], sample[:k])
+        assert same_floats(y_p[:k], ref["y"][pos])
