@@ -497,25 +497,36 @@ __global__ __launch_bounds__(256) void copy_f4_kernel(const float4* __restrict__
     for (; i < n4; i += stride) dst[i] = src[i];
 }
 
-// Segment length for the band walk: a multiple of the chunk T.  More segments fill the 256 CUs
-// more evenly (one workgroup per CU at a time: the ring takes most of the LDS), fewer segments
-// load fewer halo columns; score both and take the best.
-int choose_seglen(int N, int K, int T, int nblk, int n_cu) {
+// Segment lengths for the band walk, best first: multiples of the chunk T.  More segments fill the
+// CUs more evenly, fewer segments load fewer halo columns; score both.  `slots` is the number of
+// workgroups resident at once (CUs x workgroups per CU).
+int rank_seglens(int N, int K, int T, int nblk, int slots, int* out, int max_out) {
     const int nchunks = (N + T - 1) / T;
-    int best_len = nchunks * T;
-    double best = -1.0;
+    double best[8];
+    int n = 0;
+    if (max_out > 8) max_out = 8;
+    int last_nseg = -1;
     for (int cps = nchunks; cps >= 1; --cps) {  // chunks per segment
         const int nseg = (nchunks + cps - 1) / cps;
         if (nseg > 65535) break;
+        if (nseg == last_nseg) continue;  // same grid as a longer segment: keep the balanced one below
+        last_nseg = nseg;
+        const int cps_bal = (nchunks + nseg - 1) / nseg;  // spread the chunks evenly over nseg segments
         const long long wgs = (long long)nblk * nseg;
-        const long long rounds = (wgs + n_cu - 1) / n_cu;
-        const double fill = (double)wgs / (double)(rounds * n_cu);
-        const double halo = 1.0 / (1.0 + 0.25 * (double)(K - 1) / (double)(cps * T));
-        // a round costs cps chunks (+ prologue); prefer fuller rounds, then fewer halos
+        const long long rounds = (wgs + slots - 1) / slots;
+        const double fill = (double)wgs / (double)(rounds * slots);
+        const double halo = 1.0 / (1.0 + 0.25 * (double)(K - 1) / (double)(cps_bal * T));
         const double score = fill * halo;
-        if (score > best + 1e-9) { best = score; best_len = cps * T; }
+        int pos = n;
+        while (pos > 0 && score > best[pos - 1] + 1e-9) --pos;
+        if (pos >= max_out) continue;
+        const int stop = n < max_out ? n : max_out - 1;
+        for (int i = stop; i > pos; --i) { best[i] = best[i - 1]; out[i] = out[i - 1]; }
+        best[pos] = score;
+        out[pos] = cps_bal * T;
+        if (n < max_out) ++n;
     }
-    return best_len;
+    return n;
 }
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
@@ -530,8 +541,12 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
         if (e != hipSuccess) return e;
         attr_done = true;
     }
-    const int seglen = choose_seglen(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256);
+    int seglen = a.seglen;
+    if (seglen <= 0 || (seglen % T) != 0) {
+        if (rank_seglens(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256, &seglen, 1) < 1) return hipErrorInvalidValue;
+    }
     const int nseg = (a.N + seglen - 1) / seglen;
+    if (nseg > 65535) return hipErrorInvalidValue;
     dim3 grid(a.nblk, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.N, a.K,
                        seglen, a.stamp, a.wu, a.bias, a.clampv);
@@ -556,20 +571,42 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
 
 }  // namespace
 
-// Tile shapes of the band walk for 256-row blocks, selectable with SPDNN_BAND_SHAPE (tuning knob,
-// default 1):
+// Tile shapes of the band walk for 256-row blocks:
 //   0  16 waves x 3 outputs per chunk, 128-slot ring (128 KiB LDS, one workgroup per CU)
 //   1   8 waves x 2 outputs per chunk,  64-slot ring ( 64 KiB LDS, two workgroups per CU whose
 //      load / compute / barrier phases interleave)
-//   2   8 waves x 6 outputs per chunk, 128-slot ring (one workgroup per CU, more work per wave)
-static int band_shape() {
+// BandLaunch::shape < 0 takes SPDNN_BAND_SHAPE from the environment (default 1).  The smaller row
+// blocks (64 and 128 rows) have one shape each.
+static int env_band_shape() {
     static int shape = -1;
     if (shape < 0) {
         const char* e = getenv("SPDNN_BAND_SHAPE");
         shape = e ? atoi(e) : 1;
-        if (shape < 0 || shape > 2) shape = 1;
+        if (shape < 0 || shape > 1) shape = 1;
     }
     return shape;
+}
+
+int band_shape_count(int rl) { return rl == 4 ? 2 : 1; }
+
+static int resolve_shape(int rl, int shape) {
+    if (rl != 4) return 0;
+    if (shape < 0) return env_band_shape();
+    return shape > 1 ? 1 : shape;
+}
+
+int band_chunk_outputs(int rl, int shape) {
+    if (rl == 4) return resolve_shape(rl, shape) == 1 ? 16 : 48;
+    return 112;
+}
+
+int band_workgroups_per_cu(int rl, int shape) {
+    if (rl == 4) return resolve_shape(rl, shape) == 1 ? 2 : 1;
+    return rl == 1 ? 2 : 1;
+}
+
+int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out) {
+    return rank_seglens(N, K, band_chunk_outputs(rl, shape), nblk, n_cu * band_workgroups_per_cu(rl, shape), out, max_out);
 }
 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
@@ -577,15 +614,14 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
         !a.yin || !a.yout || !a.sel || !a.dst || !a.active || (a.wmode != 0 && !a.wv))
         return hipErrorInvalidValue;
+    BandLaunch b = a;
+    b.n_cu = (a.n_cu > 0 ? a.n_cu : 256) * band_workgroups_per_cu(a.rl, a.shape);
     switch (a.rl) {
         case 4:
-            switch (band_shape()) {
-                case 1: { BandLaunch b = a; b.n_cu = 2 * (a.n_cu > 0 ? a.n_cu : 256); return launch_band_rl<4, 8, 2, 64>(b, s); }
-                case 2: return launch_band_rl<4, 8, 6, 128>(a, s);
-                default: return launch_band_rl<4, 16, 3, 128>(a, s);
-            }
-        case 2: return launch_band_rl<2, 16, 7, 256>(a, s);
-        case 1: return launch_band_rl<1, 16, 7, 256>(a, s);
+            if (resolve_shape(4, a.shape) == 1) return launch_band_rl<4, 8, 2, 64>(b, s);
+            return launch_band_rl<4, 16, 3, 128>(b, s);
+        case 2: return launch_band_rl<2, 16, 7, 256>(b, s);
+        case 1: return launch_band_rl<1, 16, 7, 256>(b, s);
         default: return hipErrorInvalidValue;
     }
 }

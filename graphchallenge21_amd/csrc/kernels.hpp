@@ -25,6 +25,8 @@ struct BandLaunch {
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
     int n_cu;
+    int shape = -1;          // tile shape (see launch_band); < 0 = default
+    int seglen = 0;          // band positions per workgroup; 0 = heuristic
 };
 
 struct GatherLaunch {
@@ -41,6 +43,10 @@ struct GatherLaunch {
 };
 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s);
+// Tuning space of the band walk: number of tile shapes for a row-block size, and the best-ranked
+// segment lengths for a shape (used by the run-time selection in spdnn_run).
+int band_shape_count(int rl);
+int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
 
 // Active-row scan: rows with active[row] == stamp and gid[row] >= 0 survive, in order.

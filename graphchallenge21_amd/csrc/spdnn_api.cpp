@@ -159,6 +159,11 @@ struct spdnn_net {
     std::vector<char> pending; // layer has an inspection job in flight
     std::vector<int64_t> counts;
     std::vector<float> layer_ms;
+
+    // measured band-walk configuration per (row blocks, entries per row)
+    struct Tuned { int nblk, K, shape, seglen; };
+    std::vector<Tuned> tuned;
+    bool autotune = true;
 };
 
 namespace {
@@ -297,6 +302,8 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     n->counts.assign((size_t)layers, -1);
     n->layer_ms.assign((size_t)layers, 0.0f);
     n->pool.reset(new JobPool(host_threads()));
+    if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
+    if (getenv("SPDNN_BAND_SHAPE")) n->autotune = false;  // an explicit shape wins
     *out = n;
     return SPDNN_OK;
 }
@@ -421,6 +428,7 @@ int spdnn_inspect(spdnn_net* n) {
     }
     n->pool->wait_all();
     if (n->uploaded) free_device(n);  // plans changed: upload again on next use
+    n->tuned.clear();
     n->inspected = true;
     return SPDNN_OK;
 }
@@ -579,14 +587,67 @@ int spdnn_default_run_options(spdnn_run_options* o) {
     return SPDNN_OK;
 }
 
+static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp) {
+    const LayerPlan& p = n->layers[(size_t)l];
+    const DevLayer& d = n->dl[(size_t)l];
+    BandLaunch a{};
+    a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
+    a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
+    a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
+    a.shape = -1; a.seglen = 0;
+    return a;
+}
+
+static const spdnn_net::Tuned* find_tuned(const spdnn_net* n, int nblk, int K) {
+    for (const auto& t : n->tuned)
+        if (t.K == K && nblk * 8 >= t.nblk * 7 && nblk * 8 <= t.nblk * 9) return &t;
+    return nullptr;
+}
+
+// Run-time kernel selection for band layers (the measured half of the inspector's choice): time
+// each tile shape with its two best-ranked segment lengths on the real buffers of layer l and keep
+// the fastest for this row-block count.  The trial outputs land in the buffer the layer writes
+// anyway; every trial uses a fresh row stamp.
+static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk) {
+    const LayerPlan& p = n->layers[(size_t)l];
+    hipEvent_t e0, e1;
+    HIPCHK(hipEventCreate(&e0));
+    HIPCHK(hipEventCreate(&e1));
+    spdnn_net::Tuned best{nblk, p.kmax, -1, 0};
+    float best_ms = 0.0f;
+    hipError_t err = hipSuccess;
+    for (int shape = 0; shape < band_shape_count(n->rl) && err == hipSuccess; ++shape) {
+        int lens[2];
+        const int nc = band_seglen_candidates(n->N, p.kmax, nblk, n->rl, shape, n->n_cu, lens, 2);
+        for (int c = 0; c < nc && err == hipSuccess; ++c) {
+            BandLaunch a = band_args(n, l, in, out, nblk, 0);
+            a.shape = shape;
+            a.seglen = lens[c];
+            float ms = 0.0f;
+            for (int rep = 0; rep < 2 && err == hipSuccess; ++rep) {  // first launch warms the code path
+                a.stamp = ++n->stamp;
+                if (rep == 1) err = hipEventRecord(e0, n->stream);
+                if (err == hipSuccess) err = launch_band(a, n->stream);
+                if (rep == 1 && err == hipSuccess) err = hipEventRecord(e1, n->stream);
+            }
+            if (err == hipSuccess) err = hipEventSynchronize(e1);
+            if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+            if (err == hipSuccess && (best.shape < 0 || ms < best_ms)) { best.shape = shape; best.seglen = lens[c]; best_ms = ms; }
+        }
+    }
+    hipEventDestroy(e0);
+    hipEventDestroy(e1);
+    if (err != hipSuccess) return fail(SPDNN_E_DEVICE, std::string("band tuning: ") + hipGetErrorString(err));
+    if (best.shape >= 0) n->tuned.push_back(best);
+    return SPDNN_OK;
+}
+
 static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
-        BandLaunch a{};
-        a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
-        a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
-        a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
+        BandLaunch a = band_args(n, l, in, out, nblk, stamp);
+        if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) { a.shape = t->shape; a.seglen = t->seglen; }
         return launch_band(a, n->stream);
     }
     GatherLaunch g{};
@@ -636,6 +697,10 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         }
         float* out = (n->cur == n->A) ? n->C : n->A;
         const int nblk = n->carried / n->RB;
+        if (n->autotune && p.kernel == SPDNN_KERNEL_BAND && last - l + 1 >= 8 && !find_tuned(n, nblk, p.kmax)) {
+            int rc = tune_band(n, l, n->cur, out, nblk);
+            if (rc) return rc;
+        }
         const int stamp = ++n->stamp;
         if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
         HIPCHK(launch_layer(n, l, n->cur, out, nblk, stamp));
