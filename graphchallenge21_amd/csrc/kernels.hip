@@ -52,6 +52,31 @@ template <int WMODE> __device__ __forceinline__ float mac(float acc, float x, fl
     return __builtin_fmaf(x, w, acc);
 }
 
+// End of a layer kernel: stamp the rows of this lane that produced a nonzero output.  With a
+// counter, the first wave to stamp a row (atomic exchange) also counts it, one atomic add per
+// wave, so the number of active rows after the layer needs no separate pass.
+template <int RL>
+__device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict__ active, size_t row0,
+                                           int stamp, int32_t* __restrict__ count_out) {
+    if (count_out == nullptr) {
+#pragma unroll
+        for (int q = 0; q < RL; ++q)
+            if (nz[q] > 0.0f) active[row0 + q] = stamp;
+        return;
+    }
+    int newly = 0;
+#pragma unroll
+    for (int q = 0; q < RL; ++q)
+        if (nz[q] > 0.0f) newly += (atomicExch(&active[row0 + q], stamp) != stamp) ? 1 : 0;
+    newly += __shfl_down(newly, 32, 64);
+    newly += __shfl_down(newly, 16, 64);
+    newly += __shfl_down(newly, 8, 64);
+    newly += __shfl_down(newly, 4, 64);
+    newly += __shfl_down(newly, 2, 64);
+    newly += __shfl_down(newly, 1, 64);
+    if ((threadIdx.x & 63) == 0 && newly > 0) atomicAdd(count_out, newly);
+}
+
 __device__ __forceinline__ float relu_clamp(float y, float clampv) {
     // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
     return __builtin_amdgcn_fmed3f(y, 0.0f, clampv);
@@ -77,7 +102,7 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
     const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int N, int Krt, int seglen, int stamp, float wu, float bias, float clampv) {
+    int32_t* __restrict__ count_out, int N, int Krt, int seglen, int stamp, float wu, float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     using V = typename VecOf<RL>::type;
     constexpr int T = NW * OPW;
@@ -272,10 +297,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
         }
         __syncthreads();
     }
-
-#pragma unroll
-    for (int q = 0; q < RL; ++q)
-        if (nz[q] > 0.0f) active[(size_t)rb * RB + loff + q] = stamp;
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -288,7 +310,8 @@ template <int RL, int WMODE>
 __global__ __launch_bounds__(256) void gather_kernel(
     const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ cols,
     const int32_t* __restrict__ rowlen, const float* __restrict__ wv, const int32_t* __restrict__ dst,
-    int32_t* __restrict__ active, int N, int kmax, int opg, int stamp, float bias, float clampv) {
+    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int kmax, int opg, int stamp,
+    float bias, float clampv) {
     using V = typename VecOf<RL>::type;
     constexpr int RB = 64 * RL;
     const int lane = threadIdx.x & 63;
@@ -329,54 +352,53 @@ __global__ __launch_bounds__(256) void gather_kernel(
         }
         *reinterpret_cast<V*>(yout + (size_t)dst[j] * RB + loff) = arr_to_vec<RL>(y);
     }
-#pragma unroll
-    for (int q = 0; q < RL; ++q)
-        if (nz[q] > 0.0f) active[(size_t)rb * RB + loff + q] = stamp;
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
 }
 
 // ------------------------------------------------------------------------------------------
-// Active-row scan (one workgroup): wave64 ballot + popcount prefix inside a wave, an LDS scan
-// over the 16 wave totals, a running base across 1024-row chunks.  Stable: survivors keep
-// their order, as the reference's host loop does (all_network.cu:455-463).
+// Active-row scan (one workgroup of 1024 threads).  Thread t owns the contiguous strip of rows
+// [t*S, (t+1)*S): it counts its survivors, the workgroup takes an exclusive prefix over the 1024
+// counts (wave64 ballot-free shuffle scan inside a wave, LDS across the 16 waves), and every
+// thread then writes its survivors in order.  Stable: survivors keep their order, as the
+// reference's host loop does (all_network.cu:455-463).
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void scan_active_kernel(
     const int32_t* __restrict__ active, const int32_t* __restrict__ gid, int rows, int stamp,
     int32_t* __restrict__ count, int32_t* __restrict__ alive_src, int32_t* __restrict__ alive_gid) {
     __shared__ int wave_tot[16];
-    __shared__ int base_s;
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0) base_s = 0;
+    const int S = (rows + 1023) / 1024;
+    const int r0 = threadIdx.x * S;
+    const int r1 = min(rows, r0 + S);
+    int mine = 0;
+    for (int r = r0; r < r1; ++r) mine += (active[r] == stamp && gid[r] >= 0) ? 1 : 0;
+    // inclusive scan of `mine` inside the wave
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += up;
+    }
+    if (lane == 63) wave_tot[wave] = incl;
     __syncthreads();
-    for (int r0 = 0; r0 < rows; r0 += 1024) {
-        const int r = r0 + threadIdx.x;
-        int g = -1;
-        bool alive = false;
-        if (r < rows) {
-            g = gid[r];
-            alive = (active[r] == stamp) && (g >= 0);
-        }
-        const unsigned long long mask = __ballot(alive);
-        const int before = __popcll(mask & ((1ull << lane) - 1ull));
-        if (lane == 0) wave_tot[wave] = __popcll(mask);
-        __syncthreads();
-        int wbase = 0;
-        for (int w = 0; w < wave; ++w) wbase += wave_tot[w];
-        const int base = base_s;
-        if (alive) {
-            const int k = base + wbase + before;
+    int base = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const int t = wave_tot[w];
+        if (w < wave) base += t;
+        total += t;
+    }
+    int k = base + incl - mine;
+    for (int r = r0; r < r1; ++r) {
+        const int g = gid[r];
+        if (active[r] == stamp && g >= 0) {
             alive_src[k] = r;
             alive_gid[k] = g;
+            ++k;
         }
-        __syncthreads();
-        if (threadIdx.x == 0) {
-            int t = 0;
-            for (int w = 0; w < 16; ++w) t += wave_tot[w];
-            base_s = base + t;
-        }
-        __syncthreads();
     }
-    if (threadIdx.x == 0) count[0] = base_s;
+    if (threadIdx.x == 0) count[0] = total;
 }
 
 // Repack survivors into dense row blocks.  Thread = destination row slot; loops over a chunk of
@@ -548,8 +570,8 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     const int nseg = (a.N + seglen - 1) / seglen;
     if (nseg > 65535) return hipErrorInvalidValue;
     dim3 grid(a.nblk, nseg), block(NW * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.N, a.K,
-                       seglen, a.stamp, a.wu, a.bias, a.clampv);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.count_out,
+                       a.N, a.K, seglen, a.stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
 }
 
@@ -635,7 +657,7 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
     if (grid.y > 65535) return hipErrorInvalidValue;
 #define SPDNN_GATHER(RLv, WM)                                                                         \
     hipLaunchKernelGGL((gather_kernel<RLv, WM>), grid, block, 0, s, a.yin, a.yout, a.cols, a.rowlen,  \
-                       a.wv, a.dst, a.active, a.N, a.kmax, opg, a.stamp, a.bias, a.clampv)
+                       a.wv, a.dst, a.active, a.count_out, a.N, a.kmax, opg, a.stamp, a.bias, a.clampv)
     const bool exact = a.wmode != 2;
     switch (a.rl) {
         case 4: if (exact) SPDNN_GATHER(4, 1); else SPDNN_GATHER(4, 2); break;

@@ -21,6 +21,7 @@ struct BandLaunch {
     const float* wv;         // [N][K] weights in accumulation order, or nullptr (uniform exact value)
     const int32_t* dst;      // [N] physical output column per band position
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
+    int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, K, nblk, stamp, rl;
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
@@ -37,6 +38,7 @@ struct GatherLaunch {
     const float* wv;         // [N][kmax]
     const int32_t* dst;      // [N]
     int32_t* active;
+    int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, kmax, nblk, stamp, rl;
     int wmode;               // 1 fma (exact products), 2 mul then add
     float bias, clampv;

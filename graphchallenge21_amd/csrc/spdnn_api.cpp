@@ -143,6 +143,9 @@ struct spdnn_net {
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
+    int32_t* d_counts = nullptr; // per-layer active-row counters (device)
+    int32_t* h_counts = nullptr; // pinned mirror
+    std::vector<hipEvent_t> ev_count;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     std::vector<hipEvent_t> ev_layer;
 
@@ -191,6 +194,8 @@ int ensure_device(spdnn_net* n) {
     HIPCHK(hipMalloc(&n->d_count, 64));
     HIPCHK(hipMalloc(&n->d_nonfinite, 64));
     HIPCHK(hipHostMalloc(&n->h_count, 64));
+    HIPCHK(hipMalloc(&n->d_counts, (size_t)n->L * 4));
+    HIPCHK(hipHostMalloc(&n->h_counts, (size_t)n->L * 4));
     HIPCHK(hipMemset(n->d_active, 0, rows * 4));
     n->dev_ready = true;
     return SPDNN_OK;
@@ -318,6 +323,9 @@ int spdnn_destroy(spdnn_net* n) {
         hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp); hipFree(n->d_alive_src);
         hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
         hipHostFree(n->h_count);
+        hipFree(n->d_counts);
+        hipHostFree(n->h_counts);
+        for (hipEvent_t e : n->ev_count) hipEventDestroy(e);
         for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
         hipEventDestroy(n->ev_start); hipEventDestroy(n->ev_stop);
         hipStreamDestroy(n->stream);
@@ -594,7 +602,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, in
     a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
-    a.shape = -1; a.seglen = 0;
+    a.shape = -1; a.seglen = 0; a.count_out = nullptr;
     return a;
 }
 
@@ -642,17 +650,19 @@ static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk)
     return SPDNN_OK;
 }
 
-static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp) {
+static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp,
+                               int32_t* count_out) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
         BandLaunch a = band_args(n, l, in, out, nblk, stamp);
+        a.count_out = count_out;
         if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) { a.shape = t->shape; a.seglen = t->seglen; }
         return launch_band(a, n->stream);
     }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
-    g.active = n->d_active; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
+    g.active = n->d_active; g.count_out = count_out; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
     g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv;
     return launch_gather(g, n->stream);
 }
@@ -673,25 +683,47 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     float thr = opt.compact_threshold > 0.0f ? opt.compact_threshold : 0.75f;
     if (thr > 1.0f) thr = 1.0f;
 
-    if (opt.time_layers && n->ev_layer.size() < (size_t)(2 * n->L)) {
+    if (opt.time_layers) {
         while (n->ev_layer.size() < (size_t)(2 * n->L)) {
             hipEvent_t e;
             HIPCHK(hipEventCreate(&e));
             n->ev_layer.push_back(e);
         }
     }
+    while (n->ev_count.size() < (size_t)n->L) {
+        hipEvent_t e;
+        HIPCHK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+        n->ev_count.push_back(e);
+    }
     const int first = opt.first_layer, last = first + nl - 1;
     for (int l = first; l <= last; ++l) { n->counts[(size_t)l] = -1; n->layer_ms[(size_t)l] = 0.0f; }
 
+    // With bias <= 0 padding rows stay zero, so the layer kernels can count the rows they stamp
+    // (one atomic per wave) and no scan is needed for the per-layer counts.  Otherwise the scan,
+    // which masks padding rows, counts - only when counts are asked for.
+    const bool fused_count = n->bias <= 0.0f;
+    const bool scan_count = !fused_count && opt.collect_counts;
+    const bool have_counts = fused_count || scan_count;
+    if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
+
+    // Pruning never waits for the layer it just launched: the host looks at the count of the
+    // layer `lookahead` launches back (already finished in steady state).  Counts only go down
+    // (bias <= 0), so an older count is a safe upper bound for sizing a repack, and a zero count
+    // means every later layer is all zero.
+    const int lookahead = 2;
     spdnn_run_result r{};
-    int64_t entering = n->alive;  // rows entering the next layer (for the byte model)
+    const int64_t alive_at_start = n->alive;
     std::vector<int> timed;
+    int known = first;               // counts of layers < known have been read by the host
+    int64_t newest_count = -1;       // count of layer known-1
+    bool dead = n->carried == 0;
+    int last_launched = -1, last_stamp = 0;
+
     HIPCHK(hipEventRecord(n->ev_start, n->stream));
     for (int l = first; l <= last; ++l) {
         const LayerPlan& p = n->layers[(size_t)l];
         r.edges += (double)n->batch * (double)p.info.nnz;
-        if (n->carried == 0) {  // every row died earlier: the remaining outputs are all zero
-            n->counts[(size_t)l] = 0;
+        if (dead) {  // every row died earlier: the remaining outputs are all zero
             n->cur_layer = l + 1;
             continue;
         }
@@ -700,45 +732,61 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         if (n->autotune && p.kernel == SPDNN_KERNEL_BAND && last - l + 1 >= 8 && !find_tuned(n, nblk, p.kmax)) {
             int rc = tune_band(n, l, n->cur, out, nblk);
             if (rc) return rc;
+            if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + l, 0, 4, n->stream));  // the trials counted too
         }
         const int stamp = ++n->stamp;
         if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
-        HIPCHK(launch_layer(n, l, n->cur, out, nblk, stamp));
+        HIPCHK(launch_layer(n, l, n->cur, out, nblk, stamp, fused_count ? n->d_counts + l : nullptr));
         if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back(l); }
         r.layers_run++;
-        r.alg_bytes += 8.0 * (double)(opt.prune ? entering : n->batch) * (double)n->N + 8.0 * (double)p.info.nnz +
-                       4.0 * (double)(n->N + 1);
+        last_launched = l;
+        last_stamp = stamp;
         n->cur = out;
         n->cur_layer = l + 1;
-        const bool need_count = opt.prune || opt.collect_counts;
-        if (need_count || l == last) {
+        if (scan_count) {
             HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, stamp, n->d_count, n->d_alive_src,
                                       n->d_alive_gid, n->stream));
-            n->alive_list_valid = true;
-            HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
-            HIPCHK(hipStreamSynchronize(n->stream));
-            const int64_t cnt = n->h_count[0];
-            n->counts[(size_t)l] = cnt;
-            n->alive = cnt;
-            entering = cnt;
-            if (opt.prune) {
-                if (cnt == 0) {
-                    n->carried = 0;
-                } else if ((double)cnt <= (double)thr * (double)n->carried && l + 1 < n->L) {
-                    const int nb = (int)((cnt + n->RB - 1) / n->RB);
-                    if (nb * n->RB < n->carried) {
-                        float* dstbuf = (n->cur == n->A) ? n->C : n->A;
-                        HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid,
-                                             n->d_gid_tmp, n->N, n->rl, nb, n->stream));
-                        std::swap(n->d_gid, n->d_gid_tmp);
-                        n->gid_dirty = true;
-                        n->cur = dstbuf;
-                        n->carried = nb * n->RB;
-                        r.compactions++;
-                    }
-                }
+            HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
+        }
+        if (have_counts) {
+            HIPCHK(hipMemcpyAsync(n->h_counts + l, n->d_counts + l, 4, hipMemcpyDeviceToHost, n->stream));
+            HIPCHK(hipEventRecord(n->ev_count[(size_t)l], n->stream));
+        }
+        if (!opt.prune) continue;
+
+        const int upto = l - lookahead;  // newest layer whose count the host waits for
+        while (known <= upto && !dead) {
+            HIPCHK(hipEventSynchronize(n->ev_count[(size_t)known]));
+            newest_count = n->h_counts[known];
+            n->counts[(size_t)known] = newest_count;
+            if (newest_count == 0) dead = true;
+            ++known;
+        }
+        if (dead) { n->carried = 0; continue; }
+        if (newest_count > 0 && (double)newest_count <= (double)thr * (double)n->carried && l + 1 < n->L) {
+            const int nb = (int)((newest_count + n->RB - 1) / n->RB);  // upper bound of what is alive now
+            if (nb * n->RB < n->carried) {
+                float* dstbuf = (n->cur == n->A) ? n->C : n->A;
+                HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, stamp, n->d_count, n->d_alive_src,
+                                          n->d_alive_gid, n->stream));
+                HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
+                                     n->N, n->rl, nb, n->stream));
+                std::swap(n->d_gid, n->d_gid_tmp);
+                n->gid_dirty = true;
+                n->cur = dstbuf;
+                n->carried = nb * n->RB;
+                r.compactions++;
             }
         }
+    }
+    // categories of the last layer: survivor list by the scan (after a repack the row slots moved,
+    // but the stamps of the last layer were written after it, so they match the current slots)
+    n->alive_list_valid = false;
+    if (!dead && last_launched >= 0 && last_launched == last) {
+        HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, last_stamp, n->d_count, n->d_alive_src,
+                                  n->d_alive_gid, n->stream));
+        HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
+        n->alive_list_valid = true;
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
@@ -749,7 +797,25 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         n->layer_ms[(size_t)l] = ms;
         r.ms_kernels += ms;
     }
-    if (n->carried == 0) { n->alive = 0; }
+    // per-layer counts: everything that was launched has finished now
+    bool zero_seen = false;
+    for (int l = first; l <= last; ++l) {
+        if (zero_seen) { n->counts[(size_t)l] = 0; continue; }
+        if (l <= last_launched && have_counts) n->counts[(size_t)l] = n->h_counts[l];
+        else if (l > last_launched) n->counts[(size_t)l] = (last_launched >= first || n->carried == 0) ? 0 : -1;
+        if (n->counts[(size_t)l] == 0) zero_seen = true;
+    }
+    if (dead || zero_seen) { n->carried = opt.prune ? 0 : n->carried; n->alive = 0; }
+    else if (n->alive_list_valid) n->alive = n->h_count[0];
+    if (n->alive == 0) n->alive_list_valid = true;  // the empty list
+    // byte model: rows entering each launched layer
+    int64_t entering = alive_at_start;
+    for (int l = first; l <= last_launched; ++l) {
+        const LayerPlan& p = n->layers[(size_t)l];
+        r.alg_bytes += 8.0 * (double)((opt.prune && have_counts) ? entering : n->batch) * (double)n->N +
+                       8.0 * (double)p.info.nnz + 4.0 * (double)(n->N + 1);
+        if (n->counts[(size_t)l] >= 0) entering = n->counts[(size_t)l];
+    }
     r.active_rows = n->alive;
     r.carried_rows = n->carried;
     if (res) *res = r;
