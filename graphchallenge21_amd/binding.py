@@ -29,7 +29,7 @@ class LayerPlan(C.Structure):
 class RunOptions(C.Structure):
     _fields_ = [("prune", C.c_int32), ("first_layer", C.c_int32), ("n_layers", C.c_int32),
                 ("collect_counts", C.c_int32), ("time_layers", C.c_int32),
-                ("compact_threshold", C.c_float), ("reserved", C.c_int32 * 4)]
+                ("compact_threshold", C.c_float), ("fuse_layers", C.c_int32), ("reserved", C.c_int32 * 3)]
 
 
 class RunResult(C.Structure):
@@ -236,12 +236,13 @@ class Network:
 
     # inference
     def run(self, prune=True, first_layer=0, n_layers=-1, collect_counts=False, time_layers=False,
-            compact_threshold=0.75):
+            compact_threshold=0.75, fuse_layers=0):
         opt = RunOptions()
         _check(self._lib.spdnn_default_run_options(C.byref(opt)))
         opt.prune, opt.first_layer, opt.n_layers = int(prune), first_layer, n_layers
         opt.collect_counts, opt.time_layers = int(collect_counts), int(time_layers)
         opt.compact_threshold = compact_threshold
+        opt.fuse_layers = fuse_layers
         res = RunResult()
         _check(self._lib.spdnn_run(self._h, C.byref(opt), C.byref(res)))
         return res

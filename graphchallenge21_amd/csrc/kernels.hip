@@ -77,6 +77,22 @@ __device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict_
     if ((threadIdx.x & 63) == 0 && newly > 0) atomicAdd(count_out, newly);
 }
 
+// Block-level pruning: true if no row of this lane's row block was stamped by the previous layer
+// (prev_stamp 0 = do not check).  Another workgroup of the same launch (a different band segment
+// of the same row block) may already have re-stamped rows with this launch's stamp; such rows
+// were alive too.  Uniform over the workgroup; contains a barrier.
+template <int RL>
+__device__ __forceinline__ bool block_is_dead(const int32_t* active, size_t row0, int prev_stamp, int stamp) {
+    if (prev_stamp == 0) return false;
+    int any = 0;
+#pragma unroll
+    for (int q = 0; q < RL; ++q) {
+        const int a = __atomic_load_n(&active[row0 + q], __ATOMIC_RELAXED);
+        any |= (a == prev_stamp || a == stamp) ? 1 : 0;
+    }
+    return __syncthreads_or(any) == 0;
+}
+
 __device__ __forceinline__ float relu_clamp(float y, float clampv) {
     // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
     return __builtin_amdgcn_fmed3f(y, 0.0f, clampv);
@@ -99,11 +115,10 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // physical column the NEXT layer wants it in (dst), RB*4 contiguous bytes.
 // ------------------------------------------------------------------------------------------
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
-__global__ __launch_bounds__(NW * 64) void band_walk_kernel(
-    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
-    const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int Krt, int seglen, int stamp, float wu, float bias, float clampv) {
-    extern __shared__ __align__(16) unsigned char smem[];
+__device__ __forceinline__ void band_walk_body(
+    const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ sel,
+    const float* __restrict__ wv, const int32_t* __restrict__ dst, int N, int Krt, int vb, int ve,
+    float wu, float bias, float clampv, unsigned char* smem, float* nz) {
     using V = typename VecOf<RL>::type;
     constexpr int T = NW * OPW;
     constexpr int RB = 64 * RL;
@@ -116,12 +131,6 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     const int K4 = K >> 2;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int rb = blockIdx.x;
-    const int vb = blockIdx.y * seglen;
-    const int ve = min(N, vb + seglen);
-    const size_t blk = (size_t)rb * (size_t)N * RB;
-    const float* __restrict__ yin = yin_all + blk;
-    float* __restrict__ yout = yout_all + blk;
     const int loff = lane * RL;
     const unsigned char* lane_smem = smem + loff * 4;
 
@@ -135,10 +144,6 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
         }
     }
     __syncthreads();
-
-    float nz[RL];
-#pragma unroll
-    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
 
     for (int cb = vb; cb < ve; cb += T) {
         // columns of the next chunk: issue the HBM loads now, park them in registers (past the
@@ -297,7 +302,77 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
         }
         __syncthreads();
     }
-    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
+}
+
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+__global__ __launch_bounds__(NW * 64) void band_walk_kernel(
+    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
+    const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
+    int32_t* __restrict__ count_out, int N, int Krt, int seglen, int stamp, int prev_stamp, float wu, float bias,
+    float clampv) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int RB = 64 * RL;
+    const int rb = blockIdx.x;
+    const int vb = blockIdx.y * seglen;
+    const int ve = min(N, vb + seglen);
+    const size_t blk = (size_t)rb * (size_t)N * RB;
+    if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp)) return;
+    float nz[RL];
+#pragma unroll
+    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, sel, wv, dst, N, Krt, vb, ve, wu,
+                                                 bias, clampv, smem, nz);
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp, count_out);
+}
+
+// ------------------------------------------------------------------------------------------
+// Fused layer chain ("fused" variant): one workgroup keeps one row block and runs `nlayers`
+// consecutive BAND layers back to back in a single launch - whole band per layer, ping-pong
+// between the two work buffers.  The intermediate activations of a row block are private to the
+// workgroup (written and re-read by the same CU through L2), there is no launch, tail or global
+// barrier between layers, and a workgroup whose rows have all died stops: the rest of its chain
+// is all zero by definition.  Layers of one chain share K and the weight mode.
+// ------------------------------------------------------------------------------------------
+struct ChainLayer {
+    const uint32_t* sel;
+    const float* wv;
+    const int32_t* dst;
+    float wu;
+    int pad;
+};
+
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+__global__ __launch_bounds__(NW * 64) void band_chain_kernel(
+    const ChainLayer* __restrict__ table, int nlayers, const float* __restrict__ first_in,
+    float* __restrict__ buf_a, float* __restrict__ buf_c, int32_t* __restrict__ active,
+    int32_t* __restrict__ count_out, int N, int Krt, int stamp0, int prev_stamp, int stop_when_dead, float bias,
+    float clampv) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int RB = 64 * RL;
+    const int rb = blockIdx.x;
+    const size_t blk = (size_t)rb * (size_t)N * RB;
+    if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp0)) return;
+    const float* in = first_in + blk;
+    for (int j = 0; j < nlayers; ++j) {
+        float* out = (in == buf_a + blk) ? buf_c + blk : buf_a + blk;
+        const ChainLayer lay = table[j];
+        float nz[RL];
+#pragma unroll
+        for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.sel, lay.wv, lay.dst, N, Krt, 0, N, lay.wu, bias,
+                                                     clampv, smem, nz);
+        stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp0 + j,
+                       count_out ? count_out + j : nullptr);
+        int any = 0;
+#pragma unroll
+        for (int q = 0; q < RL; ++q) any |= (nz[q] > 0.0f) ? 1 : 0;
+        // make this layer's columns visible to the whole workgroup before the next layer reads them
+        __threadfence();
+        const int alive = __syncthreads_or(any);
+        __threadfence();
+        if (!alive && stop_when_dead) return;
+        in = out;
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -311,12 +386,13 @@ __global__ __launch_bounds__(256) void gather_kernel(
     const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ cols,
     const int32_t* __restrict__ rowlen, const float* __restrict__ wv, const int32_t* __restrict__ dst,
     int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int kmax, int opg, int stamp,
-    float bias, float clampv) {
+    int prev_stamp, float bias, float clampv) {
     using V = typename VecOf<RL>::type;
     constexpr int RB = 64 * RL;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rb = blockIdx.x;
+    if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
     const size_t blk = (size_t)rb * (size_t)N * RB;
     const float* __restrict__ yin = yin_all + blk;
     float* __restrict__ yout = yout_all + blk;
@@ -489,12 +565,14 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(
 
 __global__ void unpack_rows_kernel(const float* __restrict__ y, const int32_t* __restrict__ phys_of_col,
                                    const int32_t* __restrict__ phys_rows, int N, int RB,
-                                   float* __restrict__ rowmajor) {
+                                   const int32_t* __restrict__ active, int stamp, float* __restrict__ rowmajor) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
     if (n >= N) return;
     const int pr = phys_rows[blockIdx.y];
     float x = 0.0f;
-    if (pr >= 0) {
+    // a row that the last layer did not stamp is all zero by definition (its block may have been
+    // skipped, leaving stale data in the buffer)
+    if (pr >= 0 && (stamp == 0 || active[pr] == stamp)) {
         const int pc = phys_of_col ? phys_of_col[n] : n;
         x = y[((size_t)(pr / RB) * (size_t)N + (size_t)pc) * RB + (pr % RB)];
     }
@@ -571,7 +649,7 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     if (nseg > 65535) return hipErrorInvalidValue;
     dim3 grid(a.nblk, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.count_out,
-                       a.N, a.K, seglen, a.stamp, a.wu, a.bias, a.clampv);
+                       a.N, a.K, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
 }
 
@@ -648,6 +726,53 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     }
 }
 
+namespace {
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
+    constexpr size_t lds = (size_t)RING * 64 * RL * 4;
+    auto kern = band_chain_kernel<RL, NW, OPW, RING, WMODE, KT>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(a.nblk), dim3(NW * 64), lds, s, reinterpret_cast<const ChainLayer*>(a.table),
+                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.N, a.K, a.stamp0,
+                       a.prev_stamp, a.stop_when_dead, a.bias, a.clampv);
+    return hipGetLastError();
+}
+template <int RL, int NW, int OPW, int RING>
+hipError_t launch_chain_rl(const ChainLaunch& a, hipStream_t s) {
+    if (a.K == 32) {
+        switch (a.wmode) {
+            case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 32>(a, s);
+            case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 32>(a, s);
+            default: return launch_chain_inst<RL, NW, OPW, RING, 2, 32>(a, s);
+        }
+    }
+    switch (a.wmode) {
+        case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 0>(a, s);
+        case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 0>(a, s);
+        default: return launch_chain_inst<RL, NW, OPW, RING, 2, 0>(a, s);
+    }
+}
+}  // namespace
+
+hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
+    static_assert(sizeof(ChainLayer) == sizeof(ChainLayerDesc), "layer table layout");
+    if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 || a.nlayers < 1 ||
+        !a.table || !a.first_in || !a.buf_a || !a.buf_c || !a.active || a.buf_a == a.buf_c)
+        return hipErrorInvalidValue;
+    switch (a.rl) {
+        case 4: return launch_chain_rl<4, 16, 3, 128>(a, s);
+        case 2: return launch_chain_rl<2, 16, 7, 256>(a, s);
+        case 1: return launch_chain_rl<1, 16, 7, 256>(a, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
     if (a.N <= 0 || a.kmax < 0 || a.nblk <= 0 || !a.yin || !a.yout || !a.cols || !a.rowlen || !a.wv ||
         !a.dst || !a.active)
@@ -657,7 +782,7 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
     if (grid.y > 65535) return hipErrorInvalidValue;
 #define SPDNN_GATHER(RLv, WM)                                                                         \
     hipLaunchKernelGGL((gather_kernel<RLv, WM>), grid, block, 0, s, a.yin, a.yout, a.cols, a.rowlen,  \
-                       a.wv, a.dst, a.active, a.count_out, a.N, a.kmax, opg, a.stamp, a.bias, a.clampv)
+                       a.wv, a.dst, a.active, a.count_out, a.N, a.kmax, opg, a.stamp, a.prev_stamp, a.bias, a.clampv)
     const bool exact = a.wmode != 2;
     switch (a.rl) {
         case 4: if (exact) SPDNN_GATHER(4, 1); else SPDNN_GATHER(4, 2); break;
@@ -733,10 +858,11 @@ hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys
 }
 
 hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows, int nreq,
-                              int N, int rl, float* rowmajor, hipStream_t s) {
+                              int N, int rl, const int32_t* active, int stamp, float* rowmajor, hipStream_t s) {
     if (nreq <= 0 || nreq > 65535 || N <= 0) return hipErrorInvalidValue;
     dim3 grid((N + 255) / 256, nreq);
-    hipLaunchKernelGGL(unpack_rows_kernel, grid, dim3(256), 0, s, y, phys_of_col, phys_rows, N, 64 * rl, rowmajor);
+    hipLaunchKernelGGL(unpack_rows_kernel, grid, dim3(256), 0, s, y, phys_of_col, phys_rows, N, 64 * rl, active,
+                       stamp, rowmajor);
     return hipGetLastError();
 }
 

@@ -23,6 +23,7 @@ struct BandLaunch {
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
     int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, K, nblk, stamp, rl;
+    int prev_stamp = 0;      // stamp of the previous layer: row blocks it left without an active row are skipped (0 = off)
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
     int n_cu;
@@ -40,6 +41,7 @@ struct GatherLaunch {
     int32_t* active;
     int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, kmax, nblk, stamp, rl;
+    int prev_stamp = 0;      // as in BandLaunch
     int wmode;               // 1 fma (exact products), 2 mul then add
     float bias, clampv;
 };
@@ -50,6 +52,30 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s);
 int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
+
+// Fused layer chain: `nlayers` consecutive BAND layers (same K and weight mode) in one launch,
+// one workgroup per row block.  Layer j reads what layer j-1 wrote: the first layer reads
+// first_in, every layer writes the work buffer (buf_a / buf_c) it did not read.
+struct ChainLayerDesc {      // one entry of the device-side layer table
+    const uint32_t* sel;
+    const float* wv;
+    const int32_t* dst;
+    float wu;
+    int pad;
+};
+struct ChainLaunch {
+    const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain
+    int nlayers;
+    const float* first_in;
+    float* buf_a;
+    float* buf_c;
+    int32_t* active;
+    int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
+    int N, K, nblk, stamp0, prev_stamp, rl, wmode;
+    int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
+    float bias, clampv;
+};
+hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s);
 
 // Active-row scan: rows with active[row] == stamp and gid[row] >= 0 survive, in order.
 // Writes count[0] = number of survivors, alive_src[k] = physical row of survivor k,
@@ -75,8 +101,10 @@ hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys
                             int64_t row0, int nrows, int rl, int32_t* nonfinite, hipStream_t s);
 
 // Row-block layout to row-major for a list of physical rows (-1 gives a zero row).
+// `active`/`stamp`: rows whose stamp differs read back as zero rows (stamp 0 = no check).
 hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows,
-                              int nreq, int N, int rl, float* rowmajor, hipStream_t s);
+                              int nreq, int N, int rl, const int32_t* active, int stamp, float* rowmajor,
+                              hipStream_t s);
 
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
 hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s);

@@ -140,6 +140,7 @@ struct spdnn_net {
     void* arena = nullptr;
     std::vector<DevLayer> dl;
     float *F = nullptr, *A = nullptr, *C = nullptr;
+    int32_t* d_active_scratch = nullptr;
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
@@ -159,6 +160,10 @@ struct spdnn_net {
     int64_t alive = 0;        // rows active after the last layer run
     bool alive_list_valid = false;
     bool gid_dirty = false;   // a repack permuted d_gid since it was last initialised
+    int last_stamp = 0;       // stamp of the newest layer, valid for the current row slots (0 = none)
+    bool repacked_after_last = false;
+    int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
+    ChainLayerDesc* d_chain = nullptr;
     std::vector<char> pending; // layer has an inspection job in flight
     std::vector<int64_t> counts;
     std::vector<float> layer_ms;
@@ -187,6 +192,7 @@ int ensure_device(spdnn_net* n) {
     HIPCHK(hipEventCreate(&n->ev_stop));
     const size_t rows = (size_t)n->rows_cap;
     HIPCHK(hipMalloc(&n->d_active, rows * 4));
+    HIPCHK(hipMalloc(&n->d_active_scratch, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid_tmp, rows * 4));
     HIPCHK(hipMalloc(&n->d_alive_src, rows * 4));
@@ -233,6 +239,16 @@ int ensure_uploaded(spdnn_net* n) {
         HIPCHK(put(p.wv.data(), p.wv.size() * 4, (void**)&d.wv));
         HIPCHK(put(p.dst.data(), p.dst.size() * 4, (void**)&d.dst));
     }
+    std::vector<ChainLayerDesc> table((size_t)n->L);
+    for (int l = 0; l < n->L; ++l) {
+        table[(size_t)l].sel = n->dl[(size_t)l].sel;
+        table[(size_t)l].wv = n->dl[(size_t)l].wv;
+        table[(size_t)l].dst = n->dl[(size_t)l].dst;
+        table[(size_t)l].wu = n->layers[(size_t)l].info.value;
+        table[(size_t)l].pad = 0;
+    }
+    HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
+    HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
     const size_t fbytes = (size_t)n->rows_cap * (size_t)n->N * 4;
     HIPCHK(hipMalloc(&n->F, fbytes));
     HIPCHK(hipMalloc(&n->A, fbytes));
@@ -243,6 +259,8 @@ int ensure_uploaded(spdnn_net* n) {
 
 void free_device(spdnn_net* n) {
     if (n->arena) hipFree(n->arena);
+    if (n->d_chain) hipFree(n->d_chain);
+    n->d_chain = nullptr;
     if (n->F) hipFree(n->F);
     if (n->A) hipFree(n->A);
     if (n->C) hipFree(n->C);
@@ -262,6 +280,8 @@ void reset_state(spdnn_net* n) {
         n->gid_dirty = false;
     }
     n->cur = n->F;
+    n->last_stamp = 0;
+    n->repacked_after_last = false;
     n->cur_layer = 0;
     n->carried = ((n->batch + n->RB - 1) / n->RB) * n->RB;
     n->alive = n->batch;
@@ -309,6 +329,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     n->pool.reset(new JobPool(host_threads()));
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
     if (getenv("SPDNN_BAND_SHAPE")) n->autotune = false;  // an explicit shape wins
+    if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     *out = n;
     return SPDNN_OK;
 }
@@ -320,6 +341,7 @@ int spdnn_destroy(spdnn_net* n) {
     if (n->dev_ready) {
         hipStreamSynchronize(n->stream);
         free_device(n);
+        hipFree(n->d_active_scratch);
         hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp); hipFree(n->d_alive_src);
         hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
         hipHostFree(n->h_count);
@@ -592,6 +614,7 @@ int spdnn_default_run_options(spdnn_run_options* o) {
     o->first_layer = 0;
     o->n_layers = -1;
     o->compact_threshold = 0.75f;
+    o->fuse_layers = 0;
     return SPDNN_OK;
 }
 
@@ -602,7 +625,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, in
     a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
-    a.shape = -1; a.seglen = 0; a.count_out = nullptr;
+    a.shape = -1; a.seglen = 0; a.count_out = nullptr; a.prev_stamp = 0;
     return a;
 }
 
@@ -629,6 +652,7 @@ static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk)
         const int nc = band_seglen_candidates(n->N, p.kmax, nblk, n->rl, shape, n->n_cu, lens, 2);
         for (int c = 0; c < nc && err == hipSuccess; ++c) {
             BandLaunch a = band_args(n, l, in, out, nblk, 0);
+            a.active = n->d_active_scratch;  // trials must not disturb the real row stamps
             a.shape = shape;
             a.seglen = lens[c];
             float ms = 0.0f;
@@ -651,18 +675,19 @@ static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk)
 }
 
 static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp,
-                               int32_t* count_out) {
+                               int prev_stamp, int32_t* count_out) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
         BandLaunch a = band_args(n, l, in, out, nblk, stamp);
         a.count_out = count_out;
+        a.prev_stamp = prev_stamp;
         if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) { a.shape = t->shape; a.seglen = t->seglen; }
         return launch_band(a, n->stream);
     }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
-    g.active = n->d_active; g.count_out = count_out; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
+    g.active = n->d_active; g.count_out = count_out; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
     g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv;
     return launch_gather(g, n->stream);
 }
@@ -678,6 +703,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     if (nl < 1 || opt.first_layer + nl > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
     if (opt.prune && n->bias > 0.0f)
         return fail(SPDNN_E_UNSUPPORTED, "pruning needs bias <= 0 (an all-zero row must stay zero)");
+    if (opt.fuse_layers < 0) return fail(SPDNN_E_ARG, "fuse_layers negative");
     if (opt.first_layer == 0) reset_state(n);
     else if (opt.first_layer != n->cur_layer) return fail(SPDNN_E_STATE, "first_layer does not continue the current state");
     float thr = opt.compact_threshold > 0.0f ? opt.compact_threshold : 0.75f;
@@ -705,96 +731,133 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     const bool scan_count = !fused_count && opt.collect_counts;
     const bool have_counts = fused_count || scan_count;
     if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
+    int fuse = opt.fuse_layers ? opt.fuse_layers : n->default_fuse;
+    if (scan_count || fuse < 2) fuse = 1;
 
-    // Pruning never waits for the layer it just launched: the host looks at the count of the
-    // layer `lookahead` launches back (already finished in steady state).  Counts only go down
+    // Pruning never waits for the launch it just made: the host looks at the counts of the launch
+    // `lookahead` launches back (already finished in steady state).  Counts only go down
     // (bias <= 0), so an older count is a safe upper bound for sizing a repack, and a zero count
     // means every later layer is all zero.
-    const int lookahead = 2;
+    const size_t lookahead = 2;
+    struct Rec { int l0, c; };
+    std::vector<Rec> recs;
+    size_t processed = 0;
     spdnn_run_result r{};
     const int64_t alive_at_start = n->alive;
-    std::vector<int> timed;
-    int known = first;               // counts of layers < known have been read by the host
-    int64_t newest_count = -1;       // count of layer known-1
+    struct Timed { int l0, c; };
+    std::vector<Timed> timed;
+    int64_t newest_count = -1;
     bool dead = n->carried == 0;
-    int last_launched = -1, last_stamp = 0;
+    int last_launched = -1;
 
     HIPCHK(hipEventRecord(n->ev_start, n->stream));
-    for (int l = first; l <= last; ++l) {
+    for (int l = first; l <= last;) {
         const LayerPlan& p = n->layers[(size_t)l];
-        r.edges += (double)n->batch * (double)p.info.nnz;
         if (dead) {  // every row died earlier: the remaining outputs are all zero
-            n->cur_layer = l + 1;
+            r.edges += (double)n->batch * (double)p.info.nnz;
+            n->cur_layer = ++l;
             continue;
         }
-        float* out = (n->cur == n->A) ? n->C : n->A;
-        const int nblk = n->carried / n->RB;
-        if (n->autotune && p.kernel == SPDNN_KERNEL_BAND && last - l + 1 >= 8 && !find_tuned(n, nblk, p.kmax)) {
-            int rc = tune_band(n, l, n->cur, out, nblk);
-            if (rc) return rc;
-            if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + l, 0, 4, n->stream));  // the trials counted too
+        // chain length: consecutive BAND layers with the same row length and weight mode
+        int c = 1;
+        if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
+            while (c < fuse && l + c <= last) {
+                const LayerPlan& q = n->layers[(size_t)(l + c)];
+                if (q.kernel != SPDNN_KERNEL_BAND || q.kmax != p.kmax || q.wmode != p.wmode) break;
+                ++c;
+            }
         }
-        const int stamp = ++n->stamp;
+        for (int j = 0; j < c; ++j) r.edges += (double)n->batch * (double)n->layers[(size_t)(l + j)].info.nnz;
+        const int nblk = n->carried / n->RB;
+        const int prev_stamp = opt.prune ? n->last_stamp : 0;
+        const float* in = n->cur;
+        float* out = (n->cur == n->A) ? n->C : n->A;
+        if (c == 1 && n->autotune && p.kernel == SPDNN_KERNEL_BAND && last - l + 1 >= 8 &&
+            !find_tuned(n, nblk, p.kmax)) {
+            int rc = tune_band(n, l, in, out, nblk);
+            if (rc) return rc;
+        }
+        const int stamp0 = n->stamp + 1;
+        n->stamp += c;
         if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
-        HIPCHK(launch_layer(n, l, n->cur, out, nblk, stamp, fused_count ? n->d_counts + l : nullptr));
-        if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back(l); }
-        r.layers_run++;
-        last_launched = l;
-        last_stamp = stamp;
+        if (c == 1) {
+            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr));
+        } else {
+            ChainLaunch ch{};
+            ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
+            ch.active = n->d_active; ch.count_out = fused_count ? n->d_counts + l : nullptr;
+            ch.N = n->N; ch.K = p.kmax; ch.nblk = nblk; ch.stamp0 = stamp0; ch.prev_stamp = prev_stamp;
+            ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = opt.prune ? 1 : 0;
+            ch.bias = n->bias; ch.clampv = n->clampv;
+            HIPCHK(launch_band_chain(ch, n->stream));
+            for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
+        }
+        if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back({l, c}); }
+        r.layers_run += c;
+        last_launched = l + c - 1;
+        n->last_stamp = stamp0 + c - 1;
         n->cur = out;
-        n->cur_layer = l + 1;
+        n->cur_layer = l + c;
         if (scan_count) {
-            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, stamp, n->d_count, n->d_alive_src,
+            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
                                       n->d_alive_gid, n->stream));
             HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
         }
         if (have_counts) {
-            HIPCHK(hipMemcpyAsync(n->h_counts + l, n->d_counts + l, 4, hipMemcpyDeviceToHost, n->stream));
-            HIPCHK(hipEventRecord(n->ev_count[(size_t)l], n->stream));
+            HIPCHK(hipMemcpyAsync(n->h_counts + l, n->d_counts + l, (size_t)c * 4, hipMemcpyDeviceToHost, n->stream));
+            HIPCHK(hipEventRecord(n->ev_count[(size_t)(l + c - 1)], n->stream));
+            recs.push_back({l, c});
         }
+        l += c;
         if (!opt.prune) continue;
 
-        const int upto = l - lookahead;  // newest layer whose count the host waits for
-        while (known <= upto && !dead) {
-            HIPCHK(hipEventSynchronize(n->ev_count[(size_t)known]));
-            newest_count = n->h_counts[known];
-            n->counts[(size_t)known] = newest_count;
-            if (newest_count == 0) dead = true;
-            ++known;
+        while (recs.size() - processed > lookahead && !dead) {
+            const Rec rc = recs[processed++];
+            HIPCHK(hipEventSynchronize(n->ev_count[(size_t)(rc.l0 + rc.c - 1)]));
+            for (int j = rc.l0; j < rc.l0 + rc.c && !dead; ++j) {
+                newest_count = n->h_counts[j];
+                if (newest_count == 0) dead = true;
+            }
         }
         if (dead) { n->carried = 0; continue; }
-        if (newest_count > 0 && (double)newest_count <= (double)thr * (double)n->carried && l + 1 < n->L) {
+        if (newest_count > 0 && (double)newest_count <= (double)thr * (double)n->carried && l < n->L) {
             const int nb = (int)((newest_count + n->RB - 1) / n->RB);  // upper bound of what is alive now
             if (nb * n->RB < n->carried) {
                 float* dstbuf = (n->cur == n->A) ? n->C : n->A;
-                HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, stamp, n->d_count, n->d_alive_src,
-                                          n->d_alive_gid, n->stream));
+                HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count,
+                                          n->d_alive_src, n->d_alive_gid, n->stream));
                 HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
                                      n->N, n->rl, nb, n->stream));
                 std::swap(n->d_gid, n->d_gid_tmp);
                 n->gid_dirty = true;
                 n->cur = dstbuf;
                 n->carried = nb * n->RB;
+                n->last_stamp = 0;  // the row slots moved: the stamps no longer describe them
+                n->repacked_after_last = true;
                 r.compactions++;
+                continue;
             }
         }
+        n->repacked_after_last = false;
     }
-    // categories of the last layer: survivor list by the scan (after a repack the row slots moved,
-    // but the stamps of the last layer were written after it, so they match the current slots)
+    // categories of the last layer: survivor list by the scan.  After a final repack the list
+    // produced for the repack is that list already.
     n->alive_list_valid = false;
-    if (!dead && last_launched >= 0 && last_launched == last) {
-        HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, last_stamp, n->d_count, n->d_alive_src,
-                                  n->d_alive_gid, n->stream));
+    if (!dead && last_launched == last) {
+        if (n->last_stamp != 0) {
+            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
+                                      n->d_alive_gid, n->stream));
+        }
         HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
         n->alive_list_valid = true;
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
     HIPCHK(hipEventElapsedTime(&r.ms_total, n->ev_start, n->ev_stop));
-    for (int l : timed) {
+    for (const Timed& t : timed) {
         float ms = 0.0f;
-        HIPCHK(hipEventElapsedTime(&ms, n->ev_layer[(size_t)(2 * l)], n->ev_layer[(size_t)(2 * l + 1)]));
-        n->layer_ms[(size_t)l] = ms;
+        HIPCHK(hipEventElapsedTime(&ms, n->ev_layer[(size_t)(2 * t.l0)], n->ev_layer[(size_t)(2 * t.l0 + 1)]));
+        for (int j = 0; j < t.c; ++j) n->layer_ms[(size_t)(t.l0 + j)] = ms / (float)t.c;
         r.ms_kernels += ms;
     }
     // per-layer counts: everything that was launched has finished now
@@ -805,7 +868,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         else if (l > last_launched) n->counts[(size_t)l] = (last_launched >= first || n->carried == 0) ? 0 : -1;
         if (n->counts[(size_t)l] == 0) zero_seen = true;
     }
-    if (dead || zero_seen) { n->carried = opt.prune ? 0 : n->carried; n->alive = 0; }
+    if (dead || zero_seen) { if (opt.prune) n->carried = 0; n->alive = 0; }
     else if (n->alive_list_valid) n->alive = n->h_count[0];
     if (n->alive == 0) n->alive_list_valid = true;  // the empty list
     // byte model: rows entering each launched layer
@@ -875,7 +938,7 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
     for (int i0 = 0; i0 < nrows && e == hipSuccess; i0 += chunk) {
         const int m = std::min(chunk, nrows - i0);
         e = hipMemcpyAsync(d_phys, phys.data() + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream);
-        if (e == hipSuccess) e = launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, d_out, n->stream);
+        if (e == hipSuccess) e = launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, n->d_active, n->last_stamp, d_out, n->stream);
         if (e == hipSuccess)
             e = hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * n->N * 4, hipMemcpyDeviceToHost, n->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(n->stream);

@@ -72,7 +72,9 @@ typedef struct spdnn_run_options {
     int32_t collect_counts;    /* 1: record the active-row count after every layer                 */
     int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
-    int32_t reserved[4];
+    int32_t fuse_layers;       /* >1: fused variant, up to that many consecutive band layers per launch
+                                  (one workgroup keeps a row block through the chain); 1 = off; 0 = default */
+    int32_t reserved[3];
 } spdnn_run_options;
 
 typedef struct spdnn_run_result {

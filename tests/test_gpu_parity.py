@@ -285,3 +285,50 @@ def test_full_batch_properties_cfg1(gc, orc):
     if k:
         pos = np.searchsorted(ref["gid"], sample[:k])
         assert same_floats(y_p[:k], ref["y"][pos])
+
+
+@pytest.mark.parametrize("prune", [True, False])
+@pytest.mark.parametrize("fuse", [4, 16])
+def test_fused_layer_chain(gc, orc, fuse, prune):
+    """The fused variant (several band layers per launch, one workgroup per row block) must give
+    what the layer-by-layer launches give: counts, categories and activations."""
+    N, L, B = 1024, 24, 3000
+    print("fused chain fuse=%d prune=%s" % (fuse, prune), flush=True)
+    layers = [orc.gen_layer_csr(5, l, N) for l in range(L)]
+    feats = orc.gen_features(5, N, 0, B, 0.10, 0.50)
+    ref = orc.infer(feats, layers, -0.3, prune=True)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(5)
+        net.inspect()
+        net.set_features_dense(feats)
+        r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+        assert r.layers_run == L
+        assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+        cats = net.categories()
+        assert np.array_equal(cats, ref["categories"])
+        assert same_floats(net.activations(cats), ref["y"])
+        dead = np.setdiff1d(np.arange(B), cats)[:64].astype(np.int32)
+        assert not net.activations(dead).any()
+        # a chain that stops in the middle of the network and is continued layer by layer
+        net.run(prune=prune, first_layer=0, n_layers=10, fuse_layers=fuse)
+        net.run(prune=prune, first_layer=10, n_layers=L - 10, fuse_layers=1)
+        assert np.array_equal(net.categories(), ref["categories"])
+        assert same_floats(net.activations(cats), ref["y"])
+
+
+def test_fused_chain_when_everything_dies(gc, orc):
+    """Literal inputs: all rows die within a few layers; workgroups leave the chain early."""
+    N, L, B = 1024, 40, 2000
+    print("fused chain, all rows die", flush=True)
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(12)]
+    ref = orc.infer(orc.gen_features(0, N, 0, B), layers, -0.3, prune=True)
+    want = [len(a) for a in ref["active_ids"]] + [0] * (L - 12)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, B)
+        for prune in (True, False):
+            r = net.run(prune=prune, collect_counts=True, fuse_layers=8)
+            assert [net.active_count(l) for l in range(L)] == want
+            assert r.active_rows == 0 and len(net.categories()) == 0
+            assert not net.activations(np.arange(50, dtype=np.int32)).any()
