@@ -366,10 +366,10 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         int any = 0;
 #pragma unroll
         for (int q = 0; q < RL; ++q) any |= (nz[q] > 0.0f) ? 1 : 0;
-        // make this layer's columns visible to the whole workgroup before the next layer reads them
-        __threadfence();
+        // The barrier (with its workgroup-scope fence) makes this layer's columns visible to the
+        // other waves of the workgroup - same CU, same L1 - before the next layer reads them.  A
+        // device-scope fence here would write back and invalidate the whole L2 of the XCD.
         const int alive = __syncthreads_or(any);
-        __threadfence();
         if (!alive && stop_when_dead) return;
         in = out;
     }
