@@ -6,7 +6,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-KERNEL_AUTO, KERNEL_GATHER, KERNEL_BAND = 0, 1, 2
+KERNEL_AUTO, KERNEL_GATHER, KERNEL_BAND, KERNEL_BLOCK = 0, 1, 2, 3
 
 _i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
@@ -72,6 +72,7 @@ def load_library():
         "spdnn_get_layer_plan": ([vp, C.c_int, C.POINTER(LayerPlan)], C.c_int),
         "spdnn_get_band_plan": ([vp, C.c_int, _i32p, _i32p, _u8p], C.c_int),
         "spdnn_get_layer_dst": ([vp, C.c_int, _i32p], C.c_int),
+        "spdnn_get_layer_slots": ([vp, C.c_int, C.POINTER(C.c_int)], C.c_int),
         "spdnn_get_input_labelling": ([vp, C.c_int, _i32p], C.c_int),
         "spdnn_hash_reorder": ([C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)], C.c_int),
         "spdnn_set_features_dense": ([vp, _f32p, C.c_int], C.c_int),
@@ -209,7 +210,13 @@ class Network:
         return in_pos, out_at, sel.reshape(self.neuron, k)
 
     def layer_dst(self, layer):
-        dst = np.empty(self.neuron, np.int32)
+        p = self.layer_plan(layer)
+        slots = self.neuron
+        if p.kernel == KERNEL_BLOCK:
+            slots = C.c_int()
+            _check(self._lib.spdnn_get_layer_slots(self._h, layer, C.byref(slots)))
+            slots = slots.value
+        dst = np.empty(slots, np.int32)
         _check(self._lib.spdnn_get_layer_dst(self._h, layer, dst))
         return dst
 

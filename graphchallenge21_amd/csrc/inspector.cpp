@@ -186,6 +186,39 @@ bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::
     return true;
 }
 
+bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                     std::vector<std::vector<int32_t>>& groups) {
+    groups.clear();
+    for (int j = 0; j < N; ++j) {
+        const int len = rowptr[j + 1] - rowptr[j];
+        if (len < 1 || len > 32) return false;
+    }
+    // order the outputs by their input list; equal lists become neighbours
+    std::vector<int32_t> order((size_t)N);
+    std::iota(order.begin(), order.end(), 0);
+    auto less = [&](int32_t a, int32_t b) {
+        const int la = rowptr[a + 1] - rowptr[a], lb = rowptr[b + 1] - rowptr[b];
+        if (la != lb) return la < lb;
+        const int c = std::memcmp(col.data() + rowptr[a], col.data() + rowptr[b], (size_t)la * sizeof(int32_t));
+        if (c != 0) return c < 0;
+        return a < b;
+    };
+    auto same = [&](int32_t a, int32_t b) {
+        const int la = rowptr[a + 1] - rowptr[a], lb = rowptr[b + 1] - rowptr[b];
+        return la == lb && std::memcmp(col.data() + rowptr[a], col.data() + rowptr[b], (size_t)la * sizeof(int32_t)) == 0;
+    };
+    std::sort(order.begin(), order.end(), less);
+    for (int i = 0; i < N;) {
+        int e = i + 1;
+        while (e < N && same(order[(size_t)i], order[(size_t)e])) ++e;
+        for (int b = i; b < e; b += 16)
+            groups.emplace_back(order.begin() + b, order.begin() + std::min(e, b + 16));
+        i = e;
+    }
+    // worth it only if an input column loaded into registers is reused by several outputs
+    return (int64_t)groups.size() * 8 <= (int64_t)N;
+}
+
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, LayerPlan& plan) {
     const int64_t nnz = rowptr[N];
@@ -226,7 +259,41 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         band = discover_band(N, K, rowptr, col, plan.in_pos, plan.out_at);
     }
 
-    if (band) {
+    std::vector<std::vector<int32_t>> groups;
+    const bool block = !band && force_kernel != SPDNN_KERNEL_GATHER && !dup && discover_blocks(N, rowptr, col, groups);
+
+    plan.ngroups = 0;
+    plan.blk_cols.clear();
+    plan.blk_cnt.clear();
+    if (block) {
+        plan.kernel = SPDNN_KERNEL_BLOCK;
+        plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
+        plan.ngroups = (int)groups.size();
+        plan.kmax = kmax;
+        plan.in_pos.resize((size_t)N);
+        std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
+        plan.out_at.assign((size_t)plan.ngroups * 16, -1);
+        plan.blk_cols.assign((size_t)plan.ngroups * 32, 0);
+        plan.blk_cnt.resize((size_t)plan.ngroups);
+        if (plan.wmode != 0) plan.wv.assign((size_t)plan.ngroups * 16 * 32, 0.0f); else plan.wv.clear();
+        plan.blk_full = true;
+        for (int g = 0; g < plan.ngroups; ++g) {
+            const int j0 = groups[(size_t)g][0];
+            const int len = rowptr[j0 + 1] - rowptr[j0];
+            plan.blk_cnt[(size_t)g] = len;
+            if (len != 32) plan.blk_full = false;
+            for (int k = 0; k < len; ++k) plan.blk_cols[(size_t)g * 32 + k] = col[rowptr[j0] + k];
+            for (size_t o = 0; o < groups[(size_t)g].size(); ++o) {
+                const int j = groups[(size_t)g][o];
+                plan.out_at[(size_t)g * 16 + o] = j;
+                if (plan.wmode != 0)
+                    for (int k = 0; k < len; ++k) plan.wv[((size_t)g * 16 + o) * 32 + k] = val[rowptr[j] + k];
+            }
+        }
+        plan.sel.clear();
+        plan.ell_col.clear();
+        plan.rowlen.clear();
+    } else if (band) {
         plan.kernel = SPDNN_KERNEL_BAND;
         plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
         plan.info.band_halo = K - 1;
@@ -265,16 +332,20 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.sel.clear();
     }
     plan.info.kernel = plan.kernel;
-    plan.info.plan_bytes = (int64_t)(plan.sel.size() + 4 * (plan.ell_col.size() + plan.rowlen.size() +
-                                                              plan.wv.size() + 2 * (size_t)N));
+    plan.info.plan_bytes = (int64_t)(plan.sel.size() + 4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
+                                                              plan.blk_cols.size() + plan.blk_cnt.size() +
+                                                              plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.set = true;
 }
 
 void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos) {
-    const size_t N = cur.out_at.size();
-    cur.dst.resize(N);
-    for (size_t s = 0; s < N; ++s) cur.dst[s] = next_in_pos ? (*next_in_pos)[cur.out_at[s]] : cur.out_at[s];
+    const size_t slots = cur.out_at.size();  // N, or 16 per group with -1 padding for BLOCK layers
+    cur.dst.resize(slots);
+    for (size_t s = 0; s < slots; ++s) {
+        const int32_t j = cur.out_at[s];
+        cur.dst[s] = j < 0 ? -1 : (next_in_pos ? (*next_in_pos)[(size_t)j] : j);
+    }
 }
 
 }  // namespace spdnn

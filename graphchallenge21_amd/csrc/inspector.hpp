@@ -27,7 +27,13 @@ struct LayerPlan {
     std::vector<uint8_t> sel;       // BAND: [N][K] input position mod 256, accumulation order
     std::vector<int32_t> ell_col;   // GATHER: [N][kmax] physical input column, accumulation order
     std::vector<int32_t> rowlen;    // GATHER: [N]
-    std::vector<float> wv;          // [N][kmax] weights in accumulation order (empty when wmode 0)
+    // BLOCK: groups of up to 16 outputs that read the same (up to 32) inputs
+    int ngroups = 0;
+    bool blk_full = false;          // every group has exactly 32 shared inputs
+    std::vector<int32_t> blk_cols;  // [ngroups][32] physical input columns, accumulation order (padded)
+    std::vector<int32_t> blk_cnt;   // [ngroups] number of shared inputs
+    std::vector<float> wv;          // weights in accumulation order: BAND [N][K], GATHER [N][kmax],
+                                    // BLOCK [ngroups*16][32] (empty when wmode 0)
     std::vector<int32_t> dst;       // [N] physical column of slot's output in the next buffer
 };
 
@@ -42,6 +48,11 @@ std::string normalize_csr(int N, const int32_t* rowptr, const int32_t* col, cons
 // band position of input i and out_at[v] the output neuron at position v.
 bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    std::vector<int32_t>& in_pos, std::vector<int32_t>& out_at);
+
+// Groups outputs whose input lists are identical (at most 16 per group, lists of at most 32).
+// Returns false when the layer has too few duplicates to be worth it.
+bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                     std::vector<std::vector<int32_t>>& groups);
 
 // Full per-layer inspection (everything except dst, which needs the next layer's labelling).
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,

@@ -432,6 +432,77 @@ __global__ __launch_bounds__(256) void gather_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
+// BLOCK kernel: groups of up to 16 outputs that read the same (up to 32) input columns - the
+// structure of the challenge's RadiX-Net layers.  A wave loads the shared columns of a group once
+// into registers (32 x RB*4 bytes) and every output of the group reuses them: no LDS, register
+// operands only, one multiply-add per VALU instruction.  The accumulation order (ascending input
+// index) is the same for every output of a group, so the code is fully unrolled.
+// ------------------------------------------------------------------------------------------
+template <int RL, int WMODE, bool FULL>
+__global__ __launch_bounds__(256) void block_kernel(
+    const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ grp_cols,
+    const int32_t* __restrict__ grp_cnt, const float* __restrict__ wv, const int32_t* __restrict__ dst,
+    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int ngroups, int gpw, int stamp,
+    int prev_stamp, float wu, float bias, float clampv) {
+    using V = typename VecOf<RL>::type;
+    constexpr int RB = 64 * RL;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rb = blockIdx.x;
+    if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
+    const size_t blk = (size_t)rb * (size_t)N * RB;
+    const float* __restrict__ yin = yin_all + blk;
+    float* __restrict__ yout = yout_all + blk;
+    const int loff = lane * RL;
+    const int g0 = (blockIdx.y * 4 + wave) * gpw;
+    const int g1 = min(ngroups, g0 + gpw);
+
+    float nz[RL];
+#pragma unroll
+    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+
+    for (int g = g0; g < g1; ++g) {
+        const int S = FULL ? 32 : grp_cnt[g];
+        const int32_t* cp = grp_cols + (size_t)g * 32;
+        float x[32][RL];
+#pragma unroll
+        for (int m = 0; m < 32; ++m) {
+            if (FULL || m < S) {
+                vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)cp[m] * RB + loff), x[m]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < RL; ++q) x[m][q] = 0.0f;
+            }
+        }
+#pragma unroll 1
+        for (int o = 0; o < 16; ++o) {
+            const int d = dst[(size_t)g * 16 + o];
+            if (d < 0) break;  // groups are filled from the front
+            const float* wp = WMODE ? wv + ((size_t)g * 16 + o) * 32 : nullptr;
+            float acc[RL];
+#pragma unroll
+            for (int q = 0; q < RL; ++q) acc[q] = 0.0f;
+#pragma unroll
+            for (int m = 0; m < 32; ++m) {
+                if (FULL || m < S) {
+                    const float w = WMODE ? wp[m] : wu;
+#pragma unroll
+                    for (int q = 0; q < RL; ++q) acc[q] = mac<WMODE>(acc[q], x[m][q], w);
+                }
+            }
+            float y[RL];
+#pragma unroll
+            for (int q = 0; q < RL; ++q) {
+                y[q] = relu_clamp(acc[q] + bias, clampv);
+                nz[q] = fmaxf(nz[q], y[q]);
+            }
+            *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
+        }
+    }
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
+}
+
+// ------------------------------------------------------------------------------------------
 // Active-row scan (one workgroup of 1024 threads).  Thread t owns the contiguous strip of rows
 // [t*S, (t+1)*S): it counts its survivors, the workgroup takes an exclusive prefix over the 1024
 // counts (wave64 ballot-free shuffle scan inside a wave, LDS across the 16 waves), and every
@@ -791,6 +862,37 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
         default: return hipErrorInvalidValue;
     }
 #undef SPDNN_GATHER
+    return hipGetLastError();
+}
+
+hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {
+    if (a.N <= 0 || a.ngroups <= 0 || a.nblk <= 0 || !a.yin || !a.yout || !a.cols || !a.cnt || !a.dst ||
+        !a.active || (a.wmode != 0 && !a.wv))
+        return hipErrorInvalidValue;
+    // groups per wave: enough workgroups to fill the chip several times over, but long enough
+    // runs per wave to amortise the launch
+    int gpw = 4;
+    while (gpw > 1 && (long long)a.nblk * ((a.ngroups + 4 * gpw - 1) / (4 * gpw)) < 2048) gpw >>= 1;
+    dim3 grid(a.nblk, (a.ngroups + 4 * gpw - 1) / (4 * gpw)), block(256);
+    if (grid.y > 65535) return hipErrorInvalidValue;
+#define SPDNN_BLOCK(RLv, WM, FL)                                                                          \
+    hipLaunchKernelGGL((block_kernel<RLv, WM, FL>), grid, block, 0, s, a.yin, a.yout, a.cols, a.cnt, a.wv, \
+                       a.dst, a.active, a.count_out, a.N, a.ngroups, gpw, a.stamp, a.prev_stamp, a.wu,     \
+                       a.bias, a.clampv)
+#define SPDNN_BLOCK_WM(RLv)                                                                 \
+    switch (a.wmode) {                                                                      \
+        case 0: if (a.full) SPDNN_BLOCK(RLv, 0, true); else SPDNN_BLOCK(RLv, 0, false); break; \
+        case 1: if (a.full) SPDNN_BLOCK(RLv, 1, true); else SPDNN_BLOCK(RLv, 1, false); break; \
+        default: if (a.full) SPDNN_BLOCK(RLv, 2, true); else SPDNN_BLOCK(RLv, 2, false); break; \
+    }
+    switch (a.rl) {
+        case 4: SPDNN_BLOCK_WM(4); break;
+        case 2: SPDNN_BLOCK_WM(2); break;
+        case 1: SPDNN_BLOCK_WM(1); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef SPDNN_BLOCK_WM
+#undef SPDNN_BLOCK
     return hipGetLastError();
 }
 

@@ -53,6 +53,22 @@ int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
 
+// BLOCK layers: groups of up to 16 outputs sharing up to 32 input columns.
+struct BlockLaunch {
+    const float* yin;
+    float* yout;
+    const int32_t* cols;     // [ngroups][32] physical input columns, accumulation order
+    const int32_t* cnt;      // [ngroups] shared inputs per group
+    const float* wv;         // [ngroups*16][32] weights, or nullptr (uniform exact value)
+    const int32_t* dst;      // [ngroups*16] physical output column, -1 = unused slot
+    int32_t* active;
+    int32_t* count_out;
+    int N, ngroups, nblk, stamp, prev_stamp, rl, wmode;
+    int full;                // 1: every group has exactly 32 shared inputs
+    float wu, bias, clampv;
+};
+hipError_t launch_block(const BlockLaunch& a, hipStream_t s);
+
 // Fused layer chain: `nlayers` consecutive BAND layers (same K and weight mode) in one launch,
 // one workgroup per row block.  Layer j reads what layer j-1 wrote: the first layer reads
 // first_in, every layer writes the work buffer (buf_a / buf_c) it did not read.

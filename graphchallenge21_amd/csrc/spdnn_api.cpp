@@ -117,6 +117,8 @@ struct DevLayer {
     int32_t* rowlen = nullptr;
     float* wv = nullptr;
     int32_t* dst = nullptr;
+    int32_t* blk_cols = nullptr;
+    int32_t* blk_cnt = nullptr;
 };
 
 }  // namespace
@@ -217,7 +219,8 @@ int ensure_uploaded(spdnn_net* n) {
     size_t total = 0;
     for (const LayerPlan& p : n->layers) {
         total += align256(p.in_pos.size() * 4) + align256(p.sel.size()) + align256(p.ell_col.size() * 4) +
-                 align256(p.rowlen.size() * 4) + align256(p.wv.size() * 4) + align256(p.dst.size() * 4);
+                 align256(p.rowlen.size() * 4) + align256(p.wv.size() * 4) + align256(p.dst.size() * 4) +
+                 align256(p.blk_cols.size() * 4) + align256(p.blk_cnt.size() * 4);
     }
     HIPCHK(hipMalloc(&n->arena, std::max<size_t>(total, 256)));
     n->dl.assign((size_t)n->L, DevLayer{});
@@ -238,6 +241,8 @@ int ensure_uploaded(spdnn_net* n) {
         HIPCHK(put(p.rowlen.data(), p.rowlen.size() * 4, (void**)&d.rowlen));
         HIPCHK(put(p.wv.data(), p.wv.size() * 4, (void**)&d.wv));
         HIPCHK(put(p.dst.data(), p.dst.size() * 4, (void**)&d.dst));
+        HIPCHK(put(p.blk_cols.data(), p.blk_cols.size() * 4, (void**)&d.blk_cols));
+        HIPCHK(put(p.blk_cnt.data(), p.blk_cnt.size() * 4, (void**)&d.blk_cnt));
     }
     std::vector<ChainLayerDesc> table((size_t)n->L);
     for (int l = 0; l < n->L; ++l) {
@@ -493,6 +498,15 @@ int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
     return SPDNN_OK;
 }
 
+int spdnn_get_layer_slots(const spdnn_net* n, int layer, int* slots) {
+    if (!n || !slots) return fail(SPDNN_E_ARG, "NULL argument");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    if (!n->layers[(size_t)layer].set) return fail(SPDNN_E_STATE, "layer has not been set");
+    *slots = (int)n->layers[(size_t)layer].out_at.size();
+    return SPDNN_OK;
+}
+
 int spdnn_get_input_labelling(const spdnn_net* n, int layer, int32_t* phys_col) {
     if (!n || !phys_col) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer > n->L) return fail(SPDNN_E_ARG, "layer out of range");
@@ -684,6 +698,14 @@ static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out,
         a.prev_stamp = prev_stamp;
         if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) { a.shape = t->shape; a.seglen = t->seglen; }
         return launch_band(a, n->stream);
+    }
+    if (p.kernel == SPDNN_KERNEL_BLOCK) {
+        BlockLaunch b{};
+        b.yin = in; b.yout = out; b.cols = d.blk_cols; b.cnt = d.blk_cnt; b.wv = d.wv; b.dst = d.dst;
+        b.active = n->d_active; b.count_out = count_out; b.N = n->N; b.ngroups = p.ngroups; b.nblk = nblk;
+        b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = p.wmode; b.full = p.blk_full ? 1 : 0;
+        b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
+        return launch_block(b, n->stream);
     }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;

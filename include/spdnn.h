@@ -50,7 +50,9 @@ enum spdnn_status {
 enum spdnn_kernel {
     SPDNN_KERNEL_AUTO = 0,
     SPDNN_KERNEL_GATHER = 1, /* general CSR/ELL gather, any sparsity pattern                      */
-    SPDNN_KERNEL_BAND = 2    /* row-succ / tiled: relabelled circulant band walked through an LDS ring */
+    SPDNN_KERNEL_BAND = 2,   /* row-succ / tiled: relabelled circulant band walked through an LDS ring */
+    SPDNN_KERNEL_BLOCK = 3   /* groups of outputs that read the same inputs (RadiX-Net style): the shared
+                                input columns are held in registers and reused by every output of the group */
 };
 
 typedef struct spdnn_layer_plan {
@@ -155,7 +157,11 @@ int spdnn_get_layer_plan(const spdnn_net* net, int layer, spdnn_layer_plan* out)
  * Any pointer may be NULL.  SPDNN_E_STATE if the layer is not a BAND layer. */
 int spdnn_get_band_plan(const spdnn_net* net, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel);
 
-/* Physical output column of every schedule slot of a layer (dst[N]); needs spdnn_inspect. */
+/* Number of schedule slots of a layer: neuron for BAND and GATHER layers, 16 per group for BLOCK
+ * layers (unused slots carry -1 in dst). */
+int spdnn_get_layer_slots(const spdnn_net* net, int layer, int* slots);
+
+/* Physical output column of every schedule slot of a layer (dst[slots]); needs spdnn_inspect. */
 int spdnn_get_layer_dst(const spdnn_net* net, int layer, int32_t* dst);
 
 /* Physical column of every neuron in the buffer layer `layer` reads (layer == layers: the

@@ -41,3 +41,29 @@ def same_floats(a, b):
     a = np.asarray(a, np.float32)
     b = np.asarray(b, np.float32)
     return a.shape == b.shape and bool(np.all((a == b) | (np.isnan(a) & np.isnan(b))))
+
+
+def radix_like_csr(rng, n, stride, values="uniform", relabel=True, run=16):
+    """RadiX-Net-like layer: the outputs of group g (16 consecutive outputs) all read the two
+    16-wide input runs [16g, 16g+16) and [16g+stride, 16g+stride+16) (mod n) - the structure the
+    reference's kernels assume after its hash reorder - optionally hidden behind random
+    relabellings of inputs and outputs, as in the raw challenge files."""
+    pin = rng.permutation(n) if relabel else np.arange(n)
+    pout = rng.permutation(n) if relabel else np.arange(n)
+    rows = [None] * n
+    for j in range(n):
+        g = j // run
+        ins = np.concatenate([np.arange(run * g, run * g + run), np.arange(run * g + stride, run * g + stride + run)]) % n
+        rows[pout[j]] = np.unique(pin[ins])
+    rowptr = np.zeros(n + 1, np.int32)
+    for j in range(n):
+        rowptr[j + 1] = rowptr[j] + len(rows[j])
+    col = np.concatenate(rows).astype(np.int32)
+    k = len(col)
+    if values == "uniform":
+        val = np.full(k, 0.0625, np.float32)
+    elif values == "pow2":
+        val = (np.ldexp(1.0, rng.integers(-6, -2, size=k)) * rng.choice([-1.0, 1.0], size=k)).astype(np.float32)
+    else:
+        val = rng.uniform(-0.1, 0.15, size=k).astype(np.float32)
+    return rowptr, col, val

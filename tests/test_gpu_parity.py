@@ -332,3 +332,32 @@ def test_fused_chain_when_everything_dies(gc, orc):
             assert [net.active_count(l) for l in range(L)] == want
             assert r.active_rows == 0 and len(net.categories()) == 0
             assert not net.activations(np.arange(50, dtype=np.int32)).any()
+
+
+@pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
+def test_block_kernel_radix_like_layers(gc, orc, values):
+    """RadiX-Net-like layers (16 outputs sharing two 16-wide input runs, hidden behind random
+    relabellings) go to the BLOCK kernel; mixed with a band layer and an irregular layer."""
+    from helpers import radix_like_csr
+    N, B = 1024, 300
+    print("block kernel values=%s" % values, flush=True)
+    rng = np.random.default_rng(17)
+    layers = [radix_like_csr(rng, N, 16 << l, values) for l in range(4)]
+    layers.append(orc.gen_layer_csr(3, 0, N))                                  # BAND
+    layers.append(radix_like_csr(rng, N, 256, values, run=8))                   # groups of 8, 16 inputs
+    layers.append(sort_rows(random_csr(rng, N, rng.integers(1, 20, size=N), "pow2")))   # GATHER
+    L = len(layers)
+    feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < 0.4)).astype(np.float32)
+    with gc.Network(N, B, L, bias=-0.2) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        kinds = [net.layer_plan(l).kernel for l in range(L)]
+        assert kinds == [gc.KERNEL_BLOCK] * 4 + [gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER]
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+        ref = orc.infer(feats, layers, -0.2, prune=True)
+        for prune in (True, False):
+            net.run(prune=prune, collect_counts=True)
+            assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+            assert np.array_equal(net.categories(), ref["categories"])

@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from helpers import random_csr, sort_rows
+from helpers import radix_like_csr, random_csr, sort_rows
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GOLD = os.path.join(ROOT, "tests", "golden")
@@ -94,9 +94,10 @@ def test_inspector_falls_back_to_gather(gc, orc):
     rng = np.random.default_rng(3)
     n = 256
     irregular = random_csr(rng, n, rng.integers(0, 20, size=n), "general")
-    # 8 entries per row AND per column but no band: output j reads inputs j, j+32, j+64, ... (mod n),
-    # i.e. 32 interleaved dense 8x8 blocks
-    cols = np.sort((np.arange(n)[:, None] + 32 * np.arange(8)[None, :]) % n, axis=1)
+    # 8 entries per row AND per column, no band and no two outputs with the same inputs:
+    # output j reads inputs (4k+1)*j + k (mod n), k = 0..7 (eight affine bijections of Z_n)
+    cols = np.sort((np.arange(n)[:, None] * (4 * np.arange(8)[None, :] + 1) + np.arange(8)[None, :]) % n, axis=1)
+    assert all(len(set(r)) == 8 for r in cols) and (np.bincount(cols.reshape(-1), minlength=n) == 8).all()
     regular_random = (np.arange(0, 8 * n + 1, 8, dtype=np.int32), cols.reshape(-1).astype(np.int32),
                       np.full(8 * n, 0.0625, np.float32))
     band = orc.gen_layer_csr(2, 0, n, 8)
@@ -119,6 +120,31 @@ def test_inspector_falls_back_to_gather(gc, orc):
         assert np.array_equal(net.input_labelling(0), np.arange(n))
         assert np.array_equal(net.layer_dst(1), net.input_labelling(2))
         assert np.array_equal(net.layer_dst(3), np.arange(n)[net.band_plan(3)[1]])
+
+
+def test_inspector_block_class(gc, orc):
+    """Outputs that read identical input lists are grouped (RadiX-Net style), whatever the
+    labelling; the plan lists every output exactly once."""
+    rng = np.random.default_rng(5)
+    n = 512
+    with gc.Network(n, 4, 3, bias=-0.3) as net:
+        net.set_layer_csr(0, *radix_like_csr(rng, n, 64, "uniform"))
+        net.set_layer_csr(1, *radix_like_csr(rng, n, 16, "general"))        # overlapping runs: 32 inputs still
+        net.set_layer_csr(2, *radix_like_csr(rng, n, 128, "pow2", run=8))   # groups of 8 outputs, 16 inputs
+        net.inspect()
+        p = [net.layer_plan(l) for l in range(3)]
+        assert [q.kernel for q in p] == [gc.KERNEL_BLOCK] * 3
+        assert (p[0].max_row_nnz, p[0].uniform_value, p[0].exact_products) == (32, 1, 1)
+        assert (p[1].uniform_value, p[1].exact_products) == (0, 0)
+        assert p[2].max_row_nnz == 16
+        for l in range(3):
+            dst = net.layer_dst(l)
+            used = dst[dst >= 0]
+            assert sorted(used.tolist()) == list(range(n))
+    with gc.Network(n, 4, 1, bias=-0.3, force_kernel=gc.KERNEL_GATHER) as net:
+        net.set_layer_csr(0, *radix_like_csr(rng, n, 64, "uniform"))
+        net.inspect()
+        assert net.layer_plan(0).kernel == gc.KERNEL_GATHER
 
 
 def test_forced_gather(gc, orc):
