@@ -361,3 +361,27 @@ def test_block_kernel_radix_like_layers(gc, orc, values):
             net.run(prune=prune, collect_counts=True)
             assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
             assert np.array_equal(net.categories(), ref["categories"])
+
+
+@pytest.mark.parametrize("N,B,L,bias", [(4096, 60000, 6, -0.35), (16384, 60000, 4, -0.4), (65536, 8192, 3, -0.45)])
+def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
+    """The wider configurations at (or near) full batch, features generated on the device with
+    survivor densities; the oracle runs a row sample (rows are independent)."""
+    print("wide N=%d B=%d" % (N, B), flush=True)
+    S = 384
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
+    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.60), layers, bias, prune=False, keep=set(range(L)))
+    rows = np.arange(S, dtype=np.int32)
+    with gc.Network(N, B, L) as net:
+        assert net.bias == pytest.approx(bias)
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, B, 0.10, 0.60)
+        for l in range(L):
+            net.run(prune=True, first_layer=l, n_layers=1)
+            cats = net.categories()
+            assert np.array_equal(cats[cats < S], ref["active_ids"][l]), "layer %d" % l
+            assert same_floats(net.activations(rows), ref["kept"][l][1]), "layer %d" % l
+        full = net.run(prune=False, collect_counts=True)
+        assert np.array_equal(net.categories()[net.categories() < S], ref["active_ids"][-1])
+        assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
