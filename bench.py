@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
+    ap.add_argument("--survivor-check", type=int, default=0, metavar="ROWS",
+                    help="extra (slow): features with densities up to 0.7 so that rows survive every layer; "
+                         "the category set of the first ROWS rows after ALL layers is compared with the oracle")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build is single-GPU (rows shard trivially, see DESIGN.md); run with --gpus 1")
@@ -159,6 +162,30 @@ def main():
         parity = {"rows": int(rows), "layers": n_check, "active_ids_equal": ok_ids,
                   "activations_bit_equal": ok_y, "max_abs_diff": max_abs}
 
+    survivor = None
+    if args.survivor_check > 0:
+        from oracle import oracle as orc
+        S = min(args.survivor_check, B)
+        net.synth_features(seed, B, 0.10, 0.70)
+        t0 = time.perf_counter()
+        rs = net.run(prune=True, collect_counts=True)
+        gpu_s = time.perf_counter() - t0
+        cats = net.categories()
+        got_y = net.activations(cats[cats < S][:64].astype(np.int32))
+        y = orc.gen_features(seed, N, 0, S, 0.10, 0.70)
+        gid = np.arange(S, dtype=np.int32)
+        t0 = time.perf_counter()
+        for l in range(L):
+            y, act = orc.layer(y, gc.synth_layer_csr(seed, l, N), bias)
+            y, gid = orc.compact(y, act, gid)
+            if l % 200 == 0:
+                log("survivor check: oracle layer %d, %d rows alive" % (l, len(gid)))
+        survivor = {"rows_checked": int(S), "layers": L, "gpu_categories_total": int(len(cats)),
+                    "oracle_categories_in_sample": int(len(gid)),
+                    "categories_equal": bool(np.array_equal(cats[cats < S], gid)),
+                    "activations_bit_equal": bool(np.array_equal(got_y, y[:64])),
+                    "gpu_pruned_run_s": gpu_s, "gpu_compactions": int(rs.compactions), "oracle_s": time.perf_counter() - t0}
+
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "band_walk_cfg4_hbm_traffic.txt")
     if os.path.exists(tpath) and args.config == "cfg4" and B == 60000:
@@ -199,6 +226,7 @@ def main():
         "layer0": {"ms": layer0_ms, "achieved_gbps": alg_bytes_launch / (layer0_ms * 1e-3) / 1e9,
                    "edges_per_s": B * float(nnz_layer) / (layer0_ms * 1e-3)},
         "parity": parity,
+        "survivor_check": survivor,
         "setup_s": {"inspector": t_inspect, "upload_and_features": t_features},
         "events_ms_per_step": ms_events / args.steps,
     }
