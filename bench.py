@@ -211,6 +211,7 @@ def main():
                         "pruning off (every layer at full batch), seed %d" % (args.config, N, L, B, bias, seed),
             "neuron": N, "layers": L, "batch": B, "bias": bias, "seed": seed,
             "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "mixed",
+            "band_tuning_rowblocks_shape_seglen": net.band_tuning(),
             "final_active_rows": sustained_final_active,
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",

@@ -85,6 +85,7 @@ def load_library():
         "spdnn_get_categories": ([vp, C.c_void_p, C.c_int64, C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_activations": ([vp, _i32p, C.c_int, _f32p], C.c_int),
         "spdnn_get_layer_times": ([vp, _f32p, C.c_int], C.c_int),
+        "spdnn_get_band_tuning": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
@@ -277,6 +278,16 @@ class Network:
         ms = np.empty(self.layers, np.float32)
         _check(self._lib.spdnn_get_layer_times(self._h, ms, self.layers))
         return ms
+
+    def band_tuning(self):
+        """[(row_blocks, shape, seglen), ...] measured so far."""
+        out, i = [], 0
+        while True:
+            a, b, c = C.c_int(), C.c_int(), C.c_int()
+            if self._lib.spdnn_get_band_tuning(self._h, i, C.byref(a), C.byref(b), C.byref(c)) != 0:
+                return out
+            out.append((a.value, b.value, c.value))
+            i += 1
 
     def write_categories(self, path):
         _check(self._lib.spdnn_write_categories(self._h, path.encode()))

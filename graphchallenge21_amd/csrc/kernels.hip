@@ -93,6 +93,12 @@ __device__ __forceinline__ bool block_is_dead(const int32_t* active, size_t row0
     return __syncthreads_or(any) == 0;
 }
 
+// Running "largest output so far" of a row.  Outputs are clamped to [0, clamp], so comparing the
+// bit patterns as signed integers orders them like the floats (one v_max_i32, no NaN handling).
+__device__ __forceinline__ float nz_merge(float nz, float y) {
+    return __int_as_float(max(__float_as_int(nz), __float_as_int(y)));
+}
+
 __device__ __forceinline__ float relu_clamp(float y, float clampv) {
     // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
     return __builtin_amdgcn_fmed3f(y, 0.0f, clampv);
@@ -287,7 +293,7 @@ __device__ __forceinline__ void band_walk_body(
 #pragma unroll
                 for (int q = 0; q < RL; ++q) {
                     y[q] = relu_clamp(acc[i][q] + bias, clampv);
-                    nz[q] = fmaxf(nz[q], y[q]);
+                    nz[q] = nz_merge(nz[q], y[q]);
                 }
                 const int d = dst[v[i]];
                 *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
@@ -424,7 +430,7 @@ __global__ __launch_bounds__(256) void gather_kernel(
 #pragma unroll
         for (int q = 0; q < RL; ++q) {
             y[q] = relu_clamp(acc[q] + bias, clampv);
-            nz[q] = fmaxf(nz[q], y[q]);
+            nz[q] = nz_merge(nz[q], y[q]);
         }
         *reinterpret_cast<V*>(yout + (size_t)dst[j] * RB + loff) = arr_to_vec<RL>(y);
     }
@@ -494,7 +500,7 @@ __global__ __launch_bounds__(256) void block_kernel(
 #pragma unroll
             for (int q = 0; q < RL; ++q) {
                 y[q] = relu_clamp(acc[q] + bias, clampv);
-                nz[q] = fmaxf(nz[q], y[q]);
+                nz[q] = nz_merge(nz[q], y[q]);
             }
             *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
         }
@@ -777,7 +783,23 @@ int band_workgroups_per_cu(int rl, int shape) {
 }
 
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out) {
-    return rank_seglens(N, K, band_chunk_outputs(rl, shape), nblk, n_cu * band_workgroups_per_cu(rl, shape), out, max_out);
+    // the two best-ranked by the fill/halo model, then a geometric ladder of segment counts:
+    // shorter segments mean more, smaller workgroups, which often balances and streams better
+    // than the model predicts - the caller measures
+    const int T = band_chunk_outputs(rl, shape);
+    int n = rank_seglens(N, K, T, nblk, n_cu * band_workgroups_per_cu(rl, shape), out, max_out < 2 ? max_out : 2);
+    const int nchunks = (N + T - 1) / T;
+    static const int ladder[] = {1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512};
+    for (int nseg : ladder) {
+        if (n >= max_out) break;
+        const int cps = (nchunks + nseg - 1) / nseg;
+        if (cps < 4 && nseg > 1) break;  // at least four chunks per workgroup
+        const int len = cps * T;
+        bool dup = false;
+        for (int i = 0; i < n; ++i) dup |= out[i] == len;
+        if (!dup) out[n++] = len;
+    }
+    return n;
 }
 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
@@ -787,6 +809,11 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     BandLaunch b = a;
     b.n_cu = (a.n_cu > 0 ? a.n_cu : 256) * band_workgroups_per_cu(a.rl, a.shape);
+    if (b.seglen <= 0) {
+        static const int env_seglen = getenv("SPDNN_BAND_SEGLEN") ? atoi(getenv("SPDNN_BAND_SEGLEN")) : 0;
+        b.seglen = env_seglen;  // tuning knob; rounded down to whole chunks, 0 = heuristic
+        if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);
+    }
     switch (a.rl) {
         case 4:
             if (resolve_shape(4, a.shape) == 1) return launch_band_rl<4, 8, 2, 64>(b, s);
@@ -983,7 +1010,7 @@ hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s) {
 
 hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s) {
     if (n_floats <= 0 || (n_floats % 4) != 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(copy_f4_kernel, dim3(256 * 16), dim3(256), 0, s, reinterpret_cast<const float4*>(src),
+    hipLaunchKernelGGL(copy_f4_kernel, dim3(65536), dim3(256), 0, s, reinterpret_cast<const float4*>(src),
                        reinterpret_cast<float4*>(dst), (long long)(n_floats / 4));
     return hipGetLastError();
 }

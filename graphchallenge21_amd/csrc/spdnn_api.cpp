@@ -650,8 +650,8 @@ static const spdnn_net::Tuned* find_tuned(const spdnn_net* n, int nblk, int K) {
 }
 
 // Run-time kernel selection for band layers (the measured half of the inspector's choice): time
-// each tile shape with its two best-ranked segment lengths on the real buffers of layer l and keep
-// the fastest for this row-block count.  The trial outputs land in the buffer the layer writes
+// each tile shape with a ladder of segment lengths on the real buffers of layer l and keep the
+// fastest for this row-block count.  The trial outputs land in the buffer the layer writes
 // anyway; every trial uses a fresh row stamp.
 static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk) {
     const LayerPlan& p = n->layers[(size_t)l];
@@ -662,19 +662,19 @@ static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk)
     float best_ms = 0.0f;
     hipError_t err = hipSuccess;
     for (int shape = 0; shape < band_shape_count(n->rl) && err == hipSuccess; ++shape) {
-        int lens[2];
-        const int nc = band_seglen_candidates(n->N, p.kmax, nblk, n->rl, shape, n->n_cu, lens, 2);
+        int lens[20];
+        const int nc = band_seglen_candidates(n->N, p.kmax, nblk, n->rl, shape, n->n_cu, lens, 20);
         for (int c = 0; c < nc && err == hipSuccess; ++c) {
             BandLaunch a = band_args(n, l, in, out, nblk, 0);
             a.active = n->d_active_scratch;  // trials must not disturb the real row stamps
             a.shape = shape;
             a.seglen = lens[c];
             float ms = 0.0f;
-            for (int rep = 0; rep < 2 && err == hipSuccess; ++rep) {  // first launch warms the code path
+            for (int rep = 0; rep < 3 && err == hipSuccess; ++rep) {  // first launch warms up, two are timed
                 a.stamp = ++n->stamp;
                 if (rep == 1) err = hipEventRecord(e0, n->stream);
                 if (err == hipSuccess) err = launch_band(a, n->stream);
-                if (rep == 1 && err == hipSuccess) err = hipEventRecord(e1, n->stream);
+                if (rep == 2 && err == hipSuccess) err = hipEventRecord(e1, n->stream);
             }
             if (err == hipSuccess) err = hipEventSynchronize(e1);
             if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
@@ -968,6 +968,16 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
     hipFree(d_phys);
     hipFree(d_out);
     if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    return SPDNN_OK;
+}
+
+int spdnn_get_band_tuning(const spdnn_net* n, int index, int* row_blocks, int* shape, int* seglen) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (index < 0 || index >= (int)n->tuned.size()) return fail(SPDNN_E_ARG, "no such tuning record");
+    const spdnn_net::Tuned& t = n->tuned[(size_t)index];
+    if (row_blocks) *row_blocks = t.nblk;
+    if (shape) *shape = t.shape;
+    if (seglen) *seglen = t.seglen;
     return SPDNN_OK;
 }
 

@@ -212,6 +212,12 @@ int spdnn_get_categories(spdnn_net* net, int32_t* ids, int64_t cap, int64_t* n);
  * (all_network.cu:521). */
 int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
 
+/* Band-walk configuration measured at run time (record `index` = 0, 1, ...; SPDNN_E_ARG past the
+ * last): row blocks it was measured for, tile shape (0: 16 waves x 3 outputs, 128-slot LDS ring,
+ * one workgroup per CU; 1: 8 waves x 2 outputs, 64-slot ring, two workgroups per CU) and band
+ * positions per workgroup. */
+int spdnn_get_band_tuning(const spdnn_net* net, int index, int* row_blocks, int* shape, int* seglen);
+
 /* Per-layer kernel milliseconds of the last run made with time_layers. */
 int spdnn_get_layer_times(const spdnn_net* net, float* ms, int n);
 
