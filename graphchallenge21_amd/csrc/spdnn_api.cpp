@@ -8,7 +8,6 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
-#include <atomic>
 #include <cmath>
 #include <condition_variable>
 #include <cstdio>
@@ -131,8 +130,6 @@ struct spdnn_net {
     int force_kernel = SPDNN_KERNEL_AUTO;
     std::vector<LayerPlan> layers;
     std::unique_ptr<JobPool> pool;
-    std::mutex err_m;
-    std::string worker_err;
     bool inspected = false;
 
     // device
@@ -163,7 +160,6 @@ struct spdnn_net {
     bool alive_list_valid = false;
     bool gid_dirty = false;   // a repack permuted d_gid since it was last initialised
     int last_stamp = 0;       // stamp of the newest layer, valid for the current row slots (0 = none)
-    bool repacked_after_last = false;
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
     ChainLayerDesc* d_chain = nullptr;
     std::vector<char> pending; // layer has an inspection job in flight
@@ -286,7 +282,6 @@ void reset_state(spdnn_net* n) {
     }
     n->cur = n->F;
     n->last_stamp = 0;
-    n->repacked_after_last = false;
     n->cur_layer = 0;
     n->carried = ((n->batch + n->RB - 1) / n->RB) * n->RB;
     n->alive = n->batch;
@@ -855,12 +850,9 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 n->cur = dstbuf;
                 n->carried = nb * n->RB;
                 n->last_stamp = 0;  // the row slots moved: the stamps no longer describe them
-                n->repacked_after_last = true;
                 r.compactions++;
-                continue;
             }
         }
-        n->repacked_after_last = false;
     }
     // categories of the last layer: survivor list by the scan.  After a final repack the list
     // produced for the repack is that list already.
