@@ -216,7 +216,45 @@ bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vecto
         i = e;
     }
     // worth it only if an input column loaded into registers is reused by several outputs
-    return (int64_t)groups.size() * 8 <= (int64_t)N;
+    if ((int64_t)groups.size() * 8 > (int64_t)N) return false;
+
+    // Chain order: put groups that share inputs next to each other (greedy nearest neighbour on
+    // the number of shared inputs), so that a wave walking consecutive groups finds the columns
+    // it re-reads still in L2.
+    const int ng = (int)groups.size();
+    std::vector<std::vector<int32_t>> users((size_t)N);  // groups reading each input
+    for (int g = 0; g < ng; ++g) {
+        const int j0 = groups[(size_t)g][0];
+        for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e) users[(size_t)col[e]].push_back(g);
+    }
+    std::vector<uint8_t> placed((size_t)ng, 0);
+    std::vector<int32_t> shared((size_t)ng, 0), touched;
+    std::vector<std::vector<int32_t>> ordered;
+    ordered.reserve((size_t)ng);
+    int next_fresh = 0;
+    for (int cur = 0, done = 0; done < ng; ++done) {
+        if (done == 0 || cur < 0) {
+            while (placed[(size_t)next_fresh]) ++next_fresh;
+            cur = next_fresh;
+        }
+        placed[(size_t)cur] = 1;
+        ordered.push_back(std::move(groups[(size_t)cur]));
+        const int j0 = ordered.back()[0];
+        touched.clear();
+        for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e)
+            for (int32_t g : users[(size_t)col[e]])
+                if (!placed[(size_t)g] && shared[(size_t)g]++ == 0) touched.push_back(g);
+        int best = -1;
+        for (int32_t g : touched) {
+            if (best < 0 || shared[(size_t)g] > shared[(size_t)best] ||
+                (shared[(size_t)g] == shared[(size_t)best] && g < best))
+                best = g;
+        }
+        for (int32_t g : touched) shared[(size_t)g] = 0;
+        cur = best;
+    }
+    groups.swap(ordered);
+    return true;
 }
 
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,

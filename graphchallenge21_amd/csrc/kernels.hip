@@ -898,7 +898,7 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     // groups per wave: enough workgroups to fill the chip several times over, but long enough
     // runs per wave to amortise the launch
-    int gpw = 4;
+    int gpw = 8;
     while (gpw > 1 && (long long)a.nblk * ((a.ngroups + 4 * gpw - 1) / (4 * gpw)) < 2048) gpw >>= 1;
     dim3 grid(a.nblk, (a.ngroups + 4 * gpw - 1) / (4 * gpw)), block(256);
     if (grid.y > 65535) return hipErrorInvalidValue;
