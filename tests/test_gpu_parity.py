@@ -385,3 +385,46 @@ def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
         full = net.run(prune=False, collect_counts=True)
         assert np.array_equal(net.categories()[net.categories() < S], ref["active_ids"][-1])
         assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
+
+
+@pytest.mark.parametrize("N,K,B", [(256, 32, 1), (256, 4, 65), (512, 12, 257), (128, 8, 40), (100, 5, 33), (2048, 36, 70)])
+def test_small_and_odd_shapes(gc, orc, N, K, B):
+    """Smallest band layers, a single row, widths that are not a multiple of 256 and rows longer
+    than 32 entries (general kernel)."""
+    print("odd shape N=%d K=%d B=%d" % (N, K, B), flush=True)
+    L = 3
+    layers = [orc.gen_layer_csr(4, l, N, K, 0.0625) for l in range(L)]
+    feats = orc.gen_features(4, N, 0, B, 0.2, 0.9)
+    with gc.Network(N, B, L, bias=-0.05) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        want = gc.KERNEL_BAND if (N % 256 == 0 and K % 4 == 0 and K <= 32) else gc.KERNEL_GATHER
+        assert all(net.layer_plan(l).kernel == want for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+        ref = orc.infer(feats, layers, -0.05, prune=True)
+        net.run(prune=True)
+        assert np.array_equal(net.categories(), ref["categories"])
+
+
+def test_empty_rows_and_single_layer(gc, orc):
+    """Outputs without any input (their value is relu(bias)) and a one-layer network."""
+    N, B = 64, 20
+    print("empty rows", flush=True)
+    rng = np.random.default_rng(2)
+    nnz = rng.integers(0, 6, size=N)
+    nnz[:5] = 0
+    csr = sort_rows(random_csr(rng, N, nnz, "general"))
+    feats = rng.uniform(0, 5, size=(B, N)).astype(np.float32)
+    feats[3] = 0
+    for bias in (-0.1, 0.2):
+        with gc.Network(N, B, 1, bias=bias) as net:
+            net.set_layer_csr(0, *csr)
+            net.inspect()
+            net.set_features_dense(feats)
+            net.run(prune=False, collect_counts=True)
+            y, act = orc.layer(feats, csr, bias)
+            assert same_floats(net.activations(np.arange(B, dtype=np.int32)), y)
+            assert np.array_equal(net.categories(), np.nonzero(act)[0])
+            assert net.active_count(0) == int(act.sum())
