@@ -428,3 +428,38 @@ def test_empty_rows_and_single_layer(gc, orc):
             assert same_floats(net.activations(np.arange(B, dtype=np.int32)), y)
             assert np.array_equal(net.categories(), np.nonzero(act)[0])
             assert net.active_count(0) == int(act.sum())
+
+
+def test_cli_driver_on_tsv_files(gc, orc, tmp_path):
+    """spdnn_network (the reference's `exe neuron batch layer` command line) on challenge-format
+    TSV files in the reference's directory layout; categories against the oracle."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(gc.lib_path()), "spdnn_network")
+    if not os.path.exists(exe):
+        pytest.skip("driver not built")
+    N, B, L = 1024, 300, 4
+    print("cli driver", flush=True)
+    data = tmp_path / "data"
+    (data / ("neuron%d" % N)).mkdir(parents=True)
+    layers = [orc.gen_layer_csr(6, l, N) for l in range(L)]
+    for l, (rowptr, col, val) in enumerate(layers):
+        with open(gc.weight_file_name(str(data), N, l), "w") as f:
+            f.writelines("%d\t%d\t%.9g\n" % (col[e] + 1, j + 1, val[e]) for j in range(N) for e in range(rowptr[j], rowptr[j + 1]))
+    feats = orc.gen_features(6, N, 0, B, 0.10, 0.55)
+    with open(data / ("sparse-images-%d.tsv" % N), "w") as f:
+        rr, cc = np.nonzero(feats)
+        f.writelines("%d\t%d\t1\n" % (r + 1, c + 1) for r, c in zip(rr, cc))
+    ref = orc.infer(feats, layers, -0.3, prune=True)
+    out = tmp_path / "categories.tsv"
+    r = subprocess.run([exe, str(N), str(B), str(L), "--data", str(data), "--categories", str(out)],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    for l in range(L):
+        assert "layer %d, batch = %d" % (l, len(ref["active_ids"][l])) in r.stdout
+    got = np.array([int(x) for x in out.read_text().split()], dtype=np.int64)
+    assert np.array_equal(got, ref["categories"] + 1)
+    # without files the driver falls back to the seeded generator
+    r = subprocess.run([exe, str(N), "200", "3", "--data", str(tmp_path / "nowhere"), "--quiet"],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "seeded generator" in r.stdout
