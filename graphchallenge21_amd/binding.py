@@ -64,6 +64,7 @@ def load_library():
         "spdnn_reference_bias": ([C.c_int, C.POINTER(C.c_float)], C.c_int),
         "spdnn_set_layer_csr": ([vp, C.c_int, _i32p, _i32p, _f32p], C.c_int),
         "spdnn_load_layer_tsv": ([vp, C.c_int, C.c_char_p], C.c_int),
+        "spdnn_load_layers_bin": ([vp, C.c_char_p, C.c_int, C.c_int, C.c_int64], C.c_int),
         "spdnn_weight_file_name": ([C.c_char_p, C.c_int, C.c_int, C.c_char_p, C.c_int], C.c_int),
         "spdnn_synth_layers": ([vp, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_float], C.c_int),
         "spdnn_synth_layer_csr": ([C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_float, _i32p, _i32p, _f32p], C.c_int),
@@ -77,6 +78,7 @@ def load_library():
         "spdnn_hash_reorder": ([C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int)], C.c_int),
         "spdnn_set_features_dense": ([vp, _f32p, C.c_int], C.c_int),
         "spdnn_load_features_tsv": ([vp, C.c_char_p, C.c_int], C.c_int),
+        "spdnn_load_features_bin": ([vp, C.c_char_p, C.c_int], C.c_int),
         "spdnn_synth_features": ([vp, C.c_uint64, C.c_int, C.c_float, C.c_float], C.c_int),
         "spdnn_synth_features_host": ([C.c_uint64, C.c_int, C.c_int64, C.c_int64, C.c_float, C.c_float, _f32p], C.c_int),
         "spdnn_default_run_options": ([C.POINTER(RunOptions)], C.c_int),
@@ -190,6 +192,10 @@ class Network:
     def load_layer_tsv(self, layer, path):
         _check(self._lib.spdnn_load_layer_tsv(self._h, layer, path.encode()))
 
+    def load_layers_bin(self, path, first=0, count=None, nnz_per_layer=0):
+        count = self.layers - first if count is None else count
+        _check(self._lib.spdnn_load_layers_bin(self._h, path.encode(), first, count, nnz_per_layer))
+
     def synth_layers(self, seed, first=0, count=None, nnz_per_row=32, value=0.0625):
         count = self.layers - first if count is None else count
         _check(self._lib.spdnn_synth_layers(self._h, seed, first, count, nnz_per_row, value))
@@ -236,6 +242,10 @@ class Network:
 
     def load_features_tsv(self, path, batch):
         _check(self._lib.spdnn_load_features_tsv(self._h, path.encode(), batch))
+        self.batch = batch
+
+    def load_features_bin(self, path, batch):
+        _check(self._lib.spdnn_load_features_bin(self._h, path.encode(), batch))
         self.batch = batch
 
     def synth_features(self, seed, batch, dmin=0.10, dmax=0.25):

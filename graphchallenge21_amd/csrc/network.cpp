@@ -9,8 +9,10 @@
 // layers on the GPU and prints "layer l, batch = n" per layer (all_network.cu:508).  Unlike the
 // reference it goes through the C ABI (include/spdnn.h): the inspector runs behind the
 // boundary, errors are reported instead of exit()ing inside the library, and the categories
-// can be written out.  When the data files are absent (or with --synthetic) the seeded
-// generator provides weights and features of the same shape.
+// can be written out.  Where the TSV files are absent but the packed files of the reference's
+// library benchmarks exist (<data>/neuron<N>.bin and <data>/sparse-images-<N>.bin,
+// benchmark/cusparse/cusparse.cu:318-383) those are read instead.  When no data files are there
+// (or with --synthetic) the seeded generator provides weights and features of the same shape.
 //
 // Options:
 //   --data DIR        data directory (default ../data, as in the reference)
@@ -89,6 +91,9 @@ int main(int argc, char** argv) {
     char wname[4096];
     CHECK(spdnn_weight_file_name(data.c_str(), neuron, 0, wname, sizeof(wname)));
     const bool from_files = !synthetic && file_exists(feat_file) && file_exists(wname);
+    const std::string feat_bin = data + "/sparse-images-" + std::to_string(neuron) + ".bin";
+    const std::string weight_bin = data + "/neuron" + std::to_string(neuron) + ".bin";
+    const bool from_bin = !synthetic && !from_files && file_exists(feat_bin) && file_exists(weight_bin);
 
     double t0 = now_s();
     if (from_files) {
@@ -97,6 +102,9 @@ int main(int argc, char** argv) {
             CHECK(spdnn_load_layer_tsv(net, l, wname));
             if (!quiet) printf("[%s] to CSR success!\n", wname);
         }
+    } else if (from_bin) {
+        CHECK(spdnn_load_layers_bin(net, weight_bin.c_str(), 0, layer, 0));
+        if (!quiet) printf("[%s] to CSR success!\n", weight_bin.c_str());
     } else {
         printf("data files not used: seeded generator, seed %llu\n", seed);
         CHECK(spdnn_synth_layers(net, seed, 0, layer, 32, 0.0625f));
@@ -112,6 +120,7 @@ int main(int argc, char** argv) {
 
     t0 = now_s();
     if (from_files) CHECK(spdnn_load_features_tsv(net, feat_file.c_str(), batch));
+    else if (from_bin) CHECK(spdnn_load_features_bin(net, feat_bin.c_str(), batch));
     else CHECK(spdnn_synth_features(net, seed, batch, dmin, dmax));
     printf("Read Input success! (%.2f s)\n", now_s() - t0);
 

@@ -403,6 +403,22 @@ int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
     return spdnn_set_layer_csr(n, layer, rp.data(), cc.data(), vv.data());
 }
 
+int spdnn_load_layers_bin(spdnn_net* n, const char* path, int first, int count, int64_t nnz_per_layer) {
+    if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
+    if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
+    const int64_t nnz = nnz_per_layer > 0 ? nnz_per_layer : (int64_t)32 * n->N;
+    if (nnz > (int64_t)INT32_MAX) return fail(SPDNN_E_ARG, "nnz_per_layer too large");
+    std::vector<int32_t> rp, cc;
+    std::vector<float> vv;
+    std::string err;
+    for (int l = first; l < first + count; ++l) {
+        if (!read_weight_bin_csr(path, n->N, l, nnz, rp, cc, vv, err)) return fail(SPDNN_E_IO, err);
+        const int rc = spdnn_set_layer_csr(n, l, rp.data(), cc.data(), vv.data());
+        if (rc) return rc;
+    }
+    return SPDNN_OK;
+}
+
 int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap) {
     if (!data_dir || !out || cap < 1) return fail(SPDNN_E_ARG, "NULL argument");
     const int w = snprintf(out, (size_t)cap, "%s/neuron%d/n%d-l%d.tsv", data_dir, neuron, neuron, layer + 1);
@@ -582,6 +598,16 @@ int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
     std::string err;
     int64_t kept = 0;
     if (!read_features_tsv_dense(path, n->N, batch, dense, &kept, err)) return fail(SPDNN_E_IO, err);
+    return spdnn_set_features_dense(n, dense.data(), batch);
+}
+
+int spdnn_load_features_bin(spdnn_net* n, const char* path, int batch) {
+    if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
+    if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
+    std::vector<float> dense;
+    std::string err;
+    int64_t kept = 0;
+    if (!read_features_bin_dense(path, n->N, batch, dense, &kept, err)) return fail(SPDNN_E_IO, err);
     return spdnn_set_features_dense(n, dense.data(), batch);
 }
 

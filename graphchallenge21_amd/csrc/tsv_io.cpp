@@ -75,4 +75,67 @@ bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vec
     return true;
 }
 
+// ---- packed binary files (benchmark/cusparse/cusparse.cu:318-383) ---------------------------
+
+static bool read_exact(FILE* f, void* dst, size_t bytes) { return bytes == 0 || fread(dst, 1, bytes, f) == bytes; }
+
+bool read_weight_bin_csr(const std::string& path, int N, int layer, int64_t nnz, std::vector<int32_t>& rowptr,
+                         std::vector<int32_t>& col, std::vector<float>& val, std::string& err) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) { err = "FILE:" + path + " does not exists."; return false; }
+    const int64_t rec = nnz * 12;
+    if (fseeko(f, (off_t)(rec * layer), SEEK_SET) != 0) { fclose(f); err = "seek failed: " + path; return false; }
+    std::vector<int32_t> r((size_t)nnz), c((size_t)nnz);
+    std::vector<float> v((size_t)nnz);
+    const bool ok = read_exact(f, r.data(), (size_t)nnz * 4) && read_exact(f, c.data(), (size_t)nnz * 4) &&
+                    read_exact(f, v.data(), (size_t)nnz * 4);
+    fclose(f);
+    if (!ok) { err = "short read (layer record " + std::to_string(layer) + "): " + path; return false; }
+    rowptr.assign((size_t)N + 1, 0);
+    for (int64_t e = 0; e < nnz; ++e) {
+        const int out = r[(size_t)e] - 1, in = c[(size_t)e] - 1;
+        if (in < 0 || in >= N || out < 0 || out >= N) { err = "neuron index out of range in " + path; return false; }
+        rowptr[(size_t)out + 1]++;
+    }
+    for (int j = 0; j < N; ++j) rowptr[j + 1] += rowptr[j];
+    col.resize((size_t)nnz);
+    val.resize((size_t)nnz);
+    std::vector<int32_t> fill(rowptr.begin(), rowptr.end() - 1);
+    for (int64_t e = 0; e < nnz; ++e) {
+        const int out = r[(size_t)e] - 1;
+        col[(size_t)fill[out]] = c[(size_t)e] - 1;
+        val[(size_t)fill[out]] = v[(size_t)e];
+        fill[out]++;
+    }
+    return true;
+}
+
+bool read_features_bin_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
+                             int64_t* kept, std::string& err) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) { err = "FILE:" + path + " does not exists."; return false; }
+    fseeko(f, 0, SEEK_END);
+    const int64_t sz = (int64_t)ftello(f);
+    fseeko(f, 0, SEEK_SET);
+    if (sz % 12 != 0) { fclose(f); err = "size is not a multiple of 12 bytes: " + path; return false; }
+    const int64_t nnz = sz / 12;
+    std::vector<int32_t> r((size_t)nnz), c((size_t)nnz);
+    std::vector<float> v((size_t)nnz);
+    const bool ok = read_exact(f, r.data(), (size_t)nnz * 4) && read_exact(f, c.data(), (size_t)nnz * 4) &&
+                    read_exact(f, v.data(), (size_t)nnz * 4);
+    fclose(f);
+    if (!ok) { err = "short read: " + path; return false; }
+    dense.assign((size_t)batch * (size_t)N, 0.0f);
+    int64_t k = 0;
+    for (int64_t e = 0; e < nnz; ++e) {
+        const int neuron = r[(size_t)e], image = c[(size_t)e];
+        if (image > batch) continue;  // cusparse.cu:376: images beyond the batch are skipped
+        if (image < 1 || neuron < 1 || neuron > N) { err = "feature index out of range in " + path; return false; }
+        dense[(size_t)(image - 1) * (size_t)N + (size_t)(neuron - 1)] = v[(size_t)e];
+        ++k;
+    }
+    if (kept) *kept = k;
+    return true;
+}
+
 }  // namespace spdnn

@@ -23,4 +23,14 @@ bool read_weight_tsv_csr(const std::string& path, int N, std::vector<int32_t>& r
 bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
                              int64_t* kept, std::string& err);
 
+// Packed binary files as the reference's library benchmarks consume them
+// (benchmark/cusparse/cusparse.cu:318-383): "neuron{N}.bin" holds one record per layer of
+// int32 row[nnz], int32 col[nnz], float32 val[nnz] (1-based; row = OUTPUT neuron = CSR row,
+// col = input neuron, nnz = 32 N in the reference); "sparse-images-{N}.bin" holds int32 row[] (neuron),
+// int32 col[] (image), float32 val[] over the whole file.  `layer` selects the record.
+bool read_weight_bin_csr(const std::string& path, int N, int layer, int64_t nnz, std::vector<int32_t>& rowptr,
+                         std::vector<int32_t>& col, std::vector<float>& val, std::string& err);
+bool read_features_bin_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
+                             int64_t* kept, std::string& err);
+
 }  // namespace spdnn

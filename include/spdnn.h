@@ -123,6 +123,13 @@ int spdnn_set_layer_csr(spdnn_net* net, int layer, const int32_t* rowptr, const 
  * COOMatrix(file, 1, false) (src/utils/matrix.h:255-282), and sets the layer. */
 int spdnn_load_layer_tsv(spdnn_net* net, int layer, const char* path);
 
+/* Reads layers [first, first+count) from a packed binary weight file "neuron<N>.bin" as the
+ * reference's library benchmarks consume it (readweights, benchmark/cusparse/cusparse.cu:318-358):
+ * one record per layer of int32 row[nnz], int32 col[nnz], float32 val[nnz], 1-based, with
+ * row = OUTPUT neuron (the CSR row there) and col = input neuron.  nnz_per_layer = 0 means
+ * 32 * neuron, the only size the reference reads. */
+int spdnn_load_layers_bin(spdnn_net* net, const char* path, int first, int count, int64_t nnz_per_layer);
+
 /* File name the reference driver uses for a layer: <dir>/neuron<N>/n<N>-l<layer+1>.tsv
  * (get_weight_file_name, src/network.cpp:14-19). */
 int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap);
@@ -181,6 +188,11 @@ int spdnn_set_features_dense(spdnn_net* net, const float* rowmajor, int batch);
 /* Sparse feature TSV in the challenge format ("row neuron value", 1-based; rows beyond batch
  * are skipped): read_input, src/network.cpp:33-54. */
 int spdnn_load_features_tsv(spdnn_net* net, const char* path, int batch);
+
+/* Packed binary features "sparse-images-<N>.bin" (readinput, benchmark/cusparse/cusparse.cu:361-383):
+ * int32 row[] = neuron, int32 col[] = image, float32 val[], 1-based, the entry count being the file
+ * size / 12; images beyond batch are skipped. */
+int spdnn_load_features_bin(spdnn_net* net, const char* path, int batch);
 
 /* Seeded Bernoulli rows generated on the device: row r has density uniform in [dmin, dmax],
  * entries are 0.0f / 1.0f.  spdnn_synth_features_host produces the same values on the host. */

@@ -2,6 +2,9 @@
 
 TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the
 CPU-baseline leg of bench.py, never by the graphchallenge21_amd package.
+
+Parity unpinned: read_weights_bin and read_features_bin follow the way the reference's library
+benchmark reads its packed files, but no such file ships with the reference to check them against.
 """
 import ctypes as C
 import os
@@ -144,6 +147,40 @@ def read_features_tsv(path, neuron, batch):
     if kept < 0:
         raise FileNotFoundError(path)
     return dense, int(kept)
+
+
+def read_weights_bin(path, neuron, layer, nnz=None):
+    """Layer record `layer` of a packed "neuron<N>.bin" as CSR (rowptr, col, val), following readweights
+    of the reference's library benchmark (benchmark/cusparse/cusparse.cu:318-358): int32 row[nnz],
+    int32 col[nnz], float32 val[nnz] per layer, 1-based; CSR row = row-1 (the output neuron of
+    C = A*B there, cusparse.cu:118-150), CSR column = col-1, entries of a row in file order."""
+    nnz = 32 * neuron if nnz is None else nnz
+    with open(path, "rb") as f:
+        f.seek(12 * nnz * layer)
+        row = np.fromfile(f, dtype="<i4", count=nnz)
+        col = np.fromfile(f, dtype="<i4", count=nnz)
+        val = np.fromfile(f, dtype="<f4", count=nnz)
+    if len(val) != nnz:
+        raise IOError("short read")
+    order = np.argsort(row, kind="stable")
+    rowptr = np.zeros(neuron + 1, dtype=np.int32)
+    np.cumsum(np.bincount(row - 1, minlength=neuron), out=rowptr[1:])
+    return rowptr, (col[order] - 1).astype(np.int32), val[order].astype(np.float32)
+
+
+def read_features_bin(path, neuron, batch):
+    """Dense batch x neuron features from a packed "sparse-images-<N>.bin" (readinput,
+    benchmark/cusparse/cusparse.cu:361-383): int32 row[] = neuron, int32 col[] = image,
+    float32 val[]; images beyond `batch` are skipped."""
+    raw = np.fromfile(path, dtype="<i4")
+    n = len(raw) // 3
+    row, col = raw[:n], raw[n:2 * n]
+    val = raw[2 * n:3 * n].view("<f4")
+    dense = np.zeros((batch, neuron), dtype=np.float32)
+    for e in range(n):                      # file order: a later duplicate overwrites an earlier one
+        if col[e] - 1 < batch:
+            dense[col[e] - 1, row[e] - 1] = val[e]
+    return dense
 
 
 def relu_clamp(x):

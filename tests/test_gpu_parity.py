@@ -463,3 +463,60 @@ def test_cli_driver_on_tsv_files(gc, orc, tmp_path):
     r = subprocess.run([exe, str(N), "200", "3", "--data", str(tmp_path / "nowhere"), "--quiet"],
                        capture_output=True, text=True, timeout=100)
     assert r.returncode == 0 and "seeded generator" in r.stdout
+
+
+def test_packed_binary_files(gc, orc, tmp_path):
+    """Weights and features in the packed binary layout the reference's library benchmarks read
+    (benchmark/cusparse/cusparse.cu:318-383), through the library and through the command-line
+    driver; the oracle reads the same files with its own reader."""
+    import os
+    import subprocess
+    N, B, L = 1024, 333, 3
+    print("packed binary", flush=True)
+    rng = np.random.default_rng(4)
+    layers = [orc.gen_layer_csr(12, l, N) for l in range(L)]
+    with open(tmp_path / ("neuron%d.bin" % N), "wb") as f:
+        for rowptr, col, val in layers:
+            row = np.repeat(np.arange(N, dtype=np.int32), np.diff(rowptr))
+            perm = rng.permutation(len(col))
+            (row[perm] + 1).astype("<i4").tofile(f)
+            (col[perm] + 1).astype("<i4").tofile(f)
+            val[perm].astype("<f4").tofile(f)
+    feats = orc.gen_features(12, N, 0, B + 20, 0.10, 0.55)     # 20 images more than the batch
+    img, neu = np.nonzero(feats)
+    perm = rng.permutation(len(img))
+    with open(tmp_path / ("sparse-images-%d.bin" % N), "wb") as f:
+        (neu[perm] + 1).astype("<i4").tofile(f)
+        (img[perm] + 1).astype("<i4").tofile(f)
+        feats[img[perm], neu[perm]].astype("<f4").tofile(f)
+    wpath, fpath = str(tmp_path / ("neuron%d.bin" % N)), str(tmp_path / ("sparse-images-%d.bin" % N))
+    ofeats = orc.read_features_bin(fpath, N, B)
+    assert np.array_equal(ofeats, feats[:B])
+    olayers = [orc.read_weights_bin(wpath, N, l) for l in range(L)]
+    ref = orc.infer(ofeats, [(rp, *_sorted_rows(rp, c, v)) for rp, c, v in olayers], -0.3, prune=True)
+    with gc.Network(N, B, L, bias=-0.3) as net:
+        net.load_layers_bin(wpath)
+        net.inspect()
+        net.load_features_bin(fpath, B)
+        net.run(prune=True, collect_counts=True)
+        assert np.array_equal(net.categories(), ref["categories"])
+        for l in range(L):
+            assert net.active_count(l) == len(ref["active_ids"][l])
+        assert np.array_equal(net.activations(ref["categories"][:50].astype(np.int32)), ref["y"][:50])
+    exe = os.path.join(os.path.dirname(gc.lib_path()), "spdnn_network")
+    if os.path.exists(exe):
+        out = tmp_path / "cat.tsv"
+        r = subprocess.run([exe, str(N), str(B), str(L), "--data", str(tmp_path), "--categories", str(out), "--quiet"],
+                           capture_output=True, text=True, timeout=100)
+        assert r.returncode == 0, r.stdout + r.stderr
+        got = np.array([int(x) for x in out.read_text().split()], dtype=np.int64)
+        assert np.array_equal(got, ref["categories"] + 1)
+
+
+def _sorted_rows(rowptr, col, val):
+    col, val = col.copy(), val.copy()
+    for j in range(len(rowptr) - 1):
+        a, b = rowptr[j], rowptr[j + 1]
+        o = np.argsort(col[a:b], kind="stable")
+        col[a:b], val[a:b] = col[a:b][o], val[a:b][o]
+    return col, val

@@ -182,6 +182,54 @@ def test_tsv_layer_through_the_library(gc, orc, tmp_path):
         assert net.layer_plan(0).nnz == 64 * 8
 
 
+def _write_weights_bin(path, layers):
+    """Packed weight file in the layout readweights of the reference's library benchmark reads
+    (benchmark/cusparse/cusparse.cu:340-347): per layer row[], col[], val[], 1-based, row = output."""
+    rng = np.random.default_rng(3)
+    with open(path, "wb") as f:
+        for rowptr, col, val in layers:
+            row = np.repeat(np.arange(len(rowptr) - 1, dtype=np.int32), np.diff(rowptr))
+            perm = rng.permutation(len(col))
+            (row[perm] + 1).astype("<i4").tofile(f)
+            (col[perm] + 1).astype("<i4").tofile(f)
+            val[perm].astype("<f4").tofile(f)
+
+
+def test_packed_binary_layers_through_the_library(gc, orc, tmp_path):
+    n = 256
+    layers = [orc.gen_layer_csr(8, l, n, 32) for l in range(3)]
+    p = tmp_path / "neuron256.bin"
+    _write_weights_bin(p, layers)
+    for l in range(3):   # the oracle's reader gives the layers back (rows sorted by input index)
+        rowptr, col, val = orc.read_weights_bin(str(p), n, l)
+        srt = [np.sort(col[rowptr[j]:rowptr[j + 1]]) for j in range(n)]
+        assert np.array_equal(rowptr, layers[l][0]) and np.array_equal(np.concatenate(srt), layers[l][1])
+        assert np.all(val == np.float32(0.0625))
+    with gc.Network(n, 4, 3, bias=-0.3) as a, gc.Network(n, 4, 3, bias=-0.3) as b:
+        a.load_layers_bin(str(p))
+        for l in range(3):
+            b.set_layer_csr(l, *layers[l])
+        a.inspect()
+        b.inspect()
+        for l in range(3):
+            assert a.layer_plan(l).kernel == gc.KERNEL_BAND
+            for x, y in zip(a.band_plan(l), b.band_plan(l)):
+                assert np.array_equal(x, y)
+            assert np.array_equal(a.layer_dst(l), b.layer_dst(l))
+        # a single record out of the middle, and the error paths
+        a.load_layers_bin(str(p), first=1, count=1)
+        with pytest.raises(gc.SpdnnError) as e:
+            a.load_layers_bin(str(tmp_path / "missing.bin"))
+        assert e.value.code == 3
+        with pytest.raises(gc.SpdnnError) as e:
+            a.load_layers_bin(str(p), first=2, count=2)
+        assert e.value.code == 1
+    with gc.Network(n, 4, 4, bias=-0.3) as c:
+        with pytest.raises(gc.SpdnnError) as e:     # the file holds three records only
+            c.load_layers_bin(str(p))
+        assert e.value.code == 3 and "short read" in e.value.message
+
+
 def test_argument_and_state_errors(gc, orc):
     E_ARG, E_STATE = 1, 2
     with pytest.raises(gc.SpdnnError) as e:
