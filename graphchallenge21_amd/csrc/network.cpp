@@ -110,13 +110,15 @@ int main(int argc, char** argv) {
         CHECK(spdnn_synth_layers(net, seed, 0, layer, 32, 0.0625f));
     }
     CHECK(spdnn_inspect(net));
-    int n_band = 0;
+    int n_band = 0, n_block = 0;
     for (int l = 0; l < layer; ++l) {
         spdnn_layer_plan p;
         CHECK(spdnn_get_layer_plan(net, l, &p));
         if (p.kernel == SPDNN_KERNEL_BAND) ++n_band;
+        if (p.kernel == SPDNN_KERNEL_BLOCK) ++n_block;
     }
-    printf("Inspector success: %d band layers, %d gather layers (%.2f s)\n", n_band, layer - n_band, now_s() - t0);
+    printf("Inspector success: %d band layers, %d block layers, %d gather layers (%.2f s)\n", n_band, n_block,
+           layer - n_band - n_block, now_s() - t0);
 
     t0 = now_s();
     if (from_files) CHECK(spdnn_load_features_tsv(net, feat_file.c_str(), batch));

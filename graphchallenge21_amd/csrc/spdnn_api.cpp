@@ -276,6 +276,10 @@ const int32_t* labelling_dev(const spdnn_net* n, int layers_done) {
 }
 
 void reset_state(spdnn_net* n) {
+    if (n->stamp > 0x60000000) {  // row stamps are launch numbers: start over long before they wrap
+        hipMemsetAsync(n->d_active, 0, (size_t)n->rows_cap * 4, n->stream);
+        n->stamp = 0;
+    }
     if (n->gid_dirty) {
         launch_iota_gid(n->d_gid, n->rows_cap, n->batch, n->stream);
         n->gid_dirty = false;
@@ -545,6 +549,7 @@ int spdnn_hash_reorder(int v, int buckets, int domain, int* out) {
 static int begin_features(spdnn_net* n, int batch) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
+    if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called (or a layer changed since)");
     int rc = ensure_uploaded(n);
     if (rc) return rc;
     n->batch = batch;

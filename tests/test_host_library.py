@@ -269,10 +269,17 @@ def test_argument_and_state_errors(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.layer_plan(1)
         assert e.value.code == E_STATE
+        with pytest.raises(gc.SpdnnError) as e:     # features need the inspected network
+            net.set_features_dense(np.zeros((4, n), np.float32))
+        assert e.value.code == E_STATE
         net.set_layer_csr(1, *good)
         net.inspect()
         with pytest.raises(gc.SpdnnError) as e:
             net.run()                               # still no features
+        assert e.value.code == E_STATE
+        net.set_layer_csr(1, *good)                 # a layer changed: inspect again before anything else
+        with pytest.raises(gc.SpdnnError) as e:
+            net.synth_features(0, 4)
         assert e.value.code == E_STATE
 
 
