@@ -387,6 +387,38 @@ def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
         assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
 
 
+@pytest.mark.parametrize("N,L,bias,S", [(4096, 480, -0.35, 512), (16384, 1920, -0.4, 96)])
+def test_full_depth_cfg2_cfg3(gc, orc, N, L, bias, S):
+    """N=4096 x 480 layers and N=16384 x 1920 layers at batch 60000, every layer, with densities up
+    to 0.7 so that rows survive to the end: pruned run against the unpruned run (size-independent)
+    and against the oracle on the first S rows through all layers."""
+    B = 60000
+    print("full depth N=%d L=%d" % (N, L), flush=True)
+    with gc.Network(N, B, L) as net:
+        assert net.bias == pytest.approx(bias)
+        net.synth_layers(0)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_BAND for l in range(0, L, 37))
+        net.synth_features(0, B, 0.10, 0.70)
+        rp = net.run(prune=True, collect_counts=True)
+        counts_p = [net.active_count(l) for l in range(L)]
+        cats_p = net.categories()
+        sample = cats_p[cats_p < S][:64].astype(np.int32)
+        y_p = net.activations(sample)
+        if N == 4096:
+            net.run(prune=False, collect_counts=True)
+            assert counts_p == [net.active_count(l) for l in range(L)]
+            assert np.array_equal(cats_p, net.categories())
+            assert same_floats(y_p, net.activations(sample))
+    print("survivors", counts_p[0], counts_p[-1], "compactions", rp.compactions, flush=True)
+    assert counts_p == sorted(counts_p, reverse=True) and 0 < counts_p[-1] < B and rp.compactions >= 1
+    assert len(cats_p) == counts_p[-1] and np.array_equal(cats_p, np.sort(cats_p))
+    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.70), lambda l: orc.gen_layer_csr(0, l, N) if l < L else None,
+                    bias, prune=True)
+    assert np.array_equal(cats_p[cats_p < S], ref["categories"])
+    assert len(sample) > 0 and same_floats(y_p, ref["y"][:len(sample)])
+
+
 @pytest.mark.parametrize("N,K,B", [(256, 32, 1), (256, 4, 65), (512, 12, 257), (128, 8, 40), (100, 5, 33), (2048, 36, 70)])
 def test_small_and_odd_shapes(gc, orc, N, K, B):
     """Smallest band layers, a single row, widths that are not a multiple of 256 and rows longer
