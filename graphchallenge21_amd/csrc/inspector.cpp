@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <array>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <numeric>
 
@@ -257,6 +258,128 @@ bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vecto
     return true;
 }
 
+bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                         const std::vector<std::vector<int32_t>>& groups, std::vector<int32_t>& in_pos,
+                         std::vector<int32_t>& out_at) {
+    const int G = 16, K = 32, R = 16;
+    if (N % 256 != 0 || (int)groups.size() * G != N) return false;
+    const int ng = N / G;
+    for (const auto& g : groups)
+        if ((int)g.size() != G || rowptr[g[0] + 1] - rowptr[g[0]] != K) return false;
+    // the two groups reading every input
+    std::vector<int32_t> user((size_t)N * 2, -1);
+    for (int g = 0; g < ng; ++g) {
+        const int j0 = groups[(size_t)g][0];
+        for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e) {
+            int32_t* u = &user[(size_t)col[e] * 2];
+            if (u[0] < 0) u[0] = g;
+            else if (u[1] < 0) u[1] = g;
+            else return false;
+        }
+    }
+    for (int i = 0; i < N; ++i) if (user[(size_t)i * 2 + 1] < 0) return false;
+    // neighbours of a group: the other reader of each of its inputs
+    auto other = [&](int g, int input) {
+        const int32_t* u = &user[(size_t)input * 2];
+        return u[0] == g ? u[1] : u[0];
+    };
+    // inputs group g shares with group h, in ascending input index
+    auto shared_with = [&](int g, int h, std::vector<int32_t>& out) {
+        out.clear();
+        const int j0 = groups[(size_t)g][0];
+        for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e)
+            if (other(g, col[e]) == h) out.push_back(col[e]);
+    };
+    in_pos.assign((size_t)N, -1);
+    out_at.assign((size_t)N, -1);
+    std::vector<uint8_t> seen((size_t)ng, 0);
+    std::vector<int32_t> cyc, run;
+    int base = 0;  // run index of the first run of the current cycle
+    for (int start = 0; start < ng; ++start) {
+        if (seen[(size_t)start]) continue;
+        // walk the cycle of groups start -> ... -> start, each sharing one run with the next
+        cyc.clear();
+        int prev = -1, cur = start;
+        for (int steps = 0;; ++steps) {
+            if (steps > ng || seen[(size_t)cur]) return false;
+            seen[(size_t)cur] = 1;
+            cyc.push_back(cur);
+            const int j0 = groups[(size_t)cur][0];
+            int a = -1, b = -1;  // the one or two groups this one shares inputs with
+            for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e) {
+                const int o = other(cur, col[e]);
+                if (o == cur) return false;
+                if (a < 0 || o == a) a = o;
+                else if (b < 0 || o == b) b = o;
+                else return false;
+            }
+            int next;
+            if (b < 0) {                 // both runs shared with the same group: a cycle of two
+                if (prev >= 0 && a != prev) return false;
+                if (prev >= 0) break;    // second group of the pair
+                next = a;
+            } else if (prev < 0) next = a;
+            else if (a == prev) next = b;
+            else if (b == prev) next = a;
+            else return false;
+            if (next == start) break;
+            prev = cur;
+            cur = next;
+        }
+        const int c = (int)cyc.size();
+        if (c < 2) return false;
+        // run i is what group i-1 and group i share; group i reads runs i and i+1 (mod c).
+        // Fold the cycle (0, c-1, 1, c-2, ...) so that the two runs of every group lie at most two
+        // run slots apart, and give group i the slot of its later run - or, for the one group
+        // whose runs sit at the fold's end, the slot after it.
+        auto fold = [&](int i) { return i < (c + 1) / 2 ? 2 * i : 2 * (c - 1 - i) + 1; };
+        for (int i = 0; i < c; ++i) {
+            const int gprev = cyc[(size_t)((i + c - 1) % c)], g = cyc[(size_t)i];
+            shared_with(g, gprev, run);
+            if (c == 2) {
+                if ((int)run.size() != 2 * R) return false;
+                if (i == 0) run.erase(run.begin(), run.begin() + R); else run.resize((size_t)R);
+            }
+            if ((int)run.size() != R) return false;
+            const int slot = base + fold(i);
+            for (int k = 0; k < R; ++k) {
+                if (in_pos[(size_t)run[(size_t)k]] >= 0) return false;
+                in_pos[(size_t)run[(size_t)k]] = slot * R + k;
+            }
+        }
+        for (int i = 0; i < c; ++i) {
+            const int fa = fold(i), fb = fold((i + 1) % c);
+            const int lo = std::min(fa, fb), hi = std::max(fa, fb);
+            int t;
+            if (hi - lo == 2) t = hi;
+            else if (lo == 0) t = 1;      // runs at fold slots 0 and 1
+            else t = c;                   // runs at the last two fold slots
+            if (c == 2) t = i == 0 ? 1 : 2;
+            const int slot = (base + t) % ng;
+            for (int o = 0; o < G; ++o) {
+                if (out_at[(size_t)slot * G + o] >= 0) return false;
+                out_at[(size_t)slot * G + o] = groups[(size_t)cyc[(size_t)i]][(size_t)o];
+            }
+        }
+        base += c;
+    }
+    if (base != ng) return false;
+    // full check of what the kernel assumes: every entry of the output at position v lies in
+    // [16*floor(v/16) - 32, 16*floor(v/16) + 15] (mod N)
+    for (int v = 0; v < N; ++v) {
+        const int j = out_at[(size_t)v];
+        if (j < 0) return false;
+        const int top = (v / G) * G + G - 1;
+        for (int e = rowptr[j]; e < rowptr[j + 1]; ++e) {
+            const int p = in_pos[(size_t)col[e]];
+            if (p < 0) return false;
+            const int back = ((top - p) % N + N) % N;
+            if (back > 2 * R + G - 1) return false;
+        }
+    }
+    return true;
+}
+
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, LayerPlan& plan) {
     const int64_t nnz = rowptr[N];
@@ -298,7 +421,17 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     }
 
     std::vector<std::vector<int32_t>> groups;
-    const bool block = !band && force_kernel != SPDNN_KERNEL_GATHER && !dup && discover_blocks(N, rowptr, col, groups);
+    bool block = !band && force_kernel != SPDNN_KERNEL_GATHER && !dup && discover_blocks(N, rowptr, col, groups);
+    int halo = K - 1;
+    // Walking the chains with the band kernel beats the BLOCK kernel from N = 4096 up (measured);
+    // below that a row block's whole input sits in L2 and the BLOCK kernel's independent waves win.
+    const char* chain_env = getenv("SPDNN_RUN_CHAINS_MIN_N");
+    const int chain_min_n = chain_env ? atoi(chain_env) : 4096;   // 0 or negative: never
+    if (block && chain_min_n > 0 && N >= chain_min_n && plan.info.regular && K == 32 && discover_run_chains(N, rowptr, col, groups, plan.in_pos, plan.out_at)) {
+        band = true;    // 16-output groups chained through shared 16-input runs: walked like a band
+        block = false;
+        halo = 32;
+    }
 
     plan.ngroups = 0;
     plan.blk_cols.clear();
@@ -334,7 +467,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     } else if (band) {
         plan.kernel = SPDNN_KERNEL_BAND;
         plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
-        plan.info.band_halo = K - 1;
+        plan.info.band_halo = halo;
         plan.sel.resize((size_t)N * K);
         if (plan.wmode != 0) plan.wv.resize((size_t)N * K); else plan.wv.clear();
         for (int v = 0; v < N; ++v) {

@@ -54,6 +54,15 @@ bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::
 bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                      std::vector<std::vector<int32_t>>& groups);
 
+// For a layer of 32 entries per row whose groups (from discover_blocks) hold exactly 16 outputs each:
+// looks for the chain structure of a RadiX-Net layer - every group reads two runs of 16 inputs and
+// every run is read by two groups, so groups and runs form cycles - and lays the cycles out so
+// that the group at band positions [16t, 16t+16) reads only positions in [16t-32, 16t+16) (mod N).
+// The result is a BAND labelling (in_pos, out_at) for a halo of 32.
+bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                         const std::vector<std::vector<int32_t>>& groups, std::vector<int32_t>& in_pos,
+                         std::vector<int32_t>& out_at);
+
 // Full per-layer inspection (everything except dst, which needs the next layer's labelling).
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, LayerPlan& plan);

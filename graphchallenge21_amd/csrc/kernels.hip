@@ -107,14 +107,17 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // ------------------------------------------------------------------------------------------
 // BAND kernel ("row-succ" / tiled variant).
 //
-// The inspector has relabelled the layer so that the output at band position v reads the K
-// input columns at positions v-K+1 .. v (mod N).  A workgroup takes one row block and one
+// The inspector has relabelled the layer so that the output at band position v reads input
+// columns at positions no further back than `halo` before the 16-aligned group of v and no later
+// than the end of that group (mod N): a circulant band, where v reads v-K+1 .. v (halo K-1), or a
+// chain of 16-output groups that each read the input runs of the two groups before them and
+// their own (halo 32).  A workgroup takes one row block and one
 // segment [vb, ve) of band positions and walks it in chunks of T = NW*OPW outputs.  The input
 // columns live in an LDS ring of RING column slots (slot = position mod RING, RING | N): while
 // the waves compute chunk c from the ring, the T columns of chunk c+1 are already in flight
 // from HBM into registers and are dropped into the ring afterwards, so every input column is
-// read from HBM once per segment (plus K-1 halo columns at the segment start) and the loads
-// overlap the arithmetic.  Needs 2*T + K - 1 <= RING.
+// read from HBM once per segment (plus the halo columns at the segment start) and the loads
+// overlap the arithmetic.  Needs 2*T + halo <= RING, T a multiple of 16.
 //
 // Per output the scalar unit streams 32 one-byte ring selectors (already in accumulation order)
 // and, unless the layer has one exact value, 32 weights; the output column is written to the
@@ -123,13 +126,13 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __device__ __forceinline__ void band_walk_body(
     const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ sel,
-    const float* __restrict__ wv, const int32_t* __restrict__ dst, int N, int Krt, int vb, int ve,
+    const float* __restrict__ wv, const int32_t* __restrict__ dst, int N, int Krt, int halo, int vb, int ve,
     float wu, float bias, float clampv, unsigned char* smem, float* nz) {
     using V = typename VecOf<RL>::type;
     constexpr int T = NW * OPW;
     constexpr int RB = 64 * RL;
     constexpr int COLB = RB * 4;
-    static_assert(2 * T + 31 <= RING, "ring too small for 32 entries per output");
+    static_assert(2 * T + 32 <= RING && T % 16 == 0, "ring too small for a halo of 32 columns");
     static_assert((RING & (RING - 1)) == 0 && RING <= 256, "ring must be a power of two <= 256");
     static_assert(KT == 0 || KT == 32, "KT is 32 (unrolled) or 0 (run-time row length)");
 
@@ -140,9 +143,9 @@ __device__ __forceinline__ void band_walk_body(
     const int loff = lane * RL;
     const unsigned char* lane_smem = smem + loff * 4;
 
-    // prologue: halo (K-1 columns before the segment, wrapping below 0) + first chunk
-    for (int c = wave; c < K - 1 + T; c += NW) {
-        const int p = vb - (K - 1) + c;
+    // prologue: halo (columns before the segment, wrapping below 0) + first chunk
+    for (int c = wave; c < halo + T; c += NW) {
+        const int p = vb - halo + c;
         if (p < ve) {
             const int g = p < 0 ? p + N : p;
             V x = *reinterpret_cast<const V*>(yin + (size_t)g * RB + loff);
@@ -314,8 +317,8 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
     const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int Krt, int seglen, int stamp, int prev_stamp, float wu, float bias,
-    float clampv) {
+    int32_t* __restrict__ count_out, int N, int Krt, int halo, int seglen, int stamp, int prev_stamp, float wu,
+    float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     const int rb = blockIdx.x;
@@ -326,8 +329,8 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     float nz[RL];
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, sel, wv, dst, N, Krt, vb, ve, wu,
-                                                 bias, clampv, smem, nz);
+    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, sel, wv, dst, N, Krt, halo, vb, ve,
+                                                 wu, bias, clampv, smem, nz);
     stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp, count_out);
 }
 
@@ -344,7 +347,7 @@ struct ChainLayer {
     const float* wv;
     const int32_t* dst;
     float wu;
-    int pad;
+    int halo;
 };
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
@@ -365,8 +368,8 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         float nz[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.sel, lay.wv, lay.dst, N, Krt, 0, N, lay.wu, bias,
-                                                     clampv, smem, nz);
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.sel, lay.wv, lay.dst, N, Krt, lay.halo, 0, N, lay.wu,
+                                                     bias, clampv, smem, nz);
         stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp0 + j,
                        count_out ? count_out + j : nullptr);
         int any = 0;
@@ -726,7 +729,7 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     if (nseg > 65535) return hipErrorInvalidValue;
     dim3 grid(a.nblk, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.count_out,
-                       a.N, a.K, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
+                       a.N, a.K, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
 }
 
@@ -805,6 +808,7 @@ int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     // host-side shape checks: what the kernel and its grid assume
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
+        a.halo < a.K - 1 || a.halo > 32 || a.halo >= a.N ||
         !a.yin || !a.yout || !a.sel || !a.dst || !a.active || (a.wmode != 0 && !a.wv))
         return hipErrorInvalidValue;
     BandLaunch b = a;

@@ -23,6 +23,7 @@ struct BandLaunch {
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
     int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, K, nblk, stamp, rl;
+    int halo;                // input columns a segment needs before its first position: K-1 .. 32
     int prev_stamp = 0;      // stamp of the previous layer: row blocks it left without an active row are skipped (0 = off)
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
@@ -77,7 +78,7 @@ struct ChainLayerDesc {      // one entry of the device-side layer table
     const float* wv;
     const int32_t* dst;
     float wu;
-    int pad;
+    int halo;   // input columns a segment needs before its first position (K-1, or 32 for run chains)
 };
 struct ChainLaunch {
     const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain

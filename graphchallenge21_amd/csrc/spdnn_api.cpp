@@ -246,7 +246,7 @@ int ensure_uploaded(spdnn_net* n) {
         table[(size_t)l].wv = n->dl[(size_t)l].wv;
         table[(size_t)l].dst = n->dl[(size_t)l].dst;
         table[(size_t)l].wu = n->layers[(size_t)l].info.value;
-        table[(size_t)l].pad = 0;
+        table[(size_t)l].halo = n->layers[(size_t)l].info.band_halo;
     }
     HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
     HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
@@ -664,6 +664,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, in
     BandLaunch a{};
     a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
+    a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
     a.shape = -1; a.seglen = 0; a.count_out = nullptr; a.prev_stamp = 0;
     return a;

@@ -67,3 +67,24 @@ def radix_like_csr(rng, n, stride, values="uniform", relabel=True, run=16):
     else:
         val = rng.uniform(-0.1, 0.15, size=k).astype(np.float32)
     return rowptr, col, val
+
+
+def hub_block_csr(rng, n, values="uniform"):
+    """Groups of 16 outputs that read their own 16-wide input run plus the shared run [0, 16):
+    identical rows inside a group, but no chain of groups (one run is read by every group)."""
+    pin, pout = rng.permutation(n), rng.permutation(n)
+    rows = [None] * n
+    for j in range(n):
+        g = j // 16
+        rows[pout[j]] = np.unique(pin[np.concatenate([np.arange(16), np.arange(16 * g, 16 * g + 16)])])
+    rowptr = np.zeros(n + 1, np.int32)
+    rowptr[1:] = np.cumsum([len(r) for r in rows])
+    col = np.concatenate(rows).astype(np.int32)
+    k = len(col)
+    if values == "uniform":
+        val = np.full(k, 0.0625, np.float32)
+    elif values == "pow2":
+        val = (np.ldexp(1.0, rng.integers(-6, -2, size=k)) * rng.choice([-1.0, 1.0], size=k)).astype(np.float32)
+    else:
+        val = rng.uniform(-0.1, 0.15, size=k).astype(np.float32)
+    return rowptr, col, val

@@ -334,18 +334,25 @@ def test_fused_chain_when_everything_dies(gc, orc):
             assert not net.activations(np.arange(50, dtype=np.int32)).any()
 
 
+@pytest.mark.parametrize("chains", [True, False])
 @pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
-def test_block_kernel_radix_like_layers(gc, orc, values):
+def test_block_kernel_radix_like_layers(gc, orc, values, chains, monkeypatch):
     """RadiX-Net-like layers (16 outputs sharing two 16-wide input runs, hidden behind random
-    relabellings) go to the BLOCK kernel; mixed with a band layer and an irregular layer."""
-    from helpers import radix_like_csr
+    relabellings) are walked as chains by the band kernel; groups without a chain go to the BLOCK
+    kernel; mixed with a circulant band layer and an irregular layer."""
+    from helpers import hub_block_csr, radix_like_csr
     N, B = 1024, 300
-    print("block kernel values=%s" % values, flush=True)
+    print("block kernel values=%s chains=%s" % (values, chains), flush=True)
+    if chains:   # by default widths below 4096 stay on the BLOCK kernel
+        monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+    rk, rh = (gc.KERNEL_BAND, 32) if chains else (gc.KERNEL_BLOCK, -1)
     rng = np.random.default_rng(17)
     layers = [radix_like_csr(rng, N, 16 << l, values) for l in range(4)]
     layers.append(orc.gen_layer_csr(3, 0, N))                                  # BAND
     layers.append(radix_like_csr(rng, N, 256, values, run=8))                   # groups of 8, 16 inputs
     layers.append(sort_rows(random_csr(rng, N, rng.integers(1, 20, size=N), "pow2")))   # GATHER
+    layers.append(hub_block_csr(rng, N, values))                               # 32 inputs, no chain
+    layers.append(radix_like_csr(rng, N, 512, values))                          # cycles of two groups
     L = len(layers)
     feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < 0.4)).astype(np.float32)
     with gc.Network(N, B, L, bias=-0.2) as net:
@@ -353,7 +360,8 @@ def test_block_kernel_radix_like_layers(gc, orc, values):
             net.set_layer_csr(l, *csr)
         net.inspect()
         kinds = [net.layer_plan(l).kernel for l in range(L)]
-        assert kinds == [gc.KERNEL_BLOCK] * 4 + [gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER]
+        assert kinds == [rk] * 4 + [gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER, gc.KERNEL_BLOCK, rk]
+        assert [net.layer_plan(l).band_halo for l in range(L)] == [rh] * 4 + [31, -1, -1, -1, rh]
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
         ref = orc.infer(feats, layers, -0.2, prune=True)

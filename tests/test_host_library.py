@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from helpers import radix_like_csr, random_csr, sort_rows
+from helpers import hub_block_csr, radix_like_csr, random_csr, sort_rows
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GOLD = os.path.join(ROOT, "tests", "golden")
@@ -47,12 +47,15 @@ def _emulate_band_layer(net, l, y_phys, value_of):
     in_pos, out_at, sel = net.band_plan(l)
     dst = net.layer_dst(l)
     k = sel.shape[1]
+    halo = net.layer_plan(l).band_halo
     out = np.zeros_like(y_phys)
     for v in range(n):
         acc = np.zeros(y_phys.shape[0], np.float32)
-        window = [(v - d) % n for d in range(k)]
+        # what the ring of a 16-output chunk holds: the chunk's own positions and the halo before it
+        top = v // 16 * 16 + 15
+        window = [(top - d) % n for d in range(halo + 16)]
         by_slot = {p % 256: p for p in window}
-        assert len(by_slot) == k
+        assert len(by_slot) == halo + 16
         for m in range(k):
             p = by_slot[int(sel[v, m])]
             acc = acc + y_phys[:, p] * value_of(v, m)
@@ -128,13 +131,13 @@ def test_inspector_block_class(gc, orc):
     rng = np.random.default_rng(5)
     n = 512
     with gc.Network(n, 4, 3, bias=-0.3) as net:
-        net.set_layer_csr(0, *radix_like_csr(rng, n, 64, "uniform"))
-        net.set_layer_csr(1, *radix_like_csr(rng, n, 16, "general"))        # overlapping runs: 32 inputs still
+        net.set_layer_csr(0, *hub_block_csr(rng, n, "uniform"))              # one run read by every group
+        net.set_layer_csr(1, *hub_block_csr(rng, n, "general"))
         net.set_layer_csr(2, *radix_like_csr(rng, n, 128, "pow2", run=8))   # groups of 8 outputs, 16 inputs
         net.inspect()
         p = [net.layer_plan(l) for l in range(3)]
         assert [q.kernel for q in p] == [gc.KERNEL_BLOCK] * 3
-        assert (p[0].max_row_nnz, p[0].uniform_value, p[0].exact_products) == (32, 1, 1)
+        assert (p[0].max_row_nnz, p[0].uniform_value, p[0].exact_products, p[0].regular) == (32, 1, 1, 0)
         assert (p[1].uniform_value, p[1].exact_products) == (0, 0)
         assert p[2].max_row_nnz == 16
         for l in range(3):
@@ -145,6 +148,51 @@ def test_inspector_block_class(gc, orc):
         net.set_layer_csr(0, *radix_like_csr(rng, n, 64, "uniform"))
         net.inspect()
         assert net.layer_plan(0).kernel == gc.KERNEL_GATHER
+    # chains of groups: BLOCK below 4096 neurons, walked by the band kernel from there up
+    for width, kind, halo in ((512, gc.KERNEL_BLOCK, -1), (4096, gc.KERNEL_BAND, 32)):
+        with gc.Network(width, 4, 1, bias=-0.3) as net:
+            net.set_layer_csr(0, *radix_like_csr(rng, width, 64, "uniform"))
+            net.inspect()
+            assert (net.layer_plan(0).kernel, net.layer_plan(0).band_halo) == (kind, halo)
+
+
+@pytest.mark.parametrize("n", [256, 768, 1024])
+def test_inspector_run_chains(gc, orc, n, monkeypatch):
+    """RadiX-Net layers - groups of 16 outputs reading two 16-wide input runs, every run read by
+    two groups - are laid out as chains and walked by the band kernel with a halo of 32: every
+    stride (one long cycle, several cycles, cycles of three and of two groups), hidden behind
+    random relabellings."""
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")   # the default keeps widths below 4096 on the BLOCK kernel
+    rng = np.random.default_rng(n)
+    strides = [16, 32, 48, 64, 80, n // 4, n // 2, n - 16]
+    if n % 3 == 0:
+        strides += [n // 3, 16 * 15]               # 16 cycles of three groups; three cycles of 16
+    L, b = len(strides), 5
+    layers = [radix_like_csr(rng, n, st, "general" if i % 2 else "uniform") for i, st in enumerate(strides)]
+    with gc.Network(n, b, L, bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        for l in range(L):
+            p = net.layer_plan(l)
+            assert (p.kernel, p.max_row_nnz, p.regular, p.band_halo) == (gc.KERNEL_BAND, 32, 1, 32), strides[l]
+            in_pos, out_at, sel = net.band_plan(l)
+            assert sorted(in_pos.tolist()) == list(range(n)) and sorted(out_at.tolist()) == list(range(n))
+            rowptr, col, _ = layers[l]
+            for v in range(n):
+                top = v // 16 * 16 + 15
+                back = (top - in_pos[col[rowptr[out_at[v]]:rowptr[out_at[v] + 1]]]) % n
+                assert back.max() <= 47, (strides[l], v)
+        feats = orc.gen_features(11, n, 0, b, 0.1, 0.5)
+        y = np.zeros_like(feats)
+        y[:, net.input_labelling(0)] = feats
+        want = feats
+        for l in range(L):
+            rowptr, col, val = layers[l]
+            _, out_at, _ = net.band_plan(l)
+            y = _emulate_band_layer(net, l, y, lambda v, m: val[rowptr[out_at[v]] + m])
+            want, _ = orc.layer(want, layers[l], -0.3)
+            assert np.array_equal(y[:, net.input_labelling(l + 1)], want), strides[l]
 
 
 def test_forced_gather(gc, orc):
