@@ -44,6 +44,19 @@ int fail(int code, const std::string& msg) {
             return fail(SPDNN_E_DEVICE, std::string(#expr) + ": " + hipGetErrorString(e_));         \
     } while (0)
 
+// Temporary device allocation / event that is released on every return path.
+struct DevTmp {
+    void* p = nullptr;
+    ~DevTmp() { if (p) hipFree(p); }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes); }
+    template <class T> T* as() const { return static_cast<T*>(p); }
+};
+struct EventTmp {
+    hipEvent_t e = nullptr;
+    ~EventTmp() { if (e) hipEventDestroy(e); }
+    hipError_t create() { return hipEventCreate(&e); }
+};
+
 // Small worker pool for the per-layer inspector jobs (bounded queue so that pending CSR copies
 // stay small).
 class JobPool {
@@ -174,8 +187,27 @@ struct spdnn_net {
 
 namespace {
 
-int ensure_device(spdnn_net* n) {
-    if (n->dev_ready) return SPDNN_OK;
+void release_device_base(spdnn_net* n) {
+    hipFree(n->d_active_scratch); hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
+    hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
+    hipFree(n->d_counts);
+    if (n->h_count) hipHostFree(n->h_count);
+    if (n->h_counts) hipHostFree(n->h_counts);
+    n->d_active_scratch = n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
+    n->d_count = n->d_nonfinite = n->d_counts = n->h_count = n->h_counts = nullptr;
+    for (hipEvent_t e : n->ev_count) hipEventDestroy(e);
+    for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
+    n->ev_count.clear();
+    n->ev_layer.clear();
+    if (n->ev_start) hipEventDestroy(n->ev_start);
+    if (n->ev_stop) hipEventDestroy(n->ev_stop);
+    if (n->stream) hipStreamDestroy(n->stream);
+    n->ev_start = n->ev_stop = nullptr;
+    n->stream = nullptr;
+    n->dev_ready = false;
+}
+
+int init_device(spdnn_net* n) {
     int cnt = 0;
     hipError_t e = hipGetDeviceCount(&cnt);
     if (e != hipSuccess || cnt < 1) return fail(SPDNN_E_DEVICE, "no HIP device available");
@@ -205,13 +237,18 @@ int ensure_device(spdnn_net* n) {
     return SPDNN_OK;
 }
 
+int ensure_device(spdnn_net* n) {
+    if (n->dev_ready) return SPDNN_OK;
+    const int rc = init_device(n);
+    if (rc != SPDNN_OK) release_device_base(n);  // nothing half-built stays behind (g_err is kept)
+    return rc;
+}
+
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-int ensure_uploaded(spdnn_net* n) {
-    if (n->uploaded) return SPDNN_OK;
-    if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
-    int rc = ensure_device(n);
-    if (rc) return rc;
+void free_device(spdnn_net* n);
+
+int upload_plans(spdnn_net* n) {
     size_t total = 0;
     for (const LayerPlan& p : n->layers) {
         total += align256(p.in_pos.size() * 4) + align256(p.sel.size()) + align256(p.ell_col.size() * 4) +
@@ -256,6 +293,16 @@ int ensure_uploaded(spdnn_net* n) {
     HIPCHK(hipMalloc(&n->C, fbytes));
     n->uploaded = true;
     return SPDNN_OK;
+}
+
+int ensure_uploaded(spdnn_net* n) {
+    if (n->uploaded) return SPDNN_OK;
+    if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
+    int rc = ensure_device(n);
+    if (rc) return rc;
+    rc = upload_plans(n);
+    if (rc != SPDNN_OK) free_device(n);
+    return rc;
 }
 
 void free_device(spdnn_net* n) {
@@ -345,16 +392,7 @@ int spdnn_destroy(spdnn_net* n) {
     if (n->dev_ready) {
         hipStreamSynchronize(n->stream);
         free_device(n);
-        hipFree(n->d_active_scratch);
-        hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp); hipFree(n->d_alive_src);
-        hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
-        hipHostFree(n->h_count);
-        hipFree(n->d_counts);
-        hipHostFree(n->h_counts);
-        for (hipEvent_t e : n->ev_count) hipEventDestroy(e);
-        for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
-        hipEventDestroy(n->ev_start); hipEventDestroy(n->ev_stop);
-        hipStreamDestroy(n->stream);
+        release_device_base(n);
     }
     delete n;
     return SPDNN_OK;
@@ -565,29 +603,24 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
     // staging chunk: a whole number of row blocks, about 256 MiB
     int64_t chunk_rows = std::max<int64_t>(RB, ((int64_t)(256 << 20) / ((int64_t)N * 4)) / RB * RB);
     chunk_rows = std::min<int64_t>(chunk_rows, n->rows_cap);
-    float* stage = nullptr;
-    HIPCHK(hipMalloc(&stage, (size_t)chunk_rows * N * 4));
+    DevTmp stage_buf;
+    HIPCHK(stage_buf.alloc((size_t)chunk_rows * N * 4));
+    float* stage = stage_buf.as<float>();
     HIPCHK(hipMemsetAsync(n->d_nonfinite, 0, 4, n->stream));
     const int padded = ((batch + RB - 1) / RB) * RB;
     for (int64_t r0 = 0; r0 < padded; r0 += chunk_rows) {
         const int64_t rows_here = std::min<int64_t>(chunk_rows, padded - r0);
         const int64_t real = std::max<int64_t>(0, std::min<int64_t>(rows_here, batch - r0));
-        if (real > 0) {
-            hipError_t e = hipMemcpyAsync(stage, rowmajor + (size_t)r0 * N, (size_t)real * N * 4,
-                                          hipMemcpyHostToDevice, n->stream);
-            if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
-        }
+        if (real > 0)
+            HIPCHK(hipMemcpyAsync(stage, rowmajor + (size_t)r0 * N, (size_t)real * N * 4, hipMemcpyHostToDevice,
+                                  n->stream));
         // rows >= real inside the chunk are written as zero by the kernel (nrows = real)
-        hipError_t e = launch_pack_rows(stage, n->F, n->dl[0].in_pos, N, r0, (int)std::max<int64_t>(real, 1),
-                                        n->rl, n->d_nonfinite, n->stream);
-        if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
-        e = hipStreamSynchronize(n->stream);
-        if (e != hipSuccess) { hipFree(stage); return fail(SPDNN_E_DEVICE, hipGetErrorString(e)); }
+        HIPCHK(launch_pack_rows(stage, n->F, n->dl[0].in_pos, N, r0, (int)std::max<int64_t>(real, 1), n->rl,
+                                n->d_nonfinite, n->stream));
+        HIPCHK(hipStreamSynchronize(n->stream));  // the staging buffer is reused by the next chunk
     }
     int32_t bad = 0;
-    hipError_t e = hipMemcpy(&bad, n->d_nonfinite, 4, hipMemcpyDeviceToHost);
-    hipFree(stage);
-    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    HIPCHK(hipMemcpy(&bad, n->d_nonfinite, 4, hipMemcpyDeviceToHost));
     if (bad) return fail(SPDNN_E_ARG, "features contain NaN or infinity");
     HIPCHK(launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
@@ -624,15 +657,14 @@ int spdnn_synth_features(spdnn_net* n, uint64_t seed, int batch, float dmin, flo
     const std::vector<int32_t>& pos = n->layers[0].in_pos;
     std::vector<int32_t> inv((size_t)n->N);
     for (int i = 0; i < n->N; ++i) inv[(size_t)pos[(size_t)i]] = i;
-    int32_t* d_inv = nullptr;
-    HIPCHK(hipMalloc(&d_inv, (size_t)n->N * 4));
-    hipError_t e = hipMemcpy(d_inv, inv.data(), (size_t)n->N * 4, hipMemcpyHostToDevice);
+    DevTmp inv_buf;
+    HIPCHK(inv_buf.alloc((size_t)n->N * 4));
+    int32_t* d_inv = inv_buf.as<int32_t>();
+    HIPCHK(hipMemcpy(d_inv, inv.data(), (size_t)n->N * 4, hipMemcpyHostToDevice));
     const int nblk = (batch + n->RB - 1) / n->RB;
-    if (e == hipSuccess) e = launch_synth_features(n->F, d_inv, n->N, batch, nblk, n->rl, seed, dmin, dmax, n->stream);
-    if (e == hipSuccess) e = launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream);
-    if (e == hipSuccess) e = hipStreamSynchronize(n->stream);
-    hipFree(d_inv);
-    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
+    HIPCHK(launch_synth_features(n->F, d_inv, n->N, batch, nblk, n->rl, seed, dmin, dmax, n->stream));
+    HIPCHK(launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream));
+    HIPCHK(hipStreamSynchronize(n->stream));
     n->have_features = true;
     reset_state(n);
     return SPDNN_OK;
@@ -682,9 +714,10 @@ static const spdnn_net::Tuned* find_tuned(const spdnn_net* n, int nblk, int K) {
 // anyway; every trial uses a fresh row stamp.
 static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk) {
     const LayerPlan& p = n->layers[(size_t)l];
-    hipEvent_t e0, e1;
-    HIPCHK(hipEventCreate(&e0));
-    HIPCHK(hipEventCreate(&e1));
+    EventTmp ev0, ev1;
+    HIPCHK(ev0.create());
+    HIPCHK(ev1.create());
+    const hipEvent_t e0 = ev0.e, e1 = ev1.e;
     spdnn_net::Tuned best{nblk, p.kmax, -1, 0};
     float best_ms = 0.0f;
     hipError_t err = hipSuccess;
@@ -708,8 +741,6 @@ static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk)
             if (err == hipSuccess && (best.shape < 0 || ms < best_ms)) { best.shape = shape; best.seglen = lens[c]; best_ms = ms; }
         }
     }
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
     if (err != hipSuccess) return fail(SPDNN_E_DEVICE, std::string("band tuning: ") + hipGetErrorString(err));
     if (best.shape >= 0) n->tuned.push_back(best);
     return SPDNN_OK;
@@ -975,23 +1006,19 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
         phys[(size_t)i] = where[(size_t)rows[i]];
     }
     const int chunk = 4096;
-    int32_t* d_phys = nullptr;
-    float* d_out = nullptr;
-    HIPCHK(hipMalloc(&d_phys, (size_t)chunk * 4));
-    hipError_t e = hipMalloc(&d_out, (size_t)chunk * (size_t)n->N * 4);
-    if (e != hipSuccess) { hipFree(d_phys); return fail(SPDNN_E_NOMEM, hipGetErrorString(e)); }
+    DevTmp phys_buf, out_buf;
+    HIPCHK(phys_buf.alloc((size_t)chunk * 4));
+    if (out_buf.alloc((size_t)chunk * (size_t)n->N * 4) != hipSuccess) return fail(SPDNN_E_NOMEM, "out of device memory");
+    int32_t* d_phys = phys_buf.as<int32_t>();
+    float* d_out = out_buf.as<float>();
     const int32_t* lab = labelling_dev(n, n->cur_layer);
-    for (int i0 = 0; i0 < nrows && e == hipSuccess; i0 += chunk) {
+    for (int i0 = 0; i0 < nrows; i0 += chunk) {
         const int m = std::min(chunk, nrows - i0);
-        e = hipMemcpyAsync(d_phys, phys.data() + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream);
-        if (e == hipSuccess) e = launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, n->d_active, n->last_stamp, d_out, n->stream);
-        if (e == hipSuccess)
-            e = hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * n->N * 4, hipMemcpyDeviceToHost, n->stream);
-        if (e == hipSuccess) e = hipStreamSynchronize(n->stream);
+        HIPCHK(hipMemcpyAsync(d_phys, phys.data() + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream));
+        HIPCHK(launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, n->d_active, n->last_stamp, d_out, n->stream));
+        HIPCHK(hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * n->N * 4, hipMemcpyDeviceToHost, n->stream));
+        HIPCHK(hipStreamSynchronize(n->stream));
     }
-    hipFree(d_phys);
-    hipFree(d_out);
-    if (e != hipSuccess) return fail(SPDNN_E_DEVICE, hipGetErrorString(e));
     return SPDNN_OK;
 }
 
@@ -1032,23 +1059,22 @@ int spdnn_write_categories(spdnn_net* n, const char* path) {
 int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
     if (!gbps || bytes < 1024 || reps < 1) return fail(SPDNN_E_ARG, "bad argument");
     bytes &= ~(int64_t)1023;
-    float *a = nullptr, *b = nullptr;
-    hipEvent_t e0, e1;
-    HIPCHK(hipMalloc(&a, (size_t)bytes));
-    hipError_t e = hipMalloc(&b, (size_t)bytes);
-    if (e != hipSuccess) { hipFree(a); return fail(SPDNN_E_NOMEM, hipGetErrorString(e)); }
-    hipMemset(a, 0, (size_t)bytes);
-    hipEventCreate(&e0); hipEventCreate(&e1);
-    (void)launch_copy_f4(a, b, bytes / 4, nullptr);
-    hipEventRecord(e0, nullptr);
-    for (int i = 0; i < reps; ++i) (void)launch_copy_f4(a, b, bytes / 4, nullptr);
-    hipEventRecord(e1, nullptr);
-    e = hipEventSynchronize(e1);
+    DevTmp abuf, bbuf;
+    EventTmp ev0, ev1;
+    if (abuf.alloc((size_t)bytes) != hipSuccess || bbuf.alloc((size_t)bytes) != hipSuccess)
+        return fail(SPDNN_E_NOMEM, "out of device memory");
+    float *a = abuf.as<float>(), *b = bbuf.as<float>();
+    HIPCHK(hipMemset(a, 0, (size_t)bytes));
+    HIPCHK(ev0.create());
+    HIPCHK(ev1.create());
+    HIPCHK(launch_copy_f4(a, b, bytes / 4, nullptr));
+    HIPCHK(hipEventRecord(ev0.e, nullptr));
+    for (int i = 0; i < reps; ++i) HIPCHK(launch_copy_f4(a, b, bytes / 4, nullptr));
+    HIPCHK(hipEventRecord(ev1.e, nullptr));
+    HIPCHK(hipEventSynchronize(ev1.e));
     float ms = 0.0f;
-    hipEventElapsedTime(&ms, e0, e1);
-    hipEventDestroy(e0); hipEventDestroy(e1);
-    hipFree(a); hipFree(b);
-    if (e != hipSuccess || ms <= 0.0f) return fail(SPDNN_E_DEVICE, "copy benchmark failed");
+    HIPCHK(hipEventElapsedTime(&ms, ev0.e, ev1.e));
+    if (ms <= 0.0f) return fail(SPDNN_E_DEVICE, "copy benchmark failed");
     *gbps = 2.0 * (double)bytes * reps / (ms * 1e-3) / 1e9;
     return SPDNN_OK;
 }
