@@ -709,6 +709,15 @@ int rank_seglens(int N, int K, int T, int nblk, int slots, int* out, int max_out
     return n;
 }
 
+// the fill/halo model of rank_seglens for one segment length
+double seglen_score(int N, int K, int T, int nblk, int slots, int seglen) {
+    const int nseg = (N + seglen - 1) / seglen;
+    const long long wgs = (long long)nblk * nseg;
+    const long long rounds = (wgs + slots - 1) / slots;
+    const double fill = (double)wgs / (double)(rounds * slots);
+    return fill / (1.0 + 0.25 * (double)(K - 1) / (double)seglen);
+}
+
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     constexpr int T = NW * OPW;
@@ -786,11 +795,14 @@ int band_workgroups_per_cu(int rl, int shape) {
 }
 
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out) {
-    // the two best-ranked by the fill/halo model, then a geometric ladder of segment counts:
-    // shorter segments mean more, smaller workgroups, which often balances and streams better
-    // than the model predicts - the caller measures
+    // the two best-ranked by the fill/halo model, then a geometric ladder of segment counts
+    // (those the model does not rule out): shorter segments mean more, smaller workgroups, which
+    // often balances and streams better than the model predicts - the caller measures
     const int T = band_chunk_outputs(rl, shape);
-    int n = rank_seglens(N, K, T, nblk, n_cu * band_workgroups_per_cu(rl, shape), out, max_out < 2 ? max_out : 2);
+    const int slots = n_cu * band_workgroups_per_cu(rl, shape);
+    int n = rank_seglens(N, K, T, nblk, slots, out, max_out < 2 ? max_out : 2);
+    if (n < 1) return 0;
+    const double floor_score = 0.6 * seglen_score(N, K, T, nblk, slots, out[0]);  // not worth a trial below this
     const int nchunks = (N + T - 1) / T;
     static const int ladder[] = {1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256, 384, 512};
     for (int nseg : ladder) {
@@ -798,7 +810,7 @@ int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, 
         const int cps = (nchunks + nseg - 1) / nseg;
         if (cps < 4 && nseg > 1) break;  // at least four chunks per workgroup
         const int len = cps * T;
-        bool dup = false;
+        bool dup = seglen_score(N, K, T, nblk, slots, len) < floor_score;
         for (int i = 0; i < n; ++i) dup |= out[i] == len;
         if (!dup) out[n++] = len;
     }

@@ -152,7 +152,6 @@ struct spdnn_net {
     void* arena = nullptr;
     std::vector<DevLayer> dl;
     float *F = nullptr, *A = nullptr, *C = nullptr;
-    int32_t* d_active_scratch = nullptr;
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
@@ -183,20 +182,32 @@ struct spdnn_net {
     struct Tuned { int nblk, K, shape, seglen; };
     std::vector<Tuned> tuned;
     bool autotune = true;
+    // exploration in progress: real layers are launched with the candidates in turn and timed
+    struct Cand { int shape, seglen; float best_ms; int samples; };
+    struct Explore { int nblk, K, issued; std::vector<Cand> cands; };
+    struct Trial { int nblk, K, cand; hipEvent_t e0, e1; };
+    std::vector<Explore> exploring;
+    std::deque<Trial> trials;           // launched, not yet read back
+    std::vector<hipEvent_t> ev_free;    // timing events for trials
 };
 
 namespace {
 
 void release_device_base(spdnn_net* n) {
-    hipFree(n->d_active_scratch); hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
+    hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
     hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
     hipFree(n->d_counts);
     if (n->h_count) hipHostFree(n->h_count);
     if (n->h_counts) hipHostFree(n->h_counts);
-    n->d_active_scratch = n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
+    n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
     n->d_count = n->d_nonfinite = n->d_counts = n->h_count = n->h_counts = nullptr;
     for (hipEvent_t e : n->ev_count) hipEventDestroy(e);
     for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
+    for (const spdnn_net::Trial& t : n->trials) { hipEventDestroy(t.e0); hipEventDestroy(t.e1); }
+    for (hipEvent_t e : n->ev_free) hipEventDestroy(e);
+    n->trials.clear();
+    n->ev_free.clear();
+    n->exploring.clear();
     n->ev_count.clear();
     n->ev_layer.clear();
     if (n->ev_start) hipEventDestroy(n->ev_start);
@@ -222,7 +233,6 @@ int init_device(spdnn_net* n) {
     HIPCHK(hipEventCreate(&n->ev_stop));
     const size_t rows = (size_t)n->rows_cap;
     HIPCHK(hipMalloc(&n->d_active, rows * 4));
-    HIPCHK(hipMalloc(&n->d_active_scratch, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid_tmp, rows * 4));
     HIPCHK(hipMalloc(&n->d_alive_src, rows * 4));
@@ -379,7 +389,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     n->layer_ms.assign((size_t)layers, 0.0f);
     n->pool.reset(new JobPool(host_threads()));
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
-    if (getenv("SPDNN_BAND_SHAPE")) n->autotune = false;  // an explicit shape wins
+    if (getenv("SPDNN_BAND_SHAPE") || getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // explicit settings win
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     *out = n;
     return SPDNN_OK;
@@ -517,6 +527,9 @@ int spdnn_inspect(spdnn_net* n) {
     n->pool->wait_all();
     if (n->uploaded) free_device(n);  // plans changed: upload again on next use
     n->tuned.clear();
+    n->exploring.clear();
+    for (const spdnn_net::Trial& t : n->trials) { n->ev_free.push_back(t.e0); n->ev_free.push_back(t.e1); }
+    n->trials.clear();
     n->inspected = true;
     return SPDNN_OK;
 }
@@ -708,53 +721,70 @@ static const spdnn_net::Tuned* find_tuned(const spdnn_net* n, int nblk, int K) {
     return nullptr;
 }
 
-// Run-time kernel selection for band layers (the measured half of the inspector's choice): time
-// each tile shape with a ladder of segment lengths on the real buffers of layer l and keep the
-// fastest for this row-block count.  The trial outputs land in the buffer the layer writes
-// anyway; every trial uses a fresh row stamp.
-static int tune_band(spdnn_net* n, int l, const float* in, float* out, int nblk) {
-    const LayerPlan& p = n->layers[(size_t)l];
-    EventTmp ev0, ev1;
-    HIPCHK(ev0.create());
-    HIPCHK(ev1.create());
-    const hipEvent_t e0 = ev0.e, e1 = ev1.e;
-    spdnn_net::Tuned best{nblk, p.kmax, -1, 0};
-    float best_ms = 0.0f;
-    hipError_t err = hipSuccess;
-    for (int shape = 0; shape < band_shape_count(n->rl) && err == hipSuccess; ++shape) {
+static bool same_bucket(int nblk, int ref) { return nblk * 8 >= ref * 7 && nblk * 8 <= ref * 9; }
+
+// Run-time kernel selection for band layers (the measured half of the inspector's choice), at no
+// extra launches: until a configuration is known for this row-block count, the real layers are
+// launched with the candidate tile shapes and segment lengths in turn (every candidate gives the
+// same result), each launch bracketed by two events; the times are read back a few launches later
+// and after two samples of every candidate the fastest becomes the record for this row-block count.
+static spdnn_net::Explore* explore_for(spdnn_net* n, int nblk, int K) {
+    for (auto& e : n->exploring)
+        if (e.K == K && same_bucket(nblk, e.nblk)) return &e;
+    spdnn_net::Explore e{nblk, K, 0, {}};
+    for (int shape = 0; shape < band_shape_count(n->rl); ++shape) {
         int lens[20];
-        const int nc = band_seglen_candidates(n->N, p.kmax, nblk, n->rl, shape, n->n_cu, lens, 20);
-        for (int c = 0; c < nc && err == hipSuccess; ++c) {
-            BandLaunch a = band_args(n, l, in, out, nblk, 0);
-            a.active = n->d_active_scratch;  // trials must not disturb the real row stamps
-            a.shape = shape;
-            a.seglen = lens[c];
-            float ms = 0.0f;
-            for (int rep = 0; rep < 3 && err == hipSuccess; ++rep) {  // first launch warms up, two are timed
-                a.stamp = ++n->stamp;
-                if (rep == 1) err = hipEventRecord(e0, n->stream);
-                if (err == hipSuccess) err = launch_band(a, n->stream);
-                if (rep == 2 && err == hipSuccess) err = hipEventRecord(e1, n->stream);
+        const int nc = band_seglen_candidates(n->N, K, nblk, n->rl, shape, n->n_cu, lens, 20);
+        for (int c = 0; c < nc; ++c) e.cands.push_back({shape, lens[c], 0.0f, 0});
+    }
+    if (e.cands.empty()) return nullptr;
+    n->exploring.push_back(std::move(e));
+    return &n->exploring.back();
+}
+
+static const int kTrialSamples = 2;
+
+// Reads back finished trials, all of them or all but the newest `keep`.
+static int resolve_trials(spdnn_net* n, size_t keep) {
+    while (n->trials.size() > keep) {
+        const spdnn_net::Trial t = n->trials.front();
+        n->trials.pop_front();
+        float ms = 0.0f;
+        hipError_t err = hipEventSynchronize(t.e1);
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, t.e0, t.e1);
+        n->ev_free.push_back(t.e0);
+        n->ev_free.push_back(t.e1);
+        if (err != hipSuccess) return fail(SPDNN_E_DEVICE, std::string("band tuning: ") + hipGetErrorString(err));
+        for (size_t i = 0; i < n->exploring.size(); ++i) {
+            spdnn_net::Explore& e = n->exploring[i];
+            if (e.K != t.K || e.nblk != t.nblk) continue;
+            spdnn_net::Cand& c = e.cands[(size_t)t.cand];
+            if (c.samples == 0 || ms < c.best_ms) c.best_ms = ms;
+            c.samples++;
+            bool done = true;
+            for (const auto& q : e.cands) done &= q.samples >= kTrialSamples;
+            if (done) {
+                const spdnn_net::Cand* best = &e.cands[0];
+                for (const auto& q : e.cands) if (q.best_ms < best->best_ms) best = &q;
+                n->tuned.push_back({e.nblk, e.K, best->shape, best->seglen});
+                n->exploring.erase(n->exploring.begin() + (long)i);
             }
-            if (err == hipSuccess) err = hipEventSynchronize(e1);
-            if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
-            if (err == hipSuccess && (best.shape < 0 || ms < best_ms)) { best.shape = shape; best.seglen = lens[c]; best_ms = ms; }
+            break;
         }
     }
-    if (err != hipSuccess) return fail(SPDNN_E_DEVICE, std::string("band tuning: ") + hipGetErrorString(err));
-    if (best.shape >= 0) n->tuned.push_back(best);
     return SPDNN_OK;
 }
 
 static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp,
-                               int prev_stamp, int32_t* count_out) {
+                               int prev_stamp, int32_t* count_out, int shape, int seglen) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
         BandLaunch a = band_args(n, l, in, out, nblk, stamp);
         a.count_out = count_out;
         a.prev_stamp = prev_stamp;
-        if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) { a.shape = t->shape; a.seglen = t->seglen; }
+        a.shape = shape;
+        a.seglen = seglen;
         return launch_band(a, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_BLOCK) {
@@ -852,16 +882,45 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         const int prev_stamp = opt.prune ? n->last_stamp : 0;
         const float* in = n->cur;
         float* out = (n->cur == n->A) ? n->C : n->A;
-        if (c == 1 && n->autotune && p.kernel == SPDNN_KERNEL_BAND && last - l + 1 >= 8 &&
-            !find_tuned(n, nblk, p.kmax)) {
-            int rc = tune_band(n, l, in, out, nblk);
-            if (rc) return rc;
+        // band tile shape and segment length: the record for this row-block count, else the next
+        // candidate of the exploration (timed), else the launcher's own heuristic
+        int shape = -1, seglen = 0;
+        bool trial = false;
+        spdnn_net::Trial tr{};
+        if (c == 1 && p.kernel == SPDNN_KERNEL_BAND) {
+            if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) {
+                shape = t->shape;
+                seglen = t->seglen;
+            } else if (n->autotune) {
+                spdnn_net::Explore* e = explore_for(n, nblk, p.kmax);
+                if (e && e->issued < kTrialSamples * (int)e->cands.size()) {
+                    const int ci = e->issued++ % (int)e->cands.size();
+                    shape = e->cands[(size_t)ci].shape;
+                    seglen = e->cands[(size_t)ci].seglen;
+                    while (n->ev_free.size() < 2) {
+                        hipEvent_t ev;
+                        HIPCHK(hipEventCreate(&ev));
+                        n->ev_free.push_back(ev);
+                    }
+                    tr = {e->nblk, e->K, ci, n->ev_free[n->ev_free.size() - 1], n->ev_free[n->ev_free.size() - 2]};
+                    n->ev_free.resize(n->ev_free.size() - 2);
+                    trial = true;
+                }
+            }
         }
         const int stamp0 = n->stamp + 1;
         n->stamp += c;
         if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
         if (c == 1) {
-            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr));
+            if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
+            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr,
+                                shape, seglen));
+            if (trial) {
+                HIPCHK(hipEventRecord(tr.e1, n->stream));
+                n->trials.push_back(tr);
+                int rc = resolve_trials(n, 3);
+                if (rc) return rc;
+            }
         } else {
             ChainLaunch ch{};
             ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
@@ -930,6 +989,10 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
+    {
+        int rc = resolve_trials(n, 0);
+        if (rc) return rc;
+    }
     HIPCHK(hipEventElapsedTime(&r.ms_total, n->ev_start, n->ev_stop));
     for (const Timed& t : timed) {
         float ms = 0.0f;
