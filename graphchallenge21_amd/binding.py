@@ -91,6 +91,7 @@ def load_library():
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
+        "spdnn_device_memory": ([C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_device_synchronize": ([], C.c_int),
     }
     for name, (args, res) in sig.items():
@@ -149,6 +150,13 @@ def device_info():
     cu, mem = C.c_int(), C.c_int64()
     _check(load_library().spdnn_device_info(name, 256, C.byref(cu), C.byref(mem)))
     return name.value.decode(), cu.value, mem.value
+
+
+def device_memory():
+    """(free, total) device memory in bytes."""
+    free, total = C.c_int64(), C.c_int64()
+    _check(load_library().spdnn_device_memory(C.byref(free), C.byref(total)))
+    return free.value, total.value
 
 
 class Network:

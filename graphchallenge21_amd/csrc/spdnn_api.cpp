@@ -1153,6 +1153,14 @@ int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_byte
     return SPDNN_OK;
 }
 
+int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
+    size_t f = 0, t = 0;
+    HIPCHK(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (int64_t)f;
+    if (total_bytes) *total_bytes = (int64_t)t;
+    return SPDNN_OK;
+}
+
 int spdnn_device_synchronize(void) {
     HIPCHK(hipDeviceSynchronize());
     return SPDNN_OK;

@@ -245,6 +245,11 @@ int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps);
 /* Name and compute-unit count of device 0. */
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes);
 
+/* Free and total device memory of device 0 in bytes (what hipMemGetInfo reports); either pointer
+ * may be NULL.  Sizing aid: a network holds three feature buffers of rows*neuron*4 bytes plus the
+ * layer plans. */
+int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes);
+
 int spdnn_device_synchronize(void);
 
 #ifdef __cplusplus

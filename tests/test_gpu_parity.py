@@ -560,3 +560,60 @@ def _sorted_rows(rowptr, col, val):
         o = np.argsort(col[a:b], kind="stable")
         col[a:b], val[a:b] = col[a:b][o], val[a:b][o]
     return col, val
+
+
+def test_handle_lifecycle(gc, orc):
+    """Two networks alive at once with interleaved runs, features replaced between runs, a layer
+    replaced after a run (inspect again, set features again), and no device memory left behind by
+    create/run/destroy cycles."""
+    print("lifecycle", flush=True)
+    N, B, L = 512, 300, 3
+    la = [orc.gen_layer_csr(31, l, N) for l in range(L)]
+    lb = [orc.gen_layer_csr(32, l, N, 8) for l in range(L)]
+    fa = orc.gen_features(31, N, 0, B, 0.1, 0.6)
+    fb = orc.gen_features(32, N, 0, 77, 0.3, 0.9)
+    ra = orc.infer(fa, la, -0.3, prune=True)
+    rb = orc.infer(fb, lb, -0.05, prune=True)
+    with gc.Network(N, B, L, bias=-0.3) as a, gc.Network(N, B, L, bias=-0.05) as b:
+        for l in range(L):
+            a.set_layer_csr(l, *la[l])
+            b.set_layer_csr(l, *lb[l])
+        a.inspect()
+        b.inspect()
+        a.set_features_dense(fa)
+        b.set_features_dense(fb)
+        a.run(first_layer=0, n_layers=1)
+        b.run(first_layer=0, n_layers=2)
+        a.run(first_layer=1, n_layers=2)
+        b.run(first_layer=2, n_layers=1)
+        assert np.array_equal(a.categories(), ra["categories"]) and np.array_equal(b.categories(), rb["categories"])
+        # new features on the same handle (smaller batch), then the first ones again
+        a.set_features_dense(fb)
+        a.run()
+        assert np.array_equal(a.categories(), orc.infer(fb, la, -0.3, prune=True)["categories"])
+        a.set_features_dense(fa)
+        a.run()
+        assert np.array_equal(a.categories(), ra["categories"])
+        # replace a layer: everything before the next inspect is refused, then results follow the new layer
+        a.set_layer_csr(1, *lb[1])
+        with pytest.raises(gc.SpdnnError):
+            a.run()
+        a.inspect()
+        with pytest.raises(gc.SpdnnError):
+            a.run()                     # features went with the old plans
+        a.set_features_dense(fa)
+        a.run()
+        want = orc.infer(fa, [la[0], lb[1], la[2]], -0.3, prune=True)
+        assert np.array_equal(a.categories(), want["categories"])
+        k = min(20, len(want["categories"]))
+        assert same_floats(a.activations(want["categories"][:k].astype(np.int32)), want["y"][:k])
+    free0, total = gc.device_memory()
+    assert 0 < free0 <= total
+    for _ in range(4):
+        with gc.Network(4096, 4096, 2) as net:
+            net.synth_layers(1)
+            net.inspect()
+            net.synth_features(1, 4096, 0.1, 0.6)
+            net.run()
+    free1, _ = gc.device_memory()
+    assert free0 - free1 < (64 << 20), "device memory not returned: %d bytes" % (free0 - free1)
