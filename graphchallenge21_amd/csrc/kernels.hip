@@ -817,6 +817,11 @@ int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, 
     return n;
 }
 
+double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, int seglen) {
+    if (seglen <= 0) return 0.0;
+    return seglen_score(N, K, band_chunk_outputs(rl, shape), nblk, n_cu * band_workgroups_per_cu(rl, shape), seglen);
+}
+
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     // host-side shape checks: what the kernel and its grid assume
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||

@@ -52,6 +52,8 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s);
 // segment lengths for a shape (used by the run-time selection in spdnn_run).
 int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
+// the occupancy / halo model's score of one candidate (higher is better), for ordering trials
+double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, int seglen);
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
 
 // BLOCK layers: groups of up to 16 outputs sharing up to 32 input columns.

@@ -728,16 +728,24 @@ static bool same_bucket(int nblk, int ref) { return nblk * 8 >= ref * 7 && nblk 
 // launched with the candidate tile shapes and segment lengths in turn (every candidate gives the
 // same result), each launch bracketed by two events; the times are read back a few launches later
 // and after two samples of every candidate the fastest becomes the record for this row-block count.
-static spdnn_net::Explore* explore_for(spdnn_net* n, int nblk, int K) {
+static spdnn_net::Explore* explore_for(spdnn_net* n, int nblk, int K, int layers_left) {
     for (auto& e : n->exploring)
         if (e.K == K && same_bucket(nblk, e.nblk)) return &e;
     spdnn_net::Explore e{nblk, K, 0, {}};
+    std::vector<std::pair<double, spdnn_net::Cand>> scored;
     for (int shape = 0; shape < band_shape_count(n->rl); ++shape) {
         int lens[20];
         const int nc = band_seglen_candidates(n->N, K, nblk, n->rl, shape, n->n_cu, lens, 20);
-        for (int c = 0; c < nc; ++c) e.cands.push_back({shape, lens[c], 0.0f, 0});
+        for (int c = 0; c < nc; ++c)
+            scored.push_back({band_seglen_score(n->N, K, nblk, n->rl, shape, n->n_cu, lens[c]) + (shape == 1 ? 0.05 : 0.0),
+                              spdnn_net::Cand{shape, lens[c], 0.0f, 0}});
     }
-    if (e.cands.empty()) return nullptr;
+    // most promising first (the two-workgroup shape is the usual winner), so that a run too short
+    // to finish the exploration still spends its layers on good candidates
+    std::stable_sort(scored.begin(), scored.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
+    for (const auto& sc : scored) e.cands.push_back(sc.second);
+    // a new exploration needs at least one full round of candidates ahead of it
+    if (e.cands.empty() || layers_left < (int)e.cands.size()) return nullptr;
     n->exploring.push_back(std::move(e));
     return &n->exploring.back();
 }
@@ -892,7 +900,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 shape = t->shape;
                 seglen = t->seglen;
             } else if (n->autotune) {
-                spdnn_net::Explore* e = explore_for(n, nblk, p.kmax);
+                spdnn_net::Explore* e = explore_for(n, nblk, p.kmax, last - l + 1);
                 if (e && e->issued < kTrialSamples * (int)e->cands.size()) {
                     const int ci = e->issued++ % (int)e->cands.size();
                     shape = e->cands[(size_t)ci].shape;
