@@ -22,6 +22,9 @@
 //   --no-prune        keep every row through all layers
 //   --gather          force the general kernel for every layer
 //   --categories F    write the surviving row ids (1-based, one per line) to F
+//   --truth F         compare the surviving row ids with the challenge's truth file
+//                     (neuron<N>-l<L>-categories.tsv: 1-based ids, one per line); exit status 3
+//                     when they differ
 //   --quiet           no per-layer lines
 #include <sys/stat.h>
 
@@ -60,7 +63,7 @@ int main(int argc, char** argv) {
     const int neuron = atoi(argv[1]);
     const int batch = atoi(argv[2]);
     const int layer = atoi(argv[3]);
-    std::string data = "../data", cat_file;
+    std::string data = "../data", cat_file, truth_file;
     bool synthetic = false, prune = true, quiet = false, gather = false;
     unsigned long long seed = 0;
     float dmin = 0.10f, dmax = 0.25f;
@@ -73,6 +76,7 @@ int main(int argc, char** argv) {
         else if (a == "--no-prune") prune = false;
         else if (a == "--gather") gather = true;
         else if (a == "--categories" && i + 1 < argc) cat_file = argv[++i];
+        else if (a == "--truth" && i + 1 < argc) truth_file = argv[++i];
         else if (a == "--quiet") quiet = true;
         else { fprintf(stderr, "unknown option %s\n", a.c_str()); return 2; }
     }
@@ -160,7 +164,28 @@ int main(int argc, char** argv) {
         CHECK(spdnn_write_categories(net, cat_file.c_str()));
         printf("categories written to %s\n", cat_file.c_str());
     }
+    int status = 0;
+    if (!truth_file.empty()) {
+        std::vector<long long> truth;
+        FILE* f = fopen(truth_file.c_str(), "r");
+        if (!f) {
+            fprintf(stderr, "cannot read %s\n", truth_file.c_str());
+            return 1;
+        }
+        long long id;
+        while (fscanf(f, "%lld", &id) == 1) truth.push_back(id);
+        fclose(f);
+        int64_t cnt = 0;
+        CHECK(spdnn_get_categories(net, nullptr, 0, &cnt));
+        std::vector<int32_t> ids((size_t)(cnt > 0 ? cnt : 1));
+        CHECK(spdnn_get_categories(net, ids.data(), (int64_t)ids.size(), &cnt));
+        bool same = (int64_t)truth.size() == cnt;
+        for (int64_t i = 0; same && i < cnt; ++i) same = truth[(size_t)i] == (long long)ids[(size_t)i] + 1;
+        printf("Challenge %s (%lld categories, truth file holds %zu)\n", same ? "PASSED" : "FAILED", (long long)cnt,
+               truth.size());
+        if (!same) status = 3;
+    }
     CHECK(spdnn_destroy(net));
     printf("[END]...\n");
-    return 0;
+    return status;
 }

@@ -499,6 +499,15 @@ def test_cli_driver_on_tsv_files(gc, orc, tmp_path):
         assert "layer %d, batch = %d" % (l, len(ref["active_ids"][l])) in r.stdout
     got = np.array([int(x) for x in out.read_text().split()], dtype=np.int64)
     assert np.array_equal(got, ref["categories"] + 1)
+    # the written file is in the challenge's truth-file format: the driver checks itself against it
+    r = subprocess.run([exe, str(N), str(B), str(L), "--data", str(data), "--truth", str(out), "--quiet"],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0 and "Challenge PASSED" in r.stdout
+    wrong = tmp_path / "wrong.tsv"
+    wrong.write_text("".join("%d\n" % x for x in got[:-1]))
+    r = subprocess.run([exe, str(N), str(B), str(L), "--data", str(data), "--truth", str(wrong), "--quiet"],
+                       capture_output=True, text=True, timeout=100)
+    assert r.returncode == 3 and "Challenge FAILED" in r.stdout
     # without files the driver falls back to the seeded generator
     r = subprocess.run([exe, str(N), "200", "3", "--data", str(tmp_path / "nowhere"), "--quiet"],
                        capture_output=True, text=True, timeout=100)
