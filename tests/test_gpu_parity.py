@@ -172,7 +172,9 @@ def test_forced_gather_equals_band(gc, orc):
 @pytest.mark.parametrize("rl", [1, 2])
 def test_other_row_block_sizes(gc, orc, rl, monkeypatch):
     """Row blocks of 64 and 128 rows (the default is 256)."""
+    from helpers import hub_block_csr, radix_like_csr
     monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
     N, L, B = 1024, 4, 333
     print("rows per lane", rl, flush=True)
     layers = [orc.gen_layer_csr(9, l, N) for l in range(L)]
@@ -180,6 +182,17 @@ def test_other_row_block_sizes(gc, orc, rl, monkeypatch):
     with gc.Network(N, B, L) as net:
         net.synth_layers(9)
         net.inspect()
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+    # the other layer classes at this block size: run chains (one cycle, cycles of two), BLOCK, GATHER
+    rng = np.random.default_rng(rl)
+    layers = [radix_like_csr(rng, N, 16, "general"), radix_like_csr(rng, N, 512, "uniform"),
+              hub_block_csr(rng, N, "pow2"), sort_rows(random_csr(rng, N, rng.integers(1, 20, size=N), "general"))]
+    with gc.Network(N, B, 4, bias=-0.2) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert [net.layer_plan(l).kernel for l in range(4)] == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER]
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 
