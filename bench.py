@@ -61,7 +61,8 @@ def main():
                          "the category set of the first ROWS rows after ALL layers is compared with the oracle")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this build is single-GPU (rows shard trivially, see DESIGN.md); run with --gpus 1")
+        log("bench.py: this build runs on one GPU (rows never interact, so more GPUs would each take a slice "
+            "of the batch with replicated weights; that is not built); run with --gpus 1")
         return 2
 
     import graphchallenge21_amd as gc

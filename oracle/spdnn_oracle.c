@@ -268,7 +268,7 @@ int orc_get_threads(void) {
  *   epilogue      src/utils/cpu_spmm_fuse.h:46 / all_network.cu:57: bias is added once, after the
  *                 sum, then clamped; the bias is a float here (the GPU kernels take float bias,
  *                 all_network.cu:24; cpu_spmm_fuse.h:11 takes an int and so truncates -0.3 to 0,
- *                 which the BASELINE configurations do not want).
+ *                 which the challenge's biases -0.3 ... -0.45 do not want).
  *   active flag   all_network.cu:55-60: a row is active iff any of its outputs is nonzero
  *                 (`if (C[..] = __ReLU(..)) active[row] = 1`; NaN counts, -0.0 does not). */
 void orc_layer(const float* yin, int64_t nrows, int neuron,
