@@ -381,7 +381,7 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
 }
 
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
-                   const std::vector<float>& val, int force_kernel, LayerPlan& plan) {
+                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan) {
     const int64_t nnz = rowptr[N];
     int kmax = 0;
     bool rows_regular = true, dup = false;
@@ -410,6 +410,9 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.info.uniform_value = uniform ? 1 : 0;
     plan.info.value = uniform ? val[0] : 0.0f;
     plan.info.exact_products = exact ? 1 : 0;
+    // The fused multiply-add shortcut needs products that never underflow: power-of-two weights
+    // AND activations that are zero or well above the denormal range (the caller decides).
+    exact = exact && fma_ok;
     plan.info.band_halo = -1;
     plan.info.nnz = nnz;
 

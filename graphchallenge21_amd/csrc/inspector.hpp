@@ -64,8 +64,11 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
                          std::vector<int32_t>& out_at);
 
 // Full per-layer inspection (everything except dst, which needs the next layer's labelling).
+// fma_ok: nonzero activations stay far above the denormal range, so that a product with a
+// power-of-two weight is exact and a fused multiply-add rounds like multiply-then-add; when false
+// every layer uses the unfused pair.
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
-                   const std::vector<float>& val, int force_kernel, LayerPlan& plan);
+                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan);
 
 // dst[slot] = physical column (in the next buffer) of the neuron computed at `slot`.
 void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos);

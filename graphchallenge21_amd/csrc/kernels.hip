@@ -626,15 +626,19 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(
     const int n0 = blockIdx.x * 32;
     const int lb = blockIdx.y;  // row block inside the chunk
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    bool bad = false;
+    bool bad = false, tiny = false;
     for (int rr = ty; rr < RB; rr += 8) {
         const int lr = lb * RB + rr;
         float x = 0.0f;
         if (lr < nrows && n0 + tx < N) x = rowmajor[(size_t)lr * N + n0 + tx];
         if (!(fabsf(x) <= 3.4028234e38f)) bad = true;
+        // below 2^-100 a product with a power-of-two weight may underflow, where a fused
+        // multiply-add no longer rounds like multiply-then-add
+        if (x != 0.0f && fabsf(x) < 7.888609e-31f) tiny = true;
         tile[rr][tx] = x;
     }
     if (bad) nonfinite[0] = 1;
+    if (tiny) nonfinite[1] = 1;
     __syncthreads();
     const size_t blk = ((size_t)(row0 / RB) + lb) * (size_t)N * RB;
     for (int idx = threadIdx.x; idx < 32 * RB; idx += 256) {

@@ -141,6 +141,11 @@ struct spdnn_net {
     int rl = 4, RB = 256;
     int rows_cap = 0;
     int force_kernel = SPDNN_KERNEL_AUTO;
+    // With |bias| >= 2^-40 a nonzero output fl(acc + bias) is at least an ulp of the bias, far
+    // above the denormal range, so products with power-of-two weights (|w| <= 2^24 down to 2^-24)
+    // are exact.  With a zero or tiny bias activations can decay into the denormal range, where
+    // the fused multiply-add would round differently from the reference's multiply-then-add.
+    bool fma_ok = true;
     std::vector<LayerPlan> layers;
     std::unique_ptr<JobPool> pool;
     bool inspected = false;
@@ -355,7 +360,8 @@ int submit_layer(spdnn_net* n, int layer, std::shared_ptr<std::vector<int32_t>> 
     const int force = n->force_kernel;
     const int N = n->N;
     LayerPlan* plan = &n->layers[(size_t)layer];
-    n->pool->submit([=] { inspect_layer(N, *rp, *col, *val, force, *plan); });
+    const bool fma_ok = n->fma_ok;
+    n->pool->submit([=] { inspect_layer(N, *rp, *col, *val, force, fma_ok, *plan); });
     return SPDNN_OK;
 }
 
@@ -378,6 +384,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     spdnn_net* n = new (std::nothrow) spdnn_net();
     if (!n) return fail(SPDNN_E_NOMEM, "out of host memory");
     n->N = neuron; n->max_batch = max_batch; n->L = layers; n->bias = bias; n->clampv = clamp;
+    n->fma_ok = std::fabs(bias) >= 9.094947e-13f && clamp >= 9.094947e-13f;  // 2^-40
     int rl = 4;
     if (const char* e = getenv("SPDNN_ROWS_PER_LANE")) rl = atoi(e);
     if (rl != 1 && rl != 2 && rl != 4) { delete n; return fail(SPDNN_E_ARG, "SPDNN_ROWS_PER_LANE must be 1, 2 or 4"); }
@@ -500,6 +507,7 @@ int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nn
     std::fill(n->pending.begin(), n->pending.end(), 0);
     n->inspected = false;
     const int N = n->N, force = n->force_kernel;
+    const bool fma_ok = n->fma_ok;
     for (int l = first; l < first + count; ++l) {
         n->pending[(size_t)l] = 1;
         LayerPlan* plan = &n->layers[(size_t)l];
@@ -507,7 +515,7 @@ int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nn
             std::vector<int32_t> rp, cc;
             std::vector<float> vv;
             synth_layer_csr(seed, l, N, nnz_per_row, value, rp, cc, vv);
-            inspect_layer(N, rp, cc, vv, force, *plan);
+            inspect_layer(N, rp, cc, vv, force, fma_ok, *plan);
         });
     }
     return SPDNN_OK;
@@ -619,7 +627,7 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
     DevTmp stage_buf;
     HIPCHK(stage_buf.alloc((size_t)chunk_rows * N * 4));
     float* stage = stage_buf.as<float>();
-    HIPCHK(hipMemsetAsync(n->d_nonfinite, 0, 4, n->stream));
+    HIPCHK(hipMemsetAsync(n->d_nonfinite, 0, 8, n->stream));
     const int padded = ((batch + RB - 1) / RB) * RB;
     for (int64_t r0 = 0; r0 < padded; r0 += chunk_rows) {
         const int64_t rows_here = std::min<int64_t>(chunk_rows, padded - r0);
@@ -632,9 +640,10 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
                                 n->d_nonfinite, n->stream));
         HIPCHK(hipStreamSynchronize(n->stream));  // the staging buffer is reused by the next chunk
     }
-    int32_t bad = 0;
-    HIPCHK(hipMemcpy(&bad, n->d_nonfinite, 4, hipMemcpyDeviceToHost));
-    if (bad) return fail(SPDNN_E_ARG, "features contain NaN or infinity");
+    int32_t bad[2] = {0, 0};
+    HIPCHK(hipMemcpy(bad, n->d_nonfinite, 8, hipMemcpyDeviceToHost));
+    if (bad[0]) return fail(SPDNN_E_ARG, "features contain NaN or infinity");
+    if (bad[1]) return fail(SPDNN_E_ARG, "features contain nonzero values below 2^-100 in magnitude");
     HIPCHK(launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
     n->have_features = true;

@@ -639,3 +639,36 @@ def test_handle_lifecycle(gc, orc):
             net.run()
     free1, _ = gc.device_memory()
     assert free0 - free1 < (64 << 20), "device memory not returned: %d bytes" % (free0 - free1)
+
+
+def test_zero_bias_into_the_denormal_range(gc, orc):
+    """Bias 0 and power-of-two weights of 1/16, 8 per row: activations halve (at least) per layer and
+    reach the denormal range after ~120 layers, where a product no longer is exact.  The library
+    must not take the fused multiply-add shortcut there: bit-equal to the oracle on every layer."""
+    N, K, L, B = 256, 8, 140, 64
+    print("denormal range", flush=True)
+    rng = np.random.default_rng(0)
+    layers = []
+    for l in range(L):
+        rowptr, col, _ = orc.gen_layer_csr(5, l, N, K)
+        layers.append((rowptr, col, np.full(len(col), 2.0 ** -4, np.float32)))
+    feats = rng.uniform(0.3, 1.0, size=(B, N)).astype(np.float32)
+    ref = orc.infer(feats, layers, 0.0, prune=False, keep=set(range(L)))
+    assert 0 < ref["kept"][L - 1][1].max() < 1e-40          # the chain does end in denormals
+    rows = np.arange(B, dtype=np.int32)
+    with gc.Network(N, B, L, bias=0.0) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert net.layer_plan(0).kernel == gc.KERNEL_BAND and net.layer_plan(0).exact_products == 1
+        net.set_features_dense(feats)
+        for l in range(L):
+            net.run(prune=False, first_layer=l, n_layers=1)
+            if l % 10 == 9 or l > 115:
+                assert same_floats(net.activations(rows), ref["kept"][l][1]), "layer %d" % l
+        # features so small that even the first product would underflow are refused
+        tiny = feats.copy()
+        tiny[3, 7] = 1e-35
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_features_dense(tiny)
+        assert e.value.code == 1 and "2^-100" in e.value.message
