@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(
         const int lr = lb * RB + rr;
         float x = 0.0f;
         if (lr < nrows && n0 + tx < N) x = rowmajor[(size_t)lr * N + n0 + tx];
-        if (!(fabsf(x) <= 3.4028234e38f)) bad = true;
+        if (!(fabsf(x) <= 1.2676506e30f)) bad = true;  // NaN, infinity or beyond 2^100
         // below 2^-100 a product with a power-of-two weight may underflow, where a fused
         // multiply-add no longer rounds like multiply-then-add
         if (x != 0.0f && fabsf(x) < 7.888609e-31f) tiny = true;

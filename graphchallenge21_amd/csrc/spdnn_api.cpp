@@ -379,8 +379,8 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (neuron < 1 || neuron > (1 << 24)) return fail(SPDNN_E_ARG, "neuron must be in [1, 2^24]");
     if (max_batch < 1) return fail(SPDNN_E_ARG, "max_batch must be positive");
     if (layers < 1) return fail(SPDNN_E_ARG, "layers must be positive");
-    if (!std::isfinite(bias) || !(clamp > 0.0f) || !std::isfinite(clamp))
-        return fail(SPDNN_E_ARG, "bias must be finite and clamp positive");
+    if (!std::isfinite(bias) || !(clamp > 0.0f) || !(clamp <= 1.2676506e30f) || !(std::fabs(bias) <= 1.2676506e30f))
+        return fail(SPDNN_E_ARG, "bias must be finite and clamp positive, both at most 2^100 in magnitude");
     spdnn_net* n = new (std::nothrow) spdnn_net();
     if (!n) return fail(SPDNN_E_NOMEM, "out of host memory");
     n->N = neuron; n->max_batch = max_batch; n->L = layers; n->bias = bias; n->clampv = clamp;
@@ -642,7 +642,7 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
     }
     int32_t bad[2] = {0, 0};
     HIPCHK(hipMemcpy(bad, n->d_nonfinite, 8, hipMemcpyDeviceToHost));
-    if (bad[0]) return fail(SPDNN_E_ARG, "features contain NaN or infinity");
+    if (bad[0]) return fail(SPDNN_E_ARG, "features contain NaN, infinity or values above 2^100 in magnitude");
     if (bad[1]) return fail(SPDNN_E_ARG, "features contain nonzero values below 2^-100 in magnitude");
     HIPCHK(launch_iota_gid(n->d_gid, n->rows_cap, batch, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));

@@ -23,7 +23,12 @@
  *   - a handle is used by one host thread at a time.
  *   - row ids ("global ids", categories) are 0-based positions in the feature matrix that was
  *     handed over.
- *   - feature values and weights must be finite; products are expected not to underflow.
+ *   - value ranges, checked at the boundary (SPDNN_E_ARG): weights finite with |w| <= 2^21;
+ *     features finite with |x| <= 2^100 and, when nonzero, |x| >= 2^-100; bias finite, clamp
+ *     positive, both at most 2^100.  Inside these no sum of products overflows and none
+ *     underflows where that could change a rounding, so no infinity or NaN arises in the chain
+ *     and the results equal the reference's CPU arithmetic bit for bit.  (The reference's
+ *     ternary clamp would pass a NaN through, all_network.cu:8-10.)
  */
 #ifndef SPDNN_H
 #define SPDNN_H

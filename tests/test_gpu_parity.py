@@ -257,6 +257,10 @@ def test_positive_bias_and_error_paths(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.set_features_dense(bad)
         assert e.value.code == 1 and "NaN" in e.value.message
+        bad[5, 7] = 1e31                                                     # beyond 2^100
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_features_dense(bad)
+        assert e.value.code == 1 and "2^100" in e.value.message
         net.set_features_dense(feats)
         with pytest.raises(gc.SpdnnError) as e:
             net.run(prune=True)

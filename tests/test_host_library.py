@@ -287,6 +287,8 @@ def test_argument_and_state_errors(gc, orc):
         gc.Network(64, 0, 1, bias=0.0)
     with pytest.raises(gc.SpdnnError):
         gc.Network(64, 4, 1, bias=float("nan"))
+    with pytest.raises(gc.SpdnnError):
+        gc.Network(64, 4, 1, bias=-0.3, clamp=1e31)
     n = 64
     good = sort_rows(random_csr(np.random.default_rng(1), n, 4, "uniform"))
     with gc.Network(n, 4, 2, bias=-0.1) as net:
@@ -303,6 +305,10 @@ def test_argument_and_state_errors(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.set_layer_csr(0, good[0], good[1], bad_val)
         assert "non-finite" in e.value.message
+        bad_val[0] = 4.0e6                          # beyond 2^21
+        with pytest.raises(gc.SpdnnError) as e:
+            net.set_layer_csr(0, good[0], good[1], bad_val)
+        assert "2^21" in e.value.message
         bad_ptr = good[0].copy()
         bad_ptr[3] = bad_ptr[2] - 1
         with pytest.raises(gc.SpdnnError):
