@@ -676,3 +676,37 @@ def test_zero_bias_into_the_denormal_range(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.set_features_dense(tiny)
         assert e.value.code == 1 and "2^-100" in e.value.message
+
+
+def test_reference_side_binding(gc, orc, tmp_path):
+    """oracle/_ref/ref_binding is the binding a maintainer of the reference would add to its
+    driver, compiled against the reference's own host code: the reference's COOMatrix loads and
+    sorts the weight files, the features are read as its read_input does, the rest goes through
+    the C ABI.  Built only where the reference is mounted; the prebuilt program travels."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "oracle", "_ref", "ref_binding")
+    if not os.path.exists(exe):
+        pytest.skip("oracle/_ref/ref_binding not built (reference not mounted at build time)")
+    N, B, L = 1024, 200, 3
+    print("reference-side binding", flush=True)
+    data = tmp_path / "data"
+    (data / ("neuron%d" % N)).mkdir(parents=True)
+    rng = np.random.default_rng(8)
+    layers = [orc.gen_layer_csr(14, l, N) for l in range(L)]
+    for l, (rowptr, col, val) in enumerate(layers):
+        lines = ["%d\t%d\t%.9g\n" % (col[e] + 1, j + 1, val[e]) for j in range(N) for e in range(rowptr[j], rowptr[j + 1])]
+        rng.shuffle(lines)
+        with open(gc.weight_file_name(str(data), N, l), "w") as f:
+            f.writelines(lines)
+    feats = orc.gen_features(14, N, 0, B, 0.10, 0.55)
+    with open(data / ("sparse-images-%d.tsv" % N), "w") as f:
+        rr, cc = np.nonzero(feats)
+        f.writelines("%d\t%d\t1\n" % (r + 1, c + 1) for r, c in zip(rr, cc))
+    ref = orc.infer(feats, layers, -0.3, prune=True)
+    r = subprocess.run([exe, str(N), str(B), str(L), str(data), "-0.3"], capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, r.stdout + r.stderr
+    for l in range(L):
+        assert "layer %d, batch = %d" % (l, len(ref["active_ids"][l])) in r.stdout
+    got = np.array([int(x.split()[1]) for x in r.stdout.splitlines() if x.startswith("category ")], dtype=np.int64)
+    assert np.array_equal(got, ref["categories"])
