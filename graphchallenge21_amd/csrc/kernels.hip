@@ -812,7 +812,10 @@ int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, 
     for (int nseg : ladder) {
         if (n >= max_out) break;
         const int cps = (nchunks + nseg - 1) / nseg;
-        if (cps < 4 && nseg > 1) break;  // at least four chunks per workgroup
+        // at least four chunks per workgroup - unless even that leaves most of the chip idle
+        // (few row blocks): then single-chunk workgroups, which finish soonest, are candidates too
+        const bool starved = (long long)nblk * ((nchunks + 3) / 4) < 2LL * slots;
+        if (cps < (starved ? 1 : 4) && nseg > 1) break;
         const int len = cps * T;
         bool dup = seglen_score(N, K, T, nblk, slots, len) < floor_score;
         for (int i = 0; i < n; ++i) dup |= out[i] == len;
