@@ -72,6 +72,8 @@ def load_library():
         "spdnn_set_force_kernel": ([vp, C.c_int], C.c_int),
         "spdnn_get_layer_plan": ([vp, C.c_int, C.POINTER(LayerPlan)], C.c_int),
         "spdnn_get_band_plan": ([vp, C.c_int, _i32p, _i32p, _u8p], C.c_int),
+        "spdnn_get_band_pairs": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
+                                 C.POINTER(C.c_int), C.c_void_p, C.c_void_p], C.c_int),
         "spdnn_get_layer_dst": ([vp, C.c_int, _i32p], C.c_int),
         "spdnn_get_layer_slots": ([vp, C.c_int, C.POINTER(C.c_int)], C.c_int),
         "spdnn_get_input_labelling": ([vp, C.c_int, _i32p], C.c_int),
@@ -223,6 +225,17 @@ class Network:
         sel = np.empty(self.neuron * k, np.uint8)
         _check(self._lib.spdnn_get_band_plan(self._h, layer, in_pos, out_at, sel))
         return in_pos, out_at, sel.reshape(self.neuron, k)
+
+    def band_pairs(self, layer):
+        """(steps, records uint32[neuron/2][stride], weights float32[neuron/2][padded_steps][2] or None)."""
+        steps, stride, padded, has_w = C.c_int(), C.c_int(), C.c_int(), C.c_int()
+        _check(self._lib.spdnn_get_band_pairs(self._h, layer, C.byref(steps), C.byref(stride), C.byref(padded),
+                                              C.byref(has_w), None, None))
+        rec = np.empty((self.neuron // 2, stride.value), np.uint32)
+        w = np.empty((self.neuron // 2, padded.value, 2), np.float32) if has_w.value else None
+        _check(self._lib.spdnn_get_band_pairs(self._h, layer, None, None, None, None, rec.ctypes.data,
+                                              None if w is None else w.ctypes.data))
+        return steps.value, rec, w
 
     def layer_dst(self, layer):
         p = self.layer_plan(layer)

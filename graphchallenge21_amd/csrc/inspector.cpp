@@ -2,7 +2,9 @@
 
 #include <algorithm>
 #include <array>
+#include <climits>
 #include <cmath>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
@@ -468,6 +470,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
             }
         }
         plan.sel.clear();
+        plan.pairs.clear();
         plan.ell_col.clear();
         plan.rowlen.clear();
     } else if (band) {
@@ -475,14 +478,55 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
         plan.info.band_halo = halo;
         plan.sel.resize((size_t)N * K);
-        if (plan.wmode != 0) plan.wv.resize((size_t)N * K); else plan.wv.clear();
         for (int v = 0; v < N; ++v) {
             const int j = plan.out_at[v];
-            for (int k = 0; k < K; ++k) {
-                const int e = rowptr[j] + k;  // ascending input index = accumulation order
-                plan.sel[(size_t)v * K + k] = (uint8_t)(plan.in_pos[col[e]] & 255);
-                if (plan.wmode != 0) plan.wv[(size_t)v * K + k] = val[e];
+            for (int k = 0; k < K; ++k)   // ascending input index = accumulation order
+                plan.sel[(size_t)v * K + k] = (uint8_t)(plan.in_pos[col[rowptr[j] + k]] & 255);
+        }
+        // Pair records: the outputs at band positions 2u and 2u+1 add their inputs in ascending
+        // input index, so the two lists merge into one list of steps in which shared inputs appear
+        // once; per step a ring selector, a use bit per output and (unless the layer has one exact
+        // value) a weight per output, 0 where the output does not use the step.
+        const int npairs = N / 2;
+        int steps = K;
+        for (int u = 0; u < npairs; ++u) {
+            const int j0 = plan.out_at[2 * u], j1 = plan.out_at[2 * u + 1];
+            int a = rowptr[j0], b = rowptr[j1], m = 0;
+            while (a < rowptr[j0 + 1] || b < rowptr[j1 + 1]) {
+                const int ia = a < rowptr[j0 + 1] ? col[a] : INT32_MAX, ib = b < rowptr[j1 + 1] ? col[b] : INT32_MAX;
+                if (ia <= ib) ++a;
+                if (ib <= ia) ++b;
+                ++m;
             }
+            steps = std::max(steps, m);
+        }
+        int trips = (steps + 3) / 4;
+        if (K == 32 && steps <= 36) trips = 9;  // the unrolled kernel path reads fixed 16-dword records
+        const int stride = (4 + trips + 3) / 4 * 4;
+        plan.pair_steps = steps;
+        plan.pair_stride = stride;
+        plan.pair_padded = trips * 4;
+        plan.pairs.assign((size_t)npairs * stride, 0u);
+        if (plan.wmode != 0) plan.wv.assign((size_t)npairs * trips * 8, 0.0f); else plan.wv.clear();
+        for (int u = 0; u < npairs; ++u) {
+            const int j0 = plan.out_at[2 * u], j1 = plan.out_at[2 * u + 1];
+            uint32_t* rec = &plan.pairs[(size_t)u * stride];
+            uint8_t* slots = reinterpret_cast<uint8_t*>(rec + 4);
+            float* w = plan.wmode != 0 ? &plan.wv[(size_t)u * trips * 8] : nullptr;
+            uint64_t use0 = 0, use1 = 0;
+            int a = rowptr[j0], b = rowptr[j1], m = 0;
+            while (a < rowptr[j0 + 1] || b < rowptr[j1 + 1]) {
+                const int ia = a < rowptr[j0 + 1] ? col[a] : INT32_MAX, ib = b < rowptr[j1 + 1] ? col[b] : INT32_MAX;
+                const int in = std::min(ia, ib);
+                slots[m] = (uint8_t)(plan.in_pos[(size_t)in] & 255);
+                if (ia == in) { use0 |= 1ull << m; if (w) w[2 * m] = val[a]; ++a; }
+                if (ib == in) { use1 |= 1ull << m; if (w) w[2 * m + 1] = val[b]; ++b; }
+                ++m;
+            }
+            // padding steps read a column this pair reads anyway (a live ring slot), with weight 0
+            for (int t = m; t < trips * 4; ++t) slots[t] = slots[m - 1];
+            rec[0] = (uint32_t)use0; rec[1] = (uint32_t)(use0 >> 32);
+            rec[2] = (uint32_t)use1; rec[3] = (uint32_t)(use1 >> 32);
         }
         plan.ell_col.clear();
         plan.rowlen.clear();
@@ -507,10 +551,11 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         }
         plan.kmax = kw;
         plan.sel.clear();
+        plan.pairs.clear();
     }
     plan.info.kernel = plan.kernel;
-    plan.info.plan_bytes = (int64_t)(plan.sel.size() + 4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
-                                                              plan.blk_cols.size() + plan.blk_cnt.size() +
+    plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
+                                                              plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.set = true;

@@ -24,7 +24,12 @@ struct LayerPlan {
     std::vector<int32_t> in_pos;
     // neuron computed at every schedule slot (BAND: band position; GATHER: the neuron itself)
     std::vector<int32_t> out_at;
-    std::vector<uint8_t> sel;       // BAND: [N][K] input position mod 256, accumulation order
+    std::vector<uint8_t> sel;       // BAND: [N][K] input position mod 256, accumulation order (host view only)
+    // BAND, what the kernel streams: per pair of neighbouring band positions pair_stride dwords - two
+    // 64-bit use masks (output 2u, output 2u+1), then one selector byte per merged step (pair_steps
+    // of them, padded to whole dwords)
+    std::vector<uint32_t> pairs;
+    int pair_steps = 0, pair_stride = 0, pair_padded = 0;  // padded: steps a record and the weights are laid out for
     std::vector<int32_t> ell_col;   // GATHER: [N][kmax] physical input column, accumulation order
     std::vector<int32_t> rowlen;    // GATHER: [N]
     // BLOCK: groups of up to 16 outputs that read the same (up to 32) inputs
@@ -32,7 +37,7 @@ struct LayerPlan {
     bool blk_full = false;          // every group has exactly 32 shared inputs
     std::vector<int32_t> blk_cols;  // [ngroups][32] physical input columns, accumulation order (padded)
     std::vector<int32_t> blk_cnt;   // [ngroups] number of shared inputs
-    std::vector<float> wv;          // weights in accumulation order: BAND [N][K], GATHER [N][kmax],
+    std::vector<float> wv;          // weights in accumulation order: BAND [N/2][padded steps][2], GATHER [N][kmax],
                                     // BLOCK [ngroups*16][32] (empty when wmode 0)
     std::vector<int32_t> dst;       // [N] physical column of slot's output in the next buffer
 };

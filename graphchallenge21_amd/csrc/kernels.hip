@@ -119,25 +119,33 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // read from HBM once per segment (plus the halo columns at the segment start) and the loads
 // overlap the arithmetic.  Needs 2*T + halo <= RING, T a multiple of 16.
 //
-// Per output the scalar unit streams 32 one-byte ring selectors (already in accumulation order)
-// and, unless the layer has one exact value, 32 weights; the output column is written to the
-// physical column the NEXT layer wants it in (dst), RB*4 contiguous bytes.
+// Outputs are computed in PAIRS of neighbouring band positions (2u, 2u+1).  Every output adds its
+// inputs in ascending input index, so the inputs two outputs share come in the same order in
+// both: the inspector merges the two lists into one list of `steps` steps (K+1 for a circulant
+// band, K inside a group of a chain), and a wave reads each step's column from the ring ONCE and
+// feeds it to both accumulators - half the LDS reads and address arithmetic of one list per
+// output.  A step an output does not use enters it with weight 0 (adding an exact zero).
+//
+// Per pair the scalar unit streams `stride` dwords: two 64-bit use masks (output 0, output 1), then
+// the steps' one-byte ring selectors; unless the layer has one exact value also two weights per
+// step.  The output column is written to the physical column the NEXT layer wants it in (dst),
+// RB*4 contiguous bytes.
 // ------------------------------------------------------------------------------------------
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __device__ __forceinline__ void band_walk_body(
-    const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ sel,
-    const float* __restrict__ wv, const int32_t* __restrict__ dst, int N, int Krt, int halo, int vb, int ve,
-    float wu, float bias, float clampv, unsigned char* smem, float* nz) {
+    const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs,
+    const float* __restrict__ pw, const int32_t* __restrict__ dst, int N, int steps, int stride, int halo,
+    int vb, int ve, float wu, float bias, float clampv, unsigned char* smem, float* nz) {
     using V = typename VecOf<RL>::type;
     constexpr int T = NW * OPW;
+    constexpr int PPW = OPW / 2;  // pairs per wave and chunk
     constexpr int RB = 64 * RL;
     constexpr int COLB = RB * 4;
     static_assert(2 * T + 32 <= RING && T % 16 == 0, "ring too small for a halo of 32 columns");
     static_assert((RING & (RING - 1)) == 0 && RING <= 256, "ring must be a power of two <= 256");
-    static_assert(KT == 0 || KT == 32, "KT is 32 (unrolled) or 0 (run-time row length)");
+    static_assert(OPW % 2 == 0, "outputs are computed in pairs");
+    static_assert(KT == 0 || KT == 36, "KT is 36 (up to 36 steps, unrolled, 16-dword pair records) or 0 (run-time)");
 
-    const int K = KT ? KT : Krt;
-    const int K4 = K >> 2;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int loff = lane * RL;
@@ -154,6 +162,7 @@ __device__ __forceinline__ void band_walk_body(
     }
     __syncthreads();
 
+    const int last_pair = (ve - 1) >> 1;
     for (int cb = vb; cb < ve; cb += T) {
         // columns of the next chunk: issue the HBM loads now, park them in registers (past the
         // segment end the last column is loaded again and never stored)
@@ -164,142 +173,189 @@ __device__ __forceinline__ void band_walk_body(
             vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
         }
 
-        int v[OPW];
-        float acc[OPW][RL];
+        int pr[PPW];
+        float acc[PPW][2][RL];
 #pragma unroll
-        for (int i = 0; i < OPW; ++i) {
-            v[i] = min(cb + wave + i * NW, ve - 1);
+        for (int i = 0; i < PPW; ++i) {
+            pr[i] = min((cb >> 1) + wave + i * NW, last_pair);
 #pragma unroll
-            for (int q = 0; q < RL; ++q) acc[i][q] = 0.0f;
+            for (int q = 0; q < RL; ++q) acc[i][0][q] = acc[i][1][q] = 0.0f;
         }
 
-        if (KT == 32) {
-            // All 32 one-byte selectors of every output sit in scalar registers up front.  The
-            // 32 entries are processed in 16 stages of two; the LDS reads of stage s+1 are issued
-            // before the arithmetic of stage s, so a wave always has reads in flight while its
-            // multiply-adds issue.
-            uint4 sa[OPW], sb[OPW];
-            const float2* wp[OPW];
-            float2 w_cur[OPW];
+        if (KT == 36) {
+            // The whole pair record (masks + 36 selectors) sits in scalar registers up front.  The
+            // LDS read of step s+2 is issued before the arithmetic of step s, so a wave always has
+            // reads in flight while its multiply-adds issue.  Steps 32..35 exist only if steps > 32.
+            uint4 mk[PPW], sa[PPW], sb[PPW];
+            uint32_t sc[PPW];
+            const float4* wp[PPW];
+            float4 w_cur[PPW][2];
 #pragma unroll
-            for (int i = 0; i < OPW; ++i) {
-                const uint4* sp = reinterpret_cast<const uint4*>(sel + (size_t)v[i] * 8);
-                sa[i] = sp[0];
-                sb[i] = sp[1];
+            for (int i = 0; i < PPW; ++i) {
+                const uint4* rec = reinterpret_cast<const uint4*>(pairs + (size_t)pr[i] * 16);
+                mk[i] = rec[0];
+                sa[i] = rec[1];
+                sb[i] = rec[2];
+                sc[i] = pairs[(size_t)pr[i] * 16 + 12];
                 if (WMODE) {
-                    wp[i] = reinterpret_cast<const float2*>(wv + (size_t)v[i] * 32);
-                    w_cur[i] = wp[i][0];
+                    wp[i] = reinterpret_cast<const float4*>(pw + (size_t)pr[i] * 72);
+                    w_cur[i][0] = wp[i][0];
+                    w_cur[i][1] = wp[i][1];
                 }
             }
-            float xbuf[2][2 * OPW][RL];
+            float xb[3][PPW][RL];
+            float4 w_nxt[PPW][2];
 #define SPDNN_SLOT(i, e)                                                                              \
-    ((((((e) >> 2) & 3) == 0 ? ((e) < 16 ? sa[i].x : sb[i].x)                                          \
-       : (((e) >> 2) & 3) == 1 ? ((e) < 16 ? sa[i].y : sb[i].y)                                        \
-       : (((e) >> 2) & 3) == 2 ? ((e) < 16 ? sa[i].z : sb[i].z)                                        \
-                               : ((e) < 16 ? sa[i].w : sb[i].w)) >> (8 * ((e) & 3))) & (RING - 1))
+    (((((e) >> 2) == 0 ? sa[i].x : ((e) >> 2) == 1 ? sa[i].y : ((e) >> 2) == 2 ? sa[i].z                \
+       : ((e) >> 2) == 3 ? sa[i].w : ((e) >> 2) == 4 ? sb[i].x : ((e) >> 2) == 5 ? sb[i].y              \
+       : ((e) >> 2) == 6 ? sb[i].z : ((e) >> 2) == 7 ? sb[i].w : sc[i]) >> (8 * ((e) & 3))) & (RING - 1))
+#define SPDNN_USED(i, o, e) (((((e) < 32) ? ((o) ? mk[i].z : mk[i].x) : ((o) ? mk[i].w : mk[i].y)) >> ((e) & 31)) & 1u)
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int e = 0; e < 2; ++e)
 #pragma unroll
-                for (int i = 0; i < OPW; ++i)
-                    vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, j) * COLB),
-                                   xbuf[0][j * OPW + i]);
+                for (int i = 0; i < PPW; ++i)
+                    vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), xb[e][i]);
 #pragma unroll
-            for (int st = 0; st < 16; ++st) {
-                float2 w_nxt[OPW];
-                if (st < 15) {
+            for (int st = 0; st < 36; ++st) {
+                if (st + 2 < 36 && (st + 2 < 32 || st + 2 < steps)) {
 #pragma unroll
-                    for (int j = 0; j < 2; ++j)
+                    for (int i = 0; i < PPW; ++i)
+                        vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, st + 2) * COLB),
+                                       xb[(st + 2) % 3][i]);
+                }
+                if (WMODE && (st & 3) == 0 && st + 4 < 36) {  // two weights per step, four steps per trip
 #pragma unroll
-                        for (int i = 0; i < OPW; ++i)
-                            vec_to_arr<RL>(*reinterpret_cast<const V*>(
-                                               lane_smem + (size_t)SPDNN_SLOT(i, 2 * (st + 1) + j) * COLB),
-                                           xbuf[(st + 1) & 1][j * OPW + i]);
-                    if (WMODE) {
-#pragma unroll
-                        for (int i = 0; i < OPW; ++i) w_nxt[i] = wp[i][st + 1];
+                    for (int i = 0; i < PPW; ++i) {
+                        w_nxt[i][0] = wp[i][(st >> 2) * 2 + 2];
+                        w_nxt[i][1] = wp[i][(st >> 2) * 2 + 3];
                     }
                 }
+                if (st < 32 || st < steps) {
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                    for (int i = 0; i < PPW; ++i) {
+                        float w0, w1;
+                        if (WMODE) {
+                            const float4 wq = w_cur[i][(st >> 1) & 1];
+                            w0 = (st & 1) ? wq.z : wq.x;
+                            w1 = (st & 1) ? wq.w : wq.y;
+                        } else {
+                            w0 = SPDNN_USED(i, 0, st) ? wu : 0.0f;
+                            w1 = SPDNN_USED(i, 1, st) ? wu : 0.0f;
+                        }
 #pragma unroll
-                    for (int i = 0; i < OPW; ++i) {
-                        float w = wu;
-                        if (WMODE) w = j == 0 ? w_cur[i].x : w_cur[i].y;
-#pragma unroll
-                        for (int q = 0; q < RL; ++q)
-                            acc[i][q] = mac<WMODE>(acc[i][q], xbuf[st & 1][j * OPW + i][q], w);
+                        for (int q = 0; q < RL; ++q) {
+                            acc[i][0][q] = mac<WMODE>(acc[i][0][q], xb[st % 3][i][q], w0);
+                            acc[i][1][q] = mac<WMODE>(acc[i][1][q], xb[st % 3][i][q], w1);
+                        }
                     }
-                if (WMODE && st < 15) {
-#pragma unroll
-                    for (int i = 0; i < OPW; ++i) w_cur[i] = w_nxt[i];
                 }
-                // pin this stage's arithmetic before the reads of the stage after next: without
-                // it the compiler issues all 32 reads of every output first and spills
+                if (WMODE && (st & 3) == 3 && st + 1 < 36) {
 #pragma unroll
-                for (int i = 0; i < OPW; ++i)
+                    for (int i = 0; i < PPW; ++i) {
+                        w_cur[i][0] = w_nxt[i][0];
+                        w_cur[i][1] = w_nxt[i][1];
+                    }
+                }
+                // pin this step's arithmetic before the reads of later steps: without it the
+                // compiler issues all reads of every pair first and spills
 #pragma unroll
-                    for (int q = 0; q < RL; ++q) asm volatile("" : "+v"(acc[i][q]) : : "memory");
+                for (int i = 0; i < PPW; ++i)
+#pragma unroll
+                    for (int q = 0; q < RL; ++q) {
+                        asm volatile("" : "+v"(acc[i][0][q]) : : "memory");
+                        asm volatile("" : "+v"(acc[i][1][q]) : : "memory");
+                    }
             }
 #undef SPDNN_SLOT
+#undef SPDNN_USED
         } else {
-            const uint32_t* sp[OPW];
-            const float4* wp[OPW];
-            uint32_t s_cur[OPW];
-            float4 w_cur[OPW];
+            // run-time step count: four steps per trip; the selectors (and weights) of the next
+            // trip are requested from the scalar cache before this trip's arithmetic starts
+            const int trips = (steps + 3) >> 2;
+            const uint32_t* sp[PPW];
+            const float4* wp[PPW];
+            uint32_t m0lo[PPW], m0hi[PPW], m1lo[PPW], m1hi[PPW], s_cur[PPW];
+            float4 w_cur[PPW][2];
 #pragma unroll
-            for (int i = 0; i < OPW; ++i) {
-                sp[i] = sel + (size_t)v[i] * K4;
+            for (int i = 0; i < PPW; ++i) {
+                const uint32_t* rec = pairs + (size_t)pr[i] * stride;
+                m0lo[i] = rec[0]; m0hi[i] = rec[1]; m1lo[i] = rec[2]; m1hi[i] = rec[3];
+                sp[i] = rec + 4;
                 s_cur[i] = sp[i][0];
                 if (WMODE) {
-                    wp[i] = reinterpret_cast<const float4*>(wv + (size_t)v[i] * K);
-                    w_cur[i] = wp[i][0];
+                    wp[i] = reinterpret_cast<const float4*>(pw + (size_t)pr[i] * (size_t)trips * 8);
+                    w_cur[i][0] = wp[i][0];
+                    w_cur[i][1] = wp[i][1];
                 }
             }
-            // 4 entries of every output per trip; the selectors (and weights) of the next trip
-            // are requested from the scalar cache before this trip's arithmetic starts
 #pragma unroll 1
-            for (int m4 = 0; m4 < K4; ++m4) {
-                uint32_t s_nxt[OPW];
-                float4 w_nxt[OPW];
-                const int mn = min(m4 + 1, K4 - 1);
+            for (int m4 = 0; m4 < trips; ++m4) {
+                uint32_t s_nxt[PPW];
+                float4 w_nxt[PPW][2];
+                const int mn = min(m4 + 1, trips - 1);
 #pragma unroll
-                for (int i = 0; i < OPW; ++i) {
+                for (int i = 0; i < PPW; ++i) {
                     s_nxt[i] = sp[i][mn];
-                    if (WMODE) w_nxt[i] = wp[i][mn];
+                    if (WMODE) {
+                        w_nxt[i][0] = wp[i][2 * mn];
+                        w_nxt[i][1] = wp[i][2 * mn + 1];
+                    }
                 }
 #pragma unroll
                 for (int b = 0; b < 4; ++b) {
+                    const int e = m4 * 4 + b;
+                    if (e < steps) {
 #pragma unroll
-                    for (int i = 0; i < OPW; ++i) {
-                        const uint32_t slot = (s_cur[i] >> (8 * b)) & (RING - 1);
-                        V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
-                        float x[RL];
-                        vec_to_arr<RL>(xv, x);
-                        float w = wu;
-                        if (WMODE) w = b == 0 ? w_cur[i].x : b == 1 ? w_cur[i].y : b == 2 ? w_cur[i].z : w_cur[i].w;
+                        for (int i = 0; i < PPW; ++i) {
+                            const uint32_t slot = (s_cur[i] >> (8 * b)) & (RING - 1);
+                            V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
+                            float x[RL];
+                            vec_to_arr<RL>(xv, x);
+                            float w0, w1;
+                            if (WMODE) {
+                                const float4 wq = w_cur[i][b >> 1];
+                                w0 = (b & 1) ? wq.z : wq.x;
+                                w1 = (b & 1) ? wq.w : wq.y;
+                            } else {
+                                const uint32_t u0 = ((e < 32 ? m0lo[i] : m0hi[i]) >> (e & 31)) & 1u;
+                                const uint32_t u1 = ((e < 32 ? m1lo[i] : m1hi[i]) >> (e & 31)) & 1u;
+                                w0 = u0 ? wu : 0.0f;
+                                w1 = u1 ? wu : 0.0f;
+                            }
 #pragma unroll
-                        for (int q = 0; q < RL; ++q) acc[i][q] = mac<WMODE>(acc[i][q], x[q], w);
+                            for (int q = 0; q < RL; ++q) {
+                                acc[i][0][q] = mac<WMODE>(acc[i][0][q], x[q], w0);
+                                acc[i][1][q] = mac<WMODE>(acc[i][1][q], x[q], w1);
+                            }
+                        }
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < OPW; ++i) {
+                for (int i = 0; i < PPW; ++i) {
                     s_cur[i] = s_nxt[i];
-                    if (WMODE) w_cur[i] = w_nxt[i];
+                    if (WMODE) {
+                        w_cur[i][0] = w_nxt[i][0];
+                        w_cur[i][1] = w_nxt[i][1];
+                    }
                 }
             }
         }
 
 #pragma unroll
-        for (int i = 0; i < OPW; ++i) {
-            if (cb + wave + i * NW < ve) {
-                float y[RL];
+        for (int i = 0; i < PPW; ++i) {
 #pragma unroll
-                for (int q = 0; q < RL; ++q) {
-                    y[q] = relu_clamp(acc[i][q] + bias, clampv);
-                    nz[q] = nz_merge(nz[q], y[q]);
+            for (int o = 0; o < 2; ++o) {
+                const int v = cb + 2 * (wave + i * NW) + o;
+                if (v < ve) {
+                    float y[RL];
+#pragma unroll
+                    for (int q = 0; q < RL; ++q) {
+                        y[q] = relu_clamp(acc[i][o][q] + bias, clampv);
+                        nz[q] = nz_merge(nz[q], y[q]);
+                    }
+                    const int d = dst[v];
+                    *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
                 }
-                const int d = dst[v[i]];
-                *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
             }
         }
 
@@ -315,10 +371,10 @@ __device__ __forceinline__ void band_walk_body(
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
-    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ sel,
-    const float* __restrict__ wv, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int Krt, int halo, int seglen, int stamp, int prev_stamp, float wu,
-    float bias, float clampv) {
+    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ pairs,
+    const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
+    int32_t* __restrict__ count_out, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
+    float wu, float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     const int rb = blockIdx.x;
@@ -329,8 +385,8 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     float nz[RL];
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, sel, wv, dst, N, Krt, halo, vb, ve,
-                                                 wu, bias, clampv, smem, nz);
+    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, pairs, pw, dst, N, steps, stride, halo,
+                                                 vb, ve, wu, bias, clampv, smem, nz);
     stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp, count_out);
 }
 
@@ -343,18 +399,20 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
 // is all zero by definition.  Layers of one chain share K and the weight mode.
 // ------------------------------------------------------------------------------------------
 struct ChainLayer {
-    const uint32_t* sel;
-    const float* wv;
+    const uint32_t* pairs;
+    const float* pw;
     const int32_t* dst;
     float wu;
     int halo;
+    int steps;
+    int stride;
 };
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
     const ChainLayer* __restrict__ table, int nlayers, const float* __restrict__ first_in,
     float* __restrict__ buf_a, float* __restrict__ buf_c, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int Krt, int stamp0, int prev_stamp, int stop_when_dead, float bias,
+    int32_t* __restrict__ count_out, int N, int stamp0, int prev_stamp, int stop_when_dead, float bias,
     float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
@@ -368,8 +426,8 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         float nz[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.sel, lay.wv, lay.dst, N, Krt, lay.halo, 0, N, lay.wu,
-                                                     bias, clampv, smem, nz);
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+                                                     lay.halo, 0, N, lay.wu, bias, clampv, smem, nz);
         stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp0 + j,
                        count_out ? count_out + j : nullptr);
         int any = 0;
@@ -741,18 +799,18 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     const int nseg = (a.N + seglen - 1) / seglen;
     if (nseg > 65535) return hipErrorInvalidValue;
     dim3 grid(a.nblk, nseg), block(NW * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.sel, a.wv, a.dst, a.active, a.count_out,
-                       a.N, a.K, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
+    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_out,
+                       a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
 }
 
 template <int RL, int NW, int OPW, int RING>
 hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
-    if (a.K == 32) {
+    if (band_unrolled(a.K, a.steps, a.stride)) {
         switch (a.wmode) {
-            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 32>(a, s);
-            case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 32>(a, s);
-            default: return launch_band_inst<RL, NW, OPW, RING, 2, 32>(a, s);
+            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 36>(a, s);
+            case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36>(a, s);
+            default: return launch_band_inst<RL, NW, OPW, RING, 2, 36>(a, s);
         }
     }
     switch (a.wmode) {
@@ -764,38 +822,22 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
 
 }  // namespace
 
-// Tile shapes of the band walk for 256-row blocks:
-//   0  16 waves x 3 outputs per chunk, 128-slot ring (128 KiB LDS, one workgroup per CU)
-//   1   8 waves x 2 outputs per chunk,  64-slot ring ( 64 KiB LDS, two workgroups per CU whose
-//      load / compute / barrier phases interleave)
-// BandLaunch::shape < 0 takes SPDNN_BAND_SHAPE from the environment (default 1).  The smaller row
-// blocks (64 and 128 rows) have one shape each.
-static int env_band_shape() {
-    static int shape = -1;
-    if (shape < 0) {
-        const char* e = getenv("SPDNN_BAND_SHAPE");
-        shape = e ? atoi(e) : 1;
-        if (shape < 0 || shape > 1) shape = 1;
-    }
-    return shape;
-}
+// 32 entries per output and at most 36 merged steps per pair in 16-dword records: the unrolled path
+bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36 && stride == 16; }
 
-int band_shape_count(int rl) { return rl == 4 ? 2 : 1; }
-
-static int resolve_shape(int rl, int shape) {
-    if (rl != 4) return 0;
-    if (shape < 0) return env_band_shape();
-    return shape > 1 ? 1 : shape;
-}
+// Tile shape of the band walk: 256-row blocks use 8 waves x 2 outputs (one pair) per chunk and a
+// 64-slot ring (64 KiB LDS, two workgroups per CU whose load / compute / barrier phases
+// interleave); 64- and 128-row blocks use 16 waves x 6 outputs and a 256-slot ring.
+int band_shape_count(int rl) { (void)rl; return 1; }
 
 int band_chunk_outputs(int rl, int shape) {
-    if (rl == 4) return resolve_shape(rl, shape) == 1 ? 16 : 48;
-    return 112;
+    (void)shape;
+    return rl == 4 ? 16 : 96;
 }
 
 int band_workgroups_per_cu(int rl, int shape) {
-    if (rl == 4) return resolve_shape(rl, shape) == 1 ? 2 : 1;
-    return rl == 1 ? 2 : 1;
+    (void)shape;
+    return rl == 2 ? 1 : 2;
 }
 
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out) {
@@ -832,8 +874,9 @@ double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, in
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     // host-side shape checks: what the kernel and its grid assume
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
-        a.halo < a.K - 1 || a.halo > 32 || a.halo >= a.N ||
-        !a.yin || !a.yout || !a.sel || !a.dst || !a.active || (a.wmode != 0 && !a.wv))
+        a.halo < a.K - 1 || a.halo > 32 || a.halo >= a.N || a.steps < a.K || a.steps > 2 * a.K ||
+        a.stride < 4 + (a.steps + 3) / 4 || (a.stride % 4) != 0 ||
+        !a.yin || !a.yout || !a.pairs || !a.dst || !a.active || (a.wmode != 0 && !a.pw))
         return hipErrorInvalidValue;
     BandLaunch b = a;
     b.n_cu = (a.n_cu > 0 ? a.n_cu : 256) * band_workgroups_per_cu(a.rl, a.shape);
@@ -843,11 +886,9 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
         if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);
     }
     switch (a.rl) {
-        case 4:
-            if (resolve_shape(4, a.shape) == 1) return launch_band_rl<4, 8, 2, 64>(b, s);
-            return launch_band_rl<4, 16, 3, 128>(b, s);
-        case 2: return launch_band_rl<2, 16, 7, 256>(b, s);
-        case 1: return launch_band_rl<1, 16, 7, 256>(b, s);
+        case 4: return launch_band_rl<4, 8, 2, 64>(b, s);
+        case 2: return launch_band_rl<2, 16, 6, 256>(b, s);
+        case 1: return launch_band_rl<1, 16, 6, 256>(b, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -865,17 +906,17 @@ hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
         attr_done = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.nblk), dim3(NW * 64), lds, s, reinterpret_cast<const ChainLayer*>(a.table),
-                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.N, a.K, a.stamp0,
+                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.N, a.stamp0,
                        a.prev_stamp, a.stop_when_dead, a.bias, a.clampv);
     return hipGetLastError();
 }
 template <int RL, int NW, int OPW, int RING>
 hipError_t launch_chain_rl(const ChainLaunch& a, hipStream_t s) {
-    if (a.K == 32) {
+    if (a.unrolled) {
         switch (a.wmode) {
-            case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 32>(a, s);
-            case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 32>(a, s);
-            default: return launch_chain_inst<RL, NW, OPW, RING, 2, 32>(a, s);
+            case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 36>(a, s);
+            case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 36>(a, s);
+            default: return launch_chain_inst<RL, NW, OPW, RING, 2, 36>(a, s);
         }
     }
     switch (a.wmode) {
@@ -892,9 +933,9 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
         !a.table || !a.first_in || !a.buf_a || !a.buf_c || !a.active || a.buf_a == a.buf_c)
         return hipErrorInvalidValue;
     switch (a.rl) {
-        case 4: return launch_chain_rl<4, 16, 3, 128>(a, s);
-        case 2: return launch_chain_rl<2, 16, 7, 256>(a, s);
-        case 1: return launch_chain_rl<1, 16, 7, 256>(a, s);
+        case 4: return launch_chain_rl<4, 8, 2, 64>(a, s);
+        case 2: return launch_chain_rl<2, 16, 6, 256>(a, s);
+        case 1: return launch_chain_rl<1, 16, 6, 256>(a, s);
         default: return hipErrorInvalidValue;
     }
 }

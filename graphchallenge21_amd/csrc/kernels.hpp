@@ -17,12 +17,15 @@ namespace spdnn {
 struct BandLaunch {
     const float* yin;        // input buffer (row-block layout, labelled by the layer's band order)
     float* yout;             // output buffer (labelled for the next layer through dst)
-    const uint32_t* sel;     // [N][K/4] packed ring selectors in accumulation order
-    const float* wv;         // [N][K] weights in accumulation order, or nullptr (uniform exact value)
+    const uint32_t* pairs;   // [N/2][stride] per pair of neighbouring outputs: 2 x 64-bit use masks, then one
+                             // ring selector byte per merged step, in accumulation order
+    const float* pw;         // [N/2][4*ceil(steps/4)][2] weights per step and output (0 where unused), or
+                             // nullptr (uniform exact value)
     const int32_t* dst;      // [N] physical output column per band position
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
     int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
     int N, K, nblk, stamp, rl;
+    int steps, stride;       // merged steps per pair (K .. 2K); dwords per pair record (multiple of 4)
     int halo;                // input columns a segment needs before its first position: K-1 .. 32
     int prev_stamp = 0;      // stamp of the previous layer: row blocks it left without an active row are skipped (0 = off)
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
@@ -50,6 +53,7 @@ struct GatherLaunch {
 hipError_t launch_band(const BandLaunch& a, hipStream_t s);
 // Tuning space of the band walk: number of tile shapes for a row-block size, and the best-ranked
 // segment lengths for a shape (used by the run-time selection in spdnn_run).
+bool band_unrolled(int K, int steps, int stride);
 int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 // the occupancy / halo model's score of one candidate (higher is better), for ordering trials
@@ -76,11 +80,13 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s);
 // one workgroup per row block.  Layer j reads what layer j-1 wrote: the first layer reads
 // first_in, every layer writes the work buffer (buf_a / buf_c) it did not read.
 struct ChainLayerDesc {      // one entry of the device-side layer table
-    const uint32_t* sel;
-    const float* wv;
+    const uint32_t* pairs;
+    const float* pw;
     const int32_t* dst;
     float wu;
     int halo;   // input columns a segment needs before its first position (K-1, or 32 for run chains)
+    int steps;  // merged steps per pair
+    int stride; // dwords per pair record
 };
 struct ChainLaunch {
     const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain
@@ -91,6 +97,7 @@ struct ChainLaunch {
     int32_t* active;
     int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
     int N, K, nblk, stamp0, prev_stamp, rl, wmode;
+    int unrolled;                 // every layer of the chain fits the unrolled path (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
     float bias, clampv;
 };

@@ -124,7 +124,7 @@ int host_threads() {
 
 struct DevLayer {
     int32_t* in_pos = nullptr;
-    uint32_t* sel = nullptr;
+    uint32_t* pairs = nullptr;
     int32_t* ell = nullptr;
     int32_t* rowlen = nullptr;
     float* wv = nullptr;
@@ -266,7 +266,7 @@ void free_device(spdnn_net* n);
 int upload_plans(spdnn_net* n) {
     size_t total = 0;
     for (const LayerPlan& p : n->layers) {
-        total += align256(p.in_pos.size() * 4) + align256(p.sel.size()) + align256(p.ell_col.size() * 4) +
+        total += align256(p.in_pos.size() * 4) + align256(p.pairs.size() * 4) + align256(p.ell_col.size() * 4) +
                  align256(p.rowlen.size() * 4) + align256(p.wv.size() * 4) + align256(p.dst.size() * 4) +
                  align256(p.blk_cols.size() * 4) + align256(p.blk_cnt.size() * 4);
     }
@@ -284,7 +284,7 @@ int upload_plans(spdnn_net* n) {
         const LayerPlan& p = n->layers[(size_t)l];
         DevLayer& d = n->dl[(size_t)l];
         HIPCHK(put(p.in_pos.data(), p.in_pos.size() * 4, (void**)&d.in_pos));
-        HIPCHK(put(p.sel.data(), p.sel.size(), (void**)&d.sel));
+        HIPCHK(put(p.pairs.data(), p.pairs.size() * 4, (void**)&d.pairs));
         HIPCHK(put(p.ell_col.data(), p.ell_col.size() * 4, (void**)&d.ell));
         HIPCHK(put(p.rowlen.data(), p.rowlen.size() * 4, (void**)&d.rowlen));
         HIPCHK(put(p.wv.data(), p.wv.size() * 4, (void**)&d.wv));
@@ -294,8 +294,10 @@ int upload_plans(spdnn_net* n) {
     }
     std::vector<ChainLayerDesc> table((size_t)n->L);
     for (int l = 0; l < n->L; ++l) {
-        table[(size_t)l].sel = n->dl[(size_t)l].sel;
-        table[(size_t)l].wv = n->dl[(size_t)l].wv;
+        table[(size_t)l].pairs = n->dl[(size_t)l].pairs;
+        table[(size_t)l].pw = n->dl[(size_t)l].wv;
+        table[(size_t)l].steps = n->layers[(size_t)l].pair_steps;
+        table[(size_t)l].stride = n->layers[(size_t)l].pair_stride;
         table[(size_t)l].dst = n->dl[(size_t)l].dst;
         table[(size_t)l].wu = n->layers[(size_t)l].info.value;
         table[(size_t)l].halo = n->layers[(size_t)l].info.band_halo;
@@ -396,7 +398,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     n->layer_ms.assign((size_t)layers, 0.0f);
     n->pool.reset(new JobPool(host_threads()));
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
-    if (getenv("SPDNN_BAND_SHAPE") || getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // explicit settings win
+    if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     *out = n;
     return SPDNN_OK;
@@ -563,6 +565,22 @@ int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t*
     return SPDNN_OK;
 }
 
+int spdnn_get_band_pairs(const spdnn_net* n, int layer, int* steps, int* stride, int* padded_steps,
+                         int* has_weights, uint32_t* records, float* weights) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    const LayerPlan& p = n->layers[(size_t)layer];
+    if (!p.set || p.kernel != SPDNN_KERNEL_BAND) return fail(SPDNN_E_STATE, "not a BAND layer");
+    if (steps) *steps = p.pair_steps;
+    if (stride) *stride = p.pair_stride;
+    if (padded_steps) *padded_steps = p.pair_padded;
+    if (has_weights) *has_weights = p.wmode != 0 ? 1 : 0;
+    if (records) std::copy(p.pairs.begin(), p.pairs.end(), records);
+    if (weights) std::copy(p.wv.begin(), p.wv.end(), weights);
+    return SPDNN_OK;
+}
+
 int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
     if (!n || !dst) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
@@ -716,7 +734,8 @@ static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, in
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     BandLaunch a{};
-    a.yin = in; a.yout = out; a.sel = d.sel; a.wv = d.wv; a.dst = d.dst; a.active = n->d_active;
+    a.yin = in; a.yout = out; a.pairs = d.pairs; a.pw = d.wv; a.dst = d.dst; a.active = n->d_active;
+    a.steps = p.pair_steps; a.stride = p.pair_stride;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
@@ -746,10 +765,10 @@ static spdnn_net::Explore* explore_for(spdnn_net* n, int nblk, int K, int layers
         int lens[20];
         const int nc = band_seglen_candidates(n->N, K, nblk, n->rl, shape, n->n_cu, lens, 20);
         for (int c = 0; c < nc; ++c)
-            scored.push_back({band_seglen_score(n->N, K, nblk, n->rl, shape, n->n_cu, lens[c]) + (shape == 1 ? 0.05 : 0.0),
+            scored.push_back({band_seglen_score(n->N, K, nblk, n->rl, shape, n->n_cu, lens[c]),
                               spdnn_net::Cand{shape, lens[c], 0.0f, 0}});
     }
-    // most promising first (the two-workgroup shape is the usual winner), so that a run too short
+    // most promising first, so that a run too short
     // to finish the exploration still spends its layers on good candidates
     std::stable_sort(scored.begin(), scored.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
     for (const auto& sc : scored) e.cands.push_back(sc.second);
@@ -890,7 +909,9 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
             while (c < fuse && l + c <= last) {
                 const LayerPlan& q = n->layers[(size_t)(l + c)];
-                if (q.kernel != SPDNN_KERNEL_BAND || q.kmax != p.kmax || q.wmode != p.wmode) break;
+                if (q.kernel != SPDNN_KERNEL_BAND || q.kmax != p.kmax || q.wmode != p.wmode ||
+                    band_unrolled(q.kmax, q.pair_steps, q.pair_stride) != band_unrolled(p.kmax, p.pair_steps, p.pair_stride))
+                    break;
                 ++c;
             }
         }
@@ -944,6 +965,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             ch.active = n->d_active; ch.count_out = fused_count ? n->d_counts + l : nullptr;
             ch.N = n->N; ch.K = p.kmax; ch.nblk = nblk; ch.stamp0 = stamp0; ch.prev_stamp = prev_stamp;
             ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = opt.prune ? 1 : 0;
+            ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
             ch.bias = n->bias; ch.clampv = n->clampv;
             HIPCHK(launch_band_chain(ch, n->stream));
             for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote

@@ -67,7 +67,8 @@ typedef struct spdnn_layer_plan {
     int32_t uniform_value;   /* 1: all values equal `value`                                       */
     float   value;
     int32_t exact_products;  /* 1: every value is 0 or +-2^e, so x*w is exact and fma == mul+add  */
-    int32_t band_halo;       /* BAND: extra input columns a tile needs (max_row_nnz-1); else -1   */
+    int32_t band_halo;       /* BAND: input columns a segment needs before its first position
+                                (max_row_nnz-1 for a circulant band, 32 for run chains); else -1  */
     int64_t nnz;
     int64_t plan_bytes;      /* device bytes held for this layer                                  */
 } spdnn_layer_plan;
@@ -174,6 +175,18 @@ int spdnn_get_band_plan(const spdnn_net* net, int layer, int32_t* in_pos, int32_
 int spdnn_get_layer_slots(const spdnn_net* net, int layer, int* slots);
 
 /* Physical output column of every schedule slot of a layer (dst[slots]); needs spdnn_inspect. */
+/* What the band kernel streams for a BAND layer: one record per pair of neighbouring band positions
+ * (2u, 2u+1).  The two outputs add their inputs in ascending input index, so their lists merge into
+ * one list of *steps steps in which a shared input appears once.  A record is *stride dwords: the
+ * 64-bit use mask of output 2u (low dword first), the use mask of output 2u+1, then one byte per
+ * step = band position of the step's input mod 256 (padded with repeats of the last step).
+ * *has_weights tells whether the kernel streams weights (0: the layer has one exact value and the
+ * arithmetic takes it from the use masks).  `records` (neuron/2 * *stride dwords) and `weights`
+ * (neuron/2 * *padded_steps * 2 floats when *has_weights: per step the weight for output 2u and for
+ * output 2u+1, 0 where unused) may be NULL, like every out-parameter. */
+int spdnn_get_band_pairs(const spdnn_net* net, int layer, int* steps, int* stride, int* padded_steps,
+                         int* has_weights, uint32_t* records, float* weights);
+
 int spdnn_get_layer_dst(const spdnn_net* net, int layer, int32_t* dst);
 
 /* Physical column of every neuron in the buffer layer `layer` reads (layer == layers: the
@@ -230,9 +243,9 @@ int spdnn_get_categories(spdnn_net* net, int32_t* ids, int64_t cap, int64_t* n);
 int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
 
 /* Band-walk configuration measured at run time (record `index` = 0, 1, ...; SPDNN_E_ARG past the
- * last): row blocks it was measured for, tile shape (0: 16 waves x 3 outputs, 128-slot LDS ring,
- * one workgroup per CU; 1: 8 waves x 2 outputs, 64-slot ring, two workgroups per CU) and band
- * positions per workgroup. */
+ * last): row blocks it was measured for, index of the tile shape (one shape per row-block size at
+ * present: 8 waves x one output pair and a 64-slot LDS ring for 256-row blocks) and band positions
+ * per workgroup. */
 int spdnn_get_band_tuning(const spdnn_net* net, int index, int* row_blocks, int* shape, int* seglen);
 
 /* Per-layer kernel milliseconds of the last run made with time_layers. */

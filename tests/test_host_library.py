@@ -93,6 +93,63 @@ def test_inspector_band_plan_reproduces_oracle(gc, orc):
             assert np.array_equal(y[:, net.input_labelling(l + 1)], want)
 
 
+def _emulate_band_pairs(net, l, y_phys, uniform_value):
+    """CPU emulation of the band kernel from the pair records it streams: per pair of neighbouring
+    band positions one merged list of steps; a step's column is read once and added into the
+    accumulators of the outputs whose use bit is set."""
+    n = net.neuron
+    steps, rec, w = net.band_pairs(l)
+    halo = net.layer_plan(l).band_halo
+    dst = net.layer_dst(l)
+    out = np.zeros_like(y_phys)
+    slots = rec[:, 4:].copy().view(np.uint8)
+    for u in range(n // 2):
+        use = [int(rec[u, 0]) | int(rec[u, 1]) << 32, int(rec[u, 2]) | int(rec[u, 3]) << 32]
+        top = (2 * u) // 16 * 16 + 15
+        by_slot = {p % 256: p for p in ((top - d) % n for d in range(halo + 16))}
+        acc = [np.zeros(y_phys.shape[0], np.float32), np.zeros(y_phys.shape[0], np.float32)]
+        for m in range(steps):
+            x = y_phys[:, by_slot[int(slots[u, m])]]
+            for o in (0, 1):
+                if w is not None:
+                    acc[o] = acc[o] + x * w[u, m, o]            # 0 where the output does not use the step
+                    assert (w[u, m, o] != 0) == bool(use[o] >> m & 1) or w[u, m, o] == 0
+                elif use[o] >> m & 1:
+                    acc[o] = acc[o] + x * np.float32(uniform_value)
+        assert all(use[o] >> steps == 0 for o in (0, 1))
+        for o in (0, 1):
+            y = acc[o] + np.float32(net.bias)
+            out[:, dst[2 * u + o]] = np.where(y < 0, np.float32(0), np.where(y > 32, np.float32(32), y))
+    return out
+
+
+def test_band_pair_records_reproduce_oracle(gc, orc, monkeypatch):
+    """The merged step lists of output pairs, for circulant bands (33 steps for 32 entries, 9 for
+    8), run chains (32 steps) and general weights, emulated on the CPU against the oracle."""
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+    n, b = 512, 5
+    rng = np.random.default_rng(21)
+    band8 = orc.gen_layer_csr(4, 1, n, 8)
+    layers = [orc.gen_layer_csr(4, 0, n), radix_like_csr(rng, n, 64, "uniform"), band8,
+              (band8[0], band8[1], rng.uniform(-0.1, 0.15, size=len(band8[1])).astype(np.float32)),
+              radix_like_csr(rng, n, 16, "general")]
+    with gc.Network(n, b, len(layers), bias=-0.1) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert [net.band_pairs(l)[0] for l in range(len(layers))] == [33, 32, 9, 9, 32]
+        assert [net.band_pairs(l)[1].shape[1] for l in range(len(layers))] == [16, 16, 8, 8, 16]
+        assert [net.band_pairs(l)[2] is None for l in range(len(layers))] == [True, True, True, False, False]
+        feats = orc.gen_features(4, n, 0, b, 0.2, 0.7) * np.float32(1.7)
+        y = np.zeros_like(feats)
+        y[:, net.input_labelling(0)] = feats
+        want = feats
+        for l, csr in enumerate(layers):
+            y = _emulate_band_pairs(net, l, y, 0.0625)
+            want, _ = orc.layer(want, csr, -0.1)
+            assert np.array_equal(y[:, net.input_labelling(l + 1)], want), l
+
+
 def test_inspector_falls_back_to_gather(gc, orc):
     rng = np.random.default_rng(3)
     n = 256
