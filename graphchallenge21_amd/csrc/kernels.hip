@@ -150,6 +150,9 @@ __device__ __forceinline__ void band_walk_body(
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int loff = lane * RL;
     const unsigned char* lane_smem = smem + loff * 4;
+    // the layer's one weight as scalar bits: a step's effective weight (wu or 0) is then picked by
+    // integer ops on the scalar unit and feeds the multiply-add as a scalar operand
+    const uint32_t wu_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(wu));
 
     // prologue: halo (columns before the segment, wrapping below 0) + first chunk
     for (int c = wave; c < halo + T; c += NW) {
@@ -239,8 +242,8 @@ __device__ __forceinline__ void band_walk_body(
                             w0 = (st & 1) ? wq.z : wq.x;
                             w1 = (st & 1) ? wq.w : wq.y;
                         } else {
-                            w0 = SPDNN_USED(i, 0, st) ? wu : 0.0f;
-                            w1 = SPDNN_USED(i, 1, st) ? wu : 0.0f;
+                            w0 = __uint_as_float(wu_bits & (0u - SPDNN_USED(i, 0, st)));
+                            w1 = __uint_as_float(wu_bits & (0u - SPDNN_USED(i, 1, st)));
                         }
 #pragma unroll
                         for (int q = 0; q < RL; ++q) {
@@ -319,8 +322,8 @@ __device__ __forceinline__ void band_walk_body(
                             } else {
                                 const uint32_t u0 = ((e < 32 ? m0lo[i] : m0hi[i]) >> (e & 31)) & 1u;
                                 const uint32_t u1 = ((e < 32 ? m1lo[i] : m1hi[i]) >> (e & 31)) & 1u;
-                                w0 = u0 ? wu : 0.0f;
-                                w1 = u1 ? wu : 0.0f;
+                                w0 = __uint_as_float(wu_bits & (0u - u0));
+                                w1 = __uint_as_float(wu_bits & (0u - u1));
                             }
 #pragma unroll
                             for (int q = 0; q < RL; ++q) {
@@ -377,8 +380,10 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     float wu, float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
-    const int rb = blockIdx.x;
-    const int vb = blockIdx.y * seglen;
+    // segments vary fastest: the workgroups of one row block run together, so the columns they
+    // scatter into (and the halo columns they share) stay in few pages and in L2
+    const int rb = blockIdx.y;
+    const int vb = blockIdx.x * seglen;
     const int ve = min(N, vb + seglen);
     const size_t blk = (size_t)rb * (size_t)N * RB;
     if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp)) return;
@@ -797,8 +802,8 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
         if (rank_seglens(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256, &seglen, 1) < 1) return hipErrorInvalidValue;
     }
     const int nseg = (a.N + seglen - 1) / seglen;
-    if (nseg > 65535) return hipErrorInvalidValue;
-    dim3 grid(a.nblk, nseg), block(NW * 64);
+    if (a.nblk > 65535) return hipErrorInvalidValue;
+    dim3 grid(nseg, a.nblk), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_out,
                        a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
