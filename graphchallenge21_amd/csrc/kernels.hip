@@ -380,10 +380,10 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     float wu, float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
-    // segments vary fastest: the workgroups of one row block run together, so the columns they
-    // scatter into (and the halo columns they share) stay in few pages and in L2
-    const int rb = blockIdx.y;
-    const int vb = blockIdx.x * seglen;
+    // row blocks vary fastest (measured: launching the segments of one row block together
+    // instead is slower on live data and reads more from HBM)
+    const int rb = blockIdx.x;
+    const int vb = blockIdx.y * seglen;
     const int ve = min(N, vb + seglen);
     const size_t blk = (size_t)rb * (size_t)N * RB;
     if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp)) return;
@@ -802,8 +802,8 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
         if (rank_seglens(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256, &seglen, 1) < 1) return hipErrorInvalidValue;
     }
     const int nseg = (a.N + seglen - 1) / seglen;
-    if (a.nblk > 65535) return hipErrorInvalidValue;
-    dim3 grid(nseg, a.nblk), block(NW * 64);
+    if (nseg > 65535) return hipErrorInvalidValue;
+    dim3 grid(a.nblk, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_out,
                        a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv);
     return hipGetLastError();
