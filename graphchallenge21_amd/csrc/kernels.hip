@@ -20,6 +20,11 @@ namespace spdnn {
 
 namespace {
 
+// Start of row block rb of a feature buffer: block rb >> 1 of the half rb & 1.
+__device__ __forceinline__ float* block_base(const Feat& f, int rb, size_t block_floats) {
+    return ((rb & 1) ? f.half[1] : f.half[0]) + (size_t)(rb >> 1) * block_floats;
+}
+
 template <int RL> struct VecOf;
 template <> struct VecOf<1> { using type = float; };
 template <> struct VecOf<2> { using type = float2; };
@@ -374,7 +379,7 @@ __device__ __forceinline__ void band_walk_body(
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
-    const float* __restrict__ yin_all, float* __restrict__ yout_all, const uint32_t* __restrict__ pairs,
+    Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
     int32_t* __restrict__ count_out, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
     float wu, float bias, float clampv) {
@@ -385,13 +390,13 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     const int rb = blockIdx.x;
     const int vb = blockIdx.y * seglen;
     const int ve = min(N, vb + seglen);
-    const size_t blk = (size_t)rb * (size_t)N * RB;
+    const size_t blkf = (size_t)N * RB;
     if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp)) return;
     float nz[RL];
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(yin_all + blk, yout_all + blk, pairs, pw, dst, N, steps, stride, halo,
-                                                 vb, ve, wu, bias, clampv, smem, nz);
+    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
+                                                 pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz);
     stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp, count_out);
 }
 
@@ -415,18 +420,19 @@ struct ChainLayer {
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
-    const ChainLayer* __restrict__ table, int nlayers, const float* __restrict__ first_in,
-    float* __restrict__ buf_a, float* __restrict__ buf_c, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int stamp0, int prev_stamp, int stop_when_dead, float bias,
-    float clampv) {
+    const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
+    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int stamp0, int prev_stamp,
+    int stop_when_dead, float bias, float clampv) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     const int rb = blockIdx.x;
-    const size_t blk = (size_t)rb * (size_t)N * RB;
+    const size_t blkf = (size_t)N * RB;
     if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp0)) return;
-    const float* in = first_in + blk;
+    float* const block_a = block_base(buf_a, rb, blkf);
+    float* const block_c = block_base(buf_c, rb, blkf);
+    const float* in = block_base(first_in, rb, blkf);
     for (int j = 0; j < nlayers; ++j) {
-        float* out = (in == buf_a + blk) ? buf_c + blk : buf_a + blk;
+        float* out = (in == block_a) ? block_c : block_a;
         const ChainLayer lay = table[j];
         float nz[RL];
 #pragma unroll
@@ -455,7 +461,7 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
 // ------------------------------------------------------------------------------------------
 template <int RL, int WMODE>
 __global__ __launch_bounds__(256) void gather_kernel(
-    const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ cols,
+    Feat yin_all, Feat yout_all, const int32_t* __restrict__ cols,
     const int32_t* __restrict__ rowlen, const float* __restrict__ wv, const int32_t* __restrict__ dst,
     int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int kmax, int opg, int stamp,
     int prev_stamp, float bias, float clampv) {
@@ -465,9 +471,8 @@ __global__ __launch_bounds__(256) void gather_kernel(
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rb = blockIdx.x;
     if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
-    const size_t blk = (size_t)rb * (size_t)N * RB;
-    const float* __restrict__ yin = yin_all + blk;
-    float* __restrict__ yout = yout_all + blk;
+    const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
+    float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
     const int loff = lane * RL;
     const int j0 = (blockIdx.y * 4 + wave) * opg;
     const int j1 = min(N, j0 + opg);
@@ -512,7 +517,7 @@ __global__ __launch_bounds__(256) void gather_kernel(
 // ------------------------------------------------------------------------------------------
 template <int RL, int WMODE, bool FULL>
 __global__ __launch_bounds__(256) void block_kernel(
-    const float* __restrict__ yin_all, float* __restrict__ yout_all, const int32_t* __restrict__ grp_cols,
+    Feat yin_all, Feat yout_all, const int32_t* __restrict__ grp_cols,
     const int32_t* __restrict__ grp_cnt, const float* __restrict__ wv, const int32_t* __restrict__ dst,
     int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int ngroups, int gpw, int stamp,
     int prev_stamp, float wu, float bias, float clampv) {
@@ -522,9 +527,8 @@ __global__ __launch_bounds__(256) void block_kernel(
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rb = blockIdx.x;
     if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
-    const size_t blk = (size_t)rb * (size_t)N * RB;
-    const float* __restrict__ yin = yin_all + blk;
-    float* __restrict__ yout = yout_all + blk;
+    const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
+    float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
     const int loff = lane * RL;
     const int g0 = (blockIdx.y * 4 + wave) * gpw;
     const int g1 = min(ngroups, g0 + gpw);
@@ -624,7 +628,7 @@ __global__ __launch_bounds__(1024) void scan_active_kernel(
 // columns.  Reads are 4-byte gathers (one per surviving row and column), writes are coalesced.
 template <int RL>
 __global__ __launch_bounds__(64 * RL) void repack_kernel(
-    const float* __restrict__ src, float* __restrict__ dstb, const int32_t* __restrict__ count,
+    Feat src, Feat dstb, const int32_t* __restrict__ count,
     const int32_t* __restrict__ alive_src, const int32_t* __restrict__ alive_gid,
     int32_t* __restrict__ gid_out, int N, int cols_per_wg) {
     constexpr int RB = 64 * RL;
@@ -633,13 +637,13 @@ __global__ __launch_bounds__(64 * RL) void repack_kernel(
     const int cnt = count[0];
     const bool live = slot < cnt;
     const int srow = live ? alive_src[slot] : 0;
-    const size_t sbase = (size_t)(srow / RB) * (size_t)N * RB + (size_t)(srow % RB);
-    const size_t dbase = (size_t)nb * (size_t)N * RB + threadIdx.x;
+    const float* sp = block_base(src, srow / RB, (size_t)N * RB) + (srow % RB);
+    float* dp = block_base(dstb, nb, (size_t)N * RB) + threadIdx.x;
     const int c0 = blockIdx.x * cols_per_wg;
     const int c1 = min(N, c0 + cols_per_wg);
     for (int c = c0; c < c1; ++c) {
-        const float x = live ? src[sbase + (size_t)c * RB] : 0.0f;
-        dstb[dbase + (size_t)c * RB] = x;
+        const float x = live ? sp[(size_t)c * RB] : 0.0f;
+        dp[(size_t)c * RB] = x;
     }
     if (blockIdx.x == 0) gid_out[slot] = live ? alive_gid[slot] : -1;
 }
@@ -659,7 +663,7 @@ __device__ __forceinline__ uint64_t sm64(uint64_t x) {
 // block and a chunk of physical columns.
 template <int RL>
 __global__ __launch_bounds__(64 * RL) void synth_features_kernel(
-    float* __restrict__ y, const int32_t* __restrict__ col_of_phys, int N, int batch, int cols_per_wg,
+    Feat y, const int32_t* __restrict__ col_of_phys, int N, int batch, int cols_per_wg,
     uint64_t kf, uint64_t lo, uint64_t span) {
     constexpr int RB = 64 * RL;
     const int rb = blockIdx.y;
@@ -671,18 +675,18 @@ __global__ __launch_bounds__(64 * RL) void synth_features_kernel(
     if (thr > 0xFFFFFFFFULL) thr = 0xFFFFFFFFULL;
     const int c0 = blockIdx.x * cols_per_wg;
     const int c1 = min(N, c0 + cols_per_wg);
-    const size_t base = (size_t)rb * (size_t)N * RB + threadIdx.x;
+    float* yp = block_base(y, rb, (size_t)N * RB) + threadIdx.x;
     for (int pc = c0; pc < c1; ++pc) {
         const int n = col_of_phys[pc];
         const uint32_t e = (uint32_t)(sm64(rk + (uint64_t)n) >> 32);
-        y[base + (size_t)pc * RB] = (real && e < (uint32_t)thr) ? 1.0f : 0.0f;
+        yp[(size_t)pc * RB] = (real && e < (uint32_t)thr) ? 1.0f : 0.0f;
     }
 }
 
 // Row-major chunk -> row-block layout, 32 columns x RB rows per workgroup through an LDS tile.
 template <int RL>
 __global__ __launch_bounds__(256) void pack_rows_kernel(
-    const float* __restrict__ rowmajor, float* __restrict__ y, const int32_t* __restrict__ phys_of_col,
+    const float* __restrict__ rowmajor, Feat y, const int32_t* __restrict__ phys_of_col,
     int N, long long row0, int nrows, int32_t* __restrict__ nonfinite) {
     constexpr int RB = 64 * RL;
     __shared__ float tile[RB][33];
@@ -703,14 +707,14 @@ __global__ __launch_bounds__(256) void pack_rows_kernel(
     if (bad) nonfinite[0] = 1;
     if (tiny) nonfinite[1] = 1;
     __syncthreads();
-    const size_t blk = ((size_t)(row0 / RB) + lb) * (size_t)N * RB;
+    float* yp = block_base(y, (int)(row0 / RB) + lb, (size_t)N * RB);
     for (int idx = threadIdx.x; idx < 32 * RB; idx += 256) {
         const int c = idx / RB, r = idx % RB;
-        if (n0 + c < N) y[blk + (size_t)phys_of_col[n0 + c] * RB + r] = tile[r][c];
+        if (n0 + c < N) yp[(size_t)phys_of_col[n0 + c] * RB + r] = tile[r][c];
     }
 }
 
-__global__ void unpack_rows_kernel(const float* __restrict__ y, const int32_t* __restrict__ phys_of_col,
+__global__ void unpack_rows_kernel(Feat y, const int32_t* __restrict__ phys_of_col,
                                    const int32_t* __restrict__ phys_rows, int N, int RB,
                                    const int32_t* __restrict__ active, int stamp, float* __restrict__ rowmajor) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
@@ -721,7 +725,7 @@ __global__ void unpack_rows_kernel(const float* __restrict__ y, const int32_t* _
     // skipped, leaving stale data in the buffer)
     if (pr >= 0 && (stamp == 0 || active[pr] == stamp)) {
         const int pc = phys_of_col ? phys_of_col[n] : n;
-        x = y[((size_t)(pr / RB) * (size_t)N + (size_t)pc) * RB + (pr % RB)];
+        x = block_base(y, pr / RB, (size_t)N * RB)[(size_t)pc * RB + (pr % RB)];
     }
     rowmajor[(size_t)blockIdx.y * N + n] = x;
 }
@@ -735,6 +739,14 @@ __global__ void fill_i32_kernel(int32_t* p, long long n, int32_t v) {
 __global__ void iota_gid_kernel(int32_t* gid, int rows, int batch) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < rows) gid[i] = i < batch ? i : -1;
+}
+
+// Streaming write into two buffers at once: even workgroups fill p, odd workgroups fill q.
+__global__ __launch_bounds__(256) void zero_pair_kernel(float4* __restrict__ p, float4* __restrict__ q, long long n4) {
+    float4* d = (blockIdx.x & 1) ? q : p;
+    long long i = (long long)(blockIdx.x >> 1) * blockDim.x + threadIdx.x;
+    const long long stride = (long long)(gridDim.x >> 1) * blockDim.x;
+    for (; i < n4; i += stride) d[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
 __global__ __launch_bounds__(256) void copy_f4_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
@@ -1005,7 +1017,7 @@ hipError_t launch_scan_active(const int32_t* active, const int32_t* gid, int row
     return hipGetLastError();
 }
 
-hipError_t launch_repack(const float* src, float* dst, const int32_t* count, const int32_t* alive_src,
+hipError_t launch_repack(const Feat& src, const Feat& dst, const int32_t* count, const int32_t* alive_src,
                          const int32_t* alive_gid, int32_t* gid_out, int N, int rl, int dst_blocks,
                          hipStream_t s) {
     if (dst_blocks <= 0 || dst_blocks > 65535 || N <= 0) return hipErrorInvalidValue;
@@ -1020,7 +1032,7 @@ hipError_t launch_repack(const float* src, float* dst, const int32_t* count, con
     return hipGetLastError();
 }
 
-hipError_t launch_synth_features(float* y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
+hipError_t launch_synth_features(const Feat& y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
                                  uint64_t seed, float dmin, float dmax, hipStream_t s) {
     if (nblk <= 0 || nblk > 65535 || N <= 0) return hipErrorInvalidValue;
     // host side of the generator definition: keys and the density range as 32.32 fixed point
@@ -1044,7 +1056,7 @@ hipError_t launch_synth_features(float* y, const int32_t* col_of_phys, int N, in
     return hipGetLastError();
 }
 
-hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys_of_col, int N, int64_t row0,
+hipError_t launch_pack_rows(const float* rowmajor, const Feat& y, const int32_t* phys_of_col, int N, int64_t row0,
                             int nrows, int rl, int32_t* nonfinite, hipStream_t s) {
     const int RB = 64 * rl;
     if (nrows <= 0 || N <= 0 || (row0 % RB) != 0) return hipErrorInvalidValue;
@@ -1060,7 +1072,7 @@ hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys
     return hipGetLastError();
 }
 
-hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows, int nreq,
+hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const int32_t* phys_rows, int nreq,
                               int N, int rl, const int32_t* active, int stamp, float* rowmajor, hipStream_t s) {
     if (nreq <= 0 || nreq > 65535 || N <= 0) return hipErrorInvalidValue;
     dim3 grid((N + 255) / 256, nreq);
@@ -1079,6 +1091,13 @@ hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s) {
 hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s) {
     if (rows <= 0) return hipSuccess;
     hipLaunchKernelGGL(iota_gid_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, gid, rows, batch);
+    return hipGetLastError();
+}
+
+hipError_t launch_zero_pair(float* p, float* q, int64_t n_floats_each, hipStream_t s) {
+    if (n_floats_each <= 0 || (n_floats_each % 4) != 0 || !p || !q) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(zero_pair_kernel, dim3(65536), dim3(256), 0, s, reinterpret_cast<float4*>(p),
+                       reinterpret_cast<float4*>(q), (long long)(n_floats_each / 4));
     return hipGetLastError();
 }
 

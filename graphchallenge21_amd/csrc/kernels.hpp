@@ -14,9 +14,20 @@
 
 namespace spdnn {
 
+// A feature buffer lives in TWO allocations: row block rb is block rb >> 1 of half[rb & 1].  Device
+// memory falls into a few large regions (a third of the memory each on MI355X), and a kernel that
+// streams through buffers whose row blocks alternate between two regions runs a fifth faster than one
+// whose buffers lie in a single region (measured: 6.1 against 5.1 TB/s for the memory skeleton of the
+// band walk); the host puts the two halves into different regions where it can.
+struct Feat {
+    float* half[2] = {nullptr, nullptr};
+    bool operator==(const Feat& o) const { return half[0] == o.half[0] && half[1] == o.half[1]; }
+    explicit operator bool() const { return half[0] != nullptr; }
+};
+
 struct BandLaunch {
-    const float* yin;        // input buffer (row-block layout, labelled by the layer's band order)
-    float* yout;             // output buffer (labelled for the next layer through dst)
+    Feat yin;                // input buffer (row-block layout, labelled by the layer's band order)
+    Feat yout;               // output buffer (labelled for the next layer through dst)
     const uint32_t* pairs;   // [N/2][stride] per pair of neighbouring outputs: 2 x 64-bit use masks, then one
                              // ring selector byte per merged step, in accumulation order
     const float* pw;         // [N/2][4*ceil(steps/4)][2] weights per step and output (0 where unused), or
@@ -36,8 +47,8 @@ struct BandLaunch {
 };
 
 struct GatherLaunch {
-    const float* yin;
-    float* yout;
+    Feat yin;
+    Feat yout;
     const int32_t* cols;     // [N][kmax] physical input columns in accumulation order
     const int32_t* rowlen;   // [N]
     const float* wv;         // [N][kmax]
@@ -62,8 +73,8 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
 
 // BLOCK layers: groups of up to 16 outputs sharing up to 32 input columns.
 struct BlockLaunch {
-    const float* yin;
-    float* yout;
+    Feat yin;
+    Feat yout;
     const int32_t* cols;     // [ngroups][32] physical input columns, accumulation order
     const int32_t* cnt;      // [ngroups] shared inputs per group
     const float* wv;         // [ngroups*16][32] weights, or nullptr (uniform exact value)
@@ -91,9 +102,9 @@ struct ChainLayerDesc {      // one entry of the device-side layer table
 struct ChainLaunch {
     const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain
     int nlayers;
-    const float* first_in;
-    float* buf_a;
-    float* buf_c;
+    Feat first_in;
+    Feat buf_a;
+    Feat buf_c;
     int32_t* active;
     int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
     int N, K, nblk, stamp0, prev_stamp, rl, wmode;
@@ -111,29 +122,32 @@ hipError_t launch_scan_active(const int32_t* active, const int32_t* gid, int row
 
 // Repack: row slot k of the destination takes physical row alive_src[k] of the source for
 // k < count[0]; the remaining slots of the last block are zero-filled; gid_out likewise (-1).
-hipError_t launch_repack(const float* src, float* dst, const int32_t* count, const int32_t* alive_src,
+hipError_t launch_repack(const Feat& src, const Feat& dst, const int32_t* count, const int32_t* alive_src,
                          const int32_t* alive_gid, int32_t* gid_out, int N, int rl, int dst_blocks,
                          hipStream_t s);
 
 // Seeded Bernoulli features written straight into the row-block layout; col_of_phys maps a
 // physical column to its neuron.
-hipError_t launch_synth_features(float* y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
+hipError_t launch_synth_features(const Feat& y, const int32_t* col_of_phys, int N, int batch, int nblk, int rl,
                                  uint64_t seed, float dmin, float dmax, hipStream_t s);
 
 // Row-major chunk [nrows][N] (nrows rows starting at row0, row0 a multiple of RB) into the
 // row-block layout with column labelling phys_of_col; rows >= batch are zero.  nonfinite[0] is
 // set to 1 if a value is NaN or infinite.
-hipError_t launch_pack_rows(const float* rowmajor, float* y, const int32_t* phys_of_col, int N,
+hipError_t launch_pack_rows(const float* rowmajor, const Feat& y, const int32_t* phys_of_col, int N,
                             int64_t row0, int nrows, int rl, int32_t* nonfinite, hipStream_t s);
 
 // Row-block layout to row-major for a list of physical rows (-1 gives a zero row).
 // `active`/`stamp`: rows whose stamp differs read back as zero rows (stamp 0 = no check).
-hipError_t launch_unpack_rows(const float* y, const int32_t* phys_of_col, const int32_t* phys_rows,
+hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const int32_t* phys_rows,
                               int nreq, int N, int rl, const int32_t* active, int stamp, float* rowmajor,
                               hipStream_t s);
 
 hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
 hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s);
 hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s);
+// zero-fills p[0..n) and q[0..n) concurrently (even / odd workgroups): a probe of whether two
+// buffers lie in the same memory region
+hipError_t launch_zero_pair(float* p, float* q, int64_t n_floats_each, hipStream_t s);
 
 }  // namespace spdnn

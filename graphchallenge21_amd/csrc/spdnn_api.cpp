@@ -156,7 +156,8 @@ struct spdnn_net {
     hipStream_t stream = nullptr;
     void* arena = nullptr;
     std::vector<DevLayer> dl;
-    float *F = nullptr, *A = nullptr, *C = nullptr;
+    Feat F, A, C;             // features as handed over, and the two work buffers the layers ping-pong between
+    std::vector<float*> feat_allocs;  // the allocations behind them
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
@@ -169,7 +170,7 @@ struct spdnn_net {
     // state
     int batch = 0;
     bool have_features = false;
-    float* cur = nullptr;
+    Feat cur;
     int cur_layer = 0;
     int carried = 0;
     int stamp = 0;
@@ -263,6 +264,90 @@ size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 void free_device(spdnn_net* n);
 
+// The feature buffers: six half-buffers (see Feat).  For large problems the halves of every buffer
+// are taken from two different memory regions.  Which allocation lies where only shows in a
+// measurement: candidates are allocated one after the other and each is swept by a streaming write
+// together with the first one - 6.0 TB/s when the two share a region, 7.2 TB/s when they do not
+// (MI355X) - until three candidates of either kind are there; the rest is freed again.  On a fresh
+// device the boundary comes after about a third of the memory.  SPDNN_REGION_PAIRING=0 switches
+// the search off, SPDNN_ALLOC_VERBOSE=1 prints the measurements.
+int alloc_feature_buffers(spdnn_net* n) {
+    const size_t half_blocks = ((size_t)n->rows_cap / (size_t)n->RB + 1) / 2;
+    const size_t half_bytes = std::max<size_t>(half_blocks, 1) * (size_t)n->N * (size_t)n->RB * 4;
+    const bool verbose = getenv("SPDNN_ALLOC_VERBOSE") != nullptr;
+    const char* env = getenv("SPDNN_REGION_PAIRING");
+    size_t free_b = 0, total_b = 0;
+    HIPCHK(hipMemGetInfo(&free_b, &total_b));
+    const size_t max_cand = std::min<size_t>(48, (size_t)((double)free_b * 0.85 / (double)half_bytes));
+    const bool search = !(env && atoi(env) == 0) && half_bytes >= ((size_t)4 << 30) && max_cand >= 12;
+
+    std::vector<float*>& c = n->feat_allocs;
+    std::vector<double> rate;  // rate[i]: candidate i swept together with candidate 0 (rate[0] unused)
+    auto fail_free = [&](int code, const std::string& msg) {
+        for (float* p : c) hipFree(p);
+        c.clear();
+        return fail(code, msg);
+    };
+    auto add = [&]() {
+        float* p = nullptr;
+        if (hipMalloc(&p, half_bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
+        c.push_back(p);
+        return true;
+    };
+    for (int i = 0; i < 6; ++i)
+        if (!add()) return fail_free(SPDNN_E_NOMEM, "out of device memory for the feature buffers");
+    int pick[6] = {0, 1, 2, 3, 4, 5};
+    if (search) {
+        EventTmp e0, e1;
+        if (e0.create() != hipSuccess || e1.create() != hipSuccess) return fail_free(SPDNN_E_DEVICE, "event creation failed");
+        const int64_t nf = (int64_t)(half_bytes / 16) * 4;
+        rate.assign(1, 0.0);
+        std::vector<int> same, other;
+        for (size_t i = 1; i < max_cand; ++i) {
+            if (i >= c.size() && !add()) break;
+            hipError_t e = launch_zero_pair(c[0], c[i], nf, n->stream);  // first touch
+            if (e == hipSuccess) e = hipEventRecord(e0.e, n->stream);
+            for (int r = 0; r < 2 && e == hipSuccess; ++r) e = launch_zero_pair(c[0], c[i], nf, n->stream);
+            if (e == hipSuccess) e = hipEventRecord(e1.e, n->stream);
+            if (e == hipSuccess) e = hipEventSynchronize(e1.e);
+            float ms = 0.0f;
+            if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0.e, e1.e);
+            if (e != hipSuccess) return fail_free(SPDNN_E_DEVICE, std::string("region probe: ") + hipGetErrorString(e));
+            rate.push_back(4.0 * (double)half_bytes / ((double)ms * 1e-3) / 1e9);
+            const double lowest = *std::min_element(rate.begin() + 1, rate.end());
+            same.assign(1, 0);
+            other.clear();
+            for (size_t k = 1; k < rate.size(); ++k) {
+                if (rate[k] > 1.10 * lowest) other.push_back((int)k);
+                else if (rate[k] < 1.05 * lowest) same.push_back((int)k);
+            }
+            if (i >= 5 && same.size() >= 3 && other.size() >= 3) break;
+        }
+        if (verbose) {
+            fprintf(stderr, "spdnn: half-buffers of %.1f GB swept together with the first, GB/s:", (double)half_bytes / 1e9);
+            for (size_t k = 1; k < rate.size(); ++k) fprintf(stderr, " %.0f", rate[k]);
+            fprintf(stderr, "\nspdnn: %zu in the first region, %zu elsewhere%s\n", same.size(), other.size(),
+                    same.size() >= 3 && other.size() >= 3 ? ": every buffer gets one half of each" : ": no pairing");
+        }
+        if (same.size() >= 3 && other.size() >= 3)
+            for (int b = 0; b < 3; ++b) { pick[2 * b] = same[(size_t)b]; pick[2 * b + 1] = other[(size_t)b]; }
+    }
+    Feat* bufs[3] = {&n->A, &n->C, &n->F};
+    for (int b = 0; b < 3; ++b) {
+        bufs[b]->half[0] = c[(size_t)pick[2 * b]];
+        bufs[b]->half[1] = c[(size_t)pick[2 * b + 1]];
+    }
+    // give back what was only a candidate
+    std::vector<float*> keep;
+    for (size_t i = 0; i < c.size(); ++i) {
+        bool used = false;
+        for (int k = 0; k < 6; ++k) used |= pick[k] == (int)i;
+        if (used) keep.push_back(c[i]); else hipFree(c[i]);
+    }
+    c.swap(keep);
+    return SPDNN_OK;
+}
+
 int upload_plans(spdnn_net* n) {
     size_t total = 0;
     for (const LayerPlan& p : n->layers) {
@@ -304,10 +389,8 @@ int upload_plans(spdnn_net* n) {
     }
     HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
     HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
-    const size_t fbytes = (size_t)n->rows_cap * (size_t)n->N * 4;
-    HIPCHK(hipMalloc(&n->F, fbytes));
-    HIPCHK(hipMalloc(&n->A, fbytes));
-    HIPCHK(hipMalloc(&n->C, fbytes));
+    int rc = alloc_feature_buffers(n);
+    if (rc) return rc;
     n->uploaded = true;
     return SPDNN_OK;
 }
@@ -326,10 +409,10 @@ void free_device(spdnn_net* n) {
     if (n->arena) hipFree(n->arena);
     if (n->d_chain) hipFree(n->d_chain);
     n->d_chain = nullptr;
-    if (n->F) hipFree(n->F);
-    if (n->A) hipFree(n->A);
-    if (n->C) hipFree(n->C);
-    n->arena = nullptr; n->F = n->A = n->C = nullptr;
+    for (float* p : n->feat_allocs) hipFree(p);
+    n->feat_allocs.clear();
+    n->arena = nullptr;
+    n->F = n->A = n->C = Feat();
     n->uploaded = false;
     n->have_features = false;
 }
@@ -730,7 +813,7 @@ int spdnn_default_run_options(spdnn_run_options* o) {
     return SPDNN_OK;
 }
 
-static BandLaunch band_args(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp) {
+static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     BandLaunch a{};
@@ -811,7 +894,7 @@ static int resolve_trials(spdnn_net* n, size_t keep) {
     return SPDNN_OK;
 }
 
-static hipError_t launch_layer(spdnn_net* n, int l, const float* in, float* out, int nblk, int stamp,
+static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
                                int prev_stamp, int32_t* count_out, int shape, int seglen) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
@@ -918,8 +1001,8 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         for (int j = 0; j < c; ++j) r.edges += (double)n->batch * (double)n->layers[(size_t)(l + j)].info.nnz;
         const int nblk = n->carried / n->RB;
         const int prev_stamp = opt.prune ? n->last_stamp : 0;
-        const float* in = n->cur;
-        float* out = (n->cur == n->A) ? n->C : n->A;
+        const Feat in = n->cur;
+        Feat out = (n->cur == n->A) ? n->C : n->A;
         // band tile shape and segment length: the record for this row-block count, else the next
         // candidate of the exploration (timed), else the launcher's own heuristic
         int shape = -1, seglen = 0;
@@ -1001,7 +1084,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         if (newest_count > 0 && (double)newest_count <= (double)thr * (double)n->carried && l < n->L) {
             const int nb = (int)((newest_count + n->RB - 1) / n->RB);  // upper bound of what is alive now
             if (nb * n->RB < n->carried) {
-                float* dstbuf = (n->cur == n->A) ? n->C : n->A;
+                const Feat dstbuf = (n->cur == n->A) ? n->C : n->A;
                 HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count,
                                           n->d_alive_src, n->d_alive_gid, n->stream));
                 HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
