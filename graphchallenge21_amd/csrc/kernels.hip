@@ -349,6 +349,18 @@ __device__ __forceinline__ void band_walk_body(
             }
         }
 
+        // The parked columns go into ring slots no wave reads during this chunk - BEFORE the outputs
+        // are stored: loads and stores share one counter on this hardware, so waiting for the parked
+        // loads after the stores were issued would also wait for the stores to be acknowledged.
+        // The write is unconditional: past the segment end it drops a copy of the last column into a
+        // slot nobody reads any more, and every path has then waited for the parked loads here, so
+        // that nothing downstream needs to wait on the memory counter again.
+#pragma unroll
+        for (int i = 0; i < OPW; ++i) {
+            const int p = cb + T + wave + i * NW;
+            *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(pf[i]);
+        }
+        asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 0; i < PPW; ++i) {
 #pragma unroll
@@ -367,12 +379,6 @@ __device__ __forceinline__ void band_walk_body(
             }
         }
 
-        // the parked columns go into ring slots no wave reads during this chunk
-#pragma unroll
-        for (int i = 0; i < OPW; ++i) {
-            const int p = cb + T + wave + i * NW;
-            if (p < ve) *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(pf[i]);
-        }
         __syncthreads();
     }
 }
