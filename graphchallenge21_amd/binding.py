@@ -93,6 +93,7 @@ def load_library():
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
+        "spdnn_get_feature_placement": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_device_memory": ([C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_device_synchronize": ([], C.c_int),
     }
@@ -236,6 +237,12 @@ class Network:
         _check(self._lib.spdnn_get_band_pairs(self._h, layer, None, None, None, None, rec.ctypes.data,
                                               None if w is None else w.ctypes.data))
         return steps.value, rec, w
+
+    def feature_placement(self):
+        """(paired, candidates): whether the buffer halves lie in different memory regions."""
+        paired, cand = C.c_int(), C.c_int()
+        _check(self._lib.spdnn_get_feature_placement(self._h, C.byref(paired), C.byref(cand)))
+        return bool(paired.value), cand.value
 
     def layer_dst(self, layer):
         p = self.layer_plan(layer)

@@ -158,6 +158,7 @@ struct spdnn_net {
     std::vector<DevLayer> dl;
     Feat F, A, C;             // features as handed over, and the two work buffers the layers ping-pong between
     std::vector<float*> feat_allocs;  // the allocations behind them
+    int feat_paired = 0, feat_candidates = 0;
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
@@ -297,6 +298,7 @@ int alloc_feature_buffers(spdnn_net* n) {
     for (int i = 0; i < 6; ++i)
         if (!add()) return fail_free(SPDNN_E_NOMEM, "out of device memory for the feature buffers");
     int pick[6] = {0, 1, 2, 3, 4, 5};
+    n->feat_paired = 0;
     if (search) {
         EventTmp e0, e1;
         if (e0.create() != hipSuccess || e1.create() != hipSuccess) return fail_free(SPDNN_E_DEVICE, "event creation failed");
@@ -329,9 +331,12 @@ int alloc_feature_buffers(spdnn_net* n) {
             fprintf(stderr, "\nspdnn: %zu in the first region, %zu elsewhere%s\n", same.size(), other.size(),
                     same.size() >= 3 && other.size() >= 3 ? ": every buffer gets one half of each" : ": no pairing");
         }
-        if (same.size() >= 3 && other.size() >= 3)
+        if (same.size() >= 3 && other.size() >= 3) {
             for (int b = 0; b < 3; ++b) { pick[2 * b] = same[(size_t)b]; pick[2 * b + 1] = other[(size_t)b]; }
+            n->feat_paired = 1;
+        }
     }
+    n->feat_candidates = (int)c.size();
     Feat* bufs[3] = {&n->A, &n->C, &n->F};
     for (int b = 0; b < 3; ++b) {
         bufs[b]->half[0] = c[(size_t)pick[2 * b]];
@@ -1272,6 +1277,14 @@ int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_byte
     if (name && cap > 0) snprintf(name, (size_t)cap, "%s (%s)", p.name, p.gcnArchName);
     if (compute_units) *compute_units = p.multiProcessorCount;
     if (hbm_bytes) *hbm_bytes = (int64_t)p.totalGlobalMem;
+    return SPDNN_OK;
+}
+
+int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (!n->uploaded) return fail(SPDNN_E_STATE, "no feature buffers yet");
+    if (paired) *paired = n->feat_paired;
+    if (candidates) *candidates = n->feat_candidates;
     return SPDNN_OK;
 }
 

@@ -263,6 +263,11 @@ int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps);
 /* Name and compute-unit count of device 0. */
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes);
 
+/* How the feature buffers were placed (after features were set): *paired = 1 if the two halves of
+ * every buffer lie in different memory regions (searched for buffers of 8 GiB and more, see
+ * SPDNN_REGION_PAIRING), *candidates = half-buffers allocated during the search (6 = no search). */
+int spdnn_get_feature_placement(const spdnn_net* net, int* paired, int* candidates);
+
 /* Free and total device memory of device 0 in bytes (what hipMemGetInfo reports); either pointer
  * may be NULL.  Sizing aid: a network holds three feature buffers of rows*neuron*4 bytes plus the
  * layer plans. */

@@ -408,6 +408,9 @@ def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
             assert np.array_equal(cats[cats < S], ref["active_ids"][l]), "layer %d" % l
             assert same_floats(net.activations(rows), ref["kept"][l][1]), "layer %d" % l
         full = net.run(prune=False, collect_counts=True)
+        paired, candidates = net.feature_placement()
+        print("feature buffers paired over two memory regions:", paired, "candidates", candidates, flush=True)
+        assert candidates >= 6 and (N == 65536 or (not paired and candidates == 6))   # searched from 8 GiB buffers up
         assert np.array_equal(net.categories()[net.categories() < S], ref["active_ids"][-1])
         assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
 
