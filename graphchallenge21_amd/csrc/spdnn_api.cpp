@@ -279,12 +279,16 @@ int alloc_feature_buffers(spdnn_net* n) {
     const char* env = getenv("SPDNN_REGION_PAIRING");
     size_t free_b = 0, total_b = 0;
     HIPCHK(hipMemGetInfo(&free_b, &total_b));
-    const size_t max_cand = std::min<size_t>(48, (size_t)((double)free_b * 0.85 / (double)half_bytes));
-    const bool search = !(env && atoi(env) == 0) && half_bytes >= ((size_t)4 << 30) && max_cand >= 12;
+    const size_t max_cand = std::min<size_t>(64, (size_t)((double)free_b * 0.85 / (double)half_bytes));
+    const char* min_env = getenv("SPDNN_REGION_PAIRING_MIN_GIB");   // smallest half-buffer worth the search
+    const double min_gib = min_env ? atof(min_env) : 1.0;
+    const bool search = !(env && atoi(env) == 0) && (double)half_bytes >= min_gib * 1073741824.0 && max_cand >= 12;
 
     std::vector<float*>& c = n->feat_allocs;
     std::vector<double> rate;  // rate[i]: candidate i swept together with candidate 0 (rate[0] unused)
+    std::vector<void*> fillers;
     auto fail_free = [&](int code, const std::string& msg) {
+        for (void* f : fillers) hipFree(f);
         for (float* p : c) hipFree(p);
         c.clear();
         return fail(code, msg);
@@ -303,35 +307,80 @@ int alloc_feature_buffers(spdnn_net* n) {
         EventTmp e0, e1;
         if (e0.create() != hipSuccess || e1.create() != hipSuccess) return fail_free(SPDNN_E_DEVICE, "event creation failed");
         const int64_t nf = (int64_t)(half_bytes / 16) * 4;
-        rate.assign(1, 0.0);
         std::vector<int> same, other;
-        for (size_t i = 1; i < max_cand; ++i) {
-            if (i >= c.size() && !add()) break;
-            hipError_t e = launch_zero_pair(c[0], c[i], nf, n->stream);  // first touch
+        // streaming-write rate of candidates a and b swept together
+        auto probe = [&](size_t a, size_t b, double* gbps) {
+            hipError_t e = launch_zero_pair(c[a], c[b], nf, n->stream);  // first touch
             if (e == hipSuccess) e = hipEventRecord(e0.e, n->stream);
-            for (int r = 0; r < 2 && e == hipSuccess; ++r) e = launch_zero_pair(c[0], c[i], nf, n->stream);
+            for (int r = 0; r < 2 && e == hipSuccess; ++r) e = launch_zero_pair(c[a], c[b], nf, n->stream);
             if (e == hipSuccess) e = hipEventRecord(e1.e, n->stream);
             if (e == hipSuccess) e = hipEventSynchronize(e1.e);
             float ms = 0.0f;
             if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0.e, e1.e);
-            if (e != hipSuccess) return fail_free(SPDNN_E_DEVICE, std::string("region probe: ") + hipGetErrorString(e));
-            rate.push_back(4.0 * (double)half_bytes / ((double)ms * 1e-3) / 1e9);
-            const double lowest = *std::min_element(rate.begin() + 1, rate.end());
-            same.assign(1, 0);
+            if (e == hipSuccess) *gbps = 4.0 * (double)half_bytes / ((double)ms * 1e-3) / 1e9;
+            return e;
+        };
+        // candidates that share the reference's region (the slow ones) and candidates that do not
+        auto classify = [&](int ref) {
+            double lowest = 0.0;
+            for (size_t k = 0; k < rate.size(); ++k)
+                if ((int)k != ref && (lowest == 0.0 || rate[k] < lowest)) lowest = rate[k];
+            same.assign(1, ref);
             other.clear();
-            for (size_t k = 1; k < rate.size(); ++k) {
+            for (size_t k = 0; k < rate.size(); ++k) {
+                if ((int)k == ref) continue;
                 if (rate[k] > 1.10 * lowest) other.push_back((int)k);
                 else if (rate[k] < 1.05 * lowest) same.push_back((int)k);
             }
-            if (i >= 5 && same.size() >= 3 && other.size() >= 3) break;
+            return same.size() >= 3 && other.size() >= 3;
+        };
+        // every step past the first six candidates advances at least 4 GiB through the memory: small
+        // half-buffers are spaced out by fillers, which are freed again below
+        const size_t filler = half_bytes < ((size_t)4 << 30) ? ((size_t)4 << 30) - half_bytes : 0;
+        const size_t budget = (size_t)((double)free_b * 0.85);
+        rate.assign(1, 0.0);
+        bool found = false;
+        int ref = 0;
+        for (size_t i = 1; i < max_cand && !found; ++i) {
+            if (i >= c.size()) {
+                if ((c.size() + 1) * half_bytes + (fillers.size() + 1) * filler > budget) break;
+                if (filler) {
+                    void* f = nullptr;
+                    if (hipMalloc(&f, filler) != hipSuccess) { (void)hipGetLastError(); break; }
+                    fillers.push_back(f);
+                }
+                if (!add()) break;
+            }
+            double r = 0.0;
+            const hipError_t e = probe(0, i, &r);
+            if (e != hipSuccess) return fail_free(SPDNN_E_DEVICE, std::string("region probe: ") + hipGetErrorString(e));
+            rate.push_back(r);
+            found = i >= 5 && classify(0);
+        }
+        if (!found && rate.size() >= 8) {
+            // The first candidate may itself straddle two regions, and then every partner looks fast.
+            // Second pass over what is allocated, against the partner that went slowest with it.
+            ref = 1;
+            for (size_t k = 2; k < rate.size(); ++k) if (rate[k] < rate[(size_t)ref]) ref = (int)k;
+            if (verbose) {
+                fprintf(stderr, "spdnn: no second region seen from candidate 0 (GB/s:");
+                for (size_t k = 1; k < rate.size(); ++k) fprintf(stderr, " %.0f", rate[k]);
+                fprintf(stderr, "), second pass against candidate %d\n", ref);
+            }
+            for (size_t k = 0; k < rate.size(); ++k) {
+                if ((int)k == ref) continue;
+                const hipError_t e = probe((size_t)ref, k, &rate[k]);
+                if (e != hipSuccess) return fail_free(SPDNN_E_DEVICE, std::string("region probe: ") + hipGetErrorString(e));
+            }
+            found = classify(ref);
         }
         if (verbose) {
-            fprintf(stderr, "spdnn: half-buffers of %.1f GB swept together with the first, GB/s:", (double)half_bytes / 1e9);
-            for (size_t k = 1; k < rate.size(); ++k) fprintf(stderr, " %.0f", rate[k]);
-            fprintf(stderr, "\nspdnn: %zu in the first region, %zu elsewhere%s\n", same.size(), other.size(),
-                    same.size() >= 3 && other.size() >= 3 ? ": every buffer gets one half of each" : ": no pairing");
+            fprintf(stderr, "spdnn: half-buffers of %.1f GB swept together with candidate %d, GB/s:", (double)half_bytes / 1e9, ref);
+            for (size_t k = 0; k < rate.size(); ++k) if ((int)k != ref) fprintf(stderr, " %.0f", rate[k]);
+            fprintf(stderr, "\nspdnn: %zu in its region, %zu elsewhere%s\n", same.size(), other.size(),
+                    found ? ": every buffer gets one half of each" : ": no pairing");
         }
-        if (same.size() >= 3 && other.size() >= 3) {
+        if (found) {
             for (int b = 0; b < 3; ++b) { pick[2 * b] = same[(size_t)b]; pick[2 * b + 1] = other[(size_t)b]; }
             n->feat_paired = 1;
         }
@@ -343,6 +392,7 @@ int alloc_feature_buffers(spdnn_net* n) {
         bufs[b]->half[1] = c[(size_t)pick[2 * b + 1]];
     }
     // give back what was only a candidate
+    for (void* f : fillers) hipFree(f);
     std::vector<float*> keep;
     for (size_t i = 0; i < c.size(); ++i) {
         bool used = false;
