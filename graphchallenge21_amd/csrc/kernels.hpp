@@ -62,9 +62,10 @@ struct GatherLaunch {
 };
 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s);
-// Tuning space of the band walk: number of tile shapes for a row-block size, and the best-ranked
-// segment lengths for a shape (used by the run-time selection in spdnn_run).
+// 32 entries per output, at most 36 merged steps per pair, 16-dword records: the unrolled kernel path
 bool band_unrolled(int K, int steps, int stride);
+// Tuning space of the band walk: number of tile shapes for a row-block size (one at present) and
+// the candidate segment lengths for a shape (used by the run-time selection in spdnn_run).
 int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 // the occupancy / halo model's score of one candidate (higher is better), for ordering trials
