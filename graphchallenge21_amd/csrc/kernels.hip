@@ -848,19 +848,21 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
 // 32 entries per output and at most 36 merged steps per pair in 16-dword records: the unrolled path
 bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36 && stride == 16; }
 
-// Tile shape of the band walk: 256-row blocks use 8 waves x 2 outputs (one pair) per chunk and a
-// 64-slot ring (64 KiB LDS, two workgroups per CU whose load / compute / barrier phases
-// interleave); 64- and 128-row blocks use 16 waves x 6 outputs and a 256-slot ring.
+// Tile shape of the band walk, the same for every row-block size: 8 waves x 2 outputs (one pair) per
+// chunk and a 64-slot ring - 64 KiB of LDS and two workgroups per CU for 256-row blocks (whose load /
+// compute / barrier phases interleave), 32 and 16 KiB and four workgroups per CU (the wave limit)
+// for 128- and 64-row blocks.  Measured at N=65536: 256-row blocks 6.0 ms per layer, 128-row blocks
+// 6.6 ms (8.8 ms with one 16-wave workgroup and a 256-slot ring per CU).
 int band_shape_count(int rl) { (void)rl; return 1; }
 
 int band_chunk_outputs(int rl, int shape) {
-    (void)shape;
-    return rl == 4 ? 16 : 96;
+    (void)rl; (void)shape;
+    return 16;
 }
 
 int band_workgroups_per_cu(int rl, int shape) {
     (void)shape;
-    return rl == 2 ? 1 : 2;
+    return rl == 4 ? 2 : 4;
 }
 
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out) {
@@ -910,8 +912,8 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     }
     switch (a.rl) {
         case 4: return launch_band_rl<4, 8, 2, 64>(b, s);
-        case 2: return launch_band_rl<2, 16, 6, 256>(b, s);
-        case 1: return launch_band_rl<1, 16, 6, 256>(b, s);
+        case 2: return launch_band_rl<2, 8, 2, 64>(b, s);
+        case 1: return launch_band_rl<1, 8, 2, 64>(b, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -957,8 +959,8 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     switch (a.rl) {
         case 4: return launch_chain_rl<4, 8, 2, 64>(a, s);
-        case 2: return launch_chain_rl<2, 16, 6, 256>(a, s);
-        case 1: return launch_chain_rl<1, 16, 6, 256>(a, s);
+        case 2: return launch_chain_rl<2, 8, 2, 64>(a, s);
+        case 1: return launch_chain_rl<1, 8, 2, 64>(a, s);
         default: return hipErrorInvalidValue;
     }
 }
