@@ -958,9 +958,11 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
         !a.table || !a.first_in || !a.buf_a || !a.buf_c || !a.active || a.buf_a == a.buf_c)
         return hipErrorInvalidValue;
     switch (a.rl) {
-        case 4: return launch_chain_rl<4, 8, 2, 64>(a, s);
-        case 2: return launch_chain_rl<2, 8, 2, 64>(a, s);
-        case 1: return launch_chain_rl<1, 8, 2, 64>(a, s);
+        // one workgroup per row block walks the whole band: 16 waves (one pair each, chunks of 32
+        // outputs, 128-slot ring) so that a CU holds as many waves as in the per-layer kernel
+        case 4: return launch_chain_rl<4, 16, 2, 128>(a, s);
+        case 2: return launch_chain_rl<2, 16, 2, 128>(a, s);
+        case 1: return launch_chain_rl<1, 16, 2, 128>(a, s);
         default: return hipErrorInvalidValue;
     }
 }
