@@ -214,6 +214,7 @@ def main():
             "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "mixed",
             "band_tuning_rowblocks_shape_seglen": net.band_tuning(),
             "feature_buffers_region_paired_candidates": list(net.feature_placement()),
+            "plan_window_device_bytes_pinned_bytes": list(net.plan_memory()),
             "final_active_rows": sustained_final_active,
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",

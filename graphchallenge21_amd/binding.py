@@ -70,6 +70,8 @@ def load_library():
         "spdnn_synth_layer_csr": ([C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_float, _i32p, _i32p, _f32p], C.c_int),
         "spdnn_inspect": ([vp], C.c_int),
         "spdnn_set_force_kernel": ([vp, C.c_int], C.c_int),
+        "spdnn_set_plan_window": ([vp, C.c_int], C.c_int),
+        "spdnn_get_plan_memory": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_layer_plan": ([vp, C.c_int, C.POINTER(LayerPlan)], C.c_int),
         "spdnn_get_band_plan": ([vp, C.c_int, _i32p, _i32p, _u8p], C.c_int),
         "spdnn_get_band_pairs": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
@@ -243,6 +245,16 @@ class Network:
         paired, cand = C.c_int(), C.c_int()
         _check(self._lib.spdnn_get_feature_placement(self._h, C.byref(paired), C.byref(cand)))
         return bool(paired.value), cand.value
+
+    def set_plan_window(self, slots):
+        """0 = every plan resident; 2..64 = that many device slots, plans streamed from pinned memory."""
+        _check(self._lib.spdnn_set_plan_window(self._h, int(slots)))
+
+    def plan_memory(self):
+        """(window, device_bytes, pinned_bytes) of the uploaded plans."""
+        w, d, h = C.c_int(), C.c_int64(), C.c_int64()
+        _check(self._lib.spdnn_get_plan_memory(self._h, C.byref(w), C.byref(d), C.byref(h)))
+        return w.value, d.value, h.value
 
     def layer_dst(self, layer):
         p = self.layer_plan(layer)

@@ -123,7 +123,6 @@ int host_threads() {
 }
 
 struct DevLayer {
-    int32_t* in_pos = nullptr;
     uint32_t* pairs = nullptr;
     int32_t* ell = nullptr;
     int32_t* rowlen = nullptr;
@@ -131,6 +130,15 @@ struct DevLayer {
     int32_t* dst = nullptr;
     int32_t* blk_cols = nullptr;
     int32_t* blk_cnt = nullptr;
+};
+
+// Where the arrays of one layer's plan lie inside its block of device memory (and inside the
+// pinned host copy of that block when plans are streamed): pairs, ell, rowlen, wv, dst, blk_cols,
+// blk_cnt, each aligned to 256 bytes.
+struct PlanLayout {
+    size_t off[7] = {0, 0, 0, 0, 0, 0, 0};
+    size_t len[7] = {0, 0, 0, 0, 0, 0, 0};
+    size_t bytes = 0;
 };
 
 }  // namespace
@@ -156,6 +164,22 @@ struct spdnn_net {
     hipStream_t stream = nullptr;
     void* arena = nullptr;
     std::vector<DevLayer> dl;
+    std::vector<PlanLayout> lay;
+    // Streamed plans (plan_window >= 2): the device holds `plan_window` slots of the largest
+    // plan's size; layer l uses slot l % plan_window.  A second stream copies the plan of layer
+    // l + plan_window from pinned host memory into the slot as soon as layer l has finished,
+    // so the copy runs under the layers in between.
+    int plan_window = 0;
+    size_t slot_bytes = 0;
+    char* h_plans = nullptr;          // pinned: all plans, back to back
+    std::vector<size_t> h_plan_off;
+    std::vector<int> slot_layer;      // layer whose plan the slot holds (or is being filled with)
+    std::vector<char> slot_busy;      // a kernel that reads the slot has been launched since it was filled
+    std::vector<hipEvent_t> ev_slot_ready, ev_slot_free;
+    hipStream_t copy_stream = nullptr;
+    // input labellings: layer 0's stays on the device, another layer's is sent when asked for
+    int32_t* d_lab = nullptr;
+    int lab_layer = -1;
     Feat F, A, C;             // features as handed over, and the two work buffers the layers ping-pong between
     std::vector<float*> feat_allocs;  // the allocations behind them
     int feat_paired = 0, feat_candidates = 0;
@@ -403,47 +427,100 @@ int alloc_feature_buffers(spdnn_net* n) {
     return SPDNN_OK;
 }
 
+PlanLayout plan_layout(const LayerPlan& p) {
+    PlanLayout y;
+    const size_t len[7] = {p.pairs.size() * 4, p.ell_col.size() * 4, p.rowlen.size() * 4, p.wv.size() * 4,
+                           p.dst.size() * 4,   p.blk_cols.size() * 4, p.blk_cnt.size() * 4};
+    for (int k = 0; k < 7; ++k) {
+        y.off[k] = y.bytes;
+        y.len[k] = len[k];
+        y.bytes += align256(len[k]);
+    }
+    return y;
+}
+
+void pack_plan(const LayerPlan& p, const PlanLayout& y, char* dst) {
+    const void* src[7] = {p.pairs.data(), p.ell_col.data(), p.rowlen.data(), p.wv.data(),
+                          p.dst.data(),   p.blk_cols.data(), p.blk_cnt.data()};
+    for (int k = 0; k < 7; ++k)
+        if (y.len[k]) memcpy(dst + y.off[k], src[k], y.len[k]);
+}
+
+DevLayer plan_at(const PlanLayout& y, char* base) {
+    DevLayer d;
+    auto at = [&](int k) -> void* { return y.len[k] ? base + y.off[k] : nullptr; };
+    d.pairs = (uint32_t*)at(0);
+    d.ell = (int32_t*)at(1);
+    d.rowlen = (int32_t*)at(2);
+    d.wv = (float*)at(3);
+    d.dst = (int32_t*)at(4);
+    d.blk_cols = (int32_t*)at(5);
+    d.blk_cnt = (int32_t*)at(6);
+    return d;
+}
+
 int upload_plans(spdnn_net* n) {
-    size_t total = 0;
-    for (const LayerPlan& p : n->layers) {
-        total += align256(p.in_pos.size() * 4) + align256(p.pairs.size() * 4) + align256(p.ell_col.size() * 4) +
-                 align256(p.rowlen.size() * 4) + align256(p.wv.size() * 4) + align256(p.dst.size() * 4) +
-                 align256(p.blk_cols.size() * 4) + align256(p.blk_cnt.size() * 4);
+    const size_t L = (size_t)n->L;
+    n->lay.assign(L, PlanLayout{});
+    size_t total = 0, largest = 0;
+    for (size_t l = 0; l < L; ++l) {
+        n->lay[l] = plan_layout(n->layers[l]);
+        total += n->lay[l].bytes;
+        largest = std::max(largest, n->lay[l].bytes);
     }
-    HIPCHK(hipMalloc(&n->arena, std::max<size_t>(total, 256)));
-    n->dl.assign((size_t)n->L, DevLayer{});
-    char* base = (char*)n->arena;
-    size_t off = 0;
-    auto put = [&](const void* src, size_t bytes, void** dptr) -> hipError_t {
-        if (bytes == 0) { *dptr = nullptr; return hipSuccess; }
-        *dptr = base + off;
-        off += align256(bytes);
-        return hipMemcpy(*dptr, src, bytes, hipMemcpyHostToDevice);
-    };
-    for (int l = 0; l < n->L; ++l) {
-        const LayerPlan& p = n->layers[(size_t)l];
-        DevLayer& d = n->dl[(size_t)l];
-        HIPCHK(put(p.in_pos.data(), p.in_pos.size() * 4, (void**)&d.in_pos));
-        HIPCHK(put(p.pairs.data(), p.pairs.size() * 4, (void**)&d.pairs));
-        HIPCHK(put(p.ell_col.data(), p.ell_col.size() * 4, (void**)&d.ell));
-        HIPCHK(put(p.rowlen.data(), p.rowlen.size() * 4, (void**)&d.rowlen));
-        HIPCHK(put(p.wv.data(), p.wv.size() * 4, (void**)&d.wv));
-        HIPCHK(put(p.dst.data(), p.dst.size() * 4, (void**)&d.dst));
-        HIPCHK(put(p.blk_cols.data(), p.blk_cols.size() * 4, (void**)&d.blk_cols));
-        HIPCHK(put(p.blk_cnt.data(), p.blk_cnt.size() * 4, (void**)&d.blk_cnt));
+    n->dl.assign(L, DevLayer{});
+    const bool streamed = n->plan_window >= 2 && (size_t)n->plan_window < L;
+    if (!streamed) {
+        HIPCHK(hipMalloc(&n->arena, std::max<size_t>(total, 256)));
+        std::vector<char> blob(largest);
+        size_t off = 0;
+        for (size_t l = 0; l < L; ++l) {
+            pack_plan(n->layers[l], n->lay[l], blob.data());
+            if (n->lay[l].bytes)
+                HIPCHK(hipMemcpy((char*)n->arena + off, blob.data(), n->lay[l].bytes, hipMemcpyHostToDevice));
+            n->dl[l] = plan_at(n->lay[l], (char*)n->arena + off);
+            off += n->lay[l].bytes;
+        }
+        std::vector<ChainLayerDesc> table(L);
+        for (size_t l = 0; l < L; ++l) {
+            table[l].pairs = n->dl[l].pairs;
+            table[l].pw = n->dl[l].wv;
+            table[l].steps = n->layers[l].pair_steps;
+            table[l].stride = n->layers[l].pair_stride;
+            table[l].dst = n->dl[l].dst;
+            table[l].wu = n->layers[l].info.value;
+            table[l].halo = n->layers[l].info.band_halo;
+        }
+        HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
+        HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
+        n->slot_bytes = 0;
+    } else {
+        const size_t S = (size_t)n->plan_window;
+        n->slot_bytes = std::max<size_t>(largest, 256);
+        HIPCHK(hipMalloc(&n->arena, S * n->slot_bytes));
+        HIPCHK(hipHostMalloc((void**)&n->h_plans, std::max<size_t>(total, 256)));
+        n->h_plan_off.assign(L, 0);
+        size_t off = 0;
+        for (size_t l = 0; l < L; ++l) {
+            n->h_plan_off[l] = off;
+            pack_plan(n->layers[l], n->lay[l], n->h_plans + off);
+            off += n->lay[l].bytes;
+            n->dl[l] = plan_at(n->lay[l], (char*)n->arena + (l % S) * n->slot_bytes);
+        }
+        n->slot_layer.assign(S, -1);
+        n->slot_busy.assign(S, 0);
+        HIPCHK(hipStreamCreateWithFlags(&n->copy_stream, hipStreamNonBlocking));
+        for (size_t k = 0; k < S; ++k) {
+            hipEvent_t e;
+            HIPCHK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            n->ev_slot_ready.push_back(e);
+            HIPCHK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+            n->ev_slot_free.push_back(e);
+        }
     }
-    std::vector<ChainLayerDesc> table((size_t)n->L);
-    for (int l = 0; l < n->L; ++l) {
-        table[(size_t)l].pairs = n->dl[(size_t)l].pairs;
-        table[(size_t)l].pw = n->dl[(size_t)l].wv;
-        table[(size_t)l].steps = n->layers[(size_t)l].pair_steps;
-        table[(size_t)l].stride = n->layers[(size_t)l].pair_stride;
-        table[(size_t)l].dst = n->dl[(size_t)l].dst;
-        table[(size_t)l].wu = n->layers[(size_t)l].info.value;
-        table[(size_t)l].halo = n->layers[(size_t)l].info.band_halo;
-    }
-    HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
-    HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
+    HIPCHK(hipMalloc(&n->d_lab, (size_t)n->N * 8));
+    HIPCHK(hipMemcpy(n->d_lab, n->layers[0].in_pos.data(), (size_t)n->N * 4, hipMemcpyHostToDevice));
+    n->lab_layer = -1;
     int rc = alloc_feature_buffers(n);
     if (rc) return rc;
     n->uploaded = true;
@@ -461,6 +538,22 @@ int ensure_uploaded(spdnn_net* n) {
 }
 
 void free_device(spdnn_net* n) {
+    if (n->copy_stream) {
+        hipStreamSynchronize(n->copy_stream);
+        hipStreamDestroy(n->copy_stream);
+        n->copy_stream = nullptr;
+    }
+    for (hipEvent_t e : n->ev_slot_ready) hipEventDestroy(e);
+    for (hipEvent_t e : n->ev_slot_free) hipEventDestroy(e);
+    n->ev_slot_ready.clear();
+    n->ev_slot_free.clear();
+    n->slot_layer.clear();
+    n->slot_busy.clear();
+    if (n->h_plans) hipHostFree(n->h_plans);
+    n->h_plans = nullptr;
+    if (n->d_lab) hipFree(n->d_lab);
+    n->d_lab = nullptr;
+    n->lab_layer = -1;
     if (n->arena) hipFree(n->arena);
     if (n->d_chain) hipFree(n->d_chain);
     n->d_chain = nullptr;
@@ -472,9 +565,62 @@ void free_device(spdnn_net* n) {
     n->have_features = false;
 }
 
+bool plans_streamed(const spdnn_net* n) { return n->copy_stream != nullptr; }
+
+// Streamed plans: starts the copy of layer l's plan into its slot (unless the slot holds it or is
+// being filled with it already).  The copy waits for the last kernel that read the slot.
+hipError_t plan_fetch(spdnn_net* n, int l) {
+    const size_t slot = (size_t)l % (size_t)n->plan_window;
+    if (n->slot_layer[slot] == l) return hipSuccess;
+    hipError_t e;
+    if (n->slot_busy[slot]) {
+        if ((e = hipStreamWaitEvent(n->copy_stream, n->ev_slot_free[slot], 0)) != hipSuccess) return e;
+    }
+    const PlanLayout& y = n->lay[(size_t)l];
+    if (y.bytes) {
+        e = hipMemcpyAsync((char*)n->arena + slot * n->slot_bytes, n->h_plans + n->h_plan_off[(size_t)l], y.bytes,
+                           hipMemcpyHostToDevice, n->copy_stream);
+        if (e != hipSuccess) return e;
+    }
+    if ((e = hipEventRecord(n->ev_slot_ready[slot], n->copy_stream)) != hipSuccess) return e;
+    n->slot_layer[slot] = l;
+    n->slot_busy[slot] = 0;
+    return hipSuccess;
+}
+
+// Before the launch of layer l: its plan is in its slot (the compute stream waits for the copy).
+hipError_t plan_acquire(spdnn_net* n, int l) {
+    if (!plans_streamed(n)) return hipSuccess;
+    hipError_t e = plan_fetch(n, l);
+    if (e != hipSuccess) return e;
+    return hipStreamWaitEvent(n->stream, n->ev_slot_ready[(size_t)l % (size_t)n->plan_window], 0);
+}
+
+// After the launch of layer l: the slot is handed to the layer that uses it next.
+hipError_t plan_release(spdnn_net* n, int l) {
+    if (!plans_streamed(n)) return hipSuccess;
+    const size_t slot = (size_t)l % (size_t)n->plan_window;
+    hipError_t e = hipEventRecord(n->ev_slot_free[slot], n->stream);
+    if (e != hipSuccess) return e;
+    n->slot_busy[slot] = 1;
+    const int next = l + n->plan_window;
+    return next < n->L ? plan_fetch(n, next) : hipSuccess;
+}
+
 // physical-column labelling of the buffer that holds the state after `layers_done` layers
-const int32_t* labelling_dev(const spdnn_net* n, int layers_done) {
-    return layers_done < n->L ? n->dl[(size_t)layers_done].in_pos : nullptr;  // nullptr = identity
+// (nullptr = identity, after the last layer); *out is device memory
+hipError_t labelling_dev(spdnn_net* n, int layers_done, const int32_t** out) {
+    if (layers_done >= n->L) { *out = nullptr; return hipSuccess; }
+    if (layers_done == 0) { *out = n->d_lab; return hipSuccess; }
+    int32_t* second = n->d_lab + n->N;
+    if (n->lab_layer != layers_done) {
+        hipError_t e = hipMemcpy(second, n->layers[(size_t)layers_done].in_pos.data(), (size_t)n->N * 4,
+                                 hipMemcpyHostToDevice);
+        if (e != hipSuccess) return e;
+        n->lab_layer = layers_done;
+    }
+    *out = second;
+    return hipSuccess;
 }
 
 void reset_state(spdnn_net* n) {
@@ -538,6 +684,10 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
     if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
+    if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
+        const int w = atoi(e);
+        if (w == 0 || (w >= 2 && w <= 64)) n->plan_window = w;
+    }
     *out = n;
     return SPDNN_OK;
 }
@@ -682,6 +832,26 @@ int spdnn_inspect(spdnn_net* n) {
     return SPDNN_OK;
 }
 
+int spdnn_set_plan_window(spdnn_net* n, int slots) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (slots != 0 && (slots < 2 || slots > 64)) return fail(SPDNN_E_ARG, "plan window is 0 (all plans resident) or 2..64 slots");
+    if (n->uploaded) return fail(SPDNN_E_STATE, "plans are on the device already: set the window before the features");
+    n->plan_window = slots;
+    return SPDNN_OK;
+}
+
+int spdnn_get_plan_memory(const spdnn_net* n, int* window, int64_t* device_bytes, int64_t* pinned_bytes) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (!n->uploaded) return fail(SPDNN_E_STATE, "plans are not on the device yet");
+    int64_t total = 0;
+    for (const PlanLayout& y : n->lay) total += (int64_t)y.bytes;
+    const bool st = plans_streamed(n);
+    if (window) *window = st ? n->plan_window : 0;
+    if (device_bytes) *device_bytes = st ? (int64_t)n->plan_window * (int64_t)n->slot_bytes : total;
+    if (pinned_bytes) *pinned_bytes = st ? total : 0;
+    return SPDNN_OK;
+}
+
 int spdnn_get_layer_plan(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
     if (!n || !out) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
@@ -792,7 +962,7 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
             HIPCHK(hipMemcpyAsync(stage, rowmajor + (size_t)r0 * N, (size_t)real * N * 4, hipMemcpyHostToDevice,
                                   n->stream));
         // rows >= real inside the chunk are written as zero by the kernel (nrows = real)
-        HIPCHK(launch_pack_rows(stage, n->F, n->dl[0].in_pos, N, r0, (int)std::max<int64_t>(real, 1), n->rl,
+        HIPCHK(launch_pack_rows(stage, n->F, n->d_lab, N, r0, (int)std::max<int64_t>(real, 1), n->rl,
                                 n->d_nonfinite, n->stream));
         HIPCHK(hipStreamSynchronize(n->stream));  // the staging buffer is reused by the next chunk
     }
@@ -1016,7 +1186,9 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     const bool have_counts = fused_count || scan_count;
     if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
     int fuse = opt.fuse_layers ? opt.fuse_layers : n->default_fuse;
-    if (scan_count || fuse < 2) fuse = 1;
+    if (scan_count || fuse < 2 || plans_streamed(n)) fuse = 1;  // a fused launch needs all its plans resident
+    if (plans_streamed(n))
+        for (int l = first; l <= last && l < first + n->plan_window; ++l) HIPCHK(plan_fetch(n, l));
 
     // Pruning never waits for the launch it just made: the host looks at the counts of the launch
     // `lookahead` launches back (already finished in steady state).  Counts only go down
@@ -1088,6 +1260,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         n->stamp += c;
         if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
         if (c == 1) {
+            HIPCHK(plan_acquire(n, l));
             if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
             HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr,
                                 shape, seglen));
@@ -1097,6 +1270,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 int rc = resolve_trials(n, 3);
                 if (rc) return rc;
             }
+            HIPCHK(plan_release(n, l));
         } else {
             ChainLaunch ch{};
             ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
@@ -1166,6 +1340,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
+    if (plans_streamed(n)) HIPCHK(hipStreamSynchronize(n->copy_stream));
     {
         int rc = resolve_trials(n, 0);
         if (rc) return rc;
@@ -1251,7 +1426,8 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
     if (out_buf.alloc((size_t)chunk * (size_t)n->N * 4) != hipSuccess) return fail(SPDNN_E_NOMEM, "out of device memory");
     int32_t* d_phys = phys_buf.as<int32_t>();
     float* d_out = out_buf.as<float>();
-    const int32_t* lab = labelling_dev(n, n->cur_layer);
+    const int32_t* lab = nullptr;
+    HIPCHK(labelling_dev(n, n->cur_layer, &lab));
     for (int i0 = 0; i0 < nrows; i0 += chunk) {
         const int m = std::min(chunk, nrows - i0);
         HIPCHK(hipMemcpyAsync(d_phys, phys.data() + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream));

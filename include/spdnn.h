@@ -162,6 +162,23 @@ int spdnn_inspect(spdnn_net* net);
  * emit the general kernel for every layer.  Must be called before the first layer is set. */
 int spdnn_set_force_kernel(spdnn_net* net, int kernel);
 
+/* Streamed plans, for networks whose plans should not (or do not) all stay in device memory: the
+ * device holds `slots` plan-sized slots (2..64; 0 = every plan resident, the default), all plans
+ * stay in pinned host memory, and a second stream copies the plan of layer l + slots into the slot
+ * of layer l as soon as layer l has finished, under the layers in between.  This is the double
+ * buffer of src/microbenchmark/out_memory.cu:318-327 (two weight/index buffers) and :367-386 (copy
+ * of layer l+1 on a memory stream while layer l runs), with events between the two streams instead
+ * of that loop's host synchronisation per layer.  Results are the same as with resident plans;
+ * launches that fuse several layers are not used.  Call before the features are handed over
+ * (SPDNN_E_STATE afterwards; spdnn_inspect after a layer change opens the choice again).  A window
+ * that is not smaller than the layer count leaves the plans resident.  Environment default:
+ * SPDNN_PLAN_WINDOW. */
+int spdnn_set_plan_window(spdnn_net* net, int slots);
+
+/* Where the plans are once they are uploaded: window (0 = resident), bytes of device memory they
+ * occupy, bytes of pinned host memory behind them (0 when resident). */
+int spdnn_get_plan_memory(const spdnn_net* net, int* window, int64_t* device_bytes, int64_t* pinned_bytes);
+
 int spdnn_get_layer_plan(const spdnn_net* net, int layer, spdnn_layer_plan* out);
 
 /* Host view of a BAND plan, for verification: position of every input neuron along the band

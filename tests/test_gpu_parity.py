@@ -197,6 +197,57 @@ def test_other_row_block_sizes(gc, orc, rl, monkeypatch):
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 
 
+@pytest.mark.parametrize("window", [2, 3])
+def test_streamed_plans(gc, orc, window, monkeypatch):
+    """Plans streamed through a window of device slots: same results as the oracle (and as resident
+    plans), in one run, in continued runs and when run again from the start."""
+    from helpers import hub_block_csr, radix_like_csr
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+    N, B = 1024, 700
+    rng = np.random.default_rng(40 + window)
+    layers = [orc.gen_layer_csr(3, 0, N), radix_like_csr(rng, N, 16, "general"), orc.gen_layer_csr(3, 2, N),
+              hub_block_csr(rng, N, "pow2"), orc.gen_layer_csr(3, 4, N),
+              sort_rows(random_csr(rng, N, rng.integers(1, 20, size=N), "general")),
+              radix_like_csr(rng, N, 512, "uniform"), orc.gen_layer_csr(3, 7, N), orc.gen_layer_csr(3, 8, N)]
+    L = len(layers)
+    feats = orc.gen_features(3, N, 0, B, 0.10, 0.6)
+    rows = np.arange(B, dtype=np.int32)
+    for prune in (False, True):
+        print("window", window, "prune", prune, flush=True)
+        ref = orc.infer(feats, layers, -0.2, prune=False, keep={L - 1})
+        with gc.Network(N, B, L, bias=-0.2) as net:
+            net.set_plan_window(window)
+            for l, csr in enumerate(layers):
+                net.set_layer_csr(l, *csr)
+            net.inspect()
+            kernels = {net.layer_plan(l).kernel for l in range(L)}
+            assert kernels == {gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER}
+            net.set_features_dense(feats)
+            w, dev_bytes, pinned = net.plan_memory()
+            assert w == window and pinned > dev_bytes > 0
+            with pytest.raises(gc.SpdnnError):
+                net.set_plan_window(0)       # too late: the plans are uploaded
+            for attempt in range(2):         # the second run starts with the slots as the first left them
+                r = net.run(prune=prune, collect_counts=True)
+                assert np.array_equal(net.categories(), ref["active_ids"][L - 1])
+                assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
+                for l in range(L):
+                    assert net.active_count(l) == len(ref["active_ids"][l])
+            _layer_by_layer(gc, orc, net, layers, feats, prune=prune)
+            # three layers, then the rest
+            net.run(prune=prune, first_layer=0, n_layers=3)
+            net.run(prune=prune, first_layer=3)
+            assert np.array_equal(net.categories(), ref["active_ids"][L - 1])
+            assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
+    # a window as long as the network leaves the plans resident
+    with gc.Network(N, B, 2, bias=-0.2) as net:
+        net.set_plan_window(2)
+        net.synth_layers(3)
+        net.inspect()
+        net.synth_features(3, B)
+        assert net.plan_memory()[0] == 0 and net.plan_memory()[2] == 0
+
+
 def test_wider_layers(gc, orc):
     """N=4096 and N=16384 at a few layers, rows sampled."""
     for N, bias in ((4096, -0.35), (16384, -0.4)):

@@ -370,6 +370,15 @@ def test_argument_and_state_errors(gc, orc):
         bad_ptr[3] = bad_ptr[2] - 1
         with pytest.raises(gc.SpdnnError):
             net.set_layer_csr(0, bad_ptr, good[1], good[2])
+        for slots in (1, -2, 65):                   # the plan window is 0 or 2..64 slots
+            with pytest.raises(gc.SpdnnError) as e:
+                net.set_plan_window(slots)
+            assert e.value.code == E_ARG
+        net.set_plan_window(2)
+        net.set_plan_window(0)
+        with pytest.raises(gc.SpdnnError) as e:
+            net.plan_memory()                       # nothing uploaded
+        assert e.value.code == E_STATE
         net.set_layer_csr(0, *good)
         with pytest.raises(gc.SpdnnError) as e:
             net.inspect()                           # layer 1 missing
