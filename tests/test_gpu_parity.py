@@ -439,6 +439,29 @@ def test_block_kernel_radix_like_layers(gc, orc, values, chains, monkeypatch):
             assert np.array_equal(net.categories(), ref["categories"])
 
 
+@pytest.mark.parametrize("N,strides", [(4096, (16, 256, 2048)), (65536, (16, 1024, 32768))])
+def test_radix_like_layers_at_challenge_widths(gc, orc, N, strides):
+    """RadiX-Net-like layers (two 16-wide input runs per group of 16 outputs, first, middle and last
+    stride of the width, behind random relabellings) at N=4096 and at the headline width: walked
+    as run chains by the band kernel under the default settings, bit-equal to the oracle."""
+    from helpers import radix_like_csr
+    B = 300
+    print("radix-like N=%d strides %s" % (N, strides), flush=True)
+    rng = np.random.default_rng(N)
+    layers = [radix_like_csr(rng, N, st, "uniform") for st in strides]
+    L = len(layers)
+    feats = (rng.uniform(0, 2, size=(B, N)) * (rng.random((B, N)) < 0.3)).astype(np.float32)
+    with gc.Network(N, B, L, bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        for l in range(L):
+            p = net.layer_plan(l)
+            assert p.kernel == gc.KERNEL_BAND and p.band_halo == 32
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=True)
+
+
 @pytest.mark.parametrize("N,B,L,bias", [(4096, 60000, 6, -0.35), (16384, 60000, 4, -0.4), (65536, 60000, 3, -0.45)])
 def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
     """The wider configurations at full batch, features generated on the device with
