@@ -13,8 +13,8 @@ by the library's seeded generator).  Reported on ONE JSON line:
   roofline     band-walk kernel: algorithmic bytes per launch (8*B*N + 8*nnz + 4*(N+1)) over the
                average launch duration measured with HIP events on the library's stream, against
                the 8 TB/s HBM peak.
-  cpu_baseline the CPU oracle (oracle/) timed on this box's host cores on a bounded row sample
-               of layer 0 of the same workload.
+  cpu_baseline the CPU oracle (oracle/) timed on this box's host cores on a bounded sample of the
+               same workload (the first layers, chained, on the first rows).
   literal      the run as configured (pruning on): edges/s as defined, layers actually launched,
                per-layer active rows; and the parity gate of a row sample against the oracle.
 """
@@ -55,6 +55,7 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="override the batch (quick runs)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
+    ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
     ap.add_argument("--survivor-check", type=int, default=0, metavar="ROWS",
                     help="extra (slow): features with densities up to 0.7 so that rows survive every layer; "
@@ -132,24 +133,26 @@ def main():
         rows = args.cpu_rows or max(256, min(B, int(7.0e10 * max(cores, 1) / 16 / (N * 32.0))) // 256 * 256)
         rows = min(rows, B)
         feats = orc.gen_features(seed, N, 0, rows, 0.10, 0.25)
-        csr0 = orc.gen_layer_csr(seed, 0, N)
-        t0 = time.perf_counter()
-        y1, act1 = orc.layer(feats, csr0, bias)
-        t_cpu = time.perf_counter() - t0
-        cpu = {"value": rows * float(nnz_layer) / t_cpu, "unit": "edges/s", "cores": cores, "kind": "port",
-               "sample": "layer 0 of the same workload on rows 0..%d (%.1f s)" % (rows - 1, t_cpu)}
-        # parity: first three layers of the sample rows, per-layer active ids and activations
+        # timed: the first layers of the same workload, chained, on the sample rows (every row kept,
+        # as in the sustained run); the first three of them are the parity reference below
+        n_cpu = min(L, args.cpu_layers)
+        n_check = min(L, 3)
         ref_ids, ref_y = [], []
         y, gid = feats, np.arange(rows, dtype=np.int32)
-        n_check = min(L, 3)
-        for l in range(n_check):
-            if l == 0:
-                yo, act = y1, act1
-            else:
-                yo, act = orc.layer(y, orc.gen_layer_csr(seed, l, N), bias)
-            ref_ids.append(gid[act != 0].copy())
-            ref_y.append((gid.copy(), yo))
+        t_cpu = 0.0
+        for l in range(max(n_cpu, n_check)):
+            csr = orc.gen_layer_csr(seed, l, N)
+            t0 = time.perf_counter()
+            yo, act = orc.layer(y, csr, bias)
+            if l < n_cpu:
+                t_cpu += time.perf_counter() - t0
+            if l < n_check:
+                ref_ids.append(gid[act != 0].copy())
+                ref_y.append((gid.copy(), yo))
             y = yo
+        cpu = {"value": rows * float(nnz_layer) * n_cpu / t_cpu, "unit": "edges/s", "cores": cores, "kind": "port",
+               "sample": "layers 0..%d of the same workload on rows 0..%d, every row kept (%.1f s)"
+                         % (n_cpu - 1, rows - 1, t_cpu)}
         ok_ids, ok_y, max_abs = True, True, 0.0
         sample = np.arange(rows, dtype=np.int32)
         for l in range(n_check):
