@@ -70,6 +70,7 @@ def load_library():
         "spdnn_synth_layer_csr": ([C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_float, _i32p, _i32p, _f32p], C.c_int),
         "spdnn_inspect": ([vp], C.c_int),
         "spdnn_set_force_kernel": ([vp, C.c_int], C.c_int),
+        "spdnn_load_layers_tsv": ([vp, C.c_char_p, C.c_int, C.c_int], C.c_int),
         "spdnn_set_plan_window": ([vp, C.c_int], C.c_int),
         "spdnn_get_plan_memory": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_layer_plan": ([vp, C.c_int, C.POINTER(LayerPlan)], C.c_int),
@@ -204,6 +205,11 @@ class Network:
 
     def load_layer_tsv(self, layer, path):
         _check(self._lib.spdnn_load_layer_tsv(self._h, layer, path.encode()))
+
+    def load_layers_tsv(self, data_dir, first=0, count=None):
+        """Layers [first, first+count) from <data_dir>/neuron<N>/n<N>-l<l+1>.tsv, parsed in parallel."""
+        count = self.layers - first if count is None else count
+        _check(self._lib.spdnn_load_layers_tsv(self._h, str(data_dir).encode(), first, count))
 
     def load_layers_bin(self, path, first=0, count=None, nnz_per_layer=0):
         count = self.layers - first if count is None else count

@@ -101,11 +101,12 @@ int main(int argc, char** argv) {
 
     double t0 = now_s();
     if (from_files) {
-        for (int l = 0; l < layer; ++l) {
-            CHECK(spdnn_weight_file_name(data.c_str(), neuron, l, wname, sizeof(wname)));
-            CHECK(spdnn_load_layer_tsv(net, l, wname));
-            if (!quiet) printf("[%s] to CSR success!\n", wname);
-        }
+        CHECK(spdnn_load_layers_tsv(net, data.c_str(), 0, layer));   // parsed by the inspector's worker threads
+        if (!quiet)
+            for (int l = 0; l < layer; ++l) {
+                CHECK(spdnn_weight_file_name(data.c_str(), neuron, l, wname, sizeof(wname)));
+                printf("[%s] to CSR success!\n", wname);
+            }
     } else if (from_bin) {
         CHECK(spdnn_load_layers_bin(net, weight_bin.c_str(), 0, layer, 0));
         if (!quiet) printf("[%s] to CSR success!\n", weight_bin.c_str());

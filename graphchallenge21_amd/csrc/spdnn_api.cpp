@@ -752,6 +752,49 @@ int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
     return spdnn_set_layer_csr(n, layer, rp.data(), cc.data(), vv.data());
 }
 
+int spdnn_load_layers_tsv(spdnn_net* n, const char* data_dir, int first, int count) {
+    if (!n || !data_dir) return fail(SPDNN_E_ARG, "NULL argument");
+    if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
+    n->pool->wait_all();
+    std::fill(n->pending.begin(), n->pending.end(), 0);
+    n->inspected = false;
+    const int N = n->N, force = n->force_kernel;
+    const bool fma_ok = n->fma_ok;
+    const std::string dir = data_dir;
+    // every worker parses, validates and inspects whole layers; the first failure by layer number is reported
+    auto errs = std::make_shared<std::vector<std::string>>((size_t)count);
+    auto codes = std::make_shared<std::vector<int>>((size_t)count, SPDNN_OK);
+    for (int l = first; l < first + count; ++l) {
+        LayerPlan* plan = &n->layers[(size_t)l];
+        const size_t k = (size_t)(l - first);
+        n->pool->submit([=] {
+            const std::string path = dir + "/neuron" + std::to_string(N) + "/n" + std::to_string(N) + "-l" +
+                                     std::to_string(l + 1) + ".tsv";
+            std::vector<int32_t> rp, cc, rp2, cc2;
+            std::vector<float> vv, vv2;
+            std::string err;
+            if (!read_weight_tsv_csr(path, N, rp, cc, vv, err)) {
+                (*errs)[k] = err;
+                (*codes)[k] = SPDNN_E_IO;
+                plan->set = false;
+                return;
+            }
+            err = normalize_csr(N, rp.data(), cc.data(), vv.data(), rp2, cc2, vv2);
+            if (!err.empty()) {
+                (*errs)[k] = path + ": " + err;
+                (*codes)[k] = SPDNN_E_ARG;
+                plan->set = false;
+                return;
+            }
+            inspect_layer(N, rp2, cc2, vv2, force, fma_ok, *plan);
+        });
+    }
+    n->pool->wait_all();
+    for (size_t k = 0; k < (size_t)count; ++k)
+        if ((*codes)[k] != SPDNN_OK) return fail((*codes)[k], (*errs)[k]);
+    return SPDNN_OK;
+}
+
 int spdnn_load_layers_bin(spdnn_net* n, const char* path, int first, int count, int64_t nnz_per_layer) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");

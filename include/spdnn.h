@@ -129,6 +129,13 @@ int spdnn_set_layer_csr(spdnn_net* net, int layer, const int32_t* rowptr, const 
  * COOMatrix(file, 1, false) (src/utils/matrix.h:255-282), and sets the layer. */
 int spdnn_load_layer_tsv(spdnn_net* net, int layer, const char* path);
 
+/* Reads layers [first, first+count) from <data_dir>/neuron<N>/n<N>-l<layer+1>.tsv (the names of
+ * get_weight_file_name, src/network.cpp:14-19) - the loop of src/network.cpp:96-120, with the
+ * files parsed, checked and inspected side by side on the library's worker threads (one layer of
+ * N=65536 is 39 MB of text, the 1920 of them 75 GB).  Returns when every layer is done; the first
+ * failing layer by number is reported (SPDNN_E_IO names the file) and stays unset. */
+int spdnn_load_layers_tsv(spdnn_net* net, const char* data_dir, int first, int count);
+
 /* Reads layers [first, first+count) from a packed binary weight file "neuron<N>.bin" as the
  * reference's library benchmarks consume it (readweights, benchmark/cusparse/cusparse.cu:318-358):
  * one record per layer of int32 row[nnz], int32 col[nnz], float32 val[nnz], 1-based, with

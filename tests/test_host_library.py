@@ -287,6 +287,46 @@ def test_tsv_layer_through_the_library(gc, orc, tmp_path):
         assert net.layer_plan(0).nnz == 64 * 8
 
 
+def test_tsv_directory_loaded_in_parallel(gc, orc, tmp_path):
+    """All layers of a data directory (the reference's file names) in one call: same plans as the
+    layers handed over one by one; a missing or broken file is reported by name."""
+    n, L = 256, 7
+    d = tmp_path / ("neuron%d" % n)
+    d.mkdir()
+    layers = [orc.gen_layer_csr(8, l, n, 8) for l in range(L)]
+    rng = np.random.default_rng(1)
+    for l, (rowptr, col, val) in enumerate(layers):
+        lines = ["%d\t%d\t%.9g\n" % (col[e] + 1, j + 1, val[e]) for j in range(n) for e in range(rowptr[j], rowptr[j + 1])]
+        rng.shuffle(lines)
+        (d / ("n%d-l%d.tsv" % (n, l + 1))).write_text("".join(lines))
+    with gc.Network(n, 4, L, bias=-0.3) as a, gc.Network(n, 4, L, bias=-0.3) as b:
+        a.load_layers_tsv(tmp_path)
+        for l, csr in enumerate(layers):
+            b.set_layer_csr(l, *csr)
+        a.inspect()
+        b.inspect()
+        for l in range(L):
+            for x, y in zip(a.band_plan(l), b.band_plan(l)):
+                assert np.array_equal(x, y)
+            assert np.array_equal(a.layer_dst(l), b.layer_dst(l))
+        # a part of the range, then a file that is not there, then one with a bad index
+        a.load_layers_tsv(tmp_path, first=2, count=3)
+        a.inspect()
+        (d / ("n%d-l4.tsv" % n)).unlink()
+        with pytest.raises(gc.SpdnnError) as e:
+            a.load_layers_tsv(tmp_path)
+        assert e.value.code == 3 and "n256-l4.tsv" in e.value.message
+        with pytest.raises(gc.SpdnnError) as e:
+            a.inspect()                                 # layer 3 stayed unset
+        assert e.value.code == 2
+        (d / ("n%d-l4.tsv" % n)).write_text("1\t%d\t0.5\n" % (n + 1))
+        with pytest.raises(gc.SpdnnError) as e:
+            a.load_layers_tsv(tmp_path)
+        assert "n256-l4.tsv" in e.value.message
+        with pytest.raises(gc.SpdnnError):
+            a.load_layers_tsv(tmp_path, first=5, count=4)
+
+
 def _write_weights_bin(path, layers):
     """Packed weight file in the layout readweights of the reference's library benchmark reads
     (benchmark/cusparse/cusparse.cu:340-347): per layer row[], col[], val[], 1-based, row = output."""
