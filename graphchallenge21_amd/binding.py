@@ -71,6 +71,7 @@ def load_library():
         "spdnn_inspect": ([vp], C.c_int),
         "spdnn_set_force_kernel": ([vp, C.c_int], C.c_int),
         "spdnn_load_layers_tsv": ([vp, C.c_char_p, C.c_int, C.c_int], C.c_int),
+        "spdnn_read_features_tsv": ([C.c_char_p, C.c_int, C.c_int, _f32p, C.POINTER(C.c_int64)], C.c_int),
         "spdnn_set_plan_window": ([vp, C.c_int], C.c_int),
         "spdnn_get_plan_memory": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_layer_plan": ([vp, C.c_int, C.POINTER(LayerPlan)], C.c_int),
@@ -143,6 +144,14 @@ def synth_features_host(seed, neuron, row_begin, nrows, dmin=0.10, dmax=0.25):
     out = np.empty((nrows, neuron), np.float32)
     _check(load_library().spdnn_synth_features_host(seed, neuron, row_begin, nrows, dmin, dmax, out))
     return out
+
+
+def read_features_tsv(path, neuron, batch):
+    """(dense batch x neuron fp32, lines stored) of a feature file in the challenge format."""
+    out = np.empty((batch, neuron), np.float32)
+    kept = C.c_int64()
+    _check(load_library().spdnn_read_features_tsv(str(path).encode(), neuron, batch, out, C.byref(kept)))
+    return out, kept.value
 
 
 def measure_copy_bandwidth(nbytes=1 << 30, reps=10):

@@ -1026,8 +1026,18 @@ int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
     std::vector<float> dense;
     std::string err;
     int64_t kept = 0;
-    if (!read_features_tsv_dense(path, n->N, batch, dense, &kept, err)) return fail(SPDNN_E_IO, err);
+    if (!read_features_tsv_dense(path, n->N, batch, dense, &kept, err, host_threads())) return fail(SPDNN_E_IO, err);
     return spdnn_set_features_dense(n, dense.data(), batch);
+}
+
+int spdnn_read_features_tsv(const char* path, int neuron, int batch, float* rowmajor, int64_t* kept) {
+    if (!path || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
+    if (neuron < 1 || batch < 1) return fail(SPDNN_E_ARG, "neuron and batch must be positive");
+    std::string err;
+    int64_t k = 0;
+    if (!read_features_tsv_into(path, neuron, batch, rowmajor, &k, err, host_threads())) return fail(SPDNN_E_IO, err);
+    if (kept) *kept = k;
+    return SPDNN_OK;
 }
 
 int spdnn_load_features_bin(spdnn_net* n, const char* path, int batch) {

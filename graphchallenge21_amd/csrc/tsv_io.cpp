@@ -1,8 +1,12 @@
 #include "tsv_io.hpp"
 
+#include <algorithm>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
+#include <thread>
 
 namespace spdnn {
 
@@ -59,18 +63,129 @@ bool read_weight_tsv_csr(const std::string& path, int N, std::vector<int32_t>& r
     return true;
 }
 
-bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
-                             int64_t* kept, std::string& err) {
-    std::vector<Triple> t;
-    if (!read_triples(path, t, err)) return false;
-    dense.assign((size_t)batch * (size_t)N, 0.0f);
-    int64_t k = 0;
-    for (const Triple& e : t) {
-        if (e.a > batch) continue;  // network.cpp:46: rows beyond the batch are skipped
-        if (e.a < 1 || e.b < 1 || e.b > N) { err = "feature index out of range in " + path; return false; }
-        dense[(size_t)(e.a - 1) * (size_t)N + (size_t)(e.b - 1)] = e.v;
-        ++k;
+namespace {
+
+// One "int int float" line starting at p (leading whitespace skipped).  Returns 1 and advances p,
+// 0 at the end of the data, -1 on a malformed line.  Plain decimal integers in the value column
+// (the challenge's feature files hold 1s) skip strtof.
+inline int parse_triple(const char*& p, const char* end, long& a, long& b, float& v) {
+    auto skip = [&] { while (p < end && (*p == ' ' || *p == '\t' || *p == '\n' || *p == '\r')) ++p; };
+    auto integer = [&](long& out) -> bool {
+        skip();
+        const char* q = p;
+        bool neg = false;
+        if (q < end && (*q == '-' || *q == '+')) { neg = *q == '-'; ++q; }
+        const char* d0 = q;
+        long x = 0;
+        while (q < end && *q >= '0' && *q <= '9' && q - d0 < 18) { x = x * 10 + (*q - '0'); ++q; }
+        if (q == d0) return false;
+        out = neg ? -x : x;
+        p = q;
+        return true;
+    };
+    skip();
+    if (p >= end) return 0;
+    if (!integer(a)) return -1;
+    if (!integer(b)) return -1;
+    skip();
+    const char* q = p;
+    long iv = 0;
+    const char* save = p;
+    if (integer(iv) && (p >= end || *p == '\n' || *p == '\r' || *p == ' ' || *p == '\t') && p - save <= 7) {
+        v = (float)iv;   // up to 6 digits and a sign: exact in fp32
+        return 1;
     }
+    p = q;
+    char* e;
+    v = strtof(p, &e);   // the buffer ends in a 0 byte, so this stops inside it
+    if (e == p) return -1;
+    p = e;
+    return 1;
+}
+
+}  // namespace
+
+bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
+                             int64_t* kept, std::string& err, int threads) {
+    dense.resize((size_t)batch * (size_t)N);
+    return read_features_tsv_into(path, N, batch, dense.data(), kept, err, threads);
+}
+
+bool read_features_tsv_into(const std::string& path, int N, int batch, float* dense, int64_t* kept,
+                            std::string& err, int threads) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) { err = "FILE:" + path + " does not exists."; return false; }
+    fseeko(f, 0, SEEK_END);
+    const int64_t sz = (int64_t)ftello(f);
+    fseeko(f, 0, SEEK_SET);
+    std::vector<char> buf((size_t)sz + 1);
+    if (sz > 0 && fread(buf.data(), 1, (size_t)sz, f) != (size_t)sz) { fclose(f); err = "short read: " + path; return false; }
+    fclose(f);
+    buf[(size_t)sz] = 0;
+    const char* base = buf.data();
+    const char* end = base + sz;
+
+    // Parts of the file, cut at line starts, are parsed side by side and stored straight into the
+    // dense matrix.  The reference keeps the LAST line of an entry that occurs twice
+    // (network.cpp:47); the parts cannot know each other's order, so a bitmap notes which entries
+    // were stored and, should any entry come twice, the file is gone through again in order.
+    const int T = (int)std::max<int64_t>(1, std::min<int64_t>(threads, sz / (1 << 20) + 1));
+    std::vector<const char*> cut((size_t)T + 1, end);
+    cut[0] = base;
+    for (int t = 1; t < T; ++t) {
+        const char* p = base + sz / T * t;
+        while (p < end && *p != '\n') ++p;
+        cut[(size_t)t] = p < end ? p + 1 : end;
+    }
+    const size_t total = (size_t)batch * (size_t)N;
+    std::fill(dense, dense + total, 0.0f);
+    std::vector<std::atomic<uint64_t>> seen(T > 1 ? (total + 63) / 64 : 0);
+    for (auto& w : seen) w.store(0, std::memory_order_relaxed);
+    std::vector<int64_t> kept_t((size_t)T, 0);
+    std::vector<int> state((size_t)T, 0);  // 1 = malformed, 2 = index out of range
+    std::atomic<bool> twice{false};
+    auto parse_range = [&](const char* p, const char* e, bool mark, int64_t& k_out, int& state_out) {
+        int64_t k = 0;
+        long a, b;
+        float v;
+        state_out = 0;
+        for (;;) {
+            const int r = parse_triple(p, e, a, b, v);
+            if (r == 0) break;
+            if (r < 0) { state_out = 1; break; }
+            if (a > batch) continue;  // network.cpp:46: rows beyond the batch are skipped
+            if (a < 1 || b < 1 || b > N) { state_out = 2; break; }
+            const size_t at = (size_t)(a - 1) * (size_t)N + (size_t)(b - 1);
+            dense[at] = v;
+            if (mark) {
+                const uint64_t bit = 1ull << (at & 63);
+                if (seen[at >> 6].fetch_or(bit, std::memory_order_relaxed) & bit) twice.store(true, std::memory_order_relaxed);
+            }
+            ++k;
+        }
+        k_out = k;
+    };
+    {
+        std::vector<std::thread> th;
+        for (int t = 1; t < T; ++t)
+            th.emplace_back([&, t] { parse_range(cut[(size_t)t], cut[(size_t)t + 1], true, kept_t[(size_t)t], state[(size_t)t]); });
+        parse_range(cut[0], cut[1], T > 1, kept_t[0], state[0]);
+        for (std::thread& x : th) x.join();
+    }
+    bool again = twice.load();
+    for (int t = 0; t < T; ++t) again |= state[(size_t)t] != 0;
+    if (again && T > 1) {
+        // an entry set twice, or a part that did not parse (a triple may straddle a line end, which
+        // the reference's stream extraction accepts): the whole file once more, in order, as one part
+        for (int t = 1; t < T; ++t) kept_t[(size_t)t] = 0;
+        parse_range(base, end, false, kept_t[0], state[0]);
+        for (int t = 1; t < T; ++t) state[(size_t)t] = 0;
+    }
+    // every other part's state is clear here: either nothing was wrong or the file was gone through as one part
+    if (state[0] == 1) { err = "malformed line in " + path; return false; }
+    if (state[0] == 2) { err = "feature index out of range in " + path; return false; }
+    int64_t k = 0;
+    for (int t = 0; t < T; ++t) k += kept_t[(size_t)t];
     if (kept) *kept = k;
     return true;
 }

@@ -19,9 +19,13 @@ bool read_weight_tsv_csr(const std::string& path, int N, std::vector<int32_t>& r
                          std::vector<int32_t>& col, std::vector<float>& val, std::string& err);
 
 // Feature file "row neuron value" (1-based) -> dense row-major batch x N; rows beyond batch are
-// skipped like the reference does.  *kept receives the number of entries stored.
+// skipped like the reference does, of an entry that occurs twice the last line counts.  *kept
+// receives the number of lines stored.  The file is parsed by up to `threads` threads.
 bool read_features_tsv_dense(const std::string& path, int N, int batch, std::vector<float>& dense,
-                             int64_t* kept, std::string& err);
+                             int64_t* kept, std::string& err, int threads = 1);
+// the same into memory of the caller (batch * N floats)
+bool read_features_tsv_into(const std::string& path, int N, int batch, float* dense, int64_t* kept,
+                            std::string& err, int threads = 1);
 
 // Packed binary files as the reference's library benchmarks consume them
 // (benchmark/cusparse/cusparse.cu:318-383): "neuron{N}.bin" holds one record per layer of

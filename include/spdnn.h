@@ -231,6 +231,13 @@ int spdnn_set_features_dense(spdnn_net* net, const float* rowmajor, int batch);
  * are skipped): read_input, src/network.cpp:33-54. */
 int spdnn_load_features_tsv(spdnn_net* net, const char* path, int batch);
 
+/* The same file into host memory: read_input of src/network.cpp:33-54 itself (dense batch x neuron,
+ * row-major, zero where the file says nothing; of an entry that occurs twice the last line counts,
+ * network.cpp:47).  *kept (may be NULL) receives the number of lines stored.  The file is parsed in
+ * parts by the library's host threads.  Host only: needs no device and no handle.  After a failure
+ * the contents of rowmajor are unspecified. */
+int spdnn_read_features_tsv(const char* path, int neuron, int batch, float* rowmajor, int64_t* kept);
+
 /* Packed binary features "sparse-images-<N>.bin" (readinput, benchmark/cusparse/cusparse.cu:361-383):
  * int32 row[] = neuron, int32 col[] = image, float32 val[], 1-based, the entry count being the file
  * size / 12; images beyond batch are skipped. */

@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from helpers import hub_block_csr, radix_like_csr, random_csr, sort_rows
+from helpers import hub_block_csr, radix_like_csr, random_csr, same_floats, sort_rows
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GOLD = os.path.join(ROOT, "tests", "golden")
@@ -325,6 +325,48 @@ def test_tsv_directory_loaded_in_parallel(gc, orc, tmp_path):
         assert "n256-l4.tsv" in e.value.message
         with pytest.raises(gc.SpdnnError):
             a.load_layers_tsv(tmp_path, first=5, count=4)
+
+
+def test_features_tsv_parsed_in_parts(gc, orc, tmp_path):
+    """A feature file of several MiB (parsed in parts by several threads) against the oracle's
+    reader: shuffled lines, rows beyond the batch, values with fractions and exponents; then the
+    same file with an entry set twice far apart (the later line must win) and with a triple that
+    straddles a line end (accepted, as stream extraction does)."""
+    N, B = 512, 1500
+    rng = np.random.default_rng(5)
+    flat = rng.choice(N * (B + 100), size=400000, replace=False)
+    rows, cols = flat // N + 1, flat % N + 1
+    vals = np.where(rng.random(len(flat)) < 0.7, 1.0, rng.uniform(0.001, 30.0, len(flat))).astype(np.float32)
+    lines = ["%d\t%d\t%s\n" % (r, c, "1" if v == 1.0 else ("%.6e" % v if i % 3 else "%.7f" % v))
+             for i, (r, c, v) in enumerate(zip(rows.tolist(), cols.tolist(), vals.tolist()))]
+    p = tmp_path / "sparse-images-512.tsv"
+    p.write_text("".join(lines))
+    assert p.stat().st_size > (4 << 20)
+    want, want_kept = orc.read_features_tsv(str(p), N, B)
+    got, kept = gc.read_features_tsv(p, N, B)
+    assert kept == want_kept == int((rows <= B).sum())
+    assert same_floats(got, want)
+    # the first entry again at the very end with another value, and a triple broken over two lines
+    r0, c0 = int(rows[rows <= B][0]), int(cols[rows <= B][0])
+    p.write_text("".join(lines) + "%d\t%d\t7.25\n" % (r0, c0) + "3\t9\n2.5\n")
+    want, want_kept = orc.read_features_tsv(str(p), N, B)
+    got, kept = gc.read_features_tsv(p, N, B)
+    assert got[r0 - 1, c0 - 1] == np.float32(7.25) and got[2, 8] == np.float32(2.5)
+    assert kept == want_kept and same_floats(got, want)
+    # errors: an index out of range in the middle, a line that is no triple, a missing file
+    bad = list(lines)
+    bad[len(bad) // 2] = "5\t%d\t1\n" % (N + 1)
+    p.write_text("".join(bad))
+    with pytest.raises(gc.SpdnnError) as e:
+        gc.read_features_tsv(p, N, B)
+    assert e.value.code == 3 and "out of range" in e.value.message
+    bad[len(bad) // 2] = "5\tx\t1\n"
+    p.write_text("".join(bad))
+    with pytest.raises(gc.SpdnnError) as e:
+        gc.read_features_tsv(p, N, B)
+    assert "malformed" in e.value.message
+    with pytest.raises(gc.SpdnnError):
+        gc.read_features_tsv(tmp_path / "nothing.tsv", N, B)
 
 
 def _write_weights_bin(path, layers):
