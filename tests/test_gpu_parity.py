@@ -722,6 +722,67 @@ def test_handle_lifecycle(gc, orc):
     assert free0 - free1 < (64 << 20), "device memory not returned: %d bytes" % (free0 - free1)
 
 
+def test_randomized_shapes_and_options(gc, orc, monkeypatch):
+    """400 seeded random cases: widths 32 ... 4096 (also not powers of two), batches around the
+    row-block sizes, 1-6 layers of every class and weight mode, bias below, at and above zero,
+    pruning, fused launches, streamed plans, all row-block sizes - final categories, activations
+    and per-layer counts against the oracle, on a first run and on a repeated one."""
+    from helpers import hub_block_csr, radix_like_csr
+    for case in range(400):
+        rng = np.random.default_rng(770000 + case)
+        N = int(rng.choice([32, 48, 64, 100, 256, 384, 1000, 1024, 2048, 4096]))
+        B = int(rng.choice([1, 3, 63, 64, 65, 255, 257, 700, 1500]))
+        L = int(rng.integers(1, 7))
+        rl = int(rng.choice([1, 2, 4]))
+        bias = float(rng.choice([-0.3, -0.05, 0.0, 0.1]))
+        prune = bool(rng.integers(0, 2)) and bias <= 0
+        fuse = int(rng.choice([0, 0, 3]))
+        window = int(rng.choice([0, 0, 2, 3]))
+        minchain = int(rng.choice([256, 4096]))
+        values = str(rng.choice(["uniform", "pow2", "general"]))
+        layers, kinds = [], []
+        for l in range(L):
+            kind = str(rng.choice(["circ", "circ", "gather", "radix", "hub"]))
+            if kind in ("radix", "hub") and (N % 32 or N < 64):
+                kind = "circ"
+            if kind == "circ":
+                rp, c, v = orc.gen_layer_csr(int(rng.integers(0, 1000)), l, N, int(min(N, rng.integers(1, 41))))
+                if values == "pow2":
+                    v = np.ldexp(1.0, rng.integers(-6, -2, size=len(v))).astype(np.float32)
+                elif values == "general":
+                    v = rng.uniform(-0.1, 0.2, size=len(v)).astype(np.float32)
+                layers.append((rp, c, v))
+            elif kind == "gather":
+                layers.append(sort_rows(random_csr(rng, N, rng.integers(0, min(N, 24), size=N), values)))
+            elif kind == "radix":
+                layers.append(radix_like_csr(rng, N, int(16 * rng.integers(1, N // 16)), values))
+            else:
+                layers.append(hub_block_csr(rng, N, values))
+            kinds.append(kind)
+        dens = float(rng.choice([0.05, 0.3, 0.8]))
+        feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < dens)).astype(np.float32)
+        what = dict(case=case, N=N, B=B, L=L, rl=rl, bias=bias, prune=prune, fuse=fuse, window=window,
+                    minchain=minchain, values=values, kinds=kinds, dens=dens)
+        if case % 50 == 0:
+            print("random case", what, flush=True)
+        monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
+        monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
+        ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
+        with gc.Network(N, B, L, bias=bias) as net:
+            if window:
+                net.set_plan_window(window)
+            for l, csr in enumerate(layers):
+                net.set_layer_csr(l, *csr)
+            net.inspect()
+            net.set_features_dense(feats)
+            for rep in range(2):
+                net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert np.array_equal(net.categories(), ref["active_ids"][L - 1]), what
+                assert same_floats(net.activations(np.arange(B, dtype=np.int32)), ref["kept"][L - 1][1]), what
+                if bias <= 0:
+                    assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]], what
+
+
 def test_zero_bias_into_the_denormal_range(gc, orc):
     """Bias 0 and power-of-two weights of 1/16, 8 per row: activations halve (at least) per layer and
     reach the denormal range after ~120 layers, where a product no longer is exact.  The library
