@@ -783,6 +783,90 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
                     assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]], what
 
 
+def test_randomized_call_sequences(gc, orc, monkeypatch):
+    """150 seeded random sequences of calls on one handle - new features of another batch size,
+    whole runs (pruned or not, fused, different compaction thresholds), continued partial runs,
+    activations of random rows, categories, a replaced layer with a new inspection - followed on
+    the side by the oracle, layer by layer."""
+    from helpers import hub_block_csr, radix_like_csr
+
+    def make_layer(rng, N, l, values):
+        kind = str(rng.choice(["circ", "circ", "gather", "radix", "hub"]))
+        if kind == "circ":
+            rp, c, v = orc.gen_layer_csr(int(rng.integers(0, 1000)), l, N, int(min(N, rng.integers(2, 41))))
+            if values == "pow2":
+                v = np.ldexp(1.0, rng.integers(-5, -2, size=len(v))).astype(np.float32)
+            elif values == "general":
+                v = rng.uniform(-0.05, 0.2, size=len(v)).astype(np.float32)
+            return rp, c, v
+        if kind == "gather":
+            return sort_rows(random_csr(rng, N, rng.integers(0, min(N, 24), size=N), values))
+        if kind == "radix":
+            return radix_like_csr(rng, N, int(16 * rng.integers(1, N // 16)), values)
+        return hub_block_csr(rng, N, values)
+
+    for case in range(150):
+        rng = np.random.default_rng(880000 + case)
+        N = int(rng.choice([64, 256, 1024, 2048]))
+        maxB = int(rng.choice([65, 300, 1100]))
+        L = int(rng.integers(2, 9))
+        bias = float(rng.choice([-0.3, -0.1, 0.0]))
+        values = str(rng.choice(["uniform", "pow2", "general"]))
+        window = int(rng.choice([0, 0, 2]))
+        monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(int(rng.choice([1, 2, 4]))))
+        monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(int(rng.choice([256, 4096]))))
+        layers = [make_layer(rng, N, l, values) for l in range(L)]
+        what = dict(case=case, N=N, maxB=maxB, L=L, bias=bias, values=values, window=window)
+        if case % 25 == 0:
+            print("random sequence", what, flush=True)
+        log = []
+        with gc.Network(N, maxB, L, bias=bias) as net:
+            if window:
+                net.set_plan_window(window)
+            for l, csr in enumerate(layers):
+                net.set_layer_csr(l, *csr)
+            net.inspect()
+            feats, done, y = None, 0, None     # done = layers applied to y so far
+            for step in range(int(rng.integers(4, 14))):
+                op = str(rng.choice(["feat", "run_all", "run_part", "acts", "cats", "replace", "threshold"]))
+                if feats is None:
+                    op = "feat"
+                log.append(op)
+                if op == "feat":
+                    B = int(rng.integers(1, maxB + 1))
+                    dens = float(rng.choice([0.02, 0.2, 0.7]))
+                    feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < dens)).astype(np.float32)
+                    net.set_features_dense(feats)
+                    y, done = feats.copy(), 0
+                elif op in ("run_all", "threshold"):
+                    thr = float(rng.choice([0.0, 0.3, 1.0])) if op == "threshold" else 0.0
+                    net.run(prune=bool(rng.integers(0, 2)), collect_counts=True, fuse_layers=int(rng.choice([0, 2, 4])),
+                            compact_threshold=thr)
+                    ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
+                    y, done = ref["kept"][L - 1][1], L
+                    assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]], (what, log)
+                elif op == "run_part":
+                    if done >= L:
+                        y, done = feats.copy(), 0
+                    nl = int(rng.integers(1, L - done + 1))
+                    net.run(prune=bool(rng.integers(0, 2)), first_layer=done, n_layers=nl, collect_counts=True)
+                    for l in range(done, done + nl):
+                        y, _ = orc.layer(y, layers[l], bias)
+                    done += nl
+                elif op == "acts":
+                    B = feats.shape[0]
+                    rows = rng.permutation(B)[: int(rng.integers(1, B + 1))].astype(np.int32)
+                    assert same_floats(net.activations(rows), y[rows]), (what, log)
+                elif op == "cats" and done > 0:
+                    assert np.array_equal(net.categories(), np.nonzero((y != 0).any(axis=1))[0]), (what, log)
+                elif op == "replace":
+                    l = int(rng.integers(0, L))
+                    layers[l] = make_layer(rng, N, l, values)
+                    net.set_layer_csr(l, *layers[l])
+                    net.inspect()
+                    feats = None
+
+
 def test_zero_bias_into_the_denormal_range(gc, orc):
     """Bias 0 and power-of-two weights of 1/16, 8 per row: activations halve (at least) per layer and
     reach the denormal range after ~120 layers, where a product no longer is exact.  The library
