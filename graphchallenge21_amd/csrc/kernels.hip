@@ -57,9 +57,34 @@ template <int WMODE> __device__ __forceinline__ float mac(float acc, float x, fl
     return __builtin_fmaf(x, w, acc);
 }
 
-// End of a layer kernel: stamp the rows of this lane that produced a nonzero output.  With a
-// counter, the first wave to stamp a row (atomic exchange) also counts it, one atomic add per
-// wave, so the number of active rows after the layer needs no separate pass.
+// Running "largest output so far" of a row.  Outputs are clamped to [0, clamp], so comparing the
+// bit patterns as signed integers orders them like the floats (one v_max_i32, no NaN handling).
+__device__ __forceinline__ float nz_merge(float nz, float y) {
+    return __int_as_float(max(__float_as_int(nz), __float_as_int(y)));
+}
+
+// End of a layer kernel: stamp the rows that produced a nonzero output.  With a counter, the
+// first to stamp a row (atomic exchange) also counts it, one atomic add per wave, so the number
+// of active rows after the layer needs no separate pass.  A row that already carries the stamp
+// (another wave or workgroup of this launch was first) is left alone: every workgroup that works
+// on a row block stamps the same 64*RL words, and exchanges on one address are served one after
+// the other, which on a small batch would take longer than the layer itself.
+__device__ __forceinline__ int stamp_one(int32_t* __restrict__ active, size_t row, int stamp) {
+    if (__atomic_load_n(&active[row], __ATOMIC_RELAXED) == stamp) return 0;
+    return atomicExch(&active[row], stamp) != stamp ? 1 : 0;
+}
+
+__device__ __forceinline__ void count_newly(int newly, int32_t* __restrict__ count_out) {
+    newly += __shfl_down(newly, 32, 64);
+    newly += __shfl_down(newly, 16, 64);
+    newly += __shfl_down(newly, 8, 64);
+    newly += __shfl_down(newly, 4, 64);
+    newly += __shfl_down(newly, 2, 64);
+    newly += __shfl_down(newly, 1, 64);
+    if ((threadIdx.x & 63) == 0 && newly > 0) atomicAdd(count_out, newly);
+}
+
+// one wave, lane = RL rows starting at row0
 template <int RL>
 __device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict__ active, size_t row0,
                                            int stamp, int32_t* __restrict__ count_out) {
@@ -72,14 +97,35 @@ __device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict_
     int newly = 0;
 #pragma unroll
     for (int q = 0; q < RL; ++q)
-        if (nz[q] > 0.0f) newly += (atomicExch(&active[row0 + q], stamp) != stamp) ? 1 : 0;
-    newly += __shfl_down(newly, 32, 64);
-    newly += __shfl_down(newly, 16, 64);
-    newly += __shfl_down(newly, 8, 64);
-    newly += __shfl_down(newly, 4, 64);
-    newly += __shfl_down(newly, 2, 64);
-    newly += __shfl_down(newly, 1, 64);
-    if ((threadIdx.x & 63) == 0 && newly > 0) atomicAdd(count_out, newly);
+        if (nz[q] > 0.0f) newly += stamp_one(active, row0 + q, stamp);
+    count_newly(newly, count_out);
+}
+
+// a workgroup of NW waves that all worked on the same 64*RL rows (block_row0 = first row): the
+// waves' results are merged through LDS (free after the last barrier of the band walk) and every
+// row is stamped by one thread.  Contains a barrier; the caller must put another one before the
+// LDS is written again.
+template <int RL, int NW>
+__device__ __forceinline__ void stamp_rows_workgroup(const float* nz, unsigned char* smem,
+                                                     int32_t* __restrict__ active, size_t block_row0, int stamp,
+                                                     int32_t* __restrict__ count_out) {
+    constexpr int RB = 64 * RL;
+    float* s = reinterpret_cast<float*>(smem);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int q = 0; q < RL; ++q) s[wave * RB + lane * RL + q] = nz[q];
+    __syncthreads();
+    int newly = 0;
+    for (int r = threadIdx.x; r < RB; r += NW * 64) {
+        float m = s[r];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) m = nz_merge(m, s[w * RB + r]);
+        if (m > 0.0f) {
+            if (count_out) newly += stamp_one(active, block_row0 + r, stamp);
+            else active[block_row0 + r] = stamp;
+        }
+    }
+    if (count_out) count_newly(newly, count_out);
 }
 
 // Block-level pruning: true if no row of this lane's row block was stamped by the previous layer
@@ -98,11 +144,6 @@ __device__ __forceinline__ bool block_is_dead(const int32_t* active, size_t row0
     return __syncthreads_or(any) == 0;
 }
 
-// Running "largest output so far" of a row.  Outputs are clamped to [0, clamp], so comparing the
-// bit patterns as signed integers orders them like the floats (one v_max_i32, no NaN handling).
-__device__ __forceinline__ float nz_merge(float nz, float y) {
-    return __int_as_float(max(__float_as_int(nz), __float_as_int(y)));
-}
 
 __device__ __forceinline__ float relu_clamp(float y, float clampv) {
     // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
@@ -403,7 +444,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
     band_walk_body<RL, NW, OPW, RING, WMODE, KT>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
                                                  pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz);
-    stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp, count_out);
+    stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, count_out);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -445,8 +486,8 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
         band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
                                                      lay.halo, 0, N, lay.wu, bias, clampv, smem, nz);
-        stamp_rows<RL>(nz, active, (size_t)rb * RB + (threadIdx.x & 63) * RL, stamp0 + j,
-                       count_out ? count_out + j : nullptr);
+        stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
+                                     count_out ? count_out + j : nullptr);
         int any = 0;
 #pragma unroll
         for (int q = 0; q < RL; ++q) any |= (nz[q] > 0.0f) ? 1 : 0;
