@@ -25,6 +25,16 @@ struct Feat {
     explicit operator bool() const { return half[0] != nullptr; }
 };
 
+// Counts of an earlier launch handed to the host: the first workgroup of a layer kernel copies
+// src[0..n) (device counters, final because that launch has finished) to dst (pinned host memory,
+// where the host polls them).  A copy command between two layer launches would cost more than
+// a small layer itself.
+struct Publish {
+    const int32_t* src = nullptr;
+    int32_t* dst = nullptr;
+    int n = 0;
+};
+
 struct BandLaunch {
     Feat yin;                // input buffer (row-block layout, labelled by the layer's band order)
     Feat yout;               // output buffer (labelled for the next layer through dst)
@@ -44,6 +54,7 @@ struct BandLaunch {
     int n_cu;
     int shape = -1;          // tile shape (see launch_band); < 0 = default
     int seglen = 0;          // band positions per workgroup; 0 = heuristic
+    Publish publish;
 };
 
 struct GatherLaunch {
@@ -59,6 +70,7 @@ struct GatherLaunch {
     int prev_stamp = 0;      // as in BandLaunch
     int wmode;               // 1 fma (exact products), 2 mul then add
     float bias, clampv;
+    Publish publish;
 };
 
 hipError_t launch_band(const BandLaunch& a, hipStream_t s);
@@ -85,6 +97,7 @@ struct BlockLaunch {
     int N, ngroups, nblk, stamp, prev_stamp, rl, wmode;
     int full;                // 1: every group has exactly 32 shared inputs
     float wu, bias, clampv;
+    Publish publish;
 };
 hipError_t launch_block(const BlockLaunch& a, hipStream_t s);
 
@@ -112,6 +125,7 @@ struct ChainLaunch {
     int unrolled;                 // every layer of the chain fits the unrolled path (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
     float bias, clampv;
+    Publish publish;
 };
 hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s);
 

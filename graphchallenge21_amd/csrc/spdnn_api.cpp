@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <condition_variable>
 #include <cstdio>
@@ -188,7 +189,6 @@ struct spdnn_net {
     int32_t* h_count = nullptr;  // pinned
     int32_t* d_counts = nullptr; // per-layer active-row counters (device)
     int32_t* h_counts = nullptr; // pinned mirror
-    std::vector<hipEvent_t> ev_count;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     std::vector<hipEvent_t> ev_layer;
 
@@ -232,14 +232,12 @@ void release_device_base(spdnn_net* n) {
     if (n->h_counts) hipHostFree(n->h_counts);
     n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
     n->d_count = n->d_nonfinite = n->d_counts = n->h_count = n->h_counts = nullptr;
-    for (hipEvent_t e : n->ev_count) hipEventDestroy(e);
     for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
     for (const spdnn_net::Trial& t : n->trials) { hipEventDestroy(t.e0); hipEventDestroy(t.e1); }
     for (hipEvent_t e : n->ev_free) hipEventDestroy(e);
     n->trials.clear();
     n->ev_free.clear();
     n->exploring.clear();
-    n->ev_count.clear();
     n->ev_layer.clear();
     if (n->ev_start) hipEventDestroy(n->ev_start);
     if (n->ev_stop) hipEventDestroy(n->ev_stop);
@@ -1173,7 +1171,7 @@ static int resolve_trials(spdnn_net* n, size_t keep) {
 }
 
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
-                               int prev_stamp, int32_t* count_out, int shape, int seglen) {
+                               int prev_stamp, int32_t* count_out, int shape, int seglen, const Publish& pub) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
@@ -1182,6 +1180,7 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         a.prev_stamp = prev_stamp;
         a.shape = shape;
         a.seglen = seglen;
+        a.publish = pub;
         return launch_band(a, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_BLOCK) {
@@ -1190,13 +1189,41 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         b.active = n->d_active; b.count_out = count_out; b.N = n->N; b.ngroups = p.ngroups; b.nblk = nblk;
         b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = p.wmode; b.full = p.blk_full ? 1 : 0;
         b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
+        b.publish = pub;
         return launch_block(b, n->stream);
     }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
     g.active = n->d_active; g.count_out = count_out; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
     g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv;
+    g.publish = pub;
     return launch_gather(g, n->stream);
+}
+
+// Waits until the counts of layers [l0, l0+c) have arrived in pinned host memory (written there
+// by the first workgroup of the launch after theirs; -1 = not yet).  Normally they are there or
+// arrive within microseconds.  The stream itself is asked only after 100 ms without them, so that
+// a failed launch ends the wait: asking puts a marker into the queue, which between two short
+// layers costs as much as a layer.
+static int wait_counts(spdnn_net* n, int l0, int c) {
+    volatile int32_t* h = n->h_counts;
+    for (int j = l0; j < l0 + c; ++j) {
+        if (h[j] >= 0) continue;
+        auto t0 = std::chrono::steady_clock::now();
+        for (unsigned spins = 1; h[j] < 0; ++spins) {
+            if ((spins & 4095) != 0) continue;
+            const auto now = std::chrono::steady_clock::now();
+            if (now - t0 < std::chrono::milliseconds(100)) continue;
+            t0 = now;
+            const hipError_t q = hipStreamQuery(n->stream);
+            if (q == hipSuccess) {
+                if (h[j] < 0) return fail(SPDNN_E_DEVICE, "layer counts were not handed over");
+            } else if (q != hipErrorNotReady) {
+                return fail(SPDNN_E_DEVICE, std::string("hipStreamQuery: ") + hipGetErrorString(q));
+            }
+        }
+    }
+    return SPDNN_OK;
 }
 
 int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
@@ -1223,11 +1250,6 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             n->ev_layer.push_back(e);
         }
     }
-    while (n->ev_count.size() < (size_t)n->L) {
-        hipEvent_t e;
-        HIPCHK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
-        n->ev_count.push_back(e);
-    }
     const int first = opt.first_layer, last = first + nl - 1;
     for (int l = first; l <= last; ++l) { n->counts[(size_t)l] = -1; n->layer_ms[(size_t)l] = 0.0f; }
 
@@ -1247,7 +1269,21 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     // `lookahead` launches back (already finished in steady state).  Counts only go down
     // (bias <= 0), so an older count is a safe upper bound for sizing a repack, and a zero count
     // means every later layer is all zero.
-    const size_t lookahead = 2;
+    // The counts reach the host without a copy command between the layers: the first workgroup of
+    // every layer launch stores the previous launch's counts into pinned host memory.
+    // How far behind depends on how long a layer runs: behind a long layer one launch in the
+    // queue keeps the device busy and a compaction should not come late; behind short layers the
+    // host needs several launches of lead or the device waits for it.
+    auto lookahead_for = [&](int carried_rows) -> size_t {
+        const double us = (double)carried_rows * (double)n->N * 8.0 / 4.0e6 + 6.0;  // at 4 TB/s, plus launch
+        return us > 200.0 ? 1 : us > 50.0 ? 2 : us > 20.0 ? 4 : 8;
+    };
+    const bool polled = have_counts && opt.prune;
+    if (polled) {
+        volatile int32_t* h = n->h_counts;
+        for (int l = first; l <= last; ++l) h[l] = -1;
+    }
+    Publish pub{};
     struct Rec { int l0, c; };
     std::vector<Rec> recs;
     size_t processed = 0;
@@ -1316,7 +1352,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             HIPCHK(plan_acquire(n, l));
             if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
             HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr,
-                                shape, seglen));
+                                shape, seglen, pub));
             if (trial) {
                 HIPCHK(hipEventRecord(tr.e1, n->stream));
                 n->trials.push_back(tr);
@@ -1332,6 +1368,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = opt.prune ? 1 : 0;
             ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
             ch.bias = n->bias; ch.clampv = n->clampv;
+            ch.publish = pub;
             HIPCHK(launch_band_chain(ch, n->stream));
             for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
         }
@@ -1346,17 +1383,20 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                                       n->d_alive_gid, n->stream));
             HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
         }
-        if (have_counts) {
-            HIPCHK(hipMemcpyAsync(n->h_counts + l, n->d_counts + l, (size_t)c * 4, hipMemcpyDeviceToHost, n->stream));
-            HIPCHK(hipEventRecord(n->ev_count[(size_t)(l + c - 1)], n->stream));
+        if (polled) {  // the next launch hands these counts over; the host looks at them two launches late
+            pub.src = n->d_counts + l;
+            pub.dst = n->h_counts + l;
+            pub.n = c;
             recs.push_back({l, c});
         }
         l += c;
         if (!opt.prune) continue;
 
+        const size_t lookahead = lookahead_for(n->carried);
         while (recs.size() - processed > lookahead && !dead) {
             const Rec rc = recs[processed++];
-            HIPCHK(hipEventSynchronize(n->ev_count[(size_t)(rc.l0 + rc.c - 1)]));
+            const int wrc = wait_counts(n, rc.l0, rc.c);
+            if (wrc) return wrc;
             for (int j = rc.l0; j < rc.l0 + rc.c && !dead; ++j) {
                 newest_count = n->h_counts[j];
                 if (newest_count == 0) dead = true;
@@ -1392,6 +1432,9 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         n->alive_list_valid = true;
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));
+    if (have_counts && last_launched >= first)   // all of them once more (the last launch's have no launch after it)
+        HIPCHK(hipMemcpyAsync(n->h_counts + first, n->d_counts + first, (size_t)(last_launched - first + 1) * 4,
+                              hipMemcpyDeviceToHost, n->stream));
     HIPCHK(hipStreamSynchronize(n->stream));
     if (plans_streamed(n)) HIPCHK(hipStreamSynchronize(n->copy_stream));
     {

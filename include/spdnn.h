@@ -255,9 +255,10 @@ int spdnn_default_run_options(spdnn_run_options* opt);
 
 /* Runs layers [first_layer, first_layer + n_layers): the layer loop of
  * test_benchmark_graph_challenge (all_network.cu:333-519).  The layer kernels count the rows they
- * leave active; with prune the host reads the count of the layer two launches back (never the
- * one just launched), stops launching once it is zero, and queues the on-device scan + repack
- * when few enough rows are left.  One host synchronisation, at the end. */
+ * leave active; with prune the host reads the count of a layer one to eight launches back (never
+ * the one just launched; the following launch stores it into pinned host memory), stops launching
+ * once it is zero, and queues the on-device scan + repack when few enough rows are left.  One host
+ * synchronisation, at the end. */
 int spdnn_run(spdnn_net* net, const spdnn_run_options* opt, spdnn_run_result* result);
 
 /* Active-row count recorded after layer `layer` of the last run (collect_counts or prune),
