@@ -144,7 +144,7 @@ __device__ __forceinline__ bool block_is_dead(const int32_t* active, size_t row0
     int any = 0;
 #pragma unroll
     for (int q = 0; q < RL; ++q) {
-        const int a = __atomic_load_n(&active[row0 + q], __ATOMIC_RELAXED);
+        const int a = active[row0 + q];  // either value means alive, so no ordering against this launch's stamps is needed
         any |= (a == prev_stamp || a == stamp) ? 1 : 0;
     }
     return __syncthreads_or(any) == 0;
