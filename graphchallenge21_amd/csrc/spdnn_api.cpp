@@ -1383,7 +1383,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                                       n->d_alive_gid, n->stream));
             HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
         }
-        if (polled) {  // the next launch hands these counts over; the host looks at them two launches late
+        if (polled) {  // the next launch hands these counts over; the host looks at them a few launches late
             pub.src = n->d_counts + l;
             pub.dst = n->h_counts + l;
             pub.n = c;
