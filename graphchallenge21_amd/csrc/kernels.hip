@@ -63,17 +63,15 @@ __device__ __forceinline__ float nz_merge(float nz, float y) {
     return __int_as_float(max(__float_as_int(nz), __float_as_int(y)));
 }
 
-// End of a layer kernel: stamp the rows that produced a nonzero output.  With a counter, the
-// first to stamp a row (atomic exchange) also counts it, one atomic add per wave, so the number
-// of active rows after the layer needs no separate pass.  A row that already carries the stamp
-// (another wave or workgroup of this launch was first) is left alone: every workgroup that works
-// on a row block stamps the same 64*RL words, and exchanges on one address are served one after
-// the other, which on a small batch would take longer than the layer itself.
-__device__ __forceinline__ int stamp_one(int32_t* __restrict__ active, size_t row, int stamp) {
-    if (__atomic_load_n(&active[row], __ATOMIC_RELAXED) == stamp) return 0;
-    return atomicExch(&active[row], stamp) != stamp ? 1 : 0;
-}
-
+// Row stamps and row counts.  At its end a layer kernel writes `stamp` (the number of its launch)
+// into active[row] of every row with a nonzero output: plain stores - all workgroups that work on
+// a row block store the same value, so no order among them matters.  How many rows a layer left
+// active is counted by the kernel of the NEXT layer: at its start the first workgroup of every row
+// block looks at the block's 64*RL stamps anyway (for pruning) and adds the number of rows that
+// carry the previous launch's stamp to that layer's counter, one atomic add per row block.
+// (Counting while stamping needs an atomic exchange per row and workgroup to find out who is
+// first; exchanges on one address are served one after the other, and on a small batch they took
+// longer than the layer itself.)
 __device__ __forceinline__ void count_newly(int newly, int32_t* __restrict__ count_out) {
     newly += __shfl_down(newly, 32, 64);
     newly += __shfl_down(newly, 16, 64);
@@ -86,25 +84,17 @@ __device__ __forceinline__ void count_newly(int newly, int32_t* __restrict__ cou
 
 // one wave, lane = RL rows starting at row0
 template <int RL>
-__device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict__ active, size_t row0,
-                                           int stamp, int32_t* __restrict__ count_out) {
-    if (count_out == nullptr) {
-#pragma unroll
-        for (int q = 0; q < RL; ++q)
-            if (nz[q] > 0.0f) active[row0 + q] = stamp;
-        return;
-    }
-    int newly = 0;
+__device__ __forceinline__ void stamp_rows(const float* nz, int32_t* __restrict__ active, size_t row0, int stamp) {
 #pragma unroll
     for (int q = 0; q < RL; ++q)
-        if (nz[q] > 0.0f) newly += stamp_one(active, row0 + q, stamp);
-    count_newly(newly, count_out);
+        if (nz[q] > 0.0f) active[row0 + q] = stamp;
 }
 
 // a workgroup of NW waves that all worked on the same 64*RL rows (block_row0 = first row): the
 // waves' results are merged through LDS (free after the last barrier of the band walk) and every
-// row is stamped by one thread.  Contains a barrier; the caller must put another one before the
-// LDS is written again.
+// row is stamped by one thread.  count_out (may be nullptr) is for a workgroup that is the only
+// one to work on its row block: it then also counts the rows it stamps.  Contains a barrier; the
+// caller must put another one before the LDS is written again.
 template <int RL, int NW>
 __device__ __forceinline__ void stamp_rows_workgroup(const float* nz, unsigned char* smem,
                                                      int32_t* __restrict__ active, size_t block_row0, int stamp,
@@ -121,8 +111,8 @@ __device__ __forceinline__ void stamp_rows_workgroup(const float* nz, unsigned c
 #pragma unroll
         for (int w = 1; w < NW; ++w) m = nz_merge(m, s[w * RB + r]);
         if (m > 0.0f) {
-            if (count_out) newly += stamp_one(active, block_row0 + r, stamp);
-            else active[block_row0 + r] = stamp;
+            active[block_row0 + r] = stamp;
+            ++newly;
         }
     }
     if (count_out) count_newly(newly, count_out);
@@ -134,20 +124,29 @@ __device__ __forceinline__ void publish_counts(const Publish& p) {
         for (int i = threadIdx.x; i < p.n; i += blockDim.x) p.dst[i] = p.src[i];
 }
 
-// Block-level pruning: true if no row of this lane's row block was stamped by the previous layer
-// (prev_stamp 0 = do not check).  Another workgroup of the same launch (a different band segment
-// of the same row block) may already have re-stamped rows with this launch's stamp; such rows
-// were alive too.  Uniform over the workgroup; contains a barrier.
+// Start of a layer kernel (every wave of the workgroup calls it; lane = RL rows from row0, so a
+// wave sees its whole row block).  prev_stamp is the stamp of the layer before (0 = none valid).
+// Rows that carry it were left active by that layer; so were rows that already carry this
+// launch's stamp (another workgroup was faster: with bias <= 0 only a row that was active can be
+// active again).  The number of such rows does not depend on when a wave looks.
+//  - counter (wave 0 of the row block's first workgroup) adds it to count_prev, if given;
+//  - with check_dead the return value says that the row block has no active row, i.e. that its
+//    outputs are all zero and the workgroup can leave (uniform over the workgroup; has a barrier).
 template <int RL>
-__device__ __forceinline__ bool block_is_dead(const int32_t* active, size_t row0, int prev_stamp, int stamp) {
+__device__ __forceinline__ bool enter_row_block(const int32_t* active, size_t row0, int prev_stamp, int stamp,
+                                                int check_dead, int32_t* __restrict__ count_prev, bool counter) {
     if (prev_stamp == 0) return false;
-    int any = 0;
+    const bool counts = counter && count_prev != nullptr;
+    if (!check_dead && !counts) return false;
+    int alive = 0;
 #pragma unroll
     for (int q = 0; q < RL; ++q) {
-        const int a = active[row0 + q];  // either value means alive, so no ordering against this launch's stamps is needed
-        any |= (a == prev_stamp || a == stamp) ? 1 : 0;
+        const int a = active[row0 + q];
+        alive += (int)__popcll(__ballot((a == prev_stamp || a == stamp) ? 1 : 0));
     }
-    return __syncthreads_or(any) == 0;
+    if (counts && (threadIdx.x & 63) == 0 && alive > 0) atomicAdd(count_prev, alive);
+    if (!check_dead) return false;
+    return __syncthreads_or(alive) == 0;
 }
 
 
@@ -434,8 +433,8 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_out, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
-    float wu, float bias, float clampv, Publish pub, int nblk) {
+    int32_t* __restrict__ count_prev, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
+    int check_dead, float wu, float bias, float clampv, Publish pub, int nblk) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     publish_counts(pub);
@@ -446,13 +445,15 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     const int vb = blockIdx.y * seglen;
     const int ve = min(N, vb + seglen);
     const size_t blkf = (size_t)N * RB;
-    if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp)) return;
+    if (enter_row_block<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp, check_dead, count_prev,
+                            blockIdx.y == 0 && threadIdx.x < 64))
+        return;
     float nz[RL];
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
     band_walk_body<RL, NW, OPW, RING, WMODE, KT>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
                                                  pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz);
-    stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, count_out);
+    stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, nullptr);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -476,14 +477,16 @@ struct ChainLayer {
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
     const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int stamp0, int prev_stamp,
-    int stop_when_dead, float bias, float clampv, Publish pub) {
+    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int32_t* __restrict__ count_prev, int N,
+    int stamp0, int prev_stamp, int check_dead, int stop_when_dead, float bias, float clampv, Publish pub) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     publish_counts(pub);
     const int rb = blockIdx.x;
     const size_t blkf = (size_t)N * RB;
-    if (block_is_dead<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp0)) return;
+    if (enter_row_block<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp0, check_dead, count_prev,
+                            threadIdx.x < 64))
+        return;
     float* const block_a = block_base(buf_a, rb, blkf);
     float* const block_c = block_base(buf_c, rb, blkf);
     const float* in = block_base(first_in, rb, blkf);
@@ -519,15 +522,17 @@ template <int RL, int WMODE>
 __global__ __launch_bounds__(256) void gather_kernel(
     Feat yin_all, Feat yout_all, const int32_t* __restrict__ cols,
     const int32_t* __restrict__ rowlen, const float* __restrict__ wv, const int32_t* __restrict__ dst,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int kmax, int opg, int stamp,
-    int prev_stamp, float bias, float clampv, Publish pub) {
+    int32_t* __restrict__ active, int32_t* __restrict__ count_prev, int N, int kmax, int opg, int stamp,
+    int prev_stamp, int check_dead, float bias, float clampv, Publish pub) {
     using V = typename VecOf<RL>::type;
     constexpr int RB = 64 * RL;
     publish_counts(pub);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rb = blockIdx.x;
-    if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
+    if (enter_row_block<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp, check_dead, count_prev,
+                            blockIdx.y == 0 && wave == 0))
+        return;
     const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
     float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
     const int loff = lane * RL;
@@ -562,7 +567,7 @@ __global__ __launch_bounds__(256) void gather_kernel(
         }
         *reinterpret_cast<V*>(yout + (size_t)dst[j] * RB + loff) = arr_to_vec<RL>(y);
     }
-    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -576,15 +581,17 @@ template <int RL, int WMODE, bool FULL>
 __global__ __launch_bounds__(256) void block_kernel(
     Feat yin_all, Feat yout_all, const int32_t* __restrict__ grp_cols,
     const int32_t* __restrict__ grp_cnt, const float* __restrict__ wv, const int32_t* __restrict__ dst,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int N, int ngroups, int gpw, int stamp,
-    int prev_stamp, float wu, float bias, float clampv, Publish pub) {
+    int32_t* __restrict__ active, int32_t* __restrict__ count_prev, int N, int ngroups, int gpw, int stamp,
+    int prev_stamp, int check_dead, float wu, float bias, float clampv, Publish pub) {
     using V = typename VecOf<RL>::type;
     constexpr int RB = 64 * RL;
     publish_counts(pub);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int rb = blockIdx.x;
-    if (block_is_dead<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp)) return;
+    if (enter_row_block<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp, check_dead, count_prev,
+                            blockIdx.y == 0 && wave == 0))
+        return;
     const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
     float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
     const int loff = lane * RL;
@@ -633,7 +640,7 @@ __global__ __launch_bounds__(256) void block_kernel(
             *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
         }
     }
-    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp, count_out);
+    stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -884,8 +891,8 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     const bool pad = a.nblk >= 3 && (a.nblk & 7) != 0 && (size_t)((a.nblk + 7) / 8) * block_bytes * 2 <= ((size_t)4 << 20);
     const int gx = pad ? (a.nblk + 7) / 8 * 8 : a.nblk;
     dim3 grid(gx, nseg), block(NW * 64);
-    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_out,
-                       a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.wu, a.bias, a.clampv, a.publish,
+    hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_prev,
+                       a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,
                        a.nblk);
     return hipGetLastError();
 }
@@ -994,8 +1001,8 @@ hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
         attr_done = true;
     }
     hipLaunchKernelGGL(kern, dim3(a.nblk), dim3(NW * 64), lds, s, reinterpret_cast<const ChainLayer*>(a.table),
-                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.N, a.stamp0,
-                       a.prev_stamp, a.stop_when_dead, a.bias, a.clampv, a.publish);
+                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.count_prev, a.N, a.stamp0,
+                       a.prev_stamp, a.check_dead, a.stop_when_dead, a.bias, a.clampv, a.publish);
     return hipGetLastError();
 }
 template <int RL, int NW, int OPW, int RING>
@@ -1039,7 +1046,7 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
     if (grid.y > 65535) return hipErrorInvalidValue;
 #define SPDNN_GATHER(RLv, WM)                                                                         \
     hipLaunchKernelGGL((gather_kernel<RLv, WM>), grid, block, 0, s, a.yin, a.yout, a.cols, a.rowlen,  \
-                       a.wv, a.dst, a.active, a.count_out, a.N, a.kmax, opg, a.stamp, a.prev_stamp, a.bias, a.clampv, \
+                       a.wv, a.dst, a.active, a.count_prev, a.N, a.kmax, opg, a.stamp, a.prev_stamp, a.check_dead, a.bias, a.clampv, \
                        a.publish)
     const bool exact = a.wmode != 2;
     switch (a.rl) {
@@ -1064,7 +1071,7 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {
     if (grid.y > 65535) return hipErrorInvalidValue;
 #define SPDNN_BLOCK(RLv, WM, FL)                                                                          \
     hipLaunchKernelGGL((block_kernel<RLv, WM, FL>), grid, block, 0, s, a.yin, a.yout, a.cols, a.cnt, a.wv, \
-                       a.dst, a.active, a.count_out, a.N, a.ngroups, gpw, a.stamp, a.prev_stamp, a.wu,     \
+                       a.dst, a.active, a.count_prev, a.N, a.ngroups, gpw, a.stamp, a.prev_stamp, a.check_dead, a.wu, \
                        a.bias, a.clampv, a.publish)
 #define SPDNN_BLOCK_WM(RLv)                                                                 \
     switch (a.wmode) {                                                                      \

@@ -44,11 +44,12 @@ struct BandLaunch {
                              // nullptr (uniform exact value)
     const int32_t* dst;      // [N] physical output column per band position
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
-    int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
+    int32_t* count_prev;     // device counter of the layer that stamped prev_stamp: this launch adds the rows that layer left active (may be nullptr)
     int N, K, nblk, stamp, rl;
     int steps, stride;       // merged steps per pair (K .. 2K); dwords per pair record (multiple of 4)
     int halo;                // input columns a segment needs before its first position: K-1 .. 32
-    int prev_stamp = 0;      // stamp of the previous layer: row blocks it left without an active row are skipped (0 = off)
+    int prev_stamp = 0;      // stamp of the previous layer if the row slots still carry it (0 = none)
+    int check_dead = 0;      // 1: row blocks the previous layer left without an active row are skipped
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
     int n_cu;
@@ -65,9 +66,10 @@ struct GatherLaunch {
     const float* wv;         // [N][kmax]
     const int32_t* dst;      // [N]
     int32_t* active;
-    int32_t* count_out;      // device counter of rows stamped by this launch (may be nullptr)
+    int32_t* count_prev;     // device counter of the layer that stamped prev_stamp: this launch adds the rows that layer left active (may be nullptr)
     int N, kmax, nblk, stamp, rl;
     int prev_stamp = 0;      // as in BandLaunch
+    int check_dead = 0;
     int wmode;               // 1 fma (exact products), 2 mul then add
     float bias, clampv;
     Publish publish;
@@ -93,8 +95,8 @@ struct BlockLaunch {
     const float* wv;         // [ngroups*16][32] weights, or nullptr (uniform exact value)
     const int32_t* dst;      // [ngroups*16] physical output column, -1 = unused slot
     int32_t* active;
-    int32_t* count_out;
-    int N, ngroups, nblk, stamp, prev_stamp, rl, wmode;
+    int32_t* count_prev;     // as in BandLaunch
+    int N, ngroups, nblk, stamp, prev_stamp, check_dead, rl, wmode;
     int full;                // 1: every group has exactly 32 shared inputs
     float wu, bias, clampv;
     Publish publish;
@@ -121,7 +123,8 @@ struct ChainLaunch {
     Feat buf_c;
     int32_t* active;
     int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
-    int N, K, nblk, stamp0, prev_stamp, rl, wmode;
+    int32_t* count_prev;          // as in BandLaunch, for the layer before the chain
+    int N, K, nblk, stamp0, prev_stamp, check_dead, rl, wmode;
     int unrolled;                 // every layer of the chain fits the unrolled path (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
     float bias, clampv;

@@ -1098,7 +1098,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
-    a.shape = -1; a.seglen = 0; a.count_out = nullptr; a.prev_stamp = 0;
+    a.shape = -1; a.seglen = 0; a.count_prev = nullptr; a.prev_stamp = 0; a.check_dead = 0;
     return a;
 }
 
@@ -1171,13 +1171,15 @@ static int resolve_trials(spdnn_net* n, size_t keep) {
 }
 
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
-                               int prev_stamp, int32_t* count_out, int shape, int seglen, const Publish& pub) {
+                               int prev_stamp, int check_dead, int32_t* count_prev, int shape, int seglen,
+                               const Publish& pub) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (p.kernel == SPDNN_KERNEL_BAND) {
         BandLaunch a = band_args(n, l, in, out, nblk, stamp);
-        a.count_out = count_out;
+        a.count_prev = count_prev;
         a.prev_stamp = prev_stamp;
+        a.check_dead = check_dead;
         a.shape = shape;
         a.seglen = seglen;
         a.publish = pub;
@@ -1186,7 +1188,7 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
     if (p.kernel == SPDNN_KERNEL_BLOCK) {
         BlockLaunch b{};
         b.yin = in; b.yout = out; b.cols = d.blk_cols; b.cnt = d.blk_cnt; b.wv = d.wv; b.dst = d.dst;
-        b.active = n->d_active; b.count_out = count_out; b.N = n->N; b.ngroups = p.ngroups; b.nblk = nblk;
+        b.active = n->d_active; b.count_prev = count_prev; b.check_dead = check_dead; b.N = n->N; b.ngroups = p.ngroups; b.nblk = nblk;
         b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = p.wmode; b.full = p.blk_full ? 1 : 0;
         b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
         b.publish = pub;
@@ -1194,7 +1196,7 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
     }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
-    g.active = n->d_active; g.count_out = count_out; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
+    g.active = n->d_active; g.count_prev = count_prev; g.check_dead = check_dead; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;
     g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv;
     g.publish = pub;
     return launch_gather(g, n->stream);
@@ -1294,6 +1296,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     int64_t newest_count = -1;
     bool dead = n->carried == 0;
     int last_launched = -1;
+    bool count_pending = false;  // the newest layer's rows have not been counted yet
 
     HIPCHK(hipEventRecord(n->ev_start, n->stream));
     for (int l = first; l <= last;) {
@@ -1316,7 +1319,12 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         }
         for (int j = 0; j < c; ++j) r.edges += (double)n->batch * (double)n->layers[(size_t)(l + j)].info.nnz;
         const int nblk = n->carried / n->RB;
-        const int prev_stamp = opt.prune ? n->last_stamp : 0;
+        // the layer before this launch, if the row slots still carry its stamps: its rows are
+        // counted by this launch (unless a chain or a scan has counted them already), and with
+        // pruning the row blocks it left without an active row are skipped
+        const int prev_stamp = n->last_stamp;
+        const int check_dead = opt.prune ? 1 : 0;
+        int32_t* const count_prev = (fused_count && count_pending && prev_stamp != 0) ? n->d_counts + (l - 1) : nullptr;
         const Feat in = n->cur;
         Feat out = (n->cur == n->A) ? n->C : n->A;
         // band tile shape and segment length: the record for this row-block count, else the next
@@ -1351,8 +1359,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         if (c == 1) {
             HIPCHK(plan_acquire(n, l));
             if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
-            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, fused_count ? n->d_counts + l : nullptr,
-                                shape, seglen, pub));
+            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, check_dead, count_prev, shape, seglen, pub));
             if (trial) {
                 HIPCHK(hipEventRecord(tr.e1, n->stream));
                 n->trials.push_back(tr);
@@ -1364,6 +1371,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             ChainLaunch ch{};
             ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
             ch.active = n->d_active; ch.count_out = fused_count ? n->d_counts + l : nullptr;
+            ch.count_prev = count_prev; ch.check_dead = check_dead;
             ch.N = n->N; ch.K = p.kmax; ch.nblk = nblk; ch.stamp0 = stamp0; ch.prev_stamp = prev_stamp;
             ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = opt.prune ? 1 : 0;
             ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
@@ -1383,16 +1391,21 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                                       n->d_alive_gid, n->stream));
             HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
         }
-        if (polled) {  // the next launch hands these counts over; the host looks at them a few launches late
-            pub.src = n->d_counts + l;
-            pub.dst = n->h_counts + l;
-            pub.n = c;
-            recs.push_back({l, c});
+        if (fused_count) {
+            // Counts that are final once this launch has finished: the previous layer's (counted at
+            // this launch's start) and, of a fused launch, its own layers'.  The next launch hands
+            // them to the host; this launch handed over the ones before (pub).
+            if (polled && pub.n > 0) recs.push_back({(int)(pub.src - n->d_counts), pub.n});
+            const int lo = count_prev ? l - 1 : l, hi = c == 1 ? l : l + c;
+            pub = Publish{};
+            if (polled && hi > lo) { pub.src = n->d_counts + lo; pub.dst = n->h_counts + lo; pub.n = hi - lo; }
+            count_pending = c == 1;  // a single layer's rows are counted by whatever comes next
         }
         l += c;
         if (!opt.prune) continue;
 
-        const size_t lookahead = lookahead_for(n->carried);
+        // a record is pushed when the launch that hands it over is queued, i.e. one launch late
+        const size_t lookahead = lookahead_for(n->carried) - 1;
         while (recs.size() - processed > lookahead && !dead) {
             const Rec rc = recs[processed++];
             const int wrc = wait_counts(n, rc.l0, rc.c);
@@ -1409,6 +1422,10 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 const Feat dstbuf = (n->cur == n->A) ? n->C : n->A;
                 HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count,
                                           n->d_alive_src, n->d_alive_gid, n->stream));
+                if (count_pending) {  // the scan has just counted the newest layer's rows
+                    HIPCHK(hipMemcpyAsync(n->d_counts + (l - 1), n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
+                    count_pending = false;
+                }
                 HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
                                      n->N, n->rl, nb, n->stream));
                 std::swap(n->d_gid, n->d_gid_tmp);
@@ -1429,6 +1446,8 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                                       n->d_alive_gid, n->stream));
         }
         HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
+        if (count_pending)  // no launch follows the last layer: the scan's count is its count
+            HIPCHK(hipMemcpyAsync(n->d_counts + last, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
         n->alive_list_valid = true;
     }
     HIPCHK(hipEventRecord(n->ev_stop, n->stream));

@@ -254,11 +254,11 @@ int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int6
 int spdnn_default_run_options(spdnn_run_options* opt);
 
 /* Runs layers [first_layer, first_layer + n_layers): the layer loop of
- * test_benchmark_graph_challenge (all_network.cu:333-519).  The layer kernels count the rows they
- * leave active; with prune the host reads the count of a layer one to eight launches back (never
- * the one just launched; the following launch stores it into pinned host memory), stops launching
- * once it is zero, and queues the on-device scan + repack when few enough rows are left.  One host
- * synchronisation, at the end. */
+ * test_benchmark_graph_challenge (all_network.cu:333-519).  Every layer kernel counts the rows
+ * the layer before it left active; with prune the host reads the count of a layer a few launches
+ * back (never of the one just launched; a following launch stores it into pinned host memory),
+ * stops launching once it is zero, and queues the on-device scan + repack when few enough rows
+ * are left.  One host synchronisation, at the end. */
 int spdnn_run(spdnn_net* net, const spdnn_run_options* opt, spdnn_run_result* result);
 
 /* Active-row count recorded after layer `layer` of the last run (collect_counts or prune),
