@@ -444,6 +444,28 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.ngroups = 0;
     plan.blk_cols.clear();
     plan.blk_cnt.clear();
+    plan.alt_ngroups = 0;
+    plan.alt_full = false;
+    plan.alt_cols.clear();
+    plan.alt_cnt.clear();
+    plan.alt_out_at.clear();
+    plan.alt_dst.clear();
+    if (band && halo == 32 && uniform && exact) {
+        // the BLOCK form of a run-chain layer, its columns in the band's input labelling
+        plan.alt_ngroups = (int)groups.size();
+        plan.alt_full = true;
+        plan.alt_cols.assign((size_t)plan.alt_ngroups * 32, 0);
+        plan.alt_cnt.resize((size_t)plan.alt_ngroups);
+        plan.alt_out_at.assign((size_t)plan.alt_ngroups * 16, -1);
+        for (int g = 0; g < plan.alt_ngroups; ++g) {
+            const int j0 = groups[(size_t)g][0];
+            const int len = rowptr[j0 + 1] - rowptr[j0];
+            plan.alt_cnt[(size_t)g] = len;
+            if (len != 32) plan.alt_full = false;
+            for (int k = 0; k < len; ++k) plan.alt_cols[(size_t)g * 32 + k] = plan.in_pos[(size_t)col[rowptr[j0] + k]];
+            for (size_t o = 0; o < groups[(size_t)g].size(); ++o) plan.alt_out_at[(size_t)g * 16 + o] = groups[(size_t)g][o];
+        }
+    }
     if (block) {
         plan.kernel = SPDNN_KERNEL_BLOCK;
         plan.wmode = (uniform && exact) ? 0 : (exact ? 1 : 2);
@@ -556,18 +578,23 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.info.kernel = plan.kernel;
     plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
                                                               plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
+                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.set = true;
 }
 
 void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos) {
-    const size_t slots = cur.out_at.size();  // N, or 16 per group with -1 padding for BLOCK layers
-    cur.dst.resize(slots);
-    for (size_t s = 0; s < slots; ++s) {
-        const int32_t j = cur.out_at[s];
-        cur.dst[s] = j < 0 ? -1 : (next_in_pos ? (*next_in_pos)[(size_t)j] : j);
-    }
+    auto link = [&](const std::vector<int32_t>& out_at, std::vector<int32_t>& dst) {
+        const size_t slots = out_at.size();  // N, or 16 per group with -1 padding for BLOCK layers
+        dst.resize(slots);
+        for (size_t s = 0; s < slots; ++s) {
+            const int32_t j = out_at[s];
+            dst[s] = j < 0 ? -1 : (next_in_pos ? (*next_in_pos)[(size_t)j] : j);
+        }
+    };
+    link(cur.out_at, cur.dst);
+    link(cur.alt_out_at, cur.alt_dst);
 }
 
 }  // namespace spdnn

@@ -40,6 +40,15 @@ struct LayerPlan {
     std::vector<float> wv;          // weights in accumulation order: BAND [N/2][padded steps][2], GATHER [N][kmax],
                                     // BLOCK [ngroups*16][32] (empty when wmode 0)
     std::vector<int32_t> dst;       // [N] physical column of slot's output in the next buffer
+    // A run-chain BAND layer with one exact weight value also carries its BLOCK form (same input
+    // labelling, so either kernel can run the layer): for batches whose buffers fit the on-chip
+    // caches the BLOCK kernel is the faster of the two.
+    int alt_ngroups = 0;
+    bool alt_full = false;
+    std::vector<int32_t> alt_cols;   // [alt_ngroups][32] physical input columns, accumulation order
+    std::vector<int32_t> alt_cnt;    // [alt_ngroups]
+    std::vector<int32_t> alt_out_at; // [alt_ngroups*16] output neuron of the slot, -1 = unused
+    std::vector<int32_t> alt_dst;    // [alt_ngroups*16] physical column in the next buffer
 };
 
 // Sorts every row of the CSR by input index (stable) and validates it.  Returns an empty

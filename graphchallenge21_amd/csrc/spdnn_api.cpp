@@ -131,14 +131,18 @@ struct DevLayer {
     int32_t* dst = nullptr;
     int32_t* blk_cols = nullptr;
     int32_t* blk_cnt = nullptr;
+    int32_t* alt_cols = nullptr;   // the BLOCK form of a run-chain BAND layer (see LayerPlan)
+    int32_t* alt_cnt = nullptr;
+    int32_t* alt_dst = nullptr;
 };
 
 // Where the arrays of one layer's plan lie inside its block of device memory (and inside the
 // pinned host copy of that block when plans are streamed): pairs, ell, rowlen, wv, dst, blk_cols,
-// blk_cnt, each aligned to 256 bytes.
+// blk_cnt, alt_cols, alt_cnt, alt_dst, each aligned to 256 bytes.
+constexpr int kPlanArrays = 10;
 struct PlanLayout {
-    size_t off[7] = {0, 0, 0, 0, 0, 0, 0};
-    size_t len[7] = {0, 0, 0, 0, 0, 0, 0};
+    size_t off[kPlanArrays] = {};
+    size_t len[kPlanArrays] = {};
     size_t bytes = 0;
 };
 
@@ -204,6 +208,7 @@ struct spdnn_net {
     bool gid_dirty = false;   // a repack permuted d_gid since it was last initialised
     int last_stamp = 0;       // stamp of the newest layer, valid for the current row slots (0 = none)
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
+    int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     ChainLayerDesc* d_chain = nullptr;
     std::vector<char> pending; // layer has an inspection job in flight
     std::vector<int64_t> counts;
@@ -427,9 +432,10 @@ int alloc_feature_buffers(spdnn_net* n) {
 
 PlanLayout plan_layout(const LayerPlan& p) {
     PlanLayout y;
-    const size_t len[7] = {p.pairs.size() * 4, p.ell_col.size() * 4, p.rowlen.size() * 4, p.wv.size() * 4,
-                           p.dst.size() * 4,   p.blk_cols.size() * 4, p.blk_cnt.size() * 4};
-    for (int k = 0; k < 7; ++k) {
+    const size_t len[kPlanArrays] = {p.pairs.size() * 4,    p.ell_col.size() * 4,  p.rowlen.size() * 4,   p.wv.size() * 4,
+                                     p.dst.size() * 4,      p.blk_cols.size() * 4, p.blk_cnt.size() * 4,  p.alt_cols.size() * 4,
+                                     p.alt_cnt.size() * 4,  p.alt_dst.size() * 4};
+    for (int k = 0; k < kPlanArrays; ++k) {
         y.off[k] = y.bytes;
         y.len[k] = len[k];
         y.bytes += align256(len[k]);
@@ -438,9 +444,9 @@ PlanLayout plan_layout(const LayerPlan& p) {
 }
 
 void pack_plan(const LayerPlan& p, const PlanLayout& y, char* dst) {
-    const void* src[7] = {p.pairs.data(), p.ell_col.data(), p.rowlen.data(), p.wv.data(),
-                          p.dst.data(),   p.blk_cols.data(), p.blk_cnt.data()};
-    for (int k = 0; k < 7; ++k)
+    const void* src[kPlanArrays] = {p.pairs.data(),   p.ell_col.data(),  p.rowlen.data(),  p.wv.data(),      p.dst.data(),
+                                    p.blk_cols.data(), p.blk_cnt.data(), p.alt_cols.data(), p.alt_cnt.data(), p.alt_dst.data()};
+    for (int k = 0; k < kPlanArrays; ++k)
         if (y.len[k]) memcpy(dst + y.off[k], src[k], y.len[k]);
 }
 
@@ -454,6 +460,9 @@ DevLayer plan_at(const PlanLayout& y, char* base) {
     d.dst = (int32_t*)at(4);
     d.blk_cols = (int32_t*)at(5);
     d.blk_cnt = (int32_t*)at(6);
+    d.alt_cols = (int32_t*)at(7);
+    d.alt_cnt = (int32_t*)at(8);
+    d.alt_dst = (int32_t*)at(9);
     return d;
 }
 
@@ -682,6 +691,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
     if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
+    if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
     if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
         const int w = atoi(e);
         if (w == 0 || (w >= 2 && w <= 64)) n->plan_window = w;
@@ -1170,11 +1180,29 @@ static int resolve_trials(spdnn_net* n, size_t keep) {
     return SPDNN_OK;
 }
 
+// A run-chain BAND layer also has a BLOCK form.  The band walk reads every input column once from
+// HBM and wins on large batches; the BLOCK kernel reads every column twice, needs no staging and no
+// barriers, and wins while the batch's buffers stay in the on-chip caches (measured cross-over:
+// rows x neurons = 2^26, i.e. 256 MiB per buffer - N=4096: 64 row blocks of 256, N=16384: 16).
+static bool use_block_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
+    return p.kernel == SPDNN_KERNEL_BAND && p.alt_ngroups > 0 &&
+           (int64_t)nblk * (int64_t)n->RB * (int64_t)n->N < n->block_form_max_elems;
+}
+
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
                                int prev_stamp, int check_dead, int32_t* count_prev, int shape, int seglen,
                                const Publish& pub) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
+    if (use_block_form(n, p, nblk)) {
+        BlockLaunch b{};
+        b.yin = in; b.yout = out; b.cols = d.alt_cols; b.cnt = d.alt_cnt; b.wv = nullptr; b.dst = d.alt_dst;
+        b.active = n->d_active; b.count_prev = count_prev; b.check_dead = check_dead; b.N = n->N; b.ngroups = p.alt_ngroups; b.nblk = nblk;
+        b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = 0; b.full = p.alt_full ? 1 : 0;
+        b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
+        b.publish = pub;
+        return launch_block(b, n->stream);
+    }
     if (p.kernel == SPDNN_KERNEL_BAND) {
         BandLaunch a = band_args(n, l, in, out, nblk, stamp);
         a.count_prev = count_prev;
@@ -1332,7 +1360,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         int shape = -1, seglen = 0;
         bool trial = false;
         spdnn_net::Trial tr{};
-        if (c == 1 && p.kernel == SPDNN_KERNEL_BAND) {
+        if (c == 1 && p.kernel == SPDNN_KERNEL_BAND && !use_block_form(n, p, nblk)) {
             if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) {
                 shape = t->shape;
                 seglen = t->seglen;

@@ -411,8 +411,9 @@ def test_block_kernel_radix_like_layers(gc, orc, values, chains, monkeypatch):
     from helpers import hub_block_csr, radix_like_csr
     N, B = 1024, 300
     print("block kernel values=%s chains=%s" % (values, chains), flush=True)
-    if chains:   # by default widths below 4096 stay on the BLOCK kernel
+    if chains:   # by default widths below 4096 stay on the BLOCK kernel, and small batches take the BLOCK form
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+        monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", "0")
     rk, rh = (gc.KERNEL_BAND, 32) if chains else (gc.KERNEL_BLOCK, -1)
     rng = np.random.default_rng(17)
     layers = [radix_like_csr(rng, N, 16 << l, values) for l in range(4)]
@@ -439,14 +440,17 @@ def test_block_kernel_radix_like_layers(gc, orc, values, chains, monkeypatch):
             assert np.array_equal(net.categories(), ref["categories"])
 
 
+@pytest.mark.parametrize("form", ["band", "block"])
 @pytest.mark.parametrize("N,strides", [(4096, (16, 256, 2048)), (65536, (16, 1024, 32768))])
-def test_radix_like_layers_at_challenge_widths(gc, orc, N, strides):
+def test_radix_like_layers_at_challenge_widths(gc, orc, N, strides, form, monkeypatch):
     """RadiX-Net-like layers (two 16-wide input runs per group of 16 outputs, first, middle and last
-    stride of the width, behind random relabellings) at N=4096 and at the headline width: walked
-    as run chains by the band kernel under the default settings, bit-equal to the oracle."""
+    stride of the width, behind random relabellings) at N=4096 and at the headline width: planned
+    as run chains for the band kernel under the default settings, and run in both of their forms -
+    the band walk (what large batches get) and the BLOCK form (what small batches get)."""
     from helpers import radix_like_csr
     B = 300
-    print("radix-like N=%d strides %s" % (N, strides), flush=True)
+    monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", "0" if form == "band" else str(1 << 40))
+    print("radix-like N=%d strides %s form %s" % (N, strides, form), flush=True)
     rng = np.random.default_rng(N)
     layers = [radix_like_csr(rng, N, st, "uniform") for st in strides]
     L = len(layers)
@@ -767,6 +771,7 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
             print("random case", what, flush=True)
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
+        monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))   # run chains: band walk or BLOCK form
         ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
         with gc.Network(N, B, L, bias=bias) as net:
             if window:
@@ -815,6 +820,7 @@ def test_randomized_call_sequences(gc, orc, monkeypatch):
         window = int(rng.choice([0, 0, 2]))
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(int(rng.choice([1, 2, 4]))))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(int(rng.choice([256, 4096]))))
+        monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))
         layers = [make_layer(rng, N, l, values) for l in range(L)]
         what = dict(case=case, N=N, maxB=maxB, L=L, bias=bias, values=values, window=window)
         if case % 25 == 0:
