@@ -1303,10 +1303,12 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     // every layer launch stores the previous launch's counts into pinned host memory.
     // How far behind depends on how long a layer runs: behind a long layer one launch in the
     // queue keeps the device busy and a compaction should not come late; behind short layers the
-    // host needs several launches of lead or the device waits for it.
+    // host needs a lead of a few launches or the device waits for it (measured: leads of 2 to 32
+    // launches give the same time per layer; every launch of lead is one more launch made in vain
+    // once all rows have died).
     auto lookahead_for = [&](int carried_rows) -> size_t {
         const double us = (double)carried_rows * (double)n->N * 8.0 / 4.0e6 + 6.0;  // at 4 TB/s, plus launch
-        return us > 200.0 ? 1 : us > 50.0 ? 2 : us > 20.0 ? 4 : 8;
+        return us > 200.0 ? 1 : 3;
     };
     const bool polled = have_counts && opt.prune;
     if (polled) {
