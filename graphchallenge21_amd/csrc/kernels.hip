@@ -644,49 +644,49 @@ __global__ __launch_bounds__(256) void block_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// Active-row scan (one workgroup of 1024 threads).  Thread t owns the contiguous strip of rows
-// [t*S, (t+1)*S): it counts its survivors, the workgroup takes an exclusive prefix over the 1024
-// counts (wave64 ballot-free shuffle scan inside a wave, LDS across the 16 waves), and every
-// thread then writes its survivors in order.  Stable: survivors keep their order, as the
-// reference's host loop does (all_network.cu:455-463).
+// Active-row scan.  Workgroup b (1024 threads) owns the tile of rows [1024 b, 1024 b + 1024),
+// thread = row, so all reads are coalesced.  Its survivors go behind those of the tiles before
+// it; how many those are it counts itself (the flags of at most 58 earlier tiles, 8 bytes a row
+// from L2 - cheaper than a second launch or a chain of workgroups waiting for each other).
+// Inside the tile a survivor's place comes from the wave's ballot and an LDS sum over the 16
+// waves.  Stable: survivors keep their order, as the reference's host loop does
+// (all_network.cu:455-463).  The last workgroup writes the total.
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void scan_active_kernel(
     const int32_t* __restrict__ active, const int32_t* __restrict__ gid, int rows, int stamp,
     int32_t* __restrict__ count, int32_t* __restrict__ alive_src, int32_t* __restrict__ alive_gid) {
     __shared__ int wave_tot[16];
+    __shared__ int wave_before[16];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int S = (rows + 1023) / 1024;
-    const int r0 = threadIdx.x * S;
-    const int r1 = min(rows, r0 + S);
-    int mine = 0;
-    for (int r = r0; r < r1; ++r) mine += (active[r] == stamp && gid[r] >= 0) ? 1 : 0;
-    // inclusive scan of `mine` inside the wave
-    int incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += up;
+    const int tile = blockIdx.x;
+    int before = 0;  // survivors among this wave's 64 rows of every earlier tile
+    for (int t = 0; t < tile; ++t) {
+        const int r = t * 1024 + (int)threadIdx.x;  // < rows: an earlier tile is a full one
+        before += (int)__popcll(__ballot((active[r] == stamp && gid[r] >= 0) ? 1 : 0));
     }
-    if (lane == 63) wave_tot[wave] = incl;
+    const int r = tile * 1024 + (int)threadIdx.x;
+    const int g = r < rows ? gid[r] : -1;
+    const bool alive = r < rows && g >= 0 && active[r] == stamp;
+    const unsigned long long mask = __ballot(alive ? 1 : 0);
+    if (lane == 0) {
+        wave_tot[wave] = (int)__popcll(mask);
+        wave_before[wave] = before;
+    }
     __syncthreads();
     int base = 0, total = 0;
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
-        const int t = wave_tot[w];
-        if (w < wave) base += t;
-        total += t;
+        base += wave_before[w];
+        total += wave_before[w] + wave_tot[w];
+        if (w < wave) base += wave_tot[w];
     }
-    int k = base + incl - mine;
-    for (int r = r0; r < r1; ++r) {
-        const int g = gid[r];
-        if (active[r] == stamp && g >= 0) {
-            alive_src[k] = r;
-            alive_gid[k] = g;
-            ++k;
-        }
+    if (alive) {
+        const int k = base + (int)__popcll(mask & ((1ull << lane) - 1ull));
+        alive_src[k] = r;
+        alive_gid[k] = g;
     }
-    if (threadIdx.x == 0) count[0] = total;
+    if (tile == (int)gridDim.x - 1 && threadIdx.x == 0) count[0] = total;
 }
 
 // Repack survivors into dense row blocks.  Thread = destination row slot; loops over a chunk of
@@ -1093,8 +1093,8 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {
 hipError_t launch_scan_active(const int32_t* active, const int32_t* gid, int rows, int stamp, int32_t* count,
                               int32_t* alive_src, int32_t* alive_gid, hipStream_t s) {
     if (rows < 0 || !active || !gid || !count || !alive_src || !alive_gid) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(scan_active_kernel, dim3(1), dim3(1024), 0, s, active, gid, rows, stamp, count,
-                       alive_src, alive_gid);
+    hipLaunchKernelGGL(scan_active_kernel, dim3(std::max(1, (rows + 1023) / 1024)), dim3(1024), 0, s, active, gid, rows,
+                       stamp, count, alive_src, alive_gid);
     return hipGetLastError();
 }
 
