@@ -498,10 +498,8 @@ def test_replacing_a_layer(gc, orc):
         other.close()
 
 
-def test_driver_usage_paths():
+def test_driver_usage_paths(gc):
     exe = os.path.join(ROOT, "graphchallenge21_amd", "spdnn_network")
-    if not os.path.exists(exe):
-        pytest.skip("driver not built")
     r = subprocess.run([exe], capture_output=True, text=True)
     assert r.returncode == 0 and "Usage: exe neuron batch layer" in r.stdout      # reference network.cpp:58-61
     r = subprocess.run([exe, "1000", "10", "2"], capture_output=True, text=True)
