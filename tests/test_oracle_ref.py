@@ -14,6 +14,8 @@ GOLD = os.path.join(HERE, "golden")
 
 
 def _ref(orc):
+    if not os.path.exists(orc.REF_CHECK) and os.path.isdir("/root/reference/src/utils"):
+        orc.build(with_ref=True)   # a fresh checkout beside the mounted reference: build the harness once
     if not os.path.exists(orc.REF_CHECK):
         pytest.skip("oracle/_ref/ref_check not built (the reference is not mounted here)")
     return orc.REF_CHECK
