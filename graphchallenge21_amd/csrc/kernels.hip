@@ -795,12 +795,6 @@ __global__ void unpack_rows_kernel(Feat y, const int32_t* __restrict__ phys_of_c
     rowmajor[(size_t)blockIdx.y * N + n] = x;
 }
 
-__global__ void fill_i32_kernel(int32_t* p, long long n, int32_t v) {
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    const long long stride = (long long)gridDim.x * blockDim.x;
-    for (; i < n; i += stride) p[i] = v;
-}
-
 __global__ void iota_gid_kernel(int32_t* gid, int rows, int batch) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < rows) gid[i] = i < batch ? i : -1;
@@ -1159,13 +1153,6 @@ hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const i
     dim3 grid((N + 255) / 256, nreq);
     hipLaunchKernelGGL(unpack_rows_kernel, grid, dim3(256), 0, s, y, phys_of_col, phys_rows, N, 64 * rl, active,
                        stamp, rowmajor);
-    return hipGetLastError();
-}
-
-hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s) {
-    if (n <= 0) return hipSuccess;
-    const int blocks = (int)std::min<int64_t>((n + 255) / 256, 4096);
-    hipLaunchKernelGGL(fill_i32_kernel, dim3(blocks), dim3(256), 0, s, p, (long long)n, v);
     return hipGetLastError();
 }
 

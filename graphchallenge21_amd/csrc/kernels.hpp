@@ -161,7 +161,6 @@ hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const i
                               int nreq, int N, int rl, const int32_t* active, int stamp, float* rowmajor,
                               hipStream_t s);
 
-hipError_t launch_fill_i32(int32_t* p, int64_t n, int32_t v, hipStream_t s);
 hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s);
 hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s);
 // zero-fills p[0..n) and q[0..n) concurrently (even / odd workgroups): a probe of whether two
