@@ -861,13 +861,10 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     constexpr int T = NW * OPW;
     constexpr size_t lds = (size_t)RING * 64 * RL * 4;
     auto kern = band_walk_kernel<RL, NW, OPW, RING, WMODE, KT>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    // once per instantiation; a function-local static is initialised by one thread only
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) return attr;
     int seglen = a.seglen;
     if (seglen <= 0 || (seglen % T) != 0) {
         if (rank_seglens(a.N, a.K, T, a.nblk, a.n_cu > 0 ? a.n_cu : 256, &seglen, 1) < 1) return hipErrorInvalidValue;
@@ -987,13 +984,10 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
     constexpr size_t lds = (size_t)RING * 64 * RL * 4;
     auto kern = band_chain_kernel<RL, NW, OPW, RING, WMODE, KT>;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
+    // once per instantiation; a function-local static is initialised by one thread only
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (attr != hipSuccess) return attr;
     hipLaunchKernelGGL(kern, dim3(a.nblk), dim3(NW * 64), lds, s, reinterpret_cast<const ChainLayer*>(a.table),
                        a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.count_prev, a.N, a.stamp0,
                        a.prev_stamp, a.check_dead, a.stop_when_dead, a.bias, a.clampv, a.publish);

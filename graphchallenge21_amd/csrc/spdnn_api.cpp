@@ -1240,9 +1240,14 @@ static int wait_counts(spdnn_net* n, int l0, int c) {
     for (int j = l0; j < l0 + c; ++j) {
         if (h[j] >= 0) continue;
         auto t0 = std::chrono::steady_clock::now();
+        auto t_start = t0;
         for (unsigned spins = 1; h[j] < 0; ++spins) {
-            if ((spins & 4095) != 0) continue;
-            const auto now = std::chrono::steady_clock::now();
+            if ((spins & 255) != 0) continue;
+            auto now = std::chrono::steady_clock::now();
+            if (now - t_start < std::chrono::microseconds(300)) continue;  // short layers: poll as fast as possible
+            // behind a long layer nothing is lost by sleeping between looks: the device has its next launch queued
+            std::this_thread::sleep_for(std::chrono::microseconds(50));
+            now = std::chrono::steady_clock::now();
             if (now - t0 < std::chrono::milliseconds(100)) continue;
             t0 = now;
             const hipError_t q = hipStreamQuery(n->stream);
