@@ -308,7 +308,7 @@ int alloc_feature_buffers(spdnn_net* n) {
     HIPCHK(hipMemGetInfo(&free_b, &total_b));
     const size_t max_cand = std::min<size_t>(64, (size_t)((double)free_b * 0.85 / (double)half_bytes));
     const char* min_env = getenv("SPDNN_REGION_PAIRING_MIN_GIB");   // smallest half-buffer worth the search
-    const double min_gib = min_env ? atof(min_env) : 1.0;
+    const double min_gib = min_env ? atof(min_env) : 0.4;
     const bool search = !(env && atoi(env) == 0) && (double)half_bytes >= min_gib * 1073741824.0 && max_cand >= 12;
 
     std::vector<float*>& c = n->feat_allocs;
