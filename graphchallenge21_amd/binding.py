@@ -23,7 +23,8 @@ class SpdnnError(RuntimeError):
 class LayerPlan(C.Structure):
     _fields_ = [("kernel", C.c_int32), ("max_row_nnz", C.c_int32), ("regular", C.c_int32),
                 ("uniform_value", C.c_int32), ("value", C.c_float), ("exact_products", C.c_int32),
-                ("band_halo", C.c_int32), ("nnz", C.c_int64), ("plan_bytes", C.c_int64)]
+                ("band_halo", C.c_int32), ("nnz", C.c_int64), ("plan_bytes", C.c_int64),
+                ("block_form", C.c_int32), ("reserved", C.c_int32)]
 
 
 class RunOptions(C.Structure):

@@ -576,6 +576,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.pairs.clear();
     }
     plan.info.kernel = plan.kernel;
+    plan.info.block_form = plan.alt_ngroups > 0 ? 1 : 0;
     plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
                                                               plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
                                                               plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() +

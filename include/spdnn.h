@@ -71,6 +71,9 @@ typedef struct spdnn_layer_plan {
                                 (max_row_nnz-1 for a circulant band, 32 for run chains); else -1  */
     int64_t nnz;
     int64_t plan_bytes;      /* device bytes held for this layer                                  */
+    int32_t block_form;      /* 1: a run-chain BAND layer that also holds its BLOCK form, which
+                                spdnn_run uses on small batches                                   */
+    int32_t reserved;
 } spdnn_layer_plan;
 
 typedef struct spdnn_run_options {

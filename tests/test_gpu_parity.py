@@ -461,7 +461,7 @@ def test_radix_like_layers_at_challenge_widths(gc, orc, N, strides, form, monkey
         net.inspect()
         for l in range(L):
             p = net.layer_plan(l)
-            assert p.kernel == gc.KERNEL_BAND and p.band_halo == 32
+            assert p.kernel == gc.KERNEL_BAND and p.band_halo == 32 and p.block_form == 1
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 

@@ -233,6 +233,7 @@ def test_inspector_run_chains(gc, orc, n, monkeypatch):
         for l in range(L):
             p = net.layer_plan(l)
             assert (p.kernel, p.max_row_nnz, p.regular, p.band_halo) == (gc.KERNEL_BAND, 32, 1, 32), strides[l]
+            assert p.block_form == (0 if l % 2 else 1)   # with one exact value the layer keeps its BLOCK form too
             in_pos, out_at, sel = net.band_plan(l)
             assert sorted(in_pos.tolist()) == list(range(n)) and sorted(out_at.tolist()) == list(range(n))
             rowptr, col, _ = layers[l]
