@@ -873,6 +873,26 @@ def test_randomized_call_sequences(gc, orc, monkeypatch):
                     feats = None
 
 
+def test_out_of_device_memory(gc, orc):
+    """Feature buffers beyond the device's memory: an error code and a message, no abort, and the
+    device is usable afterwards."""
+    free0, total = gc.device_memory()
+    rows = int(total / (65536 * 4) / 2)              # three buffers of this many rows cannot fit
+    with gc.Network(65536, rows, 2, bias=-0.45) as net:
+        net.synth_layers(0)
+        net.inspect()
+        with pytest.raises(gc.SpdnnError) as e:
+            net.synth_features(0, 1000)
+        assert e.value.code == 5 and "memory" in e.value.message
+    with gc.Network(1024, 500, 3) as net:
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, 500)
+        assert net.run().layers_run >= 1
+    free1, _ = gc.device_memory()
+    assert free0 - free1 < (512 << 20)
+
+
 def test_zero_bias_into_the_denormal_range(gc, orc):
     """Bias 0 and power-of-two weights of 1/16, 8 per row: activations halve (at least) per layer and
     reach the denormal range after ~120 layers, where a product no longer is exact.  The library
