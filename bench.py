@@ -45,6 +45,30 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def radix_layer(rng, n, stride):
+    """A layer with the structure of the challenge's RadiX-Net files: the 16 outputs of group g read the
+    two 16-wide input runs [16g, 16g+16) and [16g+stride, 16g+stride+16) (mod n), hidden behind random
+    relabellings of inputs and outputs; 32 entries of 1/16 per row.  CSR with row = output neuron."""
+    pin, pout = rng.permutation(n).astype(np.int32), rng.permutation(n)
+    base = (np.arange(n) // 16 * 16)[:, None]
+    run = np.arange(16)[None, :]
+    ins = np.concatenate([base + run, (base + stride + run) % n], axis=1)
+    col = np.empty((n, 32), np.int32)
+    col[pout] = np.sort(pin[ins], axis=1)
+    return (np.arange(n + 1, dtype=np.int32) * 32, col.reshape(-1), np.full(n * 32, 0.0625, np.float32))
+
+
+def irregular_layer(rng, n, kmax=24):
+    """A layer without structure: every output reads 1..kmax random inputs with random weights."""
+    lens = rng.integers(1, kmax + 1, size=n)
+    rowptr = np.zeros(n + 1, np.int32)
+    np.cumsum(lens, out=rowptr[1:])
+    order = np.argsort(rng.random((n, n), dtype=np.float32), axis=1)[:, :kmax].astype(np.int32)
+    col = np.concatenate([np.sort(order[j, :lens[j]]) for j in range(n)]).astype(np.int32)
+    val = rng.uniform(0.02, 0.12, size=len(col)).astype(np.float32)
+    return rowptr, col, val
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -54,6 +78,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (quick runs)")
     ap.add_argument("--batch", type=int, default=0, help="override the batch (quick runs)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--structure", default="circulant", choices=["circulant", "radix", "irregular"],
+                    help="layers: the seeded permuted-stride generator (default, the configured workload), RadiX-Net-like "
+                         "layers (one per stride 16, 32, ... n/2, repeated), or layers without structure (n <= 4096)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
     ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
@@ -79,16 +106,37 @@ def main():
 
     t0 = time.time()
     net = gc.Network(N, B, L, bias=bias)
-    net.synth_layers(seed)
+    kinds = None   # the distinct layers of a structure other than the generator's, used in turn
+    if args.structure == "circulant":
+        net.synth_layers(seed)
+
+        def layer_csr(l):   # for the CPU legs only: the oracle's own generator (the library generates on its side)
+            from oracle import oracle as orc
+            return orc.gen_layer_csr(seed, l, N)
+    else:
+        rng = np.random.default_rng(seed)
+        if args.structure == "radix":
+            kinds = [radix_layer(rng, N, 16 << k) for k in range(max(1, int(np.log2(N // 16))))]
+        else:
+            if N > 4096:
+                log("bench.py: --structure irregular is for n <= 4096")
+                return 2
+            kinds = [irregular_layer(rng, N) for _ in range(4)]
+        layer_csr = lambda l: kinds[l % len(kinds)]
+        for l in range(L):
+            net.set_layer_csr(l, *layer_csr(l))
     net.inspect()
     t_inspect = time.time() - t0
     plans = [net.layer_plan(l) for l in range(L)]
     n_band = sum(1 for p in plans if p.kernel == gc.KERNEL_BAND)
-    nnz_layer = plans[0].nnz
+    kernel_names = {gc.KERNEL_BAND: "band_walk_kernel", gc.KERNEL_BLOCK: "block_kernel", gc.KERNEL_GATHER: "gather_kernel"}
+    kernels_used = sorted({kernel_names[p.kernel] for p in plans})
+    nnz_layer = float(sum(p.nnz for p in plans)) / L     # the same for every layer except with --structure irregular
     t0 = time.time()
     net.synth_features(seed, B, 0.10, 0.25)
     t_features = time.time() - t0
-    log("setup: inspector %.1f s (%d/%d layers BAND), plan upload + features %.1f s" % (t_inspect, n_band, L, t_features))
+    log("setup: inspector %.1f s (%d/%d layers BAND, kernels %s), plan upload + features %.1f s"
+        % (t_inspect, n_band, L, "+".join(kernels_used), t_features))
 
     # ---- sustained run: the timed steps ---------------------------------------------------
     for _ in range(args.warmup):
@@ -141,7 +189,7 @@ def main():
         y, gid = feats, np.arange(rows, dtype=np.int32)
         t_cpu = 0.0
         for l in range(max(n_cpu, n_check)):
-            csr = orc.gen_layer_csr(seed, l, N)
+            csr = layer_csr(l)
             t0 = time.perf_counter()
             yo, act = orc.layer(y, csr, bias)
             if l < n_cpu:
@@ -180,7 +228,7 @@ def main():
         gid = np.arange(S, dtype=np.int32)
         t0 = time.perf_counter()
         for l in range(L):
-            y, act = orc.layer(y, gc.synth_layer_csr(seed, l, N), bias)
+            y, act = orc.layer(y, layer_csr(l), bias)
             y, gid = orc.compact(y, act, gid)
             if l % 200 == 0:
                 log("survivor check: oracle layer %d, %d rows alive" % (l, len(gid)))
@@ -192,7 +240,7 @@ def main():
 
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "band_walk_cfg4_hbm_traffic.txt")
-    if os.path.exists(tpath) and args.config == "cfg4" and B == 60000:
+    if os.path.exists(tpath) and args.config == "cfg4" and B == 60000 and args.structure == "circulant":
         for line in open(tpath):
             if line.startswith("hbm_bytes_per_launch"):
                 traffic = float(line.split("=")[1])
@@ -211,10 +259,12 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": "%s sustained: N=%d, %d layers, batch %d, bias %g, 32 nnz/row of 0.0625, "
-                        "pruning off (every layer at full batch), seed %d" % (args.config, N, L, B, bias, seed),
+            "workload": "%s sustained: N=%d, %d layers%s, batch %d, bias %g, %s, "
+                        "pruning off (every layer at full batch), seed %d"
+                        % (args.config, N, L, "" if args.structure == "circulant" else " (%s)" % args.structure, B, bias,
+                           "32 nnz/row of 0.0625" if args.structure != "irregular" else "1..24 nnz/row, random weights", seed),
             "neuron": N, "layers": L, "batch": B, "bias": bias, "seed": seed,
-            "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "mixed",
+            "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "+".join(kernels_used),
             "band_tuning_rowblocks_shape_seglen": net.band_tuning(),
             "feature_buffers_region_paired_candidates": list(net.feature_placement()),
             "plan_window_device_bytes_pinned_bytes": list(net.plan_memory()),
@@ -222,7 +272,7 @@ def main():
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "kernel": "band_walk_kernel", "alg_bytes_per_launch": alg_bytes_launch,
+                     "kernel": "+".join(kernels_used), "alg_bytes_per_launch": alg_bytes_launch,
                      "avg_launch_ms": avg_launch_ms, "launches_timed": int(layer_ms.size),
                      "measured_copy_peak_gbps": copy_gbps,
                      "frac_of_measured_copy": achieved / copy_gbps if copy_gbps else None},
