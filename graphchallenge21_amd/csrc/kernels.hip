@@ -30,6 +30,35 @@ template <> struct VecOf<1> { using type = float; };
 template <> struct VecOf<2> { using type = float2; };
 template <> struct VecOf<4> { using type = float4; };
 
+// Loads and stores of feature columns that are touched once per layer (every input column of the
+// band walk, every output column of any kernel) carry the non-temporal hint: the data of one layer
+// is far larger than the caches, and without the hint it pushes out what is used again (measured on
+// the band walk at N=65536, batch 60000: 5.97 -> 5.72 ms per layer with loads and stores hinted,
+// 5.95 - 5.96 with only one of the two).
+typedef float stream_f4 __attribute__((ext_vector_type(4)));
+typedef float stream_f2 __attribute__((ext_vector_type(2)));
+template <int RL> __device__ __forceinline__ void store_stream(float* p, const float* a) {
+    if (RL == 4) {
+        const stream_f4 v = {a[0], a[1], a[2], a[3]};
+        __builtin_nontemporal_store(v, reinterpret_cast<stream_f4*>(p));
+    } else if (RL == 2) {
+        const stream_f2 v = {a[0], a[1]};
+        __builtin_nontemporal_store(v, reinterpret_cast<stream_f2*>(p));
+    } else {
+        __builtin_nontemporal_store(a[0], p);
+    }
+}
+template <int RL> __device__ __forceinline__ void load_stream(const float* p, float* a) {
+    if (RL == 4) {
+        const stream_f4 v = __builtin_nontemporal_load(reinterpret_cast<const stream_f4*>(p));
+        a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
+    } else if (RL == 2) {
+        const stream_f2 v = __builtin_nontemporal_load(reinterpret_cast<const stream_f2*>(p));
+        a[0] = v.x; a[1] = v.y;
+    } else {
+        a[0] = __builtin_nontemporal_load(p);
+    }
+}
 template <int RL> __device__ __forceinline__ void vec_to_arr(const typename VecOf<RL>::type& v, float* a);
 template <> __device__ __forceinline__ void vec_to_arr<1>(const float& v, float* a) { a[0] = v; }
 template <> __device__ __forceinline__ void vec_to_arr<2>(const float2& v, float* a) { a[0] = v.x; a[1] = v.y; }
@@ -210,8 +239,9 @@ __device__ __forceinline__ void band_walk_body(
         const int p = vb - halo + c;
         if (p < ve) {
             const int g = p < 0 ? p + N : p;
-            V x = *reinterpret_cast<const V*>(yin + (size_t)g * RB + loff);
-            *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = x;
+            float x[RL];
+            load_stream<RL>(yin + (size_t)g * RB + loff, x);
+            *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(x);
         }
     }
     __syncthreads();
@@ -224,7 +254,7 @@ __device__ __forceinline__ void band_walk_body(
 #pragma unroll
         for (int i = 0; i < OPW; ++i) {
             const int p = min(cb + T + wave + i * NW, ve - 1);
-            vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
+            load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
         }
 
         int pr[PPW];
@@ -420,7 +450,7 @@ __device__ __forceinline__ void band_walk_body(
                         nz[q] = nz_merge(nz[q], y[q]);
                     }
                     const int d = dst[v];
-                    *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
+                    store_stream<RL>(yout + (size_t)d * RB + loff, y);
                 }
             }
         }
