@@ -30,11 +30,13 @@ template <> struct VecOf<1> { using type = float; };
 template <> struct VecOf<2> { using type = float2; };
 template <> struct VecOf<4> { using type = float4; };
 
-// Loads and stores of feature columns that are touched once per layer (every input column of the
-// band walk, every output column of any kernel) carry the non-temporal hint: the data of one layer
-// is far larger than the caches, and without the hint it pushes out what is used again (measured on
-// the band walk at N=65536, batch 60000: 5.97 -> 5.72 ms per layer with loads and stores hinted,
-// 5.95 - 5.96 with only one of the two).
+// The band walk touches every input and output column once per layer.  On a large batch its loads and
+// stores carry the non-temporal hint: the data of one layer is far larger than the caches, and without
+// the hint it pushes out what is used again (measured at N=65536, batch 60000: 5.97 -> 5.72 ms per layer
+// with loads and stores hinted, 5.95 - 5.96 with only one of the two).  Small launches, whose output the
+// next layer still finds in the caches, keep the plain forms (the launcher decides); so do the BLOCK and
+// GATHER kernels, which read columns more than once (hinted stores alone: BLOCK at N=1024, batch 60000
+// 99.6 -> 101.9 us per layer, GATHER unchanged).
 typedef float stream_f4 __attribute__((ext_vector_type(4)));
 typedef float stream_f2 __attribute__((ext_vector_type(2)));
 template <int RL> __device__ __forceinline__ void store_stream(float* p, const float* a) {
@@ -215,7 +217,7 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 __device__ __forceinline__ void band_walk_body(
     const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int N, int steps, int stride, int halo,
-    int vb, int ve, float wu, float bias, float clampv, unsigned char* smem, float* nz) {
+    int vb, int ve, float wu, float bias, float clampv, unsigned char* smem, float* nz, int stream) {
     using V = typename VecOf<RL>::type;
     constexpr int T = NW * OPW;
     constexpr int PPW = OPW / 2;  // pairs per wave and chunk
@@ -240,7 +242,8 @@ __device__ __forceinline__ void band_walk_body(
         if (p < ve) {
             const int g = p < 0 ? p + N : p;
             float x[RL];
-            load_stream<RL>(yin + (size_t)g * RB + loff, x);
+            if (stream) load_stream<RL>(yin + (size_t)g * RB + loff, x);
+            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)g * RB + loff), x);
             *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(x);
         }
     }
@@ -254,7 +257,8 @@ __device__ __forceinline__ void band_walk_body(
 #pragma unroll
         for (int i = 0; i < OPW; ++i) {
             const int p = min(cb + T + wave + i * NW, ve - 1);
-            load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
+            if (stream) load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
+            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
         }
 
         int pr[PPW];
@@ -450,7 +454,8 @@ __device__ __forceinline__ void band_walk_body(
                         nz[q] = nz_merge(nz[q], y[q]);
                     }
                     const int d = dst[v];
-                    store_stream<RL>(yout + (size_t)d * RB + loff, y);
+                    if (stream) store_stream<RL>(yout + (size_t)d * RB + loff, y);
+                    else *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
                 }
             }
         }
@@ -464,7 +469,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
     int32_t* __restrict__ count_prev, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
-    int check_dead, float wu, float bias, float clampv, Publish pub, int nblk) {
+    int check_dead, float wu, float bias, float clampv, Publish pub, int nblk, int stream) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     publish_counts(pub);
@@ -482,7 +487,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
     band_walk_body<RL, NW, OPW, RING, WMODE, KT>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
-                                                 pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz);
+                                                 pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz, stream);
     stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, nullptr);
 }
 
@@ -527,7 +532,7 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
         band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
-                                                     lay.halo, 0, N, lay.wu, bias, clampv, smem, nz);
+                                                     lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
         stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
                                      count_out ? count_out + j : nullptr);
         int any = 0;
@@ -911,10 +916,16 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     const size_t block_bytes = (size_t)a.N * 64 * RL * 4;
     const bool pad = a.nblk >= 3 && (a.nblk & 7) != 0 && (size_t)((a.nblk + 7) / 8) * block_bytes * 2 <= ((size_t)4 << 20);
     const int gx = pad ? (a.nblk + 7) / 8 * 8 : a.nblk;
+    // Input and output of the launch together beyond what stays in the caches from one layer to the next: the
+    // columns are hinted as touched once (see store_stream).  Measured cross-over (N=1024 ... 16384): around
+    // 64 - 128 MiB; below it the next layer still finds this layer's output on chip and the hint costs up to 15 %.
+    const char* stream_env = getenv("SPDNN_STREAM_MIN_BYTES");   // looked up per launch: tests switch it
+    const long long stream_min = stream_env ? atoll(stream_env) : (96ll << 20);
+    const int stream = (long long)a.nblk * (long long)block_bytes * 2 >= stream_min ? 1 : 0;
     dim3 grid(gx, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_prev,
                        a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,
-                       a.nblk);
+                       a.nblk, stream);
     return hipGetLastError();
 }
 

@@ -772,6 +772,7 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
         monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))   # run chains: band walk or BLOCK form
+        monkeypatch.setenv("SPDNN_STREAM_MIN_BYTES", str(int(rng.choice([0, 96 << 20]))))      # band walk with or without streaming hints
         ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
         with gc.Network(N, B, L, bias=bias) as net:
             if window:
