@@ -443,20 +443,32 @@ __device__ __forceinline__ void band_walk_body(
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int i = 0; i < PPW; ++i) {
+            const int v0 = cb + 2 * (wave + i * NW);
+            if (v0 + 1 < ve) {
+                // both outputs of the pair (the usual case: segments end at even positions)
+                float y0[RL], y1[RL];
 #pragma unroll
-            for (int o = 0; o < 2; ++o) {
-                const int v = cb + 2 * (wave + i * NW) + o;
-                if (v < ve) {
-                    float y[RL];
-#pragma unroll
-                    for (int q = 0; q < RL; ++q) {
-                        y[q] = relu_clamp(acc[i][o][q] + bias, clampv);
-                        nz[q] = nz_merge(nz[q], y[q]);
-                    }
-                    const int d = dst[v];
-                    if (stream) store_stream<RL>(yout + (size_t)d * RB + loff, y);
-                    else *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
+                for (int q = 0; q < RL; ++q) {
+                    y0[q] = relu_clamp(acc[i][0][q] + bias, clampv);
+                    y1[q] = relu_clamp(acc[i][1][q] + bias, clampv);
+                    nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));   // one three-way maximum
                 }
+                const int d0 = dst[v0], d1 = dst[v0 + 1];
+                if (stream) {
+                    store_stream<RL>(yout + (size_t)d0 * RB + loff, y0);
+                    store_stream<RL>(yout + (size_t)d1 * RB + loff, y1);
+                } else {
+                    *reinterpret_cast<V*>(yout + (size_t)d0 * RB + loff) = arr_to_vec<RL>(y0);
+                    *reinterpret_cast<V*>(yout + (size_t)d1 * RB + loff) = arr_to_vec<RL>(y1);
+                }
+            } else if (v0 < ve) {
+                float y[RL];
+#pragma unroll
+                for (int q = 0; q < RL; ++q) {
+                    y[q] = relu_clamp(acc[i][0][q] + bias, clampv);
+                    nz[q] = nz_merge(nz[q], y[q]);
+                }
+                *reinterpret_cast<V*>(yout + (size_t)dst[v0] * RB + loff) = arr_to_vec<RL>(y);
             }
         }
 
