@@ -151,8 +151,10 @@ __device__ __forceinline__ void stamp_rows_workgroup(const float* nz, unsigned c
 
 // see Publish: the first workgroup of the launch hands the previous launch's counts to the host
 __device__ __forceinline__ void publish_counts(const Publish& p) {
-    if (p.n > 0 && blockIdx.x == 0 && blockIdx.y == 0)
+    if (p.n > 0 && blockIdx.x == 0 && blockIdx.y == 0) {
         for (int i = threadIdx.x; i < p.n; i += blockDim.x) p.dst[i] = p.src[i];
+        __threadfence_system();  // the host polls this memory while the kernel is still running
+    }
 }
 
 // Start of a layer kernel (every wave of the workgroup calls it; lane = RL rows from row0, so a
@@ -931,9 +933,7 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     // Input and output of the launch together beyond what stays in the caches from one layer to the next: the
     // columns are hinted as touched once (see store_stream).  Measured cross-over (N=1024 ... 16384): around
     // 64 - 128 MiB; below it the next layer still finds this layer's output on chip and the hint costs up to 15 %.
-    const char* stream_env = getenv("SPDNN_STREAM_MIN_BYTES");   // looked up per launch: tests switch it
-    const long long stream_min = stream_env ? atoll(stream_env) : (96ll << 20);
-    const int stream = (long long)a.nblk * (long long)block_bytes * 2 >= stream_min ? 1 : 0;
+    const int stream = (long long)a.nblk * (long long)block_bytes * 2 >= a.stream_min_bytes ? 1 : 0;
     dim3 grid(gx, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_prev,
                        a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,

@@ -55,6 +55,8 @@ struct BandLaunch {
     int n_cu;
     int shape = -1;          // tile shape (see launch_band); < 0 = default
     int seglen = 0;          // band positions per workgroup; 0 = heuristic
+    long long stream_min_bytes = 96ll << 20;  // launches that read + write at least this much hint their
+                                              // column loads and stores as touched once
     Publish publish;
 };
 

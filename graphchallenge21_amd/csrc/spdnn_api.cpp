@@ -207,8 +207,15 @@ struct spdnn_net {
     bool alive_list_valid = false;
     bool gid_dirty = false;   // a repack permuted d_gid since it was last initialised
     int last_stamp = 0;       // stamp of the newest layer, valid for the current row slots (0 = none)
+    // A launch that skips row blocks without an active row leaves those blocks of its output buffer
+    // unwritten (they hold an older layer's values).  Consumers that look at the stamps never read
+    // them; a later launch that does not look (pruning off) would.  Set by launches that may skip,
+    // cleared when every carried block has been written again (new run, repack).
+    bool blocks_skipped = false;
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
+    long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
+    long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
     ChainLayerDesc* d_chain = nullptr;
     std::vector<char> pending; // layer has an inspection job in flight
     std::vector<int64_t> counts;
@@ -273,9 +280,10 @@ int init_device(spdnn_net* n) {
     HIPCHK(hipMalloc(&n->d_alive_gid, rows * 4));
     HIPCHK(hipMalloc(&n->d_count, 64));
     HIPCHK(hipMalloc(&n->d_nonfinite, 64));
-    HIPCHK(hipHostMalloc(&n->h_count, 64));
+    // coherent: the layer kernels store counts here and the host reads them while kernels still run
+    HIPCHK(hipHostMalloc(&n->h_count, 64, hipHostMallocCoherent | hipHostMallocMapped));
     HIPCHK(hipMalloc(&n->d_counts, (size_t)n->L * 4));
-    HIPCHK(hipHostMalloc(&n->h_counts, (size_t)n->L * 4));
+    HIPCHK(hipHostMalloc(&n->h_counts, (size_t)n->L * 4, hipHostMallocCoherent | hipHostMallocMapped));
     HIPCHK(hipMemset(n->d_active, 0, rows * 4));
     n->dev_ready = true;
     return SPDNN_OK;
@@ -641,6 +649,7 @@ void reset_state(spdnn_net* n) {
     }
     n->cur = n->F;
     n->last_stamp = 0;
+    n->blocks_skipped = false;
     n->cur_layer = 0;
     n->carried = ((n->batch + n->RB - 1) / n->RB) * n->RB;
     n->alive = n->batch;
@@ -692,6 +701,8 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
+    if (const char* e = getenv("SPDNN_STREAM_MIN_BYTES")) n->stream_min_bytes = atoll(e);
+    if (const char* e = getenv("SPDNN_COUNT_TIMEOUT_MS")) n->count_timeout_ms = std::max(1ll, atoll(e));
     if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
         const int w = atoi(e);
         if (w == 0 || (w >= 2 && w <= 64)) n->plan_window = w;
@@ -1109,6 +1120,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
     a.shape = -1; a.seglen = 0; a.count_prev = nullptr; a.prev_stamp = 0; a.check_dead = 0;
+    a.stream_min_bytes = n->stream_min_bytes;
     return a;
 }
 
@@ -1234,7 +1246,8 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
 // by the first workgroup of the launch after theirs; -1 = not yet).  Normally they are there or
 // arrive within microseconds.  The stream itself is asked only after 100 ms without them, so that
 // a failed launch ends the wait: asking puts a marker into the queue, which between two short
-// layers costs as much as a layer.
+// layers costs as much as a layer.  The wait is bounded: after count_timeout_ms without the counts
+// of one layer (a kernel that never finishes) the call gives up with SPDNN_E_DEVICE.
 static int wait_counts(spdnn_net* n, int l0, int c) {
     volatile int32_t* h = n->h_counts;
     for (int j = l0; j < l0 + c; ++j) {
@@ -1250,6 +1263,9 @@ static int wait_counts(spdnn_net* n, int l0, int c) {
             now = std::chrono::steady_clock::now();
             if (now - t0 < std::chrono::milliseconds(100)) continue;
             t0 = now;
+            if (now - t_start > std::chrono::milliseconds(n->count_timeout_ms))
+                return fail(SPDNN_E_DEVICE, "timed out waiting for the active-row count of layer " + std::to_string(j) +
+                                                " (the device did not finish the launch)");
             const hipError_t q = hipStreamQuery(n->stream);
             if (q == hipSuccess) {
                 if (h[j] < 0) return fail(SPDNN_E_DEVICE, "layer counts were not handed over");
@@ -1358,7 +1374,10 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         // counted by this launch (unless a chain or a scan has counted them already), and with
         // pruning the row blocks it left without an active row are skipped
         const int prev_stamp = n->last_stamp;
-        const int check_dead = opt.prune ? 1 : 0;
+        // (a run without pruning that continues a pruned one keeps skipping: the blocks skipped
+        // so far hold stale values, and with bias <= 0 a dead row stays dead, so skipping is exact)
+        const int check_dead = (opt.prune || n->blocks_skipped) ? 1 : 0;
+        if (check_dead && (prev_stamp != 0 || c > 1)) n->blocks_skipped = true;
         int32_t* const count_prev = (fused_count && count_pending && prev_stamp != 0) ? n->d_counts + (l - 1) : nullptr;
         const Feat in = n->cur;
         Feat out = (n->cur == n->A) ? n->C : n->A;
@@ -1408,7 +1427,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             ch.active = n->d_active; ch.count_out = fused_count ? n->d_counts + l : nullptr;
             ch.count_prev = count_prev; ch.check_dead = check_dead;
             ch.N = n->N; ch.K = p.kmax; ch.nblk = nblk; ch.stamp0 = stamp0; ch.prev_stamp = prev_stamp;
-            ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = opt.prune ? 1 : 0;
+            ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = check_dead;
             ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
             ch.bias = n->bias; ch.clampv = n->clampv;
             ch.publish = pub;
@@ -1468,6 +1487,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 n->cur = dstbuf;
                 n->carried = nb * n->RB;
                 n->last_stamp = 0;  // the row slots moved: the stamps no longer describe them
+                n->blocks_skipped = false;  // every carried block has just been written
                 r.compactions++;
             }
         }

@@ -493,11 +493,13 @@ def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
         assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
 
 
-@pytest.mark.parametrize("N,L,bias,S", [(4096, 480, -0.35, 512), (16384, 1920, -0.4, 96)])
-def test_full_depth_cfg2_cfg3(gc, orc, N, L, bias, S):
-    """N=4096 x 480 layers and N=16384 x 1920 layers at batch 60000, every layer, with densities up
-    to 0.7 so that rows survive to the end: pruned run against the unpruned run (size-independent)
-    and against the oracle on the first S rows through all layers."""
+@pytest.mark.parametrize("N,L,bias,S", [(4096, 480, -0.35, 512), (16384, 1920, -0.4, 96), (65536, 1920, -0.45, 96)],
+                         ids=["cfg2", "cfg3", "cfg4"])
+def test_full_depth_cfg2_cfg3_cfg4(gc, orc, N, L, bias, S):
+    """N=4096 x 480 layers, N=16384 x 1920 layers and the headline N=65536 x 1920 layers at batch
+    60000, every layer, with densities up to 0.7 so that rows survive to the end: pruned run against
+    the unpruned run (size-independent, N=4096) and against the oracle on the first S rows through
+    all layers (categories inside the sample, and the survivors' activations bit for bit)."""
     B = 60000
     print("full depth N=%d L=%d" % (N, L), flush=True)
     with gc.Network(N, B, L) as net:
@@ -519,10 +521,91 @@ def test_full_depth_cfg2_cfg3(gc, orc, N, L, bias, S):
     print("survivors", counts_p[0], counts_p[-1], "compactions", rp.compactions, flush=True)
     assert counts_p == sorted(counts_p, reverse=True) and 0 < counts_p[-1] < B and rp.compactions >= 1
     assert len(cats_p) == counts_p[-1] and np.array_equal(cats_p, np.sort(cats_p))
-    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.70), lambda l: orc.gen_layer_csr(0, l, N) if l < L else None,
-                    bias, prune=True)
+    def layer_of(l):
+        if l % 240 == 0:
+            print("  oracle layer", l, flush=True)    # a long leg (N=65536: about 100 s): keep the log moving
+        return orc.gen_layer_csr(0, l, N) if l < L else None
+
+    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.70), layer_of, bias, prune=True)
     assert np.array_equal(cats_p[cats_p < S], ref["categories"])
     assert len(sample) > 0 and same_floats(y_p, ref["y"][:len(sample)])
+
+
+@pytest.mark.parametrize("name,N,L,bias", [("cfg1", 1024, 120, -0.30), ("cfg2", 4096, 480, -0.35),
+                                           ("cfg3", 16384, 1920, -0.40), ("cfg4", 65536, 1920, -0.45)])
+def test_literal_configs_full_batch(gc, orc, name, N, L, bias):
+    """The configurations as written: batch 60000, seed 0, feature density U[0.10, 0.25] per row.
+    Every row dies within a few layers, so the final category set is empty and parity is checked
+    per layer: for the layers before everything has died, the active ids inside an oracle row
+    sample and the sample's activations (bit for bit); afterwards zero rows; and the whole-network
+    pruned run must report the same per-layer counts and no categories."""
+    B, S, seed = 60000, 2048, 0
+    print("literal %s: N=%d L=%d B=%d" % (name, N, L, B), flush=True)
+    head = 10                                    # every row is dead long before this layer
+    layers = [orc.gen_layer_csr(seed, l, N) for l in range(head)]
+    ref = orc.infer(orc.gen_features(seed, N, 0, S, 0.10, 0.25), layers, bias, prune=False, keep=set(range(head)))
+    ref_counts = [len(a) for a in ref["active_ids"]]
+    assert ref_counts[0] > 0 and ref_counts[-1] == 0, ref_counts
+    rows = np.arange(S, dtype=np.int32)
+    with gc.Network(N, B, L) as net:
+        assert net.bias == pytest.approx(bias)
+        net.synth_layers(seed)
+        net.inspect()
+        net.synth_features(seed, B, 0.10, 0.25)
+        step_counts = []
+        for l in range(head):
+            r = net.run(prune=True, first_layer=l, n_layers=1, collect_counts=True)
+            cats = net.categories()
+            step_counts.append(len(cats))
+            assert r.active_rows == len(cats) and net.active_count(l) == len(cats)
+            assert np.array_equal(cats[cats < S], ref["active_ids"][l]), "layer %d" % l
+            assert same_floats(net.activations(rows), ref["kept"][l][1]), "layer %d" % l
+            if len(cats) == 0:
+                break
+        assert step_counts[-1] == 0 and step_counts == sorted(step_counts, reverse=True)
+        r = net.run(prune=True, collect_counts=True)
+        counts = [net.active_count(l) for l in range(L)]
+        print("literal %s: active rows per layer %s, layers launched %d" % (name, counts[:len(step_counts)], r.layers_run),
+              flush=True)
+        assert counts[:len(step_counts)] == step_counts and not any(counts[len(step_counts):])
+        assert r.active_rows == 0 and len(net.categories()) == 0 and r.layers_run < L
+        assert not net.activations(rows[:64]).any()
+
+
+def test_unpruned_run_continues_a_pruned_one(gc, orc, monkeypatch):
+    """A row block whose rows have all died is skipped by pruned launches and keeps stale values in
+    the work buffers.  A run without pruning that continues from there must not bring them back:
+    64-row blocks, 65 rows, the last block holds one row that dies at once while the others live."""
+    monkeypatch.setenv("SPDNN_ROWS_PER_LANE", "1")
+    N, L, B = 256, 8, 65
+    rng = np.random.default_rng(4)
+    layers = [orc.gen_layer_csr(11, l, N) for l in range(L)]
+    feats = (rng.random((B, N)) < 0.6).astype(np.float32) * 2.0
+    # the last row is alive after layer 0 and dead after layer 1: layer 1 writes its zeros into one
+    # work buffer, the other one keeps the row's nonzero layer-0 output in a block that is skipped from then on
+    for _ in range(200):
+        cand = (rng.random((1, N)) < 0.2).astype(np.float32)
+        probe = orc.infer(cand, layers[:2], -0.3, prune=False)
+        if len(probe["active_ids"][0]) == 1 and len(probe["active_ids"][1]) == 0:
+            break
+    else:
+        raise AssertionError("no candidate row dies exactly at layer 1")
+    feats[64] = cand[0]
+    ref = orc.infer(feats, layers, -0.3, prune=False, keep=set(range(L)))
+    assert 64 in ref["active_ids"][0] and 64 not in ref["active_ids"][1] and len(ref["active_ids"][L - 1]) == 64
+    rows = np.arange(B, dtype=np.int32)
+    for split in (2, 3, 4):
+        with gc.Network(N, B, L, bias=-0.3) as net:
+            for l, csr in enumerate(layers):
+                net.set_layer_csr(l, *csr)
+            net.inspect()
+            net.set_features_dense(feats)
+            r = net.run(prune=True, first_layer=0, n_layers=split, collect_counts=True, compact_threshold=0.01)
+            assert r.compactions == 0
+            net.run(prune=False, first_layer=split, n_layers=L - split, collect_counts=True)
+            assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]], split
+            assert np.array_equal(net.categories(), ref["active_ids"][L - 1]), split
+            assert same_floats(net.activations(rows), ref["kept"][L - 1][1]), split
 
 
 @pytest.mark.parametrize("N,K,B", [(256, 32, 1), (256, 4, 65), (512, 12, 257), (128, 8, 40), (100, 5, 33), (2048, 36, 70)])
