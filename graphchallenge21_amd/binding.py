@@ -93,6 +93,7 @@ def load_library():
         "spdnn_get_active_count": ([vp, C.c_int, C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_categories": ([vp, C.c_void_p, C.c_int64, C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_activations": ([vp, _i32p, C.c_int, _f32p], C.c_int),
+        "spdnn_get_activations_noalloc": ([vp, _i32p, C.c_int, _f32p], C.c_int),
         "spdnn_get_layer_times": ([vp, _f32p, C.c_int], C.c_int),
         "spdnn_get_band_tuning": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
@@ -338,6 +339,14 @@ class Network:
         out = np.empty((len(rows), self.neuron), np.float32)
         if len(rows):
             _check(self._lib.spdnn_get_activations(self._h, rows, len(rows), out))
+        return out
+
+    def activations_noalloc(self, rows):
+        """spdnn_get_activations_noalloc: the same rows through the library's static scratch memory."""
+        rows = np.ascontiguousarray(rows, np.int32)
+        out = np.empty((len(rows), self.neuron), np.float32)
+        if len(rows):
+            _check(self._lib.spdnn_get_activations_noalloc(self._h, rows, len(rows), out))
         return out
 
     def layer_times(self):

@@ -844,6 +844,24 @@ __global__ void unpack_rows_kernel(Feat y, const int32_t* __restrict__ phys_of_c
     rowmajor[(size_t)blockIdx.y * N + n] = x;
 }
 
+// Row lookup on the device (for callers that cannot allocate): where[g] = physical row that carries
+// global id g, -1 for a row that is not carried any more.  fill first, then scatter.
+__global__ void fill_i32_kernel(int32_t* __restrict__ p, int n, int32_t v) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+__global__ void scatter_where_kernel(const int32_t* __restrict__ gid, int carried, int batch, int32_t* __restrict__ where) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= carried) return;
+    const int g = gid[r];
+    if (g >= 0 && g < batch) where[g] = r;
+}
+__global__ void lookup_rows_kernel(const int32_t* __restrict__ ids, int n, const int32_t* __restrict__ where,
+                                   int32_t* __restrict__ phys) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) phys[i] = where[ids[i]];
+}
+
 __global__ void iota_gid_kernel(int32_t* gid, int rows, int batch) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < rows) gid[i] = i < batch ? i : -1;
@@ -1200,6 +1218,20 @@ hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const i
     dim3 grid((N + 255) / 256, nreq);
     hipLaunchKernelGGL(unpack_rows_kernel, grid, dim3(256), 0, s, y, phys_of_col, phys_rows, N, 64 * rl, active,
                        stamp, rowmajor);
+    return hipGetLastError();
+}
+
+hipError_t launch_row_table(const int32_t* gid, int carried, int batch, int32_t* where, hipStream_t s) {
+    if (batch <= 0 || carried < 0 || !where || (carried > 0 && !gid)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((batch + 255) / 256), dim3(256), 0, s, where, batch, -1);
+    if (carried > 0)
+        hipLaunchKernelGGL(scatter_where_kernel, dim3((carried + 255) / 256), dim3(256), 0, s, gid, carried, batch, where);
+    return hipGetLastError();
+}
+
+hipError_t launch_lookup_rows(const int32_t* ids, int n, const int32_t* where, int32_t* phys, hipStream_t s) {
+    if (n <= 0 || !ids || !where || !phys) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(lookup_rows_kernel, dim3((n + 255) / 256), dim3(256), 0, s, ids, n, where, phys);
     return hipGetLastError();
 }
 

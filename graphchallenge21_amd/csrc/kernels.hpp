@@ -164,6 +164,10 @@ hipError_t launch_unpack_rows(const Feat& y, const int32_t* phys_of_col, const i
                               hipStream_t s);
 
 hipError_t launch_iota_gid(int32_t* gid, int rows, int batch, hipStream_t s);
+// where[g] = physical row (< carried) whose global id is g, -1 if none, for g in [0, batch)
+hipError_t launch_row_table(const int32_t* gid, int carried, int batch, int32_t* where, hipStream_t s);
+// phys[i] = where[ids[i]] (ids already checked against the batch on the host)
+hipError_t launch_lookup_rows(const int32_t* ids, int n, const int32_t* where, int32_t* phys, hipStream_t s);
 hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s);
 // zero-fills p[0..n) and q[0..n) concurrently (even / odd workgroups): a probe of whether two
 // buffers lie in the same memory region

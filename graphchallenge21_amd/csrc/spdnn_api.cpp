@@ -45,6 +45,43 @@ int fail(int code, const std::string& msg) {
             return fail(SPDNN_E_DEVICE, std::string(#expr) + ": " + hipGetErrorString(e_));         \
     } while (0)
 
+// Scratch memory of spdnn_get_activations_noalloc, the one entry point that allocates nothing: a
+// row table (global id -> physical row), the ids and physical rows of one pass, and the row-major
+// staging rows of one pass.  Each GPU holds its own copy of the array until the process ends.  In
+// host code the array's name is only a stand-in for the symbol: the device address is looked up
+// once per device (scratch_base) and everything on the host side uses that pointer.
+constexpr size_t kScratchTableRows = (size_t)1 << 20;              // rows (batch) the row table holds
+constexpr size_t kScratchPassRows = 16384;                         // requested rows per pass at most
+constexpr size_t kScratchStageBytes = (size_t)8 << 20;             // staging rows of one pass
+constexpr size_t kScratchTableOff = 0;
+constexpr size_t kScratchIdsOff = kScratchTableRows * 4;
+constexpr size_t kScratchPhysOff = kScratchIdsOff + kScratchPassRows * 4;
+constexpr size_t kScratchStageOff = kScratchPhysOff + kScratchPassRows * 4;
+constexpr size_t kScratchBytes = kScratchStageOff + kScratchStageBytes;  // 12.1 MiB
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 16;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device, looked up on the first call per device.
+hipError_t scratch_base(unsigned char** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lk(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        if (!p) return hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = static_cast<unsigned char*>(p);
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+
 // Temporary device allocation / event that is released on every return path.
 struct DevTmp {
     void* p = nullptr;
@@ -269,6 +306,8 @@ int init_device(spdnn_net* n) {
     if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
         return fail(SPDNN_E_DEVICE, std::string("kernels are built for gfx950, device is ") + p.gcnArchName);
     n->n_cu = p.multiProcessorCount;
+    unsigned char* scratch_ptr = nullptr;
+    HIPCHK(scratch_base(&scratch_ptr));  // set-up, with the device current: later calls only read the pointer
     HIPCHK(hipStreamCreate(&n->stream));
     HIPCHK(hipEventCreate(&n->ev_start));
     HIPCHK(hipEventCreate(&n->ev_stop));
@@ -1604,6 +1643,44 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
         HIPCHK(launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, n->d_active, n->last_stamp, d_out, n->stream));
         HIPCHK(hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * n->N * 4, hipMemcpyDeviceToHost, n->stream));
         HIPCHK(hipStreamSynchronize(n->stream));
+    }
+    return SPDNN_OK;
+}
+
+int spdnn_get_activations_noalloc(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+    if (!n || !rows || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
+    if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
+    if (nrows < 0) return fail(SPDNN_E_ARG, "nrows negative");
+    if (nrows == 0) return SPDNN_OK;
+    if ((size_t)n->batch > kScratchTableRows)
+        return fail(SPDNN_E_UNSUPPORTED, "spdnn_get_activations_noalloc serves batches of at most " +
+                                             std::to_string(kScratchTableRows) + " rows (this one has " +
+                                             std::to_string(n->batch) + "); use spdnn_get_activations");
+    const size_t row_bytes = (size_t)n->N * 4;
+    if (row_bytes > kScratchStageBytes)
+        return fail(SPDNN_E_UNSUPPORTED, "spdnn_get_activations_noalloc serves rows of at most " +
+                                             std::to_string(kScratchStageBytes / 4) + " neurons (this network has " +
+                                             std::to_string(n->N) + "); use spdnn_get_activations");
+    for (int i = 0; i < nrows; ++i)
+        if (rows[i] < 0 || rows[i] >= n->batch) return fail(SPDNN_E_ARG, "row id out of range");
+    unsigned char* base = nullptr;
+    HIPCHK(scratch_base(&base));
+    int32_t* const d_where = reinterpret_cast<int32_t*>(base + kScratchTableOff);
+    int32_t* const d_ids = reinterpret_cast<int32_t*>(base + kScratchIdsOff);
+    int32_t* const d_phys = reinterpret_cast<int32_t*>(base + kScratchPhysOff);
+    float* const d_out = reinterpret_cast<float*>(base + kScratchStageOff);
+    // the table keeps the last call's contents: written anew (every entry, then the carried rows)
+    HIPCHK(launch_row_table(n->d_gid, n->carried, n->batch, d_where, n->stream));
+    const int32_t* lab = nullptr;
+    HIPCHK(labelling_dev(n, n->cur_layer, &lab));
+    const int chunk = (int)std::min<size_t>(kScratchPassRows, kScratchStageBytes / row_bytes);
+    for (int i0 = 0; i0 < nrows; i0 += chunk) {
+        const int m = std::min(chunk, nrows - i0);
+        HIPCHK(hipMemcpyAsync(d_ids, rows + i0, (size_t)m * 4, hipMemcpyHostToDevice, n->stream));
+        HIPCHK(launch_lookup_rows(d_ids, m, d_where, d_phys, n->stream));
+        HIPCHK(launch_unpack_rows(n->cur, lab, d_phys, m, n->N, n->rl, n->d_active, n->last_stamp, d_out, n->stream));
+        HIPCHK(hipMemcpyAsync(rowmajor + (size_t)i0 * n->N, d_out, (size_t)m * row_bytes, hipMemcpyDeviceToHost, n->stream));
+        HIPCHK(hipStreamSynchronize(n->stream));  // the staging rows are reused by the next pass
     }
     return SPDNN_OK;
 }

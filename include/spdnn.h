@@ -277,6 +277,19 @@ int spdnn_get_categories(spdnn_net* net, int32_t* ids, int64_t cap, int64_t* n);
  * (all_network.cu:521). */
 int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
 
+/* spdnn_get_activations for callers that cannot allocate device memory (code under HIP graph
+ * capture around it, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and results as spdnn_get_activations, but where that call allocates
+ * its row list and its row-major staging rows for every call, this one calls no hipMalloc / hipFree:
+ * it works in a 12.1 MiB scratch array that is part of the library's device code (one copy per GPU,
+ * held until the process ends): a row table (global id -> physical row, filled by two small
+ * kernels at every call), the ids of one pass and 8 MiB of staging rows.
+ * Limits: batch <= 1048576 rows and neuron <= 2097152 (one row must fit the staging rows);
+ * beyond them SPDNN_E_UNSUPPORTED.  All handles of a process share one GPU's scratch array: calls
+ * that overlap in time on one GPU (from several host threads or handles) race and must be
+ * serialised by the caller. */
+int spdnn_get_activations_noalloc(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
+
 /* Band-walk configuration measured at run time (record `index` = 0, 1, ...; SPDNN_E_ARG past the
  * last): row blocks it was measured for, index of the tile shape (one shape per row-block size at
  * present: 8 waves x one output pair and a 64-slot LDS ring for 256-row blocks) and band positions
