@@ -84,6 +84,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
     ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
+    ap.add_argument("--no-live", action="store_true", help="skip the sustained pass on live data")
     ap.add_argument("--survivor-check", type=int, default=0, metavar="ROWS",
                     help="extra (slow): features with densities up to 0.7 so that rows survive every layer; "
                          "the category set of the first ROWS rows after ALL layers is compared with the oracle")
@@ -170,7 +171,27 @@ def main():
     lit_categories = int(lit.active_rows)
 
     # ---- measured copy bandwidth --------------------------------------------------------------
-    copy_gbps = gc.measure_copy_bandwidth(1 << 32, 5)
+    copy_gbps = gc.measure_copy_bandwidth(1 << 32, 5)          # two plain 4 GiB allocations
+    try:
+        buffer_copy_gbps = net.buffer_copy_bandwidth(3)            # the work buffers where they lie
+    except gc.SpdnnError:
+        buffer_copy_gbps = None
+    net.synth_features(seed, B, 0.10, 0.25)                    # the probe resets the state
+
+    # ---- live data: the same sustained run on features whose rows survive (densities up to 0.7) --
+    live = None
+    if not args.no_live:
+        net.synth_features(seed, B, 0.10, 0.70)
+        net.run(prune=False, time_layers=True, n_layers=min(L, 40))
+        rl = net.run(prune=False, time_layers=True)
+        lms = net.layer_times().copy()
+        live_ms = float(lms.mean())
+        live = {"workload": "same layers, features of density U[0.10,0.70] (rows survive every layer), pruning off, one pass",
+                "avg_launch_ms": live_ms, "achieved": alg_bytes_launch / (live_ms * 1e-3) / 1e9,
+                "frac": alg_bytes_launch / (live_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "unit": "GB/s",
+                "launches_timed": int(lms.size), "rows_nonzero_at_end": int(rl.active_rows),
+                "edges_per_s": edges / (rl.ms_total * 1e-3)}
+        net.synth_features(seed, B, 0.10, 0.25)
 
     # ---- CPU baseline + parity gate on a row sample ---------------------------------------------
     cpu = None
@@ -201,16 +222,41 @@ def main():
         cpu = {"value": rows * float(nnz_layer) * n_cpu / t_cpu, "unit": "edges/s", "cores": cores, "kind": "port",
                "sample": "layers 0..%d of the same workload on rows 0..%d, every row kept (%.1f s)"
                          % (n_cpu - 1, rows - 1, t_cpu)}
+        # one thread (the reference's CPU checker is single-threaded): layer 0 on a sixteenth of the sample
+        r1 = max(64, rows // 16)
+        orc.set_threads(1)
+        t0 = time.perf_counter()
+        orc.layer(feats[:r1], layer_csr(0), bias)
+        t1 = time.perf_counter() - t0
+        orc.set_threads(cores)
+        cpu["single_thread"] = {"value": r1 * float(nnz_layer) / t1, "unit": "edges/s", "cores": 1,
+                                "sample": "layer 0 on rows 0..%d (%.1f s)" % (r1 - 1, t1)}
+        if args.structure == "circulant":
+            # the reference's own CPU-runnable configuration in full: N=1024, 120 layers, batch 6000
+            n0, l0, b0, bias0 = CONFIGS["cfg0"]
+            lay0 = [orc.gen_layer_csr(seed, l, n0) for l in range(l0)]
+            f0 = orc.gen_features(seed, n0, 0, b0, 0.10, 0.25)
+            t0 = time.perf_counter()
+            res_p = orc.infer(f0, lay0, bias0, prune=True)
+            tp = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            orc.infer(f0, lay0, bias0, prune=False)
+            tu = time.perf_counter() - t0
+            e0 = float(b0) * n0 * 32 * l0
+            cpu["cfg0_full"] = {"cores": cores, "edges": e0, "pruned_s": tp, "pruned_edges_per_s": e0 / tp,
+                                "unpruned_s": tu, "unpruned_edges_per_s": e0 / tu,
+                                "categories": int(len(res_p["active_ids"][-1]))}
         ok_ids, ok_y, max_abs = True, True, 0.0
         sample = np.arange(rows, dtype=np.int32)
         for l in range(n_check):
             net.run(prune=True, first_layer=l, n_layers=1, collect_counts=True)
             cats = net.categories()
             ok_ids &= bool(np.array_equal(cats[cats < rows], ref_ids[l]))
-            got = net.activations(sample[: min(rows, 1024)])
-            want = ref_y[l][1][: min(rows, 1024)]
-            ok_y &= bool(np.array_equal(got, want))
-            max_abs = max(max_abs, float(np.abs(got - want).max()))
+            for c0 in range(0, rows, 2048):   # the whole sample, a chunk of rows at a time
+                got = net.activations(sample[c0:c0 + 2048])
+                want = ref_y[l][1][c0:c0 + 2048]
+                ok_y &= bool(np.array_equal(got, want))
+                max_abs = max(max_abs, float(np.abs(got - want).max()))
         parity = {"rows": int(rows), "layers": n_check, "active_ids_equal": ok_ids,
                   "activations_bit_equal": ok_y, "max_abs_diff": max_abs}
 
@@ -238,12 +284,14 @@ def main():
                     "activations_bit_equal": bool(np.array_equal(got_y, y[:64])),
                     "gpu_pruned_run_s": gpu_s, "gpu_compactions": int(rs.compactions), "oracle_s": time.perf_counter() - t0}
 
-    traffic = None
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "band_walk_cfg4_hbm_traffic.txt")
     if os.path.exists(tpath) and args.config == "cfg4" and B == 60000 and args.structure == "circulant":
         for line in open(tpath):
             if line.startswith("hbm_bytes_per_launch"):
                 traffic = float(line.split("=")[1])
+                traffic_source = ("profiles/band_walk_cfg4_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                                  "command, kept as text; not measured by this process")
 
     out = {
         "metric": METRIC,
@@ -271,11 +319,15 @@ def main():
             "final_active_rows": sustained_final_active,
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "+".join(kernels_used), "alg_bytes_per_launch": alg_bytes_launch,
                      "avg_launch_ms": avg_launch_ms, "launches_timed": int(layer_ms.size),
-                     "measured_copy_peak_gbps": copy_gbps,
-                     "frac_of_measured_copy": achieved / copy_gbps if copy_gbps else None},
+                     "data": "all-zero activations from layer 2 on (bias -0.45 kills every row of the configured features); "
+                             "see roofline_live for the same run on live data",
+                     "copy_kernel_gbps_plain_allocations": copy_gbps,
+                     "copy_kernel_gbps_work_buffers": buffer_copy_gbps,
+                     "frac_of_work_buffer_copy": achieved / buffer_copy_gbps if buffer_copy_gbps else None},
+        "roofline_live": live,
         "cpu_baseline": cpu,
         "literal": {"workload": "same inputs, pruning on", "edges_per_s": edges / (lit.ms_total * 1e-3),
                     "ms": lit.ms_total, "layers_launched": int(lit.layers_run), "compactions": int(lit.compactions),

@@ -98,6 +98,7 @@ def load_library():
         "spdnn_get_band_tuning": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
+        "spdnn_measure_buffer_copy_bandwidth": ([vp, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_get_feature_placement": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_device_memory": ([C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
@@ -348,6 +349,12 @@ class Network:
         if len(rows):
             _check(self._lib.spdnn_get_activations_noalloc(self._h, rows, len(rows), out))
         return out
+
+    def buffer_copy_bandwidth(self, reps=3):
+        """GB/s (read + written) of a plain copy of one work buffer into the other."""
+        g = C.c_double()
+        _check(self._lib.spdnn_measure_buffer_copy_bandwidth(self._h, reps, C.byref(g)))
+        return g.value
 
     def layer_times(self):
         ms = np.empty(self.layers, np.float32)

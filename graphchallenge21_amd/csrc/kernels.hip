@@ -875,6 +875,18 @@ __global__ __launch_bounds__(256) void zero_pair_kernel(float4* __restrict__ p, 
     for (; i < n4; i += stride) d[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 }
 
+// Copy of two buffers at once: even workgroups copy p0 -> q0, odd workgroups p1 -> q1 (the access
+// pattern of a layer kernel over feature buffers whose halves lie in two memory regions).
+__global__ __launch_bounds__(256) void copy_pair_kernel(const stream_f4* __restrict__ p0, stream_f4* __restrict__ q0,
+                                                        const stream_f4* __restrict__ p1, stream_f4* __restrict__ q1,
+                                                        long long n4) {
+    const stream_f4* s = (blockIdx.x & 1) ? p1 : p0;
+    stream_f4* d = (blockIdx.x & 1) ? q1 : q0;
+    long long i = (long long)(blockIdx.x >> 1) * blockDim.x + threadIdx.x;
+    const long long stride = (long long)(gridDim.x >> 1) * blockDim.x;
+    for (; i < n4; i += stride) __builtin_nontemporal_store(__builtin_nontemporal_load(&s[i]), &d[i]);
+}
+
 __global__ __launch_bounds__(256) void copy_f4_kernel(const float4* __restrict__ src, float4* __restrict__ dst,
                                                       long long n4) {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1245,6 +1257,15 @@ hipError_t launch_zero_pair(float* p, float* q, int64_t n_floats_each, hipStream
     if (n_floats_each <= 0 || (n_floats_each % 4) != 0 || !p || !q) return hipErrorInvalidValue;
     hipLaunchKernelGGL(zero_pair_kernel, dim3(65536), dim3(256), 0, s, reinterpret_cast<float4*>(p),
                        reinterpret_cast<float4*>(q), (long long)(n_floats_each / 4));
+    return hipGetLastError();
+}
+
+hipError_t launch_copy_pair(const Feat& src, const Feat& dst, int64_t n_floats_each, hipStream_t s) {
+    if (n_floats_each <= 0 || (n_floats_each % 4) != 0 || !src || !dst || !src.half[1] || !dst.half[1])
+        return hipErrorInvalidValue;
+    hipLaunchKernelGGL(copy_pair_kernel, dim3(65536), dim3(256), 0, s, reinterpret_cast<const stream_f4*>(src.half[0]),
+                       reinterpret_cast<stream_f4*>(dst.half[0]), reinterpret_cast<const stream_f4*>(src.half[1]),
+                       reinterpret_cast<stream_f4*>(dst.half[1]), (long long)(n_floats_each / 4));
     return hipGetLastError();
 }
 

@@ -169,6 +169,8 @@ hipError_t launch_row_table(const int32_t* gid, int carried, int batch, int32_t*
 // phys[i] = where[ids[i]] (ids already checked against the batch on the host)
 hipError_t launch_lookup_rows(const int32_t* ids, int n, const int32_t* where, int32_t* phys, hipStream_t s);
 hipError_t launch_copy_f4(const float* src, float* dst, int64_t n_floats, hipStream_t s);
+// copies both halves of src to the halves of dst concurrently (even / odd workgroups), n floats each
+hipError_t launch_copy_pair(const Feat& src, const Feat& dst, int64_t n_floats_each, hipStream_t s);
 // zero-fills p[0..n) and q[0..n) concurrently (even / odd workgroups): a probe of whether two
 // buffers lie in the same memory region
 hipError_t launch_zero_pair(float* p, float* q, int64_t n_floats_each, hipStream_t s);

@@ -1742,6 +1742,28 @@ int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
     return SPDNN_OK;
 }
 
+int spdnn_measure_buffer_copy_bandwidth(spdnn_net* n, int reps, double* gbps) {
+    if (!n || !gbps || reps < 1) return fail(SPDNN_E_ARG, "bad argument");
+    if (!n->uploaded || !n->have_features) return fail(SPDNN_E_STATE, "no feature buffers yet: set features first");
+    const int nblk = (n->batch + n->RB - 1) / n->RB;
+    const int64_t half_floats = (int64_t)((nblk + 1) / 2) * n->N * n->RB;
+    EventTmp ev0, ev1;
+    HIPCHK(ev0.create());
+    HIPCHK(ev1.create());
+    // the work buffers hold nothing a caller can still ask for once the state is reset
+    reset_state(n);
+    HIPCHK(launch_copy_pair(n->A, n->C, half_floats, n->stream));
+    HIPCHK(hipEventRecord(ev0.e, n->stream));
+    for (int i = 0; i < reps; ++i) HIPCHK(launch_copy_pair(n->A, n->C, half_floats, n->stream));
+    HIPCHK(hipEventRecord(ev1.e, n->stream));
+    HIPCHK(hipEventSynchronize(ev1.e));
+    float ms = 0.0f;
+    HIPCHK(hipEventElapsedTime(&ms, ev0.e, ev1.e));
+    if (ms <= 0.0f) return fail(SPDNN_E_DEVICE, "copy benchmark failed");
+    *gbps = 4.0 * (double)half_floats * 4.0 * reps / (ms * 1e-3) / 1e9;
+    return SPDNN_OK;
+}
+
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
     int cnt = 0;
     if (hipGetDeviceCount(&cnt) != hipSuccess || cnt < 1) return fail(SPDNN_E_DEVICE, "no HIP device available");

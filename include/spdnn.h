@@ -308,6 +308,12 @@ int spdnn_write_categories(spdnn_net* net, const char* path);
  * plain float4 copy kernel over `bytes` bytes: the box's practical HBM peak. */
 int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps);
 
+/* The same measurement over the network's own work buffers (one copied to the other, the rows of
+ * the current batch): the copy rate a layer kernel could reach at best with these buffers where
+ * they lie (their halves may sit in two memory regions, see spdnn_get_feature_placement).
+ * Needs features; the state of the network is reset as at the start of a run from layer 0. */
+int spdnn_measure_buffer_copy_bandwidth(spdnn_net* net, int reps, double* gbps);
+
 /* Name and compute-unit count of device 0. */
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes);
 
