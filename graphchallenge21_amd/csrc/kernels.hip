@@ -183,6 +183,25 @@ __device__ __forceinline__ bool enter_row_block(const int32_t* active, size_t ro
 }
 
 
+// One input column (64 lanes x 16 bytes) straight from global memory into an LDS column slot,
+// without passing through vector registers: lane i's 16 bytes land at lds_col + 16 i, which is
+// the layout of a 256-row column.  The transfer is counted like any vector memory load.
+template <int STREAM>
+__device__ __forceinline__ void column_to_lds(const float* gsrc_lane, unsigned char* lds_col) {
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)gsrc_lane,
+        (__attribute__((address_space(3))) void*)lds_col, 16, 0, STREAM ? 2 : 0);
+}
+__device__ __forceinline__ void wait_vector_memory() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Workgroup barrier of the band walk.  With columns sent straight into the ring the waves wait for
+// their transfers themselves (wait_vector_memory) BEFORE they store their outputs; the fence of
+// __syncthreads() would wait on the vector memory counter again behind those stores, i.e. for the
+// stores' acknowledgement, once per chunk.  The bare barrier only orders the LDS traffic.
+template <int DMA> __device__ __forceinline__ void ring_barrier() {
+    if (DMA) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else __syncthreads();
+}
+
 __device__ __forceinline__ float relu_clamp(float y, float clampv) {
     // median(y, 0, clamp): 0 below 0, clamp above clamp, y in between (inputs are finite).
     return __builtin_amdgcn_fmed3f(y, 0.0f, clampv);
@@ -215,7 +234,7 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // step.  The output column is written to the physical column the NEXT layer wants it in (dst),
 // RB*4 contiguous bytes.
 // ------------------------------------------------------------------------------------------
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
 __device__ __forceinline__ void band_walk_body(
     const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int N, int steps, int stride, int halo,
@@ -239,27 +258,40 @@ __device__ __forceinline__ void band_walk_body(
     const uint32_t wu_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(wu));
 
     // prologue: halo (columns before the segment, wrapping below 0) + first chunk
+    static_assert(DMA == 0 || RL == 4, "direct loads into the ring move 16 bytes per lane");
     for (int c = wave; c < halo + T; c += NW) {
         const int p = vb - halo + c;
         if (p < ve) {
             const int g = p < 0 ? p + N : p;
+            if (DMA) {
+                unsigned char* slot = smem + (size_t)(p & (RING - 1)) * COLB;
+                if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
+                else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+                continue;
+            }
             float x[RL];
             if (stream) load_stream<RL>(yin + (size_t)g * RB + loff, x);
             else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)g * RB + loff), x);
             *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(x);
         }
     }
-    __syncthreads();
+    if (DMA) wait_vector_memory();
+    ring_barrier<DMA>();
 
     const int last_pair = (ve - 1) >> 1;
     for (int cb = vb; cb < ve; cb += T) {
         // columns of the next chunk: issue the HBM loads now, park them in registers (past the
-        // segment end the last column is loaded again and never stored)
+        // segment end the last column is loaded again and never stored) - or, DMA, send them
+        // straight into the ring slots no wave reads during this chunk
         float pf[OPW][RL];
 #pragma unroll
         for (int i = 0; i < OPW; ++i) {
             const int p = min(cb + T + wave + i * NW, ve - 1);
-            if (stream) load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
+            if (DMA) {
+                unsigned char* slot = smem + (size_t)((cb + T + wave + i * NW) & (RING - 1)) * COLB;
+                if (stream) column_to_lds<1>(yin + (size_t)p * RB + loff, slot);
+                else column_to_lds<0>(yin + (size_t)p * RB + loff, slot);
+            } else if (stream) load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
             else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
         }
 
@@ -437,10 +469,14 @@ __device__ __forceinline__ void band_walk_body(
         // The write is unconditional: past the segment end it drops a copy of the last column into a
         // slot nobody reads any more, and every path has then waited for the parked loads here, so
         // that nothing downstream needs to wait on the memory counter again.
+        if (DMA) {
+            wait_vector_memory();  // the columns sent to the ring at the top of the chunk (and older stores)
+        } else {
 #pragma unroll
-        for (int i = 0; i < OPW; ++i) {
-            const int p = cb + T + wave + i * NW;
-            *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(pf[i]);
+            for (int i = 0; i < OPW; ++i) {
+                const int p = cb + T + wave + i * NW;
+                *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(pf[i]);
+            }
         }
         asm volatile("" ::: "memory");
 #pragma unroll
@@ -474,11 +510,11 @@ __device__ __forceinline__ void band_walk_body(
             }
         }
 
-        __syncthreads();
+        ring_barrier<DMA>();
     }
 }
 
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
@@ -500,7 +536,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     float nz[RL];
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-    band_walk_body<RL, NW, OPW, RING, WMODE, KT>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
+    band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
                                                  pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz, stream);
     stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, nullptr);
 }
@@ -545,7 +581,7 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         float nz[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT, 0>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
                                                      lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
         stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
                                      count_out ? count_out + j : nullptr);
@@ -935,11 +971,11 @@ double seglen_score(int N, int K, int T, int nblk, int slots, int seglen) {
     return fill / (1.0 + 0.25 * (double)(K - 1) / (double)seglen);
 }
 
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
 hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     constexpr int T = NW * OPW;
     constexpr size_t lds = (size_t)RING * 64 * RL * 4;
-    auto kern = band_walk_kernel<RL, NW, OPW, RING, WMODE, KT>;
+    auto kern = band_walk_kernel<RL, NW, OPW, RING, WMODE, KT, DMA>;
     // once per instantiation; a function-local static is initialised by one thread only
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -971,19 +1007,19 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     return hipGetLastError();
 }
 
-template <int RL, int NW, int OPW, int RING>
+template <int RL, int NW, int OPW, int RING, int DMA>
 hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
     if (band_unrolled(a.K, a.steps, a.stride)) {
         switch (a.wmode) {
-            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 36>(a, s);
-            case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36>(a, s);
-            default: return launch_band_inst<RL, NW, OPW, RING, 2, 36>(a, s);
+            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 36, DMA>(a, s);
+            case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36, DMA>(a, s);
+            default: return launch_band_inst<RL, NW, OPW, RING, 2, 36, DMA>(a, s);
         }
     }
     switch (a.wmode) {
-        case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 0>(a, s);
-        case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 0>(a, s);
-        default: return launch_band_inst<RL, NW, OPW, RING, 2, 0>(a, s);
+        case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 0, DMA>(a, s);
+        case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 0, DMA>(a, s);
+        default: return launch_band_inst<RL, NW, OPW, RING, 2, 0, DMA>(a, s);
     }
 }
 
@@ -1055,9 +1091,12 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
         if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);
     }
     switch (a.rl) {
-        case 4: return launch_band_rl<4, 8, 2, 64>(b, s);
-        case 2: return launch_band_rl<2, 8, 2, 64>(b, s);
-        case 1: return launch_band_rl<1, 8, 2, 64>(b, s);
+        case 4: {
+            static const bool dma = !(getenv("SPDNN_BAND_DIRECT_LDS") && atoi(getenv("SPDNN_BAND_DIRECT_LDS")) == 0);
+            return dma ? launch_band_rl<4, 8, 2, 64, 1>(b, s) : launch_band_rl<4, 8, 2, 64, 0>(b, s);
+        }
+        case 2: return launch_band_rl<2, 8, 2, 64, 0>(b, s);
+        case 1: return launch_band_rl<1, 8, 2, 64, 0>(b, s);
         default: return hipErrorInvalidValue;
     }
 }
