@@ -58,6 +58,16 @@ def radix_layer(rng, n, stride):
     return (np.arange(n + 1, dtype=np.int32) * 32, col.reshape(-1), np.full(n * 32, 0.0625, np.float32))
 
 
+def common_band_layer(perm):
+    """A convolution-like layer over the neuron order `perm` (common to all layers): the neuron at place t
+    reads the neurons at places t-31 .. t; 32 entries of 1/16 per row.  Consecutive layers of this kind write
+    their outputs where the next one's band reads them, so the library runs them two per launch."""
+    n = len(perm)
+    col = np.empty((n, 32), np.int32)
+    col[perm] = np.sort(perm[(np.arange(n)[:, None] - np.arange(32)[None, :]) % n], axis=1)
+    return (np.arange(n + 1, dtype=np.int32) * 32, col.reshape(-1), np.full(n * 32, 0.0625, np.float32))
+
+
 def irregular_layer(rng, n, kmax=24):
     """A layer without structure: every output reads 1..kmax random inputs with random weights."""
     lens = rng.integers(1, kmax + 1, size=n)
@@ -78,7 +88,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (quick runs)")
     ap.add_argument("--batch", type=int, default=0, help="override the batch (quick runs)")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--structure", default="circulant", choices=["circulant", "radix", "irregular"],
+    ap.add_argument("--fuse", type=int, default=0, help="spdnn_run_options.fuse_layers for the timed runs (1 = no fused launches)")
+    ap.add_argument("--structure", default="circulant", choices=["circulant", "radix", "irregular", "common-band"],
                     help="layers: the seeded permuted-stride generator (default, the configured workload), RadiX-Net-like "
                          "layers (one per stride 16, 32, ... n/2, repeated), or layers without structure (n <= 4096)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
@@ -118,6 +129,8 @@ def main():
         rng = np.random.default_rng(seed)
         if args.structure == "radix":
             kinds = [radix_layer(rng, N, 16 << k) for k in range(max(1, int(np.log2(N // 16))))]
+        elif args.structure == "common-band":
+            kinds = [common_band_layer(rng.permutation(N).astype(np.int32))]
         else:
             if N > 4096:
                 log("bench.py: --structure irregular is for n <= 4096")
@@ -141,13 +154,13 @@ def main():
 
     # ---- sustained run: the timed steps ---------------------------------------------------
     for _ in range(args.warmup):
-        net.run(prune=False, time_layers=True)
+        net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
     gc.load_library().spdnn_device_synchronize()
     layer_ms = []
     t0 = time.perf_counter()
     ms_events = 0.0
     for _ in range(args.steps):
-        r = net.run(prune=False, time_layers=True)
+        r = net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
         ms_events += r.ms_total
         layer_ms.append(net.layer_times().copy())
     gc.load_library().spdnn_device_synchronize()
@@ -182,8 +195,8 @@ def main():
     live = None
     if not args.no_live:
         net.synth_features(seed, B, 0.10, 0.70)
-        net.run(prune=False, time_layers=True, n_layers=min(L, 40))
-        rl = net.run(prune=False, time_layers=True)
+        net.run(prune=False, time_layers=True, n_layers=min(L, 40), fuse_layers=args.fuse)
+        rl = net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
         lms = net.layer_times().copy()
         live_ms = float(lms.mean())
         live = {"workload": "same layers, features of density U[0.10,0.70] (rows survive every layer), pruning off, one pass",
@@ -317,6 +330,7 @@ def main():
             "feature_buffers_region_paired_candidates": list(net.feature_placement()),
             "plan_window_device_bytes_pinned_bytes": list(net.plan_memory()),
             "final_active_rows": sustained_final_active,
+            "launches_per_pass": int(r.launches), "fused_pairs_per_pass": int(r.fused_pairs),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,

@@ -24,7 +24,7 @@ class LayerPlan(C.Structure):
     _fields_ = [("kernel", C.c_int32), ("max_row_nnz", C.c_int32), ("regular", C.c_int32),
                 ("uniform_value", C.c_int32), ("value", C.c_float), ("exact_products", C.c_int32),
                 ("band_halo", C.c_int32), ("nnz", C.c_int64), ("plan_bytes", C.c_int64),
-                ("block_form", C.c_int32), ("reserved", C.c_int32)]
+                ("block_form", C.c_int32), ("fuse_next", C.c_int32)]
 
 
 class RunOptions(C.Structure):
@@ -36,7 +36,7 @@ class RunOptions(C.Structure):
 class RunResult(C.Structure):
     _fields_ = [("layers_run", C.c_int32), ("compactions", C.c_int32), ("active_rows", C.c_int64),
                 ("carried_rows", C.c_int64), ("ms_total", C.c_float), ("ms_kernels", C.c_float),
-                ("alg_bytes", C.c_double), ("edges", C.c_double)]
+                ("alg_bytes", C.c_double), ("edges", C.c_double), ("launches", C.c_int32), ("fused_pairs", C.c_int32)]
 
 
 def lib_path():
@@ -97,6 +97,7 @@ def load_library():
         "spdnn_get_layer_times": ([vp, _f32p, C.c_int], C.c_int),
         "spdnn_get_band_tuning": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
         "spdnn_write_categories": ([vp, C.c_char_p], C.c_int),
+        "spdnn_receptive_field": ([vp, C.c_int, C.c_int, _i32p, C.c_int, _i32p, C.c_int64, C.POINTER(C.c_int64)], C.c_int),
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_measure_buffer_copy_bandwidth": ([vp, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
@@ -257,6 +258,15 @@ class Network:
         _check(self._lib.spdnn_get_band_pairs(self._h, layer, None, None, None, None, rec.ctypes.data,
                                               None if w is None else w.ctypes.data))
         return steps.value, rec, w
+
+    def receptive_field(self, first_layer, n_layers, out_neurons):
+        """Input neurons of layer first_layer that the given output neurons of layer
+        first_layer + n_layers - 1 depend on (ascending)."""
+        outs = np.ascontiguousarray(out_neurons, dtype=np.int32)
+        res = np.empty(self.neuron, np.int32)
+        cnt = C.c_int64()
+        _check(self._lib.spdnn_receptive_field(self._h, first_layer, n_layers, outs, len(outs), res, len(res), C.byref(cnt)))
+        return res[:cnt.value].copy()
 
     def feature_placement(self):
         """(paired, candidates): whether the buffer halves lie in different memory regions."""

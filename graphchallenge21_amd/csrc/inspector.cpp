@@ -192,6 +192,38 @@ bool discover_band(int N, int K, const std::vector<int32_t>& rowptr, const std::
     return true;
 }
 
+// A band labelling is fixed only up to a rotation and a reflection.  Where the layer is a band in
+// ONE labelling of its neurons - neuron j sits at the same place of the band as an input and as an
+// output, as in a chain of convolution-like layers over a common (possibly hidden) neuron order -
+// that freedom is used up here, the same way for every such layer: reflected if need be so that
+// position(j as output) == position(j as input), and rotated so that neuron 0 sits at position 0.
+// Consecutive layers of this kind then agree on the labelling of the buffer between them (the
+// first writes its outputs exactly where the second reads its inputs, dst = identity), which is
+// what lets a pair of them run as one fused launch with the intermediate tile in LDS.  Other
+// layers are left as discovered.  Returns whether the layer is of this kind.
+bool canonicalize_self_aligned_band(int N, int K, std::vector<int32_t>& in_pos, std::vector<int32_t>& out_at) {
+    std::vector<int32_t> out_pos((size_t)N);
+    for (int v = 0; v < N; ++v) out_pos[(size_t)out_at[(size_t)v]] = v;
+    auto delta = [&](int j) { return ((out_pos[(size_t)j] - in_pos[(size_t)j]) % N + N) % N; };
+    const int d0 = delta(0);
+    if (d0 != 0 && d0 != K - 1) return false;
+    for (int j = 1; j < N; ++j) if (delta(j) != d0) return false;
+    if (d0 == K - 1 && K > 1) {  // reflect: input p -> -p-(K-1), output v -> -v
+        std::vector<int32_t> oa((size_t)N);
+        for (int v = 0; v < N; ++v) oa[(size_t)((N - v) % N)] = out_at[(size_t)v];
+        out_at.swap(oa);
+        for (int i = 0; i < N; ++i) in_pos[(size_t)i] = (((-in_pos[(size_t)i] - (K - 1)) % N) + N) % N;
+    }
+    const int r = in_pos[0];
+    if (r != 0) {
+        for (int i = 0; i < N; ++i) in_pos[(size_t)i] = (in_pos[(size_t)i] - r + N) % N;
+        std::vector<int32_t> oa((size_t)N);
+        for (int v = 0; v < N; ++v) oa[(size_t)v] = out_at[(size_t)((v + r) % N)];
+        out_at.swap(oa);
+    }
+    return true;
+}
+
 bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                      std::vector<std::vector<int32_t>>& groups) {
     groups.clear();
@@ -409,6 +441,8 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     }
 
     plan.kmax = kmax;
+    plan.self_aligned = false;
+    plan.fuse_next = false;
     plan.info = spdnn_layer_plan{};
     plan.info.max_row_nnz = kmax;
     plan.info.regular = (rows_regular && cols_regular && !dup) ? 1 : 0;
@@ -426,6 +460,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     if (force_kernel != SPDNN_KERNEL_GATHER && plan.info.regular && K >= 4 && K <= 32 && (K % 4) == 0 &&
         (N % 256) == 0 && N >= 4 * K) {
         band = discover_band(N, K, rowptr, col, plan.in_pos, plan.out_at);
+        if (band) plan.self_aligned = canonicalize_self_aligned_band(N, K, plan.in_pos, plan.out_at);
     }
 
     std::vector<std::vector<int32_t>> groups;
@@ -583,6 +618,69 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.set = true;
+}
+
+void plan_adjacency(const LayerPlan& p, int N, std::vector<int32_t>& rowptr, std::vector<int32_t>& col) {
+    rowptr.assign((size_t)N + 1, 0);
+    col.clear();
+    std::vector<std::vector<int32_t>> ins((size_t)N);
+    if (p.kernel == SPDNN_KERNEL_BAND) {
+        const int K = p.kmax, halo = p.info.band_halo;
+        std::vector<int32_t> in_at((size_t)N);
+        for (int i = 0; i < N; ++i) in_at[(size_t)p.in_pos[(size_t)i]] = i;
+        for (int v = 0; v < N; ++v) {
+            // an input of position v lies in [base - halo, base + span): the one position of that
+            // range congruent to the selector mod 256
+            const int base = halo == K - 1 ? v : v / 16 * 16, lo = base - halo;
+            for (int k = 0; k < K; ++k) {
+                const int sel = p.sel[(size_t)v * K + k];
+                const int q = lo + (((sel - lo) % 256) + 256) % 256;
+                ins[(size_t)p.out_at[(size_t)v]].push_back(in_at[(size_t)(((q % N) + N) % N)]);
+            }
+        }
+    } else if (p.kernel == SPDNN_KERNEL_BLOCK) {
+        for (int g = 0; g < p.ngroups; ++g)
+            for (int o = 0; o < 16; ++o) {
+                const int j = p.out_at[(size_t)g * 16 + o];
+                if (j < 0) continue;
+                for (int k = 0; k < p.blk_cnt[(size_t)g]; ++k) ins[(size_t)j].push_back(p.blk_cols[(size_t)g * 32 + k]);
+            }
+    } else {
+        for (int j = 0; j < N; ++j)
+            for (int k = 0; k < p.rowlen[(size_t)j]; ++k) ins[(size_t)j].push_back(p.ell_col[(size_t)j * p.kmax + k]);
+    }
+    for (int j = 0; j < N; ++j) {
+        std::sort(ins[(size_t)j].begin(), ins[(size_t)j].end());
+        rowptr[(size_t)j + 1] = rowptr[(size_t)j] + (int32_t)ins[(size_t)j].size();
+        col.insert(col.end(), ins[(size_t)j].begin(), ins[(size_t)j].end());
+    }
+}
+
+void receptive_field(const LayerPlan* plans, int N, int n_layers, const int32_t* outs, int n_out,
+                     std::vector<int32_t>& inputs) {
+    std::vector<uint8_t> need((size_t)N, 0), next((size_t)N, 0);
+    for (int t = 0; t < n_out; ++t) need[(size_t)outs[t]] = 1;
+    std::vector<int32_t> rowptr, col;
+    for (int l = n_layers - 1; l >= 0; --l) {   // from the last layer of the range back to its first
+        plan_adjacency(plans[l], N, rowptr, col);
+        std::fill(next.begin(), next.end(), 0);
+        for (int j = 0; j < N; ++j)
+            if (need[(size_t)j])
+                for (int e = rowptr[(size_t)j]; e < rowptr[(size_t)j + 1]; ++e) next[(size_t)col[(size_t)e]] = 1;
+        need.swap(next);
+    }
+    inputs.clear();
+    for (int i = 0; i < N; ++i) if (need[(size_t)i]) inputs.push_back(i);
+}
+
+bool pair_fusable(const LayerPlan& a, const LayerPlan& b, int N) {
+    if (a.kernel != SPDNN_KERNEL_BAND || b.kernel != SPDNN_KERNEL_BAND) return false;
+    if (a.kmax != 32 || b.kmax != 32 || a.wmode != b.wmode) return false;
+    if (a.pair_steps > 36 || b.pair_steps > 36 || a.pair_stride != 16 || b.pair_stride != 16) return false;
+    if (a.info.band_halo > 32 || b.info.band_halo > 32 || N < 256 || (N % 256) != 0) return false;
+    if ((int)a.dst.size() != N) return false;
+    for (int v = 0; v < N; ++v) if (a.dst[(size_t)v] != v) return false;
+    return true;
 }
 
 void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos) {

@@ -49,6 +49,11 @@ struct LayerPlan {
     std::vector<int32_t> alt_cnt;    // [alt_ngroups]
     std::vector<int32_t> alt_out_at; // [alt_ngroups*16] output neuron of the slot, -1 = unused
     std::vector<int32_t> alt_dst;    // [alt_ngroups*16] physical column in the next buffer
+    // BAND: neuron j sits at the same band position as an input and as an output (see
+    // canonicalize_self_aligned_band); fuse_next: this layer writes its outputs exactly where the
+    // next layer's band reads them (dst = identity) and both fit the fused pair kernel
+    bool self_aligned = false;
+    bool fuse_next = false;
 };
 
 // Sorts every row of the CSR by input index (stable) and validates it.  Returns an empty
@@ -83,6 +88,23 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
 // every layer uses the unfused pair.
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan);
+
+// The layer's structure back from its plan: rowptr[N+1] / col[] with row = output neuron and the
+// input neurons of every row ascending.
+void plan_adjacency(const LayerPlan& plan, int N, std::vector<int32_t>& rowptr, std::vector<int32_t>& col);
+
+// Receptive field of a block of output neurons through n_layers consecutive layers (plans[0] is the
+// first of them): the input neurons of plans[0] that the outputs `outs` of plans[n_layers-1] depend
+// on, ascending.  The analysis of the reference's FuseLayer (src/fuse/fuse.h:13-53: the constructor
+// collects the entries of the last layer that lead into the block, every fuse() call carries the
+// set one layer further back).
+void receptive_field(const LayerPlan* plans, int N, int n_layers, const int32_t* outs, int n_out,
+                     std::vector<int32_t>& inputs);
+
+// Whether layers a and b (consecutive, a already linked to b) can run as one fused launch: both
+// circulant or run-chain bands of 32 entries per row in the unrolled record form with the same
+// weight mode, a's outputs landing exactly on b's band (dst = identity).
+bool pair_fusable(const LayerPlan& a, const LayerPlan& b, int N);
 
 // dst[slot] = physical column (in the next buffer) of the neuron computed at `slot`.
 void link_layers(LayerPlan& cur, const std::vector<int32_t>* next_in_pos);

@@ -598,6 +598,220 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
+// Fused pair ("fused" variant with the intermediate tile in LDS): two consecutive BAND layers A
+// and B, where A writes its outputs exactly where B's band reads them (dst of A = identity), run
+// in ONE launch and the activations between them never leave the CU.  The reference fuses the same
+// way: a tile of the last layer's outputs, the tile of the layer before sized to cover its halo,
+// the intermediate kept in shared memory (src/microbenchmark/fuse.cu:16-110, tile recurrence
+// :226-248; the analysis that says which inputs a tile needs is src/fuse/fuse.h:13-53).
+//
+// A workgroup of 16 waves takes one row block (256 rows) and a segment [vb, ve) of B's band
+// positions.  Waves 0-7 walk layer A over positions [vb-32, ve) - B's halo of up to 32 positions is
+// computed again by the workgroup of the segment before, the price of not sharing tiles between
+// workgroups - from a 64-slot LDS ring fed straight from HBM, and drop their outputs, after the
+// epilogue, into a second 64-slot ring.  Waves 8-15 walk layer B over [vb, ve) three chunks behind,
+// reading the second ring and storing to HBM.  One barrier per chunk of 16 positions; at step s
+// layer A writes ring positions [vb-32+16s, vb-16+16s) while layer B reads [vb-80+16s, vb-32+16s):
+// 64 consecutive positions, so no slot is written while it is read.
+// HBM traffic per pair of layers: one read and one write of the feature block (plus A's halo of
+// 64 columns per segment) instead of two of each.
+// ------------------------------------------------------------------------------------------
+struct PairSide {
+    float wu;
+    int halo;
+    int steps;
+};
+
+// The 2 x 4 x steps multiply-adds of one output pair for a lane's four rows, inputs from an LDS ring
+// (16-dword pair records: two 64-bit use masks, 36 one-byte ring selectors; weights per step and
+// output unless WMODE is 0).  The LDS read of step s+2 is issued before the arithmetic of step s.
+template <int WMODE>
+__device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, const uint32_t* __restrict__ pairs,
+                                                const float* __restrict__ pw, int pr, int steps, uint32_t wu_bits,
+                                                float (&acc)[2][4]) {
+    const uint4* rec = reinterpret_cast<const uint4*>(pairs + (size_t)pr * 16);
+    const uint4 mk = rec[0], sa = rec[1], sb = rec[2];
+    const uint32_t sc = pairs[(size_t)pr * 16 + 12];
+    const float4* wp = nullptr;
+    float4 w_cur[2], w_nxt[2];
+    if (WMODE) {
+        wp = reinterpret_cast<const float4*>(pw + (size_t)pr * 72);
+        w_cur[0] = wp[0];
+        w_cur[1] = wp[1];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[0][q] = acc[1][q] = 0.0f;
+    float xb[3][4];
+#define SPDNN_PSLOT(e)                                                                                   \
+    (((((e) >> 2) == 0 ? sa.x : ((e) >> 2) == 1 ? sa.y : ((e) >> 2) == 2 ? sa.z : ((e) >> 2) == 3 ? sa.w  \
+       : ((e) >> 2) == 4 ? sb.x : ((e) >> 2) == 5 ? sb.y : ((e) >> 2) == 6 ? sb.z : ((e) >> 2) == 7 ? sb.w : sc) >> (8 * ((e) & 3))) & 63u)
+#define SPDNN_PUSED(o, e) (((((e) < 32) ? ((o) ? mk.z : mk.x) : ((o) ? mk.w : mk.y)) >> ((e) & 31)) & 1u)
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+        vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(e) * 1024), xb[e]);
+#pragma unroll
+    for (int st = 0; st < 36; ++st) {
+        if (st + 2 < 36 && (st + 2 < 32 || st + 2 < steps))
+            vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(st + 2) * 1024), xb[(st + 2) % 3]);
+        if (WMODE && (st & 3) == 0 && st + 4 < 36) {
+            w_nxt[0] = wp[(st >> 2) * 2 + 2];
+            w_nxt[1] = wp[(st >> 2) * 2 + 3];
+        }
+        if (st < 32 || st < steps) {
+            float w0, w1;
+            if (WMODE) {
+                const float4 wq = w_cur[(st >> 1) & 1];
+                w0 = (st & 1) ? wq.z : wq.x;
+                w1 = (st & 1) ? wq.w : wq.y;
+            } else {
+                w0 = __uint_as_float(wu_bits & (0u - SPDNN_PUSED(0, st)));
+                w1 = __uint_as_float(wu_bits & (0u - SPDNN_PUSED(1, st)));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                acc[0][q] = mac<WMODE>(acc[0][q], xb[st % 3][q], w0);
+                acc[1][q] = mac<WMODE>(acc[1][q], xb[st % 3][q], w1);
+            }
+        }
+        if (WMODE && (st & 3) == 3 && st + 1 < 36) {
+            w_cur[0] = w_nxt[0];
+            w_cur[1] = w_nxt[1];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {   // keeps the reads of later steps behind this step's arithmetic
+            asm volatile("" : "+v"(acc[0][q]) : : "memory");
+            asm volatile("" : "+v"(acc[1][q]) : : "memory");
+        }
+    }
+#undef SPDNN_PSLOT
+#undef SPDNN_PUSED
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(1024) void band_pair_kernel(
+    Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs_a, const float* __restrict__ pw_a,
+    const uint32_t* __restrict__ pairs_b, const float* __restrict__ pw_b, PairSide A, PairSide B,
+    const int32_t* __restrict__ dst,
+    int32_t* __restrict__ active, int32_t* __restrict__ active_mid, int32_t* __restrict__ count_prev, int N,
+    int seglen, int stamp_a, int stamp_b, int prev_stamp, int check_dead, float bias, float clampv, Publish pub,
+    int nblk, int stream) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int RB = 256, COLB = 1024, T = 16;
+    unsigned char* ring_a = smem;                 // inputs of layer A, 64 column slots
+    unsigned char* ring_b = smem + 64 * COLB;     // outputs of layer A = inputs of layer B
+    publish_counts(pub);
+    if ((int)blockIdx.x >= nblk) return;
+    const int rb = blockIdx.x;
+    const int vb = blockIdx.y * seglen;
+    const int ve = min(N, vb + seglen);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int role = wave >> 3, w = wave & 7;     // role 0: layer A, role 1: layer B
+    const int loff = lane * 4;
+    if (enter_row_block<4>(active, (size_t)rb * RB + loff, prev_stamp, stamp_a, check_dead, count_prev,
+                           blockIdx.y == 0 && threadIdx.x < 64))
+        return;
+    const size_t blkf = (size_t)N * RB;
+    const float* __restrict__ yin = block_base(yin_all, rb, blkf);
+    float* __restrict__ yout = block_base(yout_all, rb, blkf);
+    const int nb = (ve - vb) / T;                 // chunks of layer B (segments are whole chunks)
+    const int na = nb + 2;                        // chunks of layer A: B's halo of 32 positions first
+    const int va0 = vb - 32;                      // first position layer A computes (may be negative: wraps)
+    float nz[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const uint32_t wu_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(role ? B.wu : A.wu));
+
+    if (role == 0) {
+        // layer A's halo and first chunk
+        for (int c = w; c < A.halo + T; c += 8) {
+            const int p = va0 - A.halo + c;
+            const int g = p < 0 ? p + N : p;
+            unsigned char* slot = ring_a + (size_t)(p & 63) * COLB;
+            if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
+            else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+        }
+        wait_vector_memory();
+    }
+    ring_barrier<1>();
+
+    for (int s = 0; s < nb + 3; ++s) {
+        if (role == 0) {
+            if (s < na) {
+                const int cb = va0 + s * T;
+                if (s + 1 < na) {
+#pragma unroll
+                    for (int i = 0; i < 2; ++i) {
+                        const int p = cb + T + w + i * 8;
+                        const int g = p < 0 ? p + N : p;
+                        unsigned char* slot = ring_a + (size_t)(p & 63) * COLB;
+                        if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
+                        else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+                    }
+                }
+                const int v0 = cb + 2 * w;
+                const int pr = (v0 < 0 ? v0 + N : v0) >> 1;
+                float acc[2][4];
+                pair_accumulate<WMODE>(ring_a + loff * 4, pairs_a, pw_a, pr, A.steps, wu_bits, acc);
+                float y0[4], y1[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    y0[q] = relu_clamp(acc[0][q] + bias, clampv);
+                    y1[q] = relu_clamp(acc[1][q] + bias, clampv);
+                    nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));
+                }
+                *reinterpret_cast<float4*>(ring_b + (size_t)(v0 & 63) * COLB + loff * 4) = arr_to_vec<4>(y0);
+                *reinterpret_cast<float4*>(ring_b + (size_t)((v0 + 1) & 63) * COLB + loff * 4) = arr_to_vec<4>(y1);
+                wait_vector_memory();   // the next chunk's columns are in ring A
+            }
+        } else if (s >= 3) {
+            const int v0 = vb + (s - 3) * T + 2 * w;
+            float acc[2][4];
+            pair_accumulate<WMODE>(ring_b + loff * 4, pairs_b, pw_b, v0 >> 1, B.steps, wu_bits, acc);
+            float y0[4], y1[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                y0[q] = relu_clamp(acc[0][q] + bias, clampv);
+                y1[q] = relu_clamp(acc[1][q] + bias, clampv);
+                nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));
+            }
+            const int d0 = dst[v0], d1 = dst[v0 + 1];
+            if (stream) {
+                store_stream<4>(yout + (size_t)d0 * RB + loff, y0);
+                store_stream<4>(yout + (size_t)d1 * RB + loff, y1);
+            } else {
+                *reinterpret_cast<float4*>(yout + (size_t)d0 * RB + loff) = arr_to_vec<4>(y0);
+                *reinterpret_cast<float4*>(yout + (size_t)d1 * RB + loff) = arr_to_vec<4>(y1);
+            }
+        }
+        ring_barrier<1>();
+    }
+
+    // row stamps: layer A's into active_mid, layer B's into active (the rings are free now)
+    float* sm = reinterpret_cast<float*>(smem);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) sm[wave * RB + loff + q] = nz[q];
+    __syncthreads();
+    if (threadIdx.x < 2 * RB) {
+        const int which = threadIdx.x >> 8, r = threadIdx.x & 255;
+        float m = sm[(which * 8) * RB + r];
+#pragma unroll
+        for (int k = 1; k < 8; ++k) m = nz_merge(m, sm[(which * 8 + k) * RB + r]);
+        if (m > 0.0f) {
+            if (which) active[(size_t)rb * RB + r] = stamp_b;
+            else active_mid[(size_t)rb * RB + r] = stamp_a;
+        }
+    }
+}
+
+// rows of [0, rows) that carry `stamp`: the count of a layer whose stamps no later launch looks at
+__global__ __launch_bounds__(256) void count_stamped_kernel(const int32_t* __restrict__ stamps, int rows, int stamp,
+                                                            int32_t* __restrict__ count_out) {
+    const int r = blockIdx.x * blockDim.x + threadIdx.x;
+    const int hit = (r < rows && stamps[r] == stamp) ? 1 : 0;
+    const int n = (int)__popcll(__ballot(hit));
+    if ((threadIdx.x & 63) == 0 && n > 0) atomicAdd(count_out, n);
+}
+
+// ------------------------------------------------------------------------------------------
 // GATHER kernel (general CSR / ELL): any sparsity pattern, any row length.  Each wave takes
 // OPG consecutive outputs of one row block and reads every input column straight from
 // global memory (L2), RB*4 contiguous bytes per read.  No reuse beyond the caches: this is the
@@ -1145,6 +1359,61 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
         case 1: return launch_chain_rl<1, 16, 2, 128>(a, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+int band_pair_seglen(int N, int nblk, int n_cu) {
+    // one workgroup per CU (128 KiB of LDS); a segment of c chunks costs c + 3 steps
+    const int slots = n_cu > 0 ? n_cu : 256;
+    const int nchunks = N / 16;
+    int best_len = N;
+    double best = -1.0;
+    for (int nseg = 1; nseg <= nchunks / 8 && nseg <= 65535; ++nseg) {
+        const int cps = (nchunks + nseg - 1) / nseg;
+        if ((nchunks + cps - 1) / cps != nseg) continue;
+        const long long wgs = (long long)nblk * nseg;
+        const long long rounds = (wgs + slots - 1) / slots;
+        const double score = (double)wgs / (double)(rounds * slots) * (double)cps / (double)(cps + 3);
+        if (score > best + 1e-9) { best = score; best_len = cps * 16; }
+    }
+    return best_len;
+}
+
+hipError_t launch_band_pair(const PairLaunch& a, hipStream_t s) {
+    if (a.N < 256 || (a.N % 256) != 0 || a.nblk <= 0 || a.rl != 4 || !a.yin || !a.yout || !a.pairs_a || !a.pairs_b ||
+        !a.dst || !a.active || !a.active_mid || a.halo_a < 0 || a.halo_a > 32 || a.halo_b < 0 || a.halo_b > 32 ||
+        a.steps_a < 32 || a.steps_a > 36 || a.steps_b < 32 || a.steps_b > 36 || (a.wmode != 0 && (!a.pw_a || !a.pw_b)))
+        return hipErrorInvalidValue;
+    int seglen = a.seglen > 0 ? a.seglen - a.seglen % 16 : 0;
+    if (seglen <= 0) seglen = band_pair_seglen(a.N, a.nblk, a.n_cu);
+    const int nseg = (a.N + seglen - 1) / seglen;
+    if (nseg > 65535) return hipErrorInvalidValue;
+    constexpr size_t lds = 128 * 1024;
+    PairSide A{a.wu_a, a.halo_a, a.steps_a}, B{a.wu_b, a.halo_b, a.steps_b};
+    const int stream = (long long)a.nblk * (long long)a.N * 1024 * 2 >= a.stream_min_bytes ? 1 : 0;
+    dim3 grid(a.nblk, nseg), block(1024);
+#define SPDNN_PAIR(WM)                                                                                              \
+    do {                                                                                                            \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(band_pair_kernel<WM>),     \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);  \
+        if (attr != hipSuccess) return attr;                                                                        \
+        hipLaunchKernelGGL(band_pair_kernel<WM>, grid, block, lds, s, a.yin, a.yout, a.pairs_a, a.pw_a, a.pairs_b,  \
+                           a.pw_b, A, B, a.dst, a.active,                                                           \
+                           a.active_mid, a.count_prev, a.N, seglen, a.stamp_a, a.stamp_b, a.prev_stamp, a.check_dead, \
+                           a.bias, a.clampv, a.publish, a.nblk, stream);                                            \
+    } while (0)
+    switch (a.wmode) {
+        case 0: SPDNN_PAIR(0); break;
+        case 1: SPDNN_PAIR(1); break;
+        default: SPDNN_PAIR(2); break;
+    }
+#undef SPDNN_PAIR
+    return hipGetLastError();
+}
+
+hipError_t launch_count_stamped(const int32_t* stamps, int rows, int stamp, int32_t* count_out, hipStream_t s) {
+    if (rows <= 0 || !stamps || !count_out) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(count_stamped_kernel, dim3((rows + 255) / 256), dim3(256), 0, s, stamps, rows, stamp, count_out);
+    return hipGetLastError();
 }
 
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {

@@ -134,6 +134,36 @@ struct ChainLaunch {
 };
 hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s);
 
+// Fused pair: two consecutive BAND layers (32 entries per row, unrolled record form, same weight
+// mode, rows per lane 4) of which the first writes its outputs exactly where the second reads them
+// (dst = identity) in one launch; the activations between them stay in LDS.  `dst` is the second
+// layer's.  Rows the first layer leaves active get stamp_a in active_mid (no other launch looks at
+// that array: count them with launch_count_stamped), rows the second leaves active stamp_b in active.
+struct PairLaunch {
+    Feat yin;
+    Feat yout;
+    const uint32_t* pairs_a;
+    const float* pw_a;
+    const uint32_t* pairs_b;
+    const float* pw_b;
+    const int32_t* dst;
+    int32_t* active;
+    int32_t* active_mid;
+    int32_t* count_prev;     // as in BandLaunch, for the layer before the pair
+    int N, nblk, rl, wmode;
+    int halo_a, steps_a, halo_b, steps_b;
+    int stamp_a, stamp_b, prev_stamp, check_dead;
+    int seglen;              // band positions of the second layer per workgroup, 0 = heuristic
+    int n_cu;
+    long long stream_min_bytes;
+    float wu_a, wu_b, bias, clampv;
+    Publish publish;
+};
+hipError_t launch_band_pair(const PairLaunch& a, hipStream_t s);
+int band_pair_seglen(int N, int nblk, int n_cu);
+// count_out += number of rows r < rows with stamps[r] == stamp
+hipError_t launch_count_stamped(const int32_t* stamps, int rows, int stamp, int32_t* count_out, hipStream_t s);
+
 // Active-row scan: rows with active[row] == stamp and gid[row] >= 0 survive, in order.
 // Writes count[0] = number of survivors, alive_src[k] = physical row of survivor k,
 // alive_gid[k] = its global id.

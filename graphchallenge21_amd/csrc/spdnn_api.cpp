@@ -225,6 +225,7 @@ struct spdnn_net {
     Feat F, A, C;             // features as handed over, and the two work buffers the layers ping-pong between
     std::vector<float*> feat_allocs;  // the allocations behind them
     int feat_paired = 0, feat_candidates = 0;
+    int32_t* d_active_mid = nullptr;  // row stamps of the first layer of a fused pair (see PairLaunch)
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
@@ -250,6 +251,9 @@ struct spdnn_net {
     // cleared when every carried block has been written again (new run, repack).
     bool blocks_skipped = false;
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
+    bool fuse_pairs = true;   // fused pairs where the inspector found them (SPDNN_FUSE_PAIRS=0: never)
+    int pair_seglen = 0;      // band positions per workgroup of a fused pair, 0 = heuristic (SPDNN_PAIR_SEGLEN)
+    int64_t pair_min_elems = 0;  // rows x neurons below which a pair runs as two launches (SPDNN_PAIR_MIN_ELEMS)
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
@@ -274,6 +278,7 @@ struct spdnn_net {
 namespace {
 
 void release_device_base(spdnn_net* n) {
+    hipFree(n->d_active_mid); n->d_active_mid = nullptr;
     hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
     hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
     hipFree(n->d_counts);
@@ -313,6 +318,8 @@ int init_device(spdnn_net* n) {
     HIPCHK(hipEventCreate(&n->ev_stop));
     const size_t rows = (size_t)n->rows_cap;
     HIPCHK(hipMalloc(&n->d_active, rows * 4));
+    HIPCHK(hipMalloc(&n->d_active_mid, rows * 4));
+    HIPCHK(hipMemset(n->d_active_mid, 0, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid, rows * 4));
     HIPCHK(hipMalloc(&n->d_gid_tmp, rows * 4));
     HIPCHK(hipMalloc(&n->d_alive_src, rows * 4));
@@ -680,6 +687,7 @@ hipError_t labelling_dev(spdnn_net* n, int layers_done, const int32_t** out) {
 void reset_state(spdnn_net* n) {
     if (n->stamp > 0x60000000) {  // row stamps are launch numbers: start over long before they wrap
         hipMemsetAsync(n->d_active, 0, (size_t)n->rows_cap * 4, n->stream);
+        hipMemsetAsync(n->d_active_mid, 0, (size_t)n->rows_cap * 4, n->stream);
         n->stamp = 0;
     }
     if (n->gid_dirty) {
@@ -739,6 +747,9 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
     if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
+    if (const char* e = getenv("SPDNN_FUSE_PAIRS")) n->fuse_pairs = atoi(e) != 0;
+    if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
+    if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
     if (const char* e = getenv("SPDNN_STREAM_MIN_BYTES")) n->stream_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_COUNT_TIMEOUT_MS")) n->count_timeout_ms = std::max(1ll, atoll(e));
@@ -924,6 +935,11 @@ int spdnn_inspect(spdnn_net* n) {
         n->pool->submit([=] { link_layers(*cur, nxt); });
     }
     n->pool->wait_all();
+    for (int l = 0; l < n->L; ++l) {
+        LayerPlan& p = n->layers[(size_t)l];
+        p.fuse_next = l + 1 < n->L && n->rl == 4 && pair_fusable(p, n->layers[(size_t)l + 1], n->N);
+        p.info.fuse_next = p.fuse_next ? 1 : 0;
+    }
     if (n->uploaded) free_device(n);  // plans changed: upload again on next use
     n->tuned.clear();
     n->exploring.clear();
@@ -996,6 +1012,23 @@ int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
     if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
     const LayerPlan& p = n->layers[(size_t)layer];
     std::copy(p.dst.begin(), p.dst.end(), dst);
+    return SPDNN_OK;
+}
+
+int spdnn_receptive_field(spdnn_net* n, int first_layer, int n_layers, const int32_t* out_neurons, int n_out,
+                          int32_t* in_neurons, int64_t cap, int64_t* count) {
+    if (!n || !count || (n_out > 0 && !out_neurons)) return fail(SPDNN_E_ARG, "NULL argument");
+    if (first_layer < 0 || n_layers < 1 || first_layer + n_layers > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
+    if (n_out < 0 || cap < 0) return fail(SPDNN_E_ARG, "negative size");
+    for (int t = 0; t < n_out; ++t)
+        if (out_neurons[t] < 0 || out_neurons[t] >= n->N) return fail(SPDNN_E_ARG, "neuron out of range");
+    n->pool->wait_all();
+    for (int l = first_layer; l < first_layer + n_layers; ++l)
+        if (!n->layers[(size_t)l].set) return fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
+    std::vector<int32_t> in;
+    receptive_field(&n->layers[(size_t)first_layer], n->N, n_layers, out_neurons, n_out, in);
+    *count = (int64_t)in.size();
+    if (in_neurons) std::copy(in.begin(), in.begin() + (size_t)std::min<int64_t>(cap, (int64_t)in.size()), in_neurons);
     return SPDNN_OK;
 }
 
@@ -1351,6 +1384,8 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     const bool have_counts = fused_count || scan_count;
     if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
     int fuse = opt.fuse_layers ? opt.fuse_layers : n->default_fuse;
+    // fused pairs: with fused launches asked for (fuse_layers >= 2, or SPDNN_FUSE_LAYERS as the default)
+    const bool pair_mode = n->fuse_pairs && !scan_count && !plans_streamed(n) && fuse >= 2;
     if (scan_count || fuse < 2 || plans_streamed(n)) fuse = 1;  // a fused launch needs all its plans resident
     if (plans_streamed(n))
         for (int l = first; l <= last && l < first + n->plan_window; ++l) HIPCHK(plan_fetch(n, l));
@@ -1398,7 +1433,12 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         }
         // chain length: consecutive BAND layers with the same row length and weight mode
         int c = 1;
-        if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
+        // a fused pair (intermediate tile in LDS) where the inspector found one; not while the band
+        // walk's BLOCK form would run the layers (small batches of run-chain layers)
+        const bool pair = pair_mode && p.fuse_next && l + 1 <= last && !use_block_form(n, p, n->carried / n->RB) &&
+                          (int64_t)(n->carried / n->RB) * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems;
+        if (pair) c = 2;
+        else if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
             while (c < fuse && l + c <= last) {
                 const LayerPlan& q = n->layers[(size_t)(l + c)];
                 if (q.kernel != SPDNN_KERNEL_BAND || q.kmax != p.kmax || q.wmode != p.wmode ||
@@ -1460,6 +1500,21 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
                 if (rc) return rc;
             }
             HIPCHK(plan_release(n, l));
+        } else if (pair) {
+            const LayerPlan& q = n->layers[(size_t)l + 1];
+            const DevLayer &da = n->dl[(size_t)l], &db = n->dl[(size_t)l + 1];
+            PairLaunch pl{};
+            pl.yin = in; pl.yout = out; pl.pairs_a = da.pairs; pl.pw_a = da.wv; pl.pairs_b = db.pairs; pl.pw_b = db.wv;
+            pl.dst = db.dst; pl.active = n->d_active; pl.active_mid = n->d_active_mid; pl.count_prev = count_prev;
+            pl.N = n->N; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = p.wmode;
+            pl.halo_a = p.info.band_halo; pl.steps_a = p.pair_steps; pl.halo_b = q.info.band_halo; pl.steps_b = q.pair_steps;
+            pl.stamp_a = stamp0; pl.stamp_b = stamp0 + 1; pl.prev_stamp = prev_stamp; pl.check_dead = check_dead;
+            pl.seglen = n->pair_seglen; pl.n_cu = n->n_cu; pl.stream_min_bytes = n->stream_min_bytes;
+            pl.wu_a = p.info.value; pl.wu_b = q.info.value; pl.bias = n->bias; pl.clampv = n->clampv;
+            pl.publish = pub;
+            HIPCHK(launch_band_pair(pl, n->stream));
+            // the first layer's rows: nobody looks at active_mid again, so they are counted here
+            if (fused_count) HIPCHK(launch_count_stamped(n->d_active_mid, n->carried, stamp0, n->d_counts + l, n->stream));
         } else {
             ChainLaunch ch{};
             ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
@@ -1475,6 +1530,8 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
         }
         if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back({l, c}); }
         r.layers_run += c;
+        r.launches += 1;
+        if (pair) r.fused_pairs += 1;
         last_launched = l + c - 1;
         n->last_stamp = stamp0 + c - 1;
         n->cur = out;
@@ -1489,10 +1546,12 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             // this launch's start) and, of a fused launch, its own layers'.  The next launch hands
             // them to the host; this launch handed over the ones before (pub).
             if (polled && pub.n > 0) recs.push_back({(int)(pub.src - n->d_counts), pub.n});
-            const int lo = count_prev ? l - 1 : l, hi = c == 1 ? l : l + c;
+            // (a chain counts all its layers itself; of a pair the first layer is counted behind the
+            // launch and the second, like a single layer, by whatever comes next)
+            const int lo = count_prev ? l - 1 : l, hi = c == 1 ? l : (pair ? l + 1 : l + c);
             pub = Publish{};
             if (polled && hi > lo) { pub.src = n->d_counts + lo; pub.dst = n->h_counts + lo; pub.n = hi - lo; }
-            count_pending = c == 1;  // a single layer's rows are counted by whatever comes next
+            count_pending = c == 1 || pair;
         }
         l += c;
         if (!opt.prune) continue;

@@ -73,7 +73,8 @@ typedef struct spdnn_layer_plan {
     int64_t plan_bytes;      /* device bytes held for this layer                                  */
     int32_t block_form;      /* 1: a run-chain BAND layer that also holds its BLOCK form, which
                                 spdnn_run uses on small batches                                   */
-    int32_t reserved;
+    int32_t fuse_next;       /* 1 (after spdnn_inspect): this layer and the next can run as one fused launch, the
+                                activations between them kept in LDS (see spdnn_run_options.fuse_layers)  */
 } spdnn_layer_plan;
 
 typedef struct spdnn_run_options {
@@ -83,8 +84,11 @@ typedef struct spdnn_run_options {
     int32_t collect_counts;    /* 1: record the active-row count after every layer                 */
     int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
-    int32_t fuse_layers;       /* >1: fused variant, up to that many consecutive band layers per launch
-                                  (one workgroup keeps a row block through the chain); 1 = off; 0 = default */
+    int32_t fuse_layers;       /* fused variants.  1 = every layer its own launch; 0 = default (the same, unless
+                                  SPDNN_FUSE_LAYERS says otherwise).  >1: pairs of layers the inspector marked
+                                  fuse_next run as one launch with the intermediate tile in LDS, and elsewhere up
+                                  to that many consecutive band layers share a launch (one workgroup keeps a row
+                                  block through the chain, the intermediates going through L2) */
     int32_t reserved[3];
 } spdnn_run_options;
 
@@ -97,6 +101,8 @@ typedef struct spdnn_run_result {
     float   ms_kernels;      /* sum of per-layer kernel times (time_layers only, else 0)          */
     double  alg_bytes;       /* sum over layers of 8*B_l*N + nnz_l*8 + 4*(N+1)                     */
     double  edges;           /* batch * nnz summed over the layers requested                      */
+    int32_t launches;        /* layer-kernel launches made (a fused launch counts once)           */
+    int32_t fused_pairs;     /* of them, fused pairs of layers (intermediate tile in LDS)         */
 } spdnn_run_result;
 
 /* ---- life cycle ------------------------------------------------------------------------- */
@@ -215,6 +221,18 @@ int spdnn_get_band_pairs(const spdnn_net* net, int layer, int* steps, int* strid
                          int* has_weights, uint32_t* records, float* weights);
 
 int spdnn_get_layer_dst(const spdnn_net* net, int layer, int32_t* dst);
+
+/* Receptive field of a block of output neurons through consecutive layers: the input neurons of layer
+ * first_layer that the neurons out_neurons[0..n_out) of layer first_layer + n_layers - 1 depend on -
+ * the analysis of the reference's FuseLayer (src/fuse/fuse.h:13-53: the constructor gathers the inputs
+ * of a block of output columns of one layer, every fuse() call carries the set one layer further
+ * back), on which its fused kernel sizes the tile of the layer before (src/microbenchmark/fuse.cu:226-248).
+ * *count receives the size of the set; in_neurons (may be NULL) its first min(*count, cap) members,
+ * ascending.  A pair of layers can keep its intermediate tile on chip only where this set stays a
+ * small multiple of the block for every block of a tiling; spdnn_inspect marks the pairs it fuses
+ * (spdnn_layer_plan.fuse_next).  Host only; needs the layers set (their inspection is waited for). */
+int spdnn_receptive_field(spdnn_net* net, int first_layer, int n_layers, const int32_t* out_neurons, int n_out,
+                          int32_t* in_neurons, int64_t cap, int64_t* count);
 
 /* Physical column of every neuron in the buffer layer `layer` reads (layer == layers: the
  * final output, always the identity). */

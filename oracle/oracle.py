@@ -17,6 +17,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 REF_CHECK = os.path.join(_HERE, "_ref", "ref_check")
 
 _i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
+_u8p = np.ctypeslib.ndpointer(dtype=np.uint8, flags="C_CONTIGUOUS")
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
 
 
@@ -61,6 +62,8 @@ def _load():
     lib.orc_layer.argtypes = [_f32p, C.c_int64, C.c_int, _i32p, _i32p, _f32p, C.c_float, _f32p, _i32p]
     lib.orc_compact.restype = C.c_int64
     lib.orc_compact.argtypes = [_f32p, C.c_int64, C.c_int, _i32p, _i32p, _f32p, _i32p]
+    lib.orc_need_access.restype = None
+    lib.orc_need_access.argtypes = [C.c_int, _i32p, _i32p, _u8p, _u8p]
     return lib
 
 
@@ -238,3 +241,16 @@ def infer(features, layers, bias, prune=True, keep=None):
         l += 1
     return {"active_ids": active_ids, "y": y, "gid": gid, "kept": kept,
             "categories": active_ids[-1] if active_ids else gid}
+
+
+def receptive_field(layers, out_neurons):
+    """Input neurons of layers[0] that the output neurons `out_neurons` of layers[-1] depend on
+    (ascending): the reference's FuseLayer, one orc_need_access step per layer from the last back."""
+    neuron = len(layers[-1][0]) - 1
+    flags = np.zeros(neuron, np.uint8)
+    flags[np.asarray(out_neurons, dtype=np.int64)] = 1
+    for rowptr, col, _ in reversed(list(layers)):
+        nxt = np.zeros(neuron, np.uint8)
+        _lib.orc_need_access(neuron, np.ascontiguousarray(rowptr, np.int32), np.ascontiguousarray(col, np.int32), flags, nxt)
+        flags = nxt
+    return np.nonzero(flags)[0].astype(np.int32)

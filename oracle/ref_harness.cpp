@@ -18,8 +18,16 @@
 //       ftxj::CpuSpmmFuse::run_and_cmp(...) (src/utils/cpu_spmm_fuse.h:11-94), same verdict.
 //   ref_check transpose_delete <neuron> <old_batch> <new_batch> <input_T.f32> <map.i32> <output.f32>
 //       ftxj::CpuTransposeDelete::run_and_cmp (src/utils/cpu_transpose_and_delete.h:11-27).
+//   ref_check need_access <block> <w_last.tsv> [<w_before.tsv> ...]
+//       ftxj::FuseLayer (src/fuse/fuse.h:8-54) over blocks of <block> consecutive columns of the
+//       first file, then fuse() with every further file, then print_need_access().  The files are
+//       loaded with COOMatrix(file, 1, true), i.e. row = first number of a line = input neuron and
+//       col = second number = output neuron, so that the class's "rows a block of columns needs"
+//       reads as "input neurons a block of output neurons needs".
+#include <set>
 #include "utils/header.h"
 #include "reorder/header.h"
+#include "fuse/fuse.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -46,7 +54,7 @@ static std::vector<int> read_i32(const char* path, size_t n) {
 }
 
 int main(int argc, char** argv) {
-    if (argc < 2) { fprintf(stderr, "usage: ref_check coo|hash|spmm|fuse|transpose_delete ...\n"); return 2; }
+    if (argc < 2) { fprintf(stderr, "usage: ref_check coo|hash|spmm|fuse|transpose_delete|need_access ...\n"); return 2; }
     std::string cmd = argv[1];
     if (cmd == "coo" && argc == 3) {
         ftxj::COOMatrix coo(argv[2], 1, false);
@@ -88,6 +96,19 @@ int main(int argc, char** argv) {
         auto map = read_i32(argv[6], (size_t)old_batch);
         auto out = read_f32(argv[7], (size_t)neuron * new_batch);
         ftxj::CpuTransposeDelete::run_and_cmp(in.data(), map.data(), old_batch, neuron, new_batch, out.data());
+        return 0;
+    }
+    if (cmd == "need_access" && argc >= 4) {
+        const int block = atoi(argv[2]);
+        ftxj::COOMatrix last(argv[3], 1, true);
+        std::vector<std::vector<int>> block_cols;
+        for (int c = 0; c < last.col_number; c += block) {
+            block_cols.push_back(std::vector<int>());
+            for (int j = c; j < c + block && j < last.col_number; ++j) block_cols.back().push_back(j);
+        }
+        ftxj::FuseLayer fuse(last, block_cols);
+        for (int i = 4; i < argc; ++i) fuse.fuse(ftxj::COOMatrix(argv[i], 1, true));
+        fuse.print_need_access();
         return 0;
     }
     fprintf(stderr, "bad arguments\n");

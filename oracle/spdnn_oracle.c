@@ -312,3 +312,18 @@ int64_t orc_compact(const float* y, int64_t nrows, int neuron, const int* active
     }
     return n;
 }
+
+/* One step of the reference's receptive-field analysis (src/fuse/fuse.h): given a set of a layer's
+ * output neurons, the set of its input neurons that an entry of the layer connects to one of them.
+ * The constructor (fuse.h:13-24) does this for the last layer of a fused group - for every output
+ * column of the block it scans all entries and inserts the row of each entry of that column - and
+ * every fuse() call (fuse.h:38-53) does it again for the layer before, starting from the set found so
+ * far.  Sets are 0/1 flags per neuron here; the layer is CSR with row = output neuron, col = input. */
+void orc_need_access(int neuron, const int* rowptr, const int* col, const unsigned char* out_flags,
+                     unsigned char* in_flags) {
+    for (int i = 0; i < neuron; ++i) in_flags[i] = 0;
+    for (int j = 0; j < neuron; ++j) {
+        if (!out_flags[j]) continue;
+        for (int e = rowptr[j]; e < rowptr[j + 1]; ++e) in_flags[col[e]] = 1;
+    }
+}

@@ -45,6 +45,10 @@ void  orc_layer(const float* yin, int64_t nrows, int neuron,
 int64_t orc_compact(const float* y, int64_t nrows, int neuron, const int* active,
                     const int* gid_in, float* y_out, int* gid_out);
 
+/* ---- fusion analysis ---- */
+void orc_need_access(int neuron, const int* rowptr, const int* col, const unsigned char* out_flags,
+                     unsigned char* in_flags);
+
 #ifdef __cplusplus
 }
 #endif

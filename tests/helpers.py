@@ -88,3 +88,23 @@ def hub_block_csr(rng, n, values="uniform"):
     else:
         val = rng.uniform(-0.1, 0.15, size=k).astype(np.float32)
     return rowptr, col, val
+
+
+def common_band_csr(rng, n, perm, values="uniform", k=32):
+    """A convolution-like layer over a neuron order common to all layers of a network: the neuron at
+    place t of the order (neuron perm[t]) reads the neurons at places t-k+1 .. t (mod n).  With a
+    random `perm` the band is hidden; consecutive layers built over the same `perm` write their
+    outputs where the next one's band reads them."""
+    rows = [None] * n
+    for t in range(n):
+        rows[perm[t]] = np.sort(perm[(t - np.arange(k)) % n])
+    rowptr = np.arange(n + 1, dtype=np.int32) * k
+    col = np.concatenate(rows).astype(np.int32)
+    m = len(col)
+    if values == "uniform":
+        val = np.full(m, 0.0625, np.float32)
+    elif values == "pow2":
+        val = (np.ldexp(1.0, rng.integers(-5, -2, size=m)) * rng.choice([-1.0, 1.0], size=m, p=[0.1, 0.9])).astype(np.float32)
+    else:
+        val = rng.uniform(-0.05, 0.15, size=m).astype(np.float32)
+    return rowptr, col, val

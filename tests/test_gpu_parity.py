@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from helpers import random_csr, same_floats, sort_rows
+from helpers import common_band_csr
 
 pytestmark = pytest.mark.gpu
 
@@ -382,6 +383,81 @@ def test_fused_layer_chain(gc, orc, fuse, prune):
         net.run(prune=prune, first_layer=10, n_layers=L - 10, fuse_layers=1)
         assert np.array_equal(net.categories(), ref["categories"])
         assert same_floats(net.activations(cats), ref["y"])
+
+
+@pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
+@pytest.mark.parametrize("N,B", [(1024, 1500), (4096, 700)])
+def test_fused_pairs_in_lds(gc, orc, N, B, values):
+    """Layers that are bands over one common neuron order run two per launch, the activations between
+    them kept in LDS (the reference's fused kernel, src/microbenchmark/fuse.cu:16-110): counts of every
+    layer - the one inside a pair included -, categories and activations must be the oracle's, with
+    and without pruning, and the same as with every layer in its own launch."""
+    print("fused pairs N=%d B=%d %s" % (N, B, values), flush=True)
+    rng = np.random.default_rng(N + B)
+    L = 7
+    perm = rng.permutation(N)
+    layers = [common_band_csr(rng, N, perm, values) for _ in range(L)]
+    feats = orc.gen_features(8, N, 0, B, 0.10, 0.60)
+    ref = orc.infer(feats, layers, -0.3, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    assert want_counts[-1] > 0 and want_counts[-1] < B
+    with gc.Network(N, B, L, bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert [net.layer_plan(l).fuse_next for l in range(L)] == [1] * (L - 1) + [0]
+        net.set_features_dense(feats)
+        cats = ref["categories"]
+        for prune in (True, False):
+            for fuse in (2, 0):
+                r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert r.layers_run == L
+                assert (r.fused_pairs, r.launches) == ((3, 4) if fuse == 2 else (0, L))
+                assert [net.active_count(l) for l in range(L)] == want_counts
+                assert np.array_equal(net.categories(), cats)
+                assert same_floats(net.activations(cats), ref["y"])
+                dead = np.setdiff1d(np.arange(B), cats)[:64].astype(np.int32)
+                assert not net.activations(dead).any()
+        # stops and continuations that cut pairs differently: (0,1) 2 | (3,4) (5,6) and (0,1) (2,3) | 4 (5,6)
+        for cut in (3, 4, 1):
+            net.run(prune=True, first_layer=0, n_layers=cut, fuse_layers=2)
+            gid, y = ref["kept"][cut - 1]
+            assert np.array_equal(net.categories(), ref["active_ids"][cut - 1])
+            assert same_floats(net.activations(gid), y)
+            r = net.run(prune=False, first_layer=cut, n_layers=L - cut, collect_counts=True, fuse_layers=2)
+            assert r.fused_pairs == (L - cut) // 2
+            assert [net.active_count(l) for l in range(cut, L)] == want_counts[cut:]
+            assert np.array_equal(net.categories(), cats)
+            assert same_floats(net.activations(cats), ref["y"])
+
+
+def test_fused_pairs_full_batch(gc, orc):
+    """The fused pair on a batch of 60000 (235 row blocks, several segments per row block, streaming
+    loads and stores): an oracle row sample through 6 layers, and the whole batch against the run
+    with one launch per layer."""
+    N, B, L, S = 4096, 60000, 6, 768
+    print("fused pairs, full batch", flush=True)
+    rng = np.random.default_rng(77)
+    perm = rng.permutation(N)
+    layers = [common_band_csr(rng, N, perm, "uniform") for _ in range(L)]
+    ref = orc.infer(orc.gen_features(9, N, 0, S, 0.10, 0.60), layers, -0.35, prune=True)
+    with gc.Network(N, B, L, bias=-0.35) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.synth_features(9, B, 0.10, 0.60)
+        r = net.run(prune=True, collect_counts=True, fuse_layers=2)
+        assert r.fused_pairs == 3 and r.launches == 3
+        counts = [net.active_count(l) for l in range(L)]
+        cats = net.categories()
+        assert np.array_equal(cats[cats < S], ref["categories"])
+        assert same_floats(net.activations(ref["categories"]), ref["y"])
+        probe = cats[:: max(1, len(cats) // 512)].astype(np.int32)
+        y_fused = net.activations(probe)
+        net.run(prune=False, collect_counts=True, fuse_layers=1)
+        assert [net.active_count(l) for l in range(L)] == counts
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(probe), y_fused)
 
 
 def test_fused_chain_when_everything_dies(gc, orc):

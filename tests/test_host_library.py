@@ -9,7 +9,7 @@ import subprocess
 import numpy as np
 import pytest
 
-from helpers import hub_block_csr, radix_like_csr, random_csr, same_floats, sort_rows
+from helpers import common_band_csr, hub_block_csr, radix_like_csr, random_csr, same_floats, sort_rows
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 GOLD = os.path.join(ROOT, "tests", "golden")
@@ -251,6 +251,62 @@ def test_inspector_run_chains(gc, orc, n, monkeypatch):
             y = _emulate_band_layer(net, l, y, lambda v, m: val[rowptr[out_at[v]] + m])
             want, _ = orc.layer(want, layers[l], -0.3)
             assert np.array_equal(y[:, net.input_labelling(l + 1)], want), strides[l]
+
+
+def test_receptive_field_of_every_layer_class(gc, orc, monkeypatch):
+    """spdnn_receptive_field (the reference's FuseLayer analysis, src/fuse/fuse.h:13-53) works from the
+    inspector's plans: compare with the oracle on the CSR that was handed over, for band, run-chain,
+    block and gather layers, through one to four layers."""
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "512")
+    rng = np.random.default_rng(21)
+    n = 512
+    layers = [orc.gen_layer_csr(3, 0, n), radix_like_csr(rng, n, 64), hub_block_csr(rng, n),
+              sort_rows(random_csr(rng, n, rng.integers(0, 9, size=n), "general")), orc.gen_layer_csr(3, 1, n)]
+    with gc.Network(n, 4, len(layers), bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        kinds = [net.layer_plan(l).kernel for l in range(len(layers))]
+        assert kinds == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER, gc.KERNEL_BAND]
+        assert net.layer_plan(1).band_halo == 32
+        for first in range(len(layers)):
+            for depth in range(1, len(layers) - first + 1):
+                for outs in (np.arange(16), np.array([7]), rng.choice(n, 40, replace=False), np.arange(n)):
+                    got = net.receptive_field(first, depth, outs)
+                    assert np.array_equal(got, orc.receptive_field(layers[first:first + depth], outs))
+        with pytest.raises(gc.SpdnnError):
+            net.receptive_field(0, len(layers) + 1, [0])
+        with pytest.raises(gc.SpdnnError):
+            net.receptive_field(0, 1, [n])
+
+
+def test_fusable_pairs_are_found_by_the_inspector(gc, orc):
+    """Layers that are bands over one common neuron order write their outputs where the next one reads
+    them: the inspector gives them one labelling (dst = identity) and marks the pairs; the receptive
+    field of a tile through such a pair is the tile plus a halo, through a pair of the generator's
+    layers (a fresh permutation per layer) it is all but the whole row."""
+    rng = np.random.default_rng(22)
+    n = 1024
+    perm = rng.permutation(n)
+    flipped = perm[::-1].copy()
+    layers = [common_band_csr(rng, n, perm), common_band_csr(rng, n, perm, "pow2"), common_band_csr(rng, n, perm, "pow2"),
+              common_band_csr(rng, n, flipped, "pow2"), orc.gen_layer_csr(4, 0, n), orc.gen_layer_csr(4, 1, n)]
+    with gc.Network(n, 4, len(layers), bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        for l in range(4):     # the same places along the band for a neuron as input and as output, neuron 0 first
+            in_pos, out_at, _ = net.band_plan(l)
+            assert in_pos[0] == 0 and np.array_equal(in_pos[out_at], np.arange(n))
+        # layers 0-1 differ in weight mode, 1-2 fuse, 2-3 are bands over opposite orders, 3-4 and 4-5 unrelated
+        assert [net.layer_plan(l).fuse_next for l in range(len(layers))] == [0, 1, 0, 0, 0, 0]
+        assert np.array_equal(net.layer_dst(0), np.arange(n)) and np.array_equal(net.layer_dst(1), np.arange(n))
+        in_pos, out_at, _ = net.band_plan(2)
+        tile = out_at[256:256 + 64]                     # 64 consecutive band positions of layer 2
+        assert len(net.receptive_field(1, 2, tile)) == 64 + 2 * 31
+        assert len(net.receptive_field(1, 1, tile)) == 64 + 31
+        in_pos, out_at, _ = net.band_plan(5)
+        assert len(net.receptive_field(4, 2, out_at[:64])) > 0.95 * n
 
 
 def test_forced_gather(gc, orc):

@@ -163,3 +163,38 @@ def test_unsorted_rows_are_sorted_by_loader(orc):
     got = orc.coo_to_csr(rows, col, val, 32)
     want = sort_rows(csr)
     assert all(np.array_equal(a, b) for a, b in zip(got, want))
+
+
+def test_receptive_field_against_boolean_matrix_products(orc):
+    """FuseLayer's analysis is reachability through the layers' patterns: compare with dense
+    boolean products of the transposed patterns, and with what a band fixes in closed form."""
+    rng = np.random.default_rng(5)
+    n = 48
+    layers = [random_csr(rng, n, rng.integers(0, 5, size=n), "general") for _ in range(3)]
+    dense = []
+    for rowptr, col, _ in layers:
+        m = np.zeros((n, n), bool)          # m[out, in]
+        for j in range(n):
+            m[j, col[rowptr[j]:rowptr[j + 1]]] = True
+        dense.append(m)
+    for outs in ([0], [3, 4, 5, 6], list(range(16, 32)), []):
+        need = np.zeros(n, bool)
+        need[outs] = True
+        for depth in (1, 2, 3):
+            v = need.copy()
+            for m in reversed(dense[3 - depth:]):
+                v = (m & v[:, None]).any(axis=0)
+            got = orc.receptive_field(layers[3 - depth:], outs)
+            assert np.array_equal(got, np.nonzero(v)[0])
+    # a band of width 8 in natural order: a tile of T outputs needs T+7 inputs through one layer,
+    # T+14 through two, and the set is the tile's places shifted back
+    n, k, t0, T = 64, 8, 20, 10
+    rowptr = np.arange(n + 1, dtype=np.int32) * k
+    col = np.sort((np.arange(n)[:, None] - np.arange(k)[None, :]) % n, axis=1).reshape(-1).astype(np.int32)
+    band = (rowptr, col, np.ones(n * k, np.float32))
+    assert np.array_equal(orc.receptive_field([band], range(t0, t0 + T)), np.arange(t0 - 7, t0 + T))
+    assert np.array_equal(orc.receptive_field([band, band], range(t0, t0 + T)), np.arange(t0 - 14, t0 + T))
+    # a permutation matrix moves the block, whatever its size
+    perm = rng.permutation(n).astype(np.int32)
+    pm = (np.arange(n + 1, dtype=np.int32), perm, np.ones(n, np.float32))
+    assert np.array_equal(orc.receptive_field([pm], [1, 2, 3]), np.sort(perm[[1, 2, 3]]))

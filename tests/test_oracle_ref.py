@@ -139,6 +139,34 @@ def test_compaction_accepted_by_reference_transpose_delete(orc, tmp_path):
     assert ok.returncode == 0 and "[Success]" in ok.stdout
 
 
+def test_receptive_field_matches_reference_fuselayer(orc, tmp_path):
+    """orc_need_access against ftxj::FuseLayer (src/fuse/fuse.h): blocks of 16 output neurons of the
+    last layer through one, two and three layers - the committed 64-neuron fixtures and random layers."""
+    ref = _ref(orc)
+    rng = np.random.default_rng(9)
+    n = 64
+    fixture = [os.path.join(GOLD, "tiny_n64-l%d.tsv" % l) for l in (1, 2)]
+    layers = []
+    for f in fixture:
+        r, c, v, nr, nc = orc.read_weight_tsv(f)
+        layers.append(orc.coo_to_csr(r, c, v, n))
+    extra = random_csr(rng, n, rng.integers(1, 6, size=n), "general")
+    path3 = str(tmp_path / "extra.tsv")
+    _write_tsv(path3, extra, rng)
+    chain = [(layers + [extra], fixture + [path3]), (layers, fixture), ([extra], [path3])]
+    for lays, files in chain:
+        # FuseLayer starts from the LAST layer and fuses the earlier ones in turn
+        out = subprocess.run([ref, "need_access", "16"] + files[::-1], check=True, capture_output=True, text=True).stdout
+        blocks = [ln for ln in out.splitlines() if ln.startswith("block b = ")]
+        assert len(blocks) == n // 16
+        for b, ln in enumerate(blocks):
+            head, _, tail = ln.partition(" : ")
+            want = [int(x) for x in tail.split(",") if x.strip()]
+            assert "size = %d" % len(want) in head
+            got = orc.receptive_field(lays, range(16 * b, 16 * b + 16))
+            assert got.tolist() == want
+
+
 def test_oracle_reproduces_committed_fixtures(orc):
     """tests/golden/: TSV layers + features -> expected activations / categories (confirmed by the
     reference's comparators when the fixture was generated)."""
