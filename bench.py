@@ -143,7 +143,8 @@ def main():
     t_inspect = time.time() - t0
     plans = [net.layer_plan(l) for l in range(L)]
     n_band = sum(1 for p in plans if p.kernel == gc.KERNEL_BAND)
-    kernel_names = {gc.KERNEL_BAND: "band_walk_kernel", gc.KERNEL_BLOCK: "block_kernel", gc.KERNEL_GATHER: "gather_kernel"}
+    kernel_names = {gc.KERNEL_BAND: "band_walk_kernel", gc.KERNEL_BLOCK: "block_kernel", gc.KERNEL_GATHER: "gather_kernel",
+                    gc.KERNEL_TILED: "tiled_kernel"}
     kernels_used = sorted({kernel_names[p.kernel] for p in plans})
     nnz_layer = float(sum(p.nnz for p in plans)) / L     # the same for every layer except with --structure irregular
     t0 = time.time()

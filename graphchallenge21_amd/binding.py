@@ -6,7 +6,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-KERNEL_AUTO, KERNEL_GATHER, KERNEL_BAND, KERNEL_BLOCK = 0, 1, 2, 3
+KERNEL_AUTO, KERNEL_GATHER, KERNEL_BAND, KERNEL_BLOCK, KERNEL_TILED = 0, 1, 2, 3, 4
 
 _i32p = np.ctypeslib.ndpointer(dtype=np.int32, flags="C_CONTIGUOUS")
 _f32p = np.ctypeslib.ndpointer(dtype=np.float32, flags="C_CONTIGUOUS")
@@ -287,7 +287,7 @@ class Network:
     def layer_dst(self, layer):
         p = self.layer_plan(layer)
         slots = self.neuron
-        if p.kernel == KERNEL_BLOCK:
+        if p.kernel in (KERNEL_BLOCK, KERNEL_TILED):
             slots = C.c_int()
             _check(self._lib.spdnn_get_layer_slots(self._h, layer, C.byref(slots)))
             slots = slots.value

@@ -417,6 +417,102 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
     return true;
 }
 
+// TILED plan (layers that are neither a band nor groups of identical rows).  Outputs are cut into
+// tiles of 1024; a tile's input columns - the union over its outputs, ascending - are staged in LDS
+// in panels of 512 columns and every output of the tile takes its inputs from there, so a column
+// is read from memory once per tile instead of once per entry (the reference's general prototype
+// stages a block's input list in shared memory the same way, src/microbenchmark/
+// row-succ-no-transpose.cu:15-71).  A wave owns 64 outputs of the tile; per panel it works through
+// `rounds` rounds of 2 entries per output (outputs with fewer entries in the panel are padded with
+// weight -0), so the outputs of a tile are sorted by length before they are dealt to the waves.
+// Accumulation order: an output's entries are ascending in input index, the union is ascending, so
+// panel after panel, entry after entry is the order of the reference's CPU checker.
+// Returns false (plan untouched) when staging would not pay: more than four reads per input column.
+bool build_tiled_plan(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                      const std::vector<float>& val, LayerPlan& plan) {
+    constexpr int TO = kTileOutputs, PC = kPanelCols, WO = 64, NWV = TO / WO;
+    if (N < 64) return false;
+    const int ntiles = (N + TO - 1) / TO;
+    // outputs in the order of the middle of their input lists, so that a tile's union stays small
+    // where the layer has locality; empty rows last
+    std::vector<int32_t> order((size_t)N);
+    std::iota(order.begin(), order.end(), 0);
+    auto mid = [&](int j) { return rowptr[j + 1] > rowptr[j] ? col[(size_t)(rowptr[j] + rowptr[j + 1]) / 2] : INT32_MAX; };
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return mid(a) < mid(b); });
+    std::vector<int32_t> out_at((size_t)ntiles * TO, -1), cols, hdr((size_t)2 * ntiles, 0), wave_hdr;
+    std::vector<float> ent;
+    std::vector<int32_t> slot_of((size_t)N, -1);
+    int64_t staged = 0;
+    int gp = 0;  // panels so far
+    for (int t = 0; t < ntiles; ++t) {
+        const int o0 = t * TO, o1 = std::min(N, o0 + TO);
+        std::vector<int32_t> outs(order.begin() + o0, order.begin() + o1);
+        std::stable_sort(outs.begin(), outs.end(), [&](int32_t a, int32_t b) {
+            return rowptr[a + 1] - rowptr[a] > rowptr[b + 1] - rowptr[b];
+        });
+        std::vector<int32_t> uni;
+        for (int32_t j : outs) uni.insert(uni.end(), col.begin() + rowptr[j], col.begin() + rowptr[j + 1]);
+        std::sort(uni.begin(), uni.end());
+        uni.erase(std::unique(uni.begin(), uni.end()), uni.end());
+        staged += (int64_t)uni.size();
+        if (staged > 4 * (int64_t)N) return false;
+        for (size_t k = 0; k < uni.size(); ++k) slot_of[(size_t)uni[k]] = (int32_t)k;
+        const int np = (int)((uni.size() + PC - 1) / PC);
+        hdr[(size_t)2 * t] = gp;
+        hdr[(size_t)2 * t + 1] = np;
+        for (size_t k = 0; k < outs.size(); ++k) out_at[(size_t)o0 + k] = outs[k];
+        for (int p = 0; p < np; ++p) {
+            for (int sl = 0; sl < PC; ++sl) {
+                const size_t k = (size_t)p * PC + sl;
+                cols.push_back(k < uni.size() ? uni[k] : uni[(size_t)p * PC]);  // padding: a column of this panel
+            }
+            for (int w = 0; w < NWV; ++w) {
+                // entries of the wave's outputs that fall into this panel
+                int maxc = 0;
+                std::vector<std::pair<int, int>> rng((size_t)WO, {0, 0});
+                for (int o = 0; o < WO; ++o) {
+                    const size_t k = (size_t)w * WO + o;
+                    if (k >= outs.size()) continue;
+                    const int j = outs[k];
+                    int b = rowptr[j], e = rowptr[j + 1];
+                    while (b < e && slot_of[(size_t)col[b]] / PC < p) ++b;
+                    int e2 = b;
+                    while (e2 < e && slot_of[(size_t)col[e2]] / PC == p) ++e2;
+                    rng[(size_t)o] = {b, e2};
+                    maxc = std::max(maxc, e2 - b);
+                }
+                const int rounds = (maxc + 1) / 2;
+                wave_hdr.push_back(rounds);
+                wave_hdr.push_back((int32_t)(ent.size() / 256));
+                for (int r = 0; r < rounds; ++r)
+                    for (int o = 0; o < WO; ++o)
+                        for (int k = 0; k < 2; ++k) {
+                            const int e = rng[(size_t)o].first + r * 2 + k;
+                            uint32_t off = 0;
+                            float wgt = -0.0f;  // padding: adds an exact zero; the sign tells it from a stored zero weight
+                            if (e < rng[(size_t)o].second) {
+                                off = (uint32_t)(slot_of[(size_t)col[e]] % PC) * 256u;
+                                wgt = val[e] == 0.0f ? 0.0f : val[e];
+                            }
+                            float f;
+                            memcpy(&f, &off, 4);
+                            ent.push_back(f);
+                            ent.push_back(wgt);
+                        }
+            }
+        }
+        gp += np;
+        if (ent.size() / 256 > (size_t)INT32_MAX / 2) return false;
+    }
+    plan.out_at.swap(out_at);
+    plan.ell_col.swap(cols);
+    plan.rowlen.swap(hdr);
+    plan.rowlen.insert(plan.rowlen.end(), wave_hdr.begin(), wave_hdr.end());
+    plan.wv.swap(ent);
+    plan.ntiles = ntiles;
+    return true;
+}
+
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan) {
     const int64_t nnz = rowptr[N];
@@ -587,6 +683,14 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         }
         plan.ell_col.clear();
         plan.rowlen.clear();
+    } else if (force_kernel != SPDNN_KERNEL_GATHER && !(getenv("SPDNN_TILED") && atoi(getenv("SPDNN_TILED")) == 0) &&
+               build_tiled_plan(N, rowptr, col, val, plan)) {
+        plan.kernel = SPDNN_KERNEL_TILED;
+        plan.wmode = exact ? 1 : 2;
+        plan.in_pos.resize((size_t)N);
+        std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
+        plan.sel.clear();
+        plan.pairs.clear();
     } else {
         plan.kernel = SPDNN_KERNEL_GATHER;
         plan.wmode = exact ? 1 : 2;
@@ -645,6 +749,26 @@ void plan_adjacency(const LayerPlan& p, int N, std::vector<int32_t>& rowptr, std
                 if (j < 0) continue;
                 for (int k = 0; k < p.blk_cnt[(size_t)g]; ++k) ins[(size_t)j].push_back(p.blk_cols[(size_t)g * 32 + k]);
             }
+    } else if (p.kernel == SPDNN_KERNEL_TILED) {
+        const int32_t* wave_hdr = p.rowlen.data() + 2 * p.ntiles;
+        for (int t = 0; t < p.ntiles; ++t) {
+            const int gp0 = p.rowlen[(size_t)2 * t], np = p.rowlen[(size_t)2 * t + 1];
+            for (int q = 0; q < np; ++q)
+                for (int w = 0; w < kTileOutputs / 64; ++w) {
+                    const int rounds = wave_hdr[((size_t)(gp0 + q) * 16 + w) * 2];
+                    const size_t blk = (size_t)wave_hdr[((size_t)(gp0 + q) * 16 + w) * 2 + 1];
+                    for (int r = 0; r < rounds; ++r)
+                        for (int o = 0; o < 64; ++o)
+                            for (int k = 0; k < 2; ++k) {
+                                const size_t at = ((blk + r) * 128 + (size_t)o * 2 + k) * 2;
+                                if (p.wv[at + 1] == 0.0f && std::signbit(p.wv[at + 1])) continue;  // padding
+                                uint32_t off;
+                                memcpy(&off, &p.wv[at], 4);
+                                const int j = p.out_at[(size_t)t * kTileOutputs + w * 64 + o];
+                                ins[(size_t)j].push_back(p.ell_col[(size_t)(gp0 + q) * kPanelCols + off / 256]);
+                            }
+                }
+        }
     } else {
         for (int j = 0; j < N; ++j)
             for (int k = 0; k < p.rowlen[(size_t)j]; ++k) ins[(size_t)j].push_back(p.ell_col[(size_t)j * p.kmax + k]);

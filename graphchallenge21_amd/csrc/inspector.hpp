@@ -14,6 +14,9 @@
 
 namespace spdnn {
 
+constexpr int kTileOutputs = 1024;  // TILED: outputs per tile (16 waves x 64)
+constexpr int kPanelCols = 512;     // TILED: input columns staged in LDS at a time
+
 struct LayerPlan {
     bool set = false;
     spdnn_layer_plan info{};
@@ -52,6 +55,11 @@ struct LayerPlan {
     // BAND: neuron j sits at the same band position as an input and as an output (see
     // canonicalize_self_aligned_band); fuse_next: this layer writes its outputs exactly where the
     // next layer's band reads them (dst = identity) and both fit the fused pair kernel
+    // TILED: out_at / dst hold ntiles x 1024 slots (-1 = unused); ell_col the panels' columns, 512 per
+    // panel (padded); rowlen first (first panel, panels) per tile, then (rounds, first entry block) per
+    // panel and wave; wv the entry blocks of 1 KiB: per round 64 outputs x 2 entries x (byte offset of
+    // the column's slot in the panel as raw bits, weight)
+    int ntiles = 0;
     bool self_aligned = false;
     bool fuse_next = false;
 };

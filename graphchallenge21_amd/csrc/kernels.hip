@@ -192,7 +192,14 @@ __device__ __forceinline__ void column_to_lds(const float* gsrc_lane, unsigned c
         (const __attribute__((address_space(1))) void*)gsrc_lane,
         (__attribute__((address_space(3))) void*)lds_col, 16, 0, STREAM ? 2 : 0);
 }
-__device__ __forceinline__ void wait_vector_memory() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// s_waitcnt vmcnt(0) (the other counters left alone: expcnt 7, lgkmcnt 15 in the gfx9 encoding), as
+// the instruction itself rather than inline text, so that the compiler's own bookkeeping of
+// outstanding direct-to-LDS loads sees it too.
+__device__ __forceinline__ void wait_vector_memory() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    asm volatile("" ::: "memory");
+}
 // Workgroup barrier of the band walk.  With columns sent straight into the ring the waves wait for
 // their transfers themselves (wait_vector_memory) BEFORE they store their outputs; the fence of
 // __syncthreads() would wait on the vector memory counter again behind those stores, i.e. for the
@@ -870,6 +877,141 @@ __global__ __launch_bounds__(256) void gather_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
+// TILED kernel (general class with reuse): a workgroup of 16 waves takes 64 feature rows (lane =
+// row: a quarter of a 256-row block) and a tile of 1024 outputs, 64 per wave, whose accumulators
+// stay in registers.  The tile's input columns (the union over its outputs, ascending) pass through
+// LDS in panels of 512 columns x 256 bytes, fed straight from global memory; every column is read
+// once per tile, whatever the number of outputs that use it.  Per panel a wave works through
+// `rounds` rounds of 2 entries per output.  An entry is an LDS byte offset and a weight; streaming
+// 8 bytes per multiply-add through the scalar cache does not work (every access misses, and the
+// cache serves few misses at a time: measured 0.69 ms per layer of 1024 neurons where the plain
+// gather takes 0.45), so the entry blocks (1 KiB per round and wave) go through LDS too: the wave
+// sends the next block into its own two-block ring while it works on the current one and reads
+// the entries back with broadcast reads (all lanes the same address).
+// Accumulation in ascending input index: panels ascend, entries inside a panel ascend; padding
+// entries carry weight -0 and add an exact zero.
+// ------------------------------------------------------------------------------------------
+__device__ __forceinline__ void column64_to_lds(const float* gsrc_lane, unsigned char* lds_col) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc_lane,
+                                     (__attribute__((address_space(3))) void*)lds_col, 4, 0, 0);
+}
+
+// 64 lanes x 16 bytes from global memory into 1 KiB of LDS, issued in a form the compiler does not
+// follow: it puts a wait for ALL vector memory traffic in front of any LDS read that might touch
+// the destination of a direct-to-LDS load it knows of, which here would be the very next read (the
+// other half of the wave's entry ring).  The caller waits itself (wait_vector_memory).
+__device__ __forceinline__ void block_to_lds_untracked(const float* gsrc_lane, unsigned char* lds_block) {
+    const uint32_t lds_off = (uint32_t)(size_t)((__attribute__((address_space(3))) unsigned char*)lds_block);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_off), "v"(gsrc_lane)
+                 : "m0", "memory");
+}
+
+template <int WMODE>
+__global__ __launch_bounds__(1024) void tiled_kernel(
+    Feat yin_all, Feat yout_all, const int32_t* __restrict__ cols, const int32_t* __restrict__ hdr,
+    const uint32_t* __restrict__ ent, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
+    int32_t* __restrict__ count_prev, int N, int ntiles, int rl, int stamp, int prev_stamp, int check_dead,
+    float bias, float clampv, Publish pub) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int PANEL_BYTES = 512 * 256;   // then 16 waves x 2 entry blocks of 1 KiB
+    publish_counts(pub);
+    const int lane = threadIdx.x & 63;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int RB = 64 * rl;
+    const int sb = blockIdx.x, rb = sb / rl, q = sb - rb * rl;
+    const int t = blockIdx.y;
+    const size_t row = (size_t)rb * RB + q * 64 + lane;
+    if (prev_stamp != 0 && (check_dead || (count_prev != nullptr && t == 0))) {
+        // Only a row block without ANY active row may be skipped (the kernels of the other classes
+        // decide per row block too, and expect the dead rows of a live block to hold zeros, which
+        // computing them gives); the count is taken per 64 rows.  Every wave reads the same stamps,
+        // so the whole workgroup takes the same way.
+        int alive_block = 0, alive_own = 0;
+        for (int i = 0; i < rl; ++i) {
+            const int a = active[(size_t)rb * RB + i * 64 + lane];
+            const int c = (int)__popcll(__ballot((a == prev_stamp || a == stamp) ? 1 : 0));
+            alive_block += c;
+            if (i == q) alive_own = c;
+        }
+        if (count_prev != nullptr && t == 0 && threadIdx.x == 0 && alive_own > 0) atomicAdd(count_prev, alive_own);
+        if (check_dead && alive_block == 0) return;
+    }
+    const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB) + q * 64 + lane;
+    float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB) + q * 64 + lane;
+    const int gp0 = hdr[2 * t], np = hdr[2 * t + 1];
+    const int32_t* __restrict__ wave_hdr = hdr + 2 * ntiles;
+    unsigned char* ring = smem + PANEL_BYTES + w * 2048;          // this wave's two entry blocks
+    const unsigned char* lane_panel = smem + lane * 4;
+
+    float acc[64];
+#pragma unroll
+    for (int o = 0; o < 64; ++o) acc[o] = 0.0f;
+
+    for (int p = 0; p < np; ++p) {
+        // the panel's columns, 32 per wave (every wave has finished the panel before: barrier below)
+        const int32_t* pc = cols + (size_t)(gp0 + p) * 512;
+#pragma unroll 4
+        for (int i = 0; i < 32; ++i) {
+            const int sl = w + 16 * i;
+            column64_to_lds(yin + (size_t)pc[sl] * RB, smem + sl * 256);
+        }
+        const int rounds = wave_hdr[((size_t)(gp0 + p) * 16 + w) * 2];
+        const float* blk = reinterpret_cast<const float*>(ent) + (size_t)wave_hdr[((size_t)(gp0 + p) * 16 + w) * 2 + 1] * 256;
+        if (rounds > 0) {
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(blk + lane * 4),
+                                             (__attribute__((address_space(3))) void*)ring, 16, 0, 0);
+        }
+        wait_vector_memory();
+        ring_barrier<1>();
+        for (int r = 0; r < rounds; ++r) {
+            if (r + 1 < rounds) block_to_lds_untracked(blk + (size_t)(r + 1) * 256 + lane * 4, ring + ((r + 1) & 1) * 1024);
+            const unsigned char* cur = ring + (r & 1) * 1024;
+#pragma unroll
+            for (int g = 0; g < 16; ++g) {     // 4 outputs at a time: entries first, then columns, then arithmetic
+                float4 m[4];
+#pragma unroll
+                for (int o = 0; o < 4; ++o) m[o] = *reinterpret_cast<const float4*>(cur + (g * 4 + o) * 16);
+                float x[4][2];
+#pragma unroll
+                for (int o = 0; o < 4; ++o) {
+                    x[o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[o].x));
+                    x[o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[o].z));
+                }
+#pragma unroll
+                for (int o = 0; o < 4; ++o) {
+                    acc[g * 4 + o] = mac<WMODE>(acc[g * 4 + o], x[o][0], m[o].y);
+                    acc[g * 4 + o] = mac<WMODE>(acc[g * 4 + o], x[o][1], m[o].w);
+                }
+            }
+            wait_vector_memory();   // the next entry block has arrived (nothing else is in flight)
+        }
+        ring_barrier<1>();          // every wave is done with the panel
+    }
+
+    float nz = 0.0f;
+#pragma unroll
+    for (int o = 0; o < 64; ++o) {
+        const int d = dst[(size_t)t * 1024 + w * 64 + o];
+        if (d >= 0) {
+            const float y = relu_clamp(acc[o] + bias, clampv);
+            nz = nz_merge(nz, y);
+            yout[(size_t)d * RB] = y;
+        }
+    }
+    float* sm = reinterpret_cast<float*>(smem);
+    sm[w * 64 + lane] = nz;
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        float m = sm[lane];
+#pragma unroll
+        for (int k = 1; k < 16; ++k) m = nz_merge(m, sm[k * 64 + lane]);
+        if (m > 0.0f) active[row] = stamp;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // BLOCK kernel: groups of up to 16 outputs that read the same (up to 32) input columns - the
 // structure of the challenge's RadiX-Net layers.  A wave loads the shared columns of a group once
 // into registers (32 x RB*4 bytes) and every output of the group reuses them: no LDS, register
@@ -1435,6 +1577,26 @@ hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
         default: return hipErrorInvalidValue;
     }
 #undef SPDNN_GATHER
+    return hipGetLastError();
+}
+
+hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s) {
+    if (a.N <= 0 || a.ntiles <= 0 || a.ntiles > 65535 || a.nblk <= 0 || a.rl < 1 || a.rl > 4 || !a.yin || !a.yout ||
+        !a.cols || !a.hdr || !a.ent || !a.dst || !a.active)
+        return hipErrorInvalidValue;
+    constexpr size_t lds = 512 * 256 + 16 * 2048;   // one panel and the waves' entry rings: all 160 KiB of a CU
+    dim3 grid(a.nblk * a.rl, a.ntiles), block(1024);
+#define SPDNN_TILED(WM)                                                                                          \
+    do {                                                                                                         \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM>),      \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+        if (attr != hipSuccess) return attr;                                                                     \
+        hipLaunchKernelGGL(tiled_kernel<WM>, grid, block, lds, s, a.yin, a.yout, a.cols, a.hdr, a.ent, a.dst,    \
+                           a.active, a.count_prev, a.N, a.ntiles, a.rl, a.stamp, a.prev_stamp, a.check_dead,     \
+                           a.bias, a.clampv, a.publish);                                                         \
+    } while (0)
+    if (a.wmode != 2) SPDNN_TILED(1); else SPDNN_TILED(2);
+#undef SPDNN_TILED
     return hipGetLastError();
 }
 

@@ -88,6 +88,22 @@ int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, 
 double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, int seglen);
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s);
 
+// TILED layers: tiles of 1024 outputs, their input columns staged in LDS panel by panel (see LayerPlan).
+struct TiledLaunch {
+    Feat yin;
+    Feat yout;
+    const int32_t* cols;     // panels' columns, 512 per panel
+    const int32_t* hdr;      // (first panel, panels) per tile, then (rounds, first entry block) per panel and wave
+    const uint32_t* ent;     // entry blocks
+    const int32_t* dst;      // [ntiles*1024] physical output column, -1 = unused slot
+    int32_t* active;
+    int32_t* count_prev;     // as in BandLaunch
+    int N, ntiles, nblk, rl, wmode, stamp, prev_stamp, check_dead;
+    float bias, clampv;
+    Publish publish;
+};
+hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s);
+
 // BLOCK layers: groups of up to 16 outputs sharing up to 32 input columns.
 struct BlockLaunch {
     Feat yin;

@@ -1306,6 +1306,14 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         b.publish = pub;
         return launch_block(b, n->stream);
     }
+    if (p.kernel == SPDNN_KERNEL_TILED) {
+        TiledLaunch t{};
+        t.yin = in; t.yout = out; t.cols = d.ell; t.hdr = d.rowlen; t.ent = reinterpret_cast<const uint32_t*>(d.wv); t.dst = d.dst;
+        t.active = n->d_active; t.count_prev = count_prev; t.check_dead = check_dead; t.prev_stamp = prev_stamp;
+        t.N = n->N; t.ntiles = p.ntiles; t.nblk = nblk; t.rl = n->rl; t.wmode = p.wmode; t.stamp = stamp;
+        t.bias = n->bias; t.clampv = n->clampv; t.publish = pub;
+        return launch_tiled(t, n->stream);
+    }
     GatherLaunch g{};
     g.yin = in; g.yout = out; g.cols = d.ell; g.rowlen = d.rowlen; g.wv = d.wv; g.dst = d.dst;
     g.active = n->d_active; g.count_prev = count_prev; g.check_dead = check_dead; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.kmax; g.nblk = nblk; g.stamp = stamp; g.rl = n->rl;

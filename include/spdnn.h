@@ -56,8 +56,10 @@ enum spdnn_kernel {
     SPDNN_KERNEL_AUTO = 0,
     SPDNN_KERNEL_GATHER = 1, /* general CSR/ELL gather, any sparsity pattern                      */
     SPDNN_KERNEL_BAND = 2,   /* row-succ / tiled: relabelled circulant band walked through an LDS ring */
-    SPDNN_KERNEL_BLOCK = 3   /* groups of outputs that read the same inputs (RadiX-Net style): the shared
+    SPDNN_KERNEL_BLOCK = 3,  /* groups of outputs that read the same inputs (RadiX-Net style): the shared
                                 input columns are held in registers and reused by every output of the group */
+    SPDNN_KERNEL_TILED = 4   /* any sparsity pattern: tiles of 1024 outputs whose input columns are staged in
+                                LDS panel by panel, every column read once per tile                          */
 };
 
 typedef struct spdnn_layer_plan {

@@ -114,11 +114,14 @@ def test_survivor_chain_with_compaction(gc, orc):
             assert not net.activations(dead).any()
 
 
+@pytest.mark.parametrize("tiled", [1, 0])
 @pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
-def test_gather_kernel_random_sparsity(gc, orc, values):
-    """Irregular rows (0..40 entries), unsorted columns: the general kernel."""
+def test_gather_kernel_random_sparsity(gc, orc, values, tiled, monkeypatch):
+    """Irregular rows (0..40 entries), unsorted columns: the general classes - tiles of outputs with
+    their input columns staged in LDS, and the plain gather."""
+    monkeypatch.setenv("SPDNN_TILED", str(tiled))
     N, L, B = 512, 3, 300
-    print("gather values=%s" % values, flush=True)
+    print("general class tiled=%d values=%s" % (tiled, values), flush=True)
     rng = np.random.default_rng(11)
     layers = [random_csr(rng, N, rng.integers(0, 41, size=N), values) for _ in range(L)]
     feats = rng.uniform(0, 4, size=(B, N)).astype(np.float32) * (rng.random((B, N)) < 0.3)
@@ -127,7 +130,7 @@ def test_gather_kernel_random_sparsity(gc, orc, values):
         for l, csr in enumerate(layers):
             net.set_layer_csr(l, *csr)
         net.inspect()
-        assert all(net.layer_plan(l).kernel == gc.KERNEL_GATHER for l in range(L))
+        assert all(net.layer_plan(l).kernel == (gc.KERNEL_TILED if tiled else gc.KERNEL_GATHER) for l in range(L))
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, [sort_rows(c) for c in layers], feats, prune=True)
 
@@ -193,7 +196,7 @@ def test_other_row_block_sizes(gc, orc, rl, monkeypatch):
         for l, csr in enumerate(layers):
             net.set_layer_csr(l, *csr)
         net.inspect()
-        assert [net.layer_plan(l).kernel for l in range(4)] == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER]
+        assert [net.layer_plan(l).kernel for l in range(4)] == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_TILED]
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 
@@ -222,7 +225,7 @@ def test_streamed_plans(gc, orc, window, monkeypatch):
                 net.set_layer_csr(l, *csr)
             net.inspect()
             kernels = {net.layer_plan(l).kernel for l in range(L)}
-            assert kernels == {gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER}
+            assert kernels == {gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_TILED}
             net.set_features_dense(feats)
             w, dev_bytes, pinned = net.plan_memory()
             assert w == window and pinned > dev_bytes > 0
@@ -505,7 +508,7 @@ def test_block_kernel_radix_like_layers(gc, orc, values, chains, monkeypatch):
             net.set_layer_csr(l, *csr)
         net.inspect()
         kinds = [net.layer_plan(l).kernel for l in range(L)]
-        assert kinds == [rk] * 4 + [gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER, gc.KERNEL_BLOCK, rk]
+        assert kinds == [rk] * 4 + [gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_TILED, gc.KERNEL_BLOCK, rk]
         assert [net.layer_plan(l).band_halo for l in range(L)] == [rh] * 4 + [31, -1, -1, -1, rh]
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
@@ -696,7 +699,7 @@ def test_small_and_odd_shapes(gc, orc, N, K, B):
         for l, csr in enumerate(layers):
             net.set_layer_csr(l, *csr)
         net.inspect()
-        want = gc.KERNEL_BAND if (N % 256 == 0 and K % 4 == 0 and K <= 32) else gc.KERNEL_GATHER
+        want = gc.KERNEL_BAND if (N % 256 == 0 and K % 4 == 0 and K <= 32) else gc.KERNEL_TILED
         assert all(net.layer_plan(l).kernel == want for l in range(L))
         net.set_features_dense(feats)
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)

@@ -150,7 +150,10 @@ def test_band_pair_records_reproduce_oracle(gc, orc, monkeypatch):
             assert np.array_equal(y[:, net.input_labelling(l + 1)], want), l
 
 
-def test_inspector_falls_back_to_gather(gc, orc):
+@pytest.mark.parametrize("tiled", [1, 0])
+def test_inspector_falls_back_to_the_general_classes(gc, orc, tiled, monkeypatch):
+    monkeypatch.setenv("SPDNN_TILED", str(tiled))
+    general = gc.KERNEL_TILED if tiled else gc.KERNEL_GATHER
     rng = np.random.default_rng(3)
     n = 256
     irregular = random_csr(rng, n, rng.integers(0, 20, size=n), "general")
@@ -168,7 +171,7 @@ def test_inspector_falls_back_to_gather(gc, orc):
         net.set_layer_csr(3, band[0], band[1], np.linspace(0.1, 0.2, len(band[1])).astype(np.float32))
         net.inspect()
         p = [net.layer_plan(l) for l in range(4)]
-        assert [q.kernel for q in p] == [gc.KERNEL_GATHER, gc.KERNEL_GATHER, gc.KERNEL_BAND, gc.KERNEL_BAND]
+        assert [q.kernel for q in p] == [general, general, gc.KERNEL_BAND, gc.KERNEL_BAND]
         assert (p[0].regular, p[0].exact_products) == (0, 0) and p[0].band_halo == -1
         assert (p[1].regular, p[1].uniform_value, p[1].exact_products) == (1, 1, 1)
         assert (p[2].max_row_nnz, p[2].band_halo) == (8, 7)
@@ -176,9 +179,12 @@ def test_inspector_falls_back_to_gather(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.band_plan(0)
         assert e.value.code == 2
-        # a gather layer reads its input in natural order; its outputs go where the next layer reads
+        # a general layer reads its input in natural order; its outputs go where the next layer reads
         assert np.array_equal(net.input_labelling(0), np.arange(n))
-        assert np.array_equal(net.layer_dst(1), net.input_labelling(2))
+        d1 = net.layer_dst(1)      # gather: one slot per neuron; tiled: 1024 slots per tile, -1 where unused
+        assert np.array_equal(np.sort(d1[d1 >= 0]), np.arange(n)) and (len(d1) == n or len(d1) == 1024)
+        if not tiled:
+            assert np.array_equal(d1, net.input_labelling(2))
         assert np.array_equal(net.layer_dst(3), np.arange(n)[net.band_plan(3)[1]])
 
 
@@ -267,7 +273,7 @@ def test_receptive_field_of_every_layer_class(gc, orc, monkeypatch):
             net.set_layer_csr(l, *csr)
         net.inspect()
         kinds = [net.layer_plan(l).kernel for l in range(len(layers))]
-        assert kinds == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_GATHER, gc.KERNEL_BAND]
+        assert kinds == [gc.KERNEL_BAND, gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_TILED, gc.KERNEL_BAND]
         assert net.layer_plan(1).band_halo == 32
         for first in range(len(layers)):
             for depth in range(1, len(layers) - first + 1):
@@ -278,6 +284,11 @@ def test_receptive_field_of_every_layer_class(gc, orc, monkeypatch):
             net.receptive_field(0, len(layers) + 1, [0])
         with pytest.raises(gc.SpdnnError):
             net.receptive_field(0, 1, [n])
+    with gc.Network(n, 4, 1, bias=-0.3, force_kernel=gc.KERNEL_GATHER) as net:
+        net.set_layer_csr(0, *layers[3])
+        net.inspect()
+        assert net.layer_plan(0).kernel == gc.KERNEL_GATHER
+        assert np.array_equal(net.receptive_field(0, 1, np.arange(40)), orc.receptive_field(layers[3:4], np.arange(40)))
 
 
 def test_fusable_pairs_are_found_by_the_inspector(gc, orc):
