@@ -968,22 +968,42 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
         for (int r = 0; r < rounds; ++r) {
             if (r + 1 < rounds) block_to_lds_untracked(blk + (size_t)(r + 1) * 256 + lane * 4, ring + ((r + 1) & 1) * 1024);
             const unsigned char* cur = ring + (r & 1) * 1024;
+            // 32 units of 2 outputs, software-pipelined three deep: while unit u does its arithmetic, the
+            // columns of unit u+1 and the entries of unit u+2 are on their way from LDS
+            float4 m[3][2];
+            float x[2][2][2];
 #pragma unroll
-            for (int g = 0; g < 16; ++g) {     // 4 outputs at a time: entries first, then columns, then arithmetic
-                float4 m[4];
+            for (int o = 0; o < 2; ++o) {
+                m[0][o] = *reinterpret_cast<const float4*>(cur + o * 16);
+                m[1][o] = *reinterpret_cast<const float4*>(cur + (2 + o) * 16);
+            }
 #pragma unroll
-                for (int o = 0; o < 4; ++o) m[o] = *reinterpret_cast<const float4*>(cur + (g * 4 + o) * 16);
-                float x[4][2];
+            for (int o = 0; o < 2; ++o) {
+                x[0][o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[0][o].x));
+                x[0][o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[0][o].z));
+            }
 #pragma unroll
-                for (int o = 0; o < 4; ++o) {
-                    x[o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[o].x));
-                    x[o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[o].z));
+            for (int u = 0; u < 32; ++u) {
+                if (u + 2 < 32) {
+#pragma unroll
+                    for (int o = 0; o < 2; ++o)
+                        m[(u + 2) % 3][o] = *reinterpret_cast<const float4*>(cur + ((u + 2) * 2 + o) * 16);
                 }
+                __builtin_amdgcn_sched_barrier(0);   // the three stages stay in this order
+                if (u + 1 < 32) {
 #pragma unroll
-                for (int o = 0; o < 4; ++o) {
-                    acc[g * 4 + o] = mac<WMODE>(acc[g * 4 + o], x[o][0], m[o].y);
-                    acc[g * 4 + o] = mac<WMODE>(acc[g * 4 + o], x[o][1], m[o].w);
+                    for (int o = 0; o < 2; ++o) {
+                        x[(u + 1) & 1][o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[(u + 1) % 3][o].x));
+                        x[(u + 1) & 1][o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[(u + 1) % 3][o].z));
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int o = 0; o < 2; ++o) {
+                    acc[u * 2 + o] = mac<WMODE>(acc[u * 2 + o], x[u & 1][o][0], m[u % 3][o].y);
+                    acc[u * 2 + o] = mac<WMODE>(acc[u * 2 + o], x[u & 1][o][1], m[u % 3][o].w);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
             wait_vector_memory();   // the next entry block has arrived (nothing else is in flight)
         }
