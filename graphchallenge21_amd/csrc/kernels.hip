@@ -241,12 +241,32 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // step.  The output column is written to the physical column the NEXT layer wants it in (dst),
 // RB*4 contiguous bytes.
 // ------------------------------------------------------------------------------------------
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_const_u4(const __attribute__((address_space(4))) uint32_t* p) {
+    const u32x4_t v = *(const __attribute__((address_space(4))) u32x4_t*)p;
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ float4 load_const_f4(const __attribute__((address_space(4))) float* p) {
+    const f32x4_t v = *(const __attribute__((address_space(4))) f32x4_t*)p;
+    return make_float4(v.x, v.y, v.z, v.w);
+}
+
+// RBL: rows per block of the LAYOUT (floats between two columns); larger than the 64*RL rows the
+// workgroup handles when it works on a part of a row block (yin / yout then point at that part).
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA, int RBL = 64 * RL>
 __device__ __forceinline__ void band_walk_body(
-    const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs,
-    const float* __restrict__ pw, const int32_t* __restrict__ dst, int N, int steps, int stride, int halo,
+    const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs_g,
+    const float* __restrict__ pw_g, const int32_t* __restrict__ dst_g, int N, int steps, int stride, int halo,
     int vb, int ve, float wu, float bias, float clampv, unsigned char* smem, float* nz, int stream) {
     using V = typename VecOf<RL>::type;
+    // The plan arrays never change while a kernel runs: read through the constant address space they
+    // come by the scalar unit also where the pointers themselves were loaded from memory (the layer
+    // table of the fused chain), instead of by vector loads with the selection arithmetic on the
+    // vector ALUs.
+    const __attribute__((address_space(4))) uint32_t* pairs = (const __attribute__((address_space(4))) uint32_t*)pairs_g;
+    const __attribute__((address_space(4))) float* pw = (const __attribute__((address_space(4))) float*)pw_g;
+    const __attribute__((address_space(4))) int32_t* dst = (const __attribute__((address_space(4))) int32_t*)dst_g;
     constexpr int T = NW * OPW;
     constexpr int PPW = OPW / 2;  // pairs per wave and chunk
     constexpr int RB = 64 * RL;
@@ -272,13 +292,13 @@ __device__ __forceinline__ void band_walk_body(
             const int g = p < 0 ? p + N : p;
             if (DMA) {
                 unsigned char* slot = smem + (size_t)(p & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
-                else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+                if (stream) column_to_lds<1>(yin + (size_t)g * RBL + loff, slot);
+                else column_to_lds<0>(yin + (size_t)g * RBL + loff, slot);
                 continue;
             }
             float x[RL];
-            if (stream) load_stream<RL>(yin + (size_t)g * RB + loff, x);
-            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)g * RB + loff), x);
+            if (stream) load_stream<RL>(yin + (size_t)g * RBL + loff, x);
+            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)g * RBL + loff), x);
             *reinterpret_cast<V*>(smem + (size_t)(p & (RING - 1)) * COLB + loff * 4) = arr_to_vec<RL>(x);
         }
     }
@@ -296,10 +316,10 @@ __device__ __forceinline__ void band_walk_body(
             const int p = min(cb + T + wave + i * NW, ve - 1);
             if (DMA) {
                 unsigned char* slot = smem + (size_t)((cb + T + wave + i * NW) & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1>(yin + (size_t)p * RB + loff, slot);
-                else column_to_lds<0>(yin + (size_t)p * RB + loff, slot);
-            } else if (stream) load_stream<RL>(yin + (size_t)p * RB + loff, pf[i]);
-            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RB + loff), pf[i]);
+                if (stream) column_to_lds<1>(yin + (size_t)p * RBL + loff, slot);
+                else column_to_lds<0>(yin + (size_t)p * RBL + loff, slot);
+            } else if (stream) load_stream<RL>(yin + (size_t)p * RBL + loff, pf[i]);
+            else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RBL + loff), pf[i]);
         }
 
         int pr[PPW];
@@ -317,19 +337,19 @@ __device__ __forceinline__ void band_walk_body(
             // reads in flight while its multiply-adds issue.  Steps 32..35 exist only if steps > 32.
             uint4 mk[PPW], sa[PPW], sb[PPW];
             uint32_t sc[PPW];
-            const float4* wp[PPW];
+            const __attribute__((address_space(4))) float* wp[PPW];
             float4 w_cur[PPW][2];
 #pragma unroll
             for (int i = 0; i < PPW; ++i) {
-                const uint4* rec = reinterpret_cast<const uint4*>(pairs + (size_t)pr[i] * 16);
-                mk[i] = rec[0];
-                sa[i] = rec[1];
-                sb[i] = rec[2];
+                const __attribute__((address_space(4))) uint32_t* rec = pairs + (size_t)pr[i] * 16;
+                mk[i] = load_const_u4(rec);
+                sa[i] = load_const_u4(rec + 4);
+                sb[i] = load_const_u4(rec + 8);
                 sc[i] = pairs[(size_t)pr[i] * 16 + 12];
                 if (WMODE) {
-                    wp[i] = reinterpret_cast<const float4*>(pw + (size_t)pr[i] * 72);
-                    w_cur[i][0] = wp[i][0];
-                    w_cur[i][1] = wp[i][1];
+                    wp[i] = pw + (size_t)pr[i] * 72;
+                    w_cur[i][0] = load_const_f4(wp[i]);
+                    w_cur[i][1] = load_const_f4(wp[i] + 4);
                 }
             }
             float xb[3][PPW][RL];
@@ -355,8 +375,8 @@ __device__ __forceinline__ void band_walk_body(
                 if (WMODE && (st & 3) == 0 && st + 4 < 36) {  // two weights per step, four steps per trip
 #pragma unroll
                     for (int i = 0; i < PPW; ++i) {
-                        w_nxt[i][0] = wp[i][(st >> 2) * 2 + 2];
-                        w_nxt[i][1] = wp[i][(st >> 2) * 2 + 3];
+                        w_nxt[i][0] = load_const_f4(wp[i] + 4 * ((st >> 2) * 2 + 2));
+                        w_nxt[i][1] = load_const_f4(wp[i] + 4 * ((st >> 2) * 2 + 3));
                     }
                 }
                 if (st < 32 || st < steps) {
@@ -401,20 +421,20 @@ __device__ __forceinline__ void band_walk_body(
             // run-time step count: four steps per trip; the selectors (and weights) of the next
             // trip are requested from the scalar cache before this trip's arithmetic starts
             const int trips = (steps + 3) >> 2;
-            const uint32_t* sp[PPW];
-            const float4* wp[PPW];
+            const __attribute__((address_space(4))) uint32_t* sp[PPW];
+            const __attribute__((address_space(4))) float* wp[PPW];
             uint32_t m0lo[PPW], m0hi[PPW], m1lo[PPW], m1hi[PPW], s_cur[PPW];
             float4 w_cur[PPW][2];
 #pragma unroll
             for (int i = 0; i < PPW; ++i) {
-                const uint32_t* rec = pairs + (size_t)pr[i] * stride;
+                const __attribute__((address_space(4))) uint32_t* rec = pairs + (size_t)pr[i] * stride;
                 m0lo[i] = rec[0]; m0hi[i] = rec[1]; m1lo[i] = rec[2]; m1hi[i] = rec[3];
                 sp[i] = rec + 4;
                 s_cur[i] = sp[i][0];
                 if (WMODE) {
-                    wp[i] = reinterpret_cast<const float4*>(pw + (size_t)pr[i] * (size_t)trips * 8);
-                    w_cur[i][0] = wp[i][0];
-                    w_cur[i][1] = wp[i][1];
+                    wp[i] = pw + (size_t)pr[i] * (size_t)trips * 8;
+                    w_cur[i][0] = load_const_f4(wp[i]);
+                    w_cur[i][1] = load_const_f4(wp[i] + 4);
                 }
             }
 #pragma unroll 1
@@ -426,8 +446,8 @@ __device__ __forceinline__ void band_walk_body(
                 for (int i = 0; i < PPW; ++i) {
                     s_nxt[i] = sp[i][mn];
                     if (WMODE) {
-                        w_nxt[i][0] = wp[i][2 * mn];
-                        w_nxt[i][1] = wp[i][2 * mn + 1];
+                        w_nxt[i][0] = load_const_f4(wp[i] + 8 * mn);
+                        w_nxt[i][1] = load_const_f4(wp[i] + 8 * mn + 4);
                     }
                 }
 #pragma unroll
@@ -500,11 +520,11 @@ __device__ __forceinline__ void band_walk_body(
                 }
                 const int d0 = dst[v0], d1 = dst[v0 + 1];
                 if (stream) {
-                    store_stream<RL>(yout + (size_t)d0 * RB + loff, y0);
-                    store_stream<RL>(yout + (size_t)d1 * RB + loff, y1);
+                    store_stream<RL>(yout + (size_t)d0 * RBL + loff, y0);
+                    store_stream<RL>(yout + (size_t)d1 * RBL + loff, y1);
                 } else {
-                    *reinterpret_cast<V*>(yout + (size_t)d0 * RB + loff) = arr_to_vec<RL>(y0);
-                    *reinterpret_cast<V*>(yout + (size_t)d1 * RB + loff) = arr_to_vec<RL>(y1);
+                    *reinterpret_cast<V*>(yout + (size_t)d0 * RBL + loff) = arr_to_vec<RL>(y0);
+                    *reinterpret_cast<V*>(yout + (size_t)d1 * RBL + loff) = arr_to_vec<RL>(y1);
                 }
             } else if (v0 < ve) {
                 float y[RL];
@@ -513,7 +533,7 @@ __device__ __forceinline__ void band_walk_body(
                     y[q] = relu_clamp(acc[i][0][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], y[q]);
                 }
-                *reinterpret_cast<V*>(yout + (size_t)dst[v0] * RB + loff) = arr_to_vec<RL>(y);
+                *reinterpret_cast<V*>(yout + (size_t)dst[v0] * RBL + loff) = arr_to_vec<RL>(y);
             }
         }
 
@@ -566,7 +586,7 @@ struct ChainLayer {
     int stride;
 };
 
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
+template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
 __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
     const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
     int32_t* __restrict__ active, int32_t* __restrict__ count_out, int32_t* __restrict__ count_prev, int N,
@@ -588,7 +608,7 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         float nz[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT, 0>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
                                                      lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
         stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
                                      count_out ? count_out + j : nullptr);
@@ -600,6 +620,54 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         // device-scope fence here would write back and invalidate the whole L2 of the XCD.
         const int alive = __syncthreads_or(any);
         if (!alive && stop_when_dead) return;
+        in = out;
+    }
+}
+
+// The fused chain on HALF row blocks of the 256-row layout: a workgroup keeps 128 rows (two per
+// lane) through the chain, so that a batch gives twice as many workgroups - two per CU at the
+// challenge's batch of 60000, whose load / compute / barrier phases interleave - at half the LDS
+// each.  A half whose rows have all died keeps computing (zeros) as long as the other half of its
+// row block may be alive: the kernels of the other classes skip or run whole row blocks and expect
+// the dead rows of a live block to hold zeros.
+template <int WMODE, int KT>
+__global__ __launch_bounds__(512) void band_chain_half_kernel(
+    const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
+    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int32_t* __restrict__ count_prev, int N,
+    int stamp0, int prev_stamp, int check_dead, float bias, float clampv, Publish pub) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int RBL = 256, RBH = 128;
+    publish_counts(pub);
+    const int rb = blockIdx.x >> 1, half = blockIdx.x & 1;
+    const int lane = threadIdx.x & 63;
+    const size_t blkf = (size_t)N * RBL;
+    const size_t row0 = (size_t)rb * RBL + half * RBH;
+    if (prev_stamp != 0 && (check_dead || count_prev != nullptr)) {
+        int alive_block = 0, alive_own = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // stamps only grow: the other half's workgroup may be layers ahead already
+            const int a = active[(size_t)rb * RBL + i * 64 + lane];
+            const int c = (int)__popcll(__ballot(a >= prev_stamp ? 1 : 0));
+            alive_block += c;
+            if ((i >> 1) == half) alive_own += c;
+        }
+        if (count_prev != nullptr && threadIdx.x == 0 && alive_own > 0) atomicAdd(count_prev, alive_own);
+        if (check_dead && alive_block == 0) return;   // every wave reads the same stamps
+    }
+    float* const block_a = block_base(buf_a, rb, blkf) + half * RBH;
+    float* const block_c = block_base(buf_c, rb, blkf) + half * RBH;
+    const float* in = block_base(first_in, rb, blkf) + half * RBH;
+    for (int j = 0; j < nlayers; ++j) {
+        float* out = (in == block_a) ? block_c : block_a;
+        const ChainLayer lay = table[j];
+        float nz[2] = {0.0f, 0.0f};
+        band_walk_body<2, 8, 2, 64, WMODE, KT, 0, RBL>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+                                                       lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
+        stamp_rows_workgroup<2, 8>(nz, smem, active, row0, stamp0 + j, count_out ? count_out + j : nullptr);
+        // the barrier (workgroup-scope fence) makes this layer's columns visible to the other waves
+        // of the workgroup before the next layer reads them
+        __syncthreads();
         in = out;
     }
 }
@@ -1481,7 +1549,7 @@ namespace {
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
 hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
     constexpr size_t lds = (size_t)RING * 64 * RL * 4;
-    auto kern = band_chain_kernel<RL, NW, OPW, RING, WMODE, KT>;
+    auto kern = band_chain_kernel<RL, NW, OPW, RING, WMODE, KT, RL == 4 ? 1 : 0>;
     // once per instantiation; a function-local static is initialised by one thread only
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -1513,12 +1581,33 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 || a.nlayers < 1 ||
         !a.table || !a.first_in || !a.buf_a || !a.buf_c || !a.active || a.buf_a == a.buf_c)
         return hipErrorInvalidValue;
+    if (a.rl == 4 && a.halves) {
+        constexpr size_t lds = 64 * 128 * 4;
+#define SPDNN_HALF(WM, KTv)                                                                                          \
+    do {                                                                                                             \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(band_chain_half_kernel<WM, KTv>), \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
+        if (attr != hipSuccess) return attr;                                                                         \
+        hipLaunchKernelGGL((band_chain_half_kernel<WM, KTv>), dim3(a.nblk * 2), dim3(512), lds, s,                   \
+                           reinterpret_cast<const ChainLayer*>(a.table), a.nlayers, a.first_in, a.buf_a, a.buf_c,    \
+                           a.active, a.count_out, a.count_prev, a.N, a.stamp0, a.prev_stamp, a.check_dead, a.bias,   \
+                           a.clampv, a.publish);                                                                     \
+    } while (0)
+        if (a.unrolled) {
+            if (a.wmode == 0) SPDNN_HALF(0, 36); else if (a.wmode == 1) SPDNN_HALF(1, 36); else SPDNN_HALF(2, 36);
+        } else {
+            if (a.wmode == 0) SPDNN_HALF(0, 0); else if (a.wmode == 1) SPDNN_HALF(1, 0); else SPDNN_HALF(2, 0);
+        }
+#undef SPDNN_HALF
+        return hipGetLastError();
+    }
     switch (a.rl) {
-        // one workgroup per row block walks the whole band: 16 waves (one pair each, chunks of 32
-        // outputs, 128-slot ring) so that a CU holds as many waves as in the per-layer kernel
-        case 4: return launch_chain_rl<4, 16, 2, 128>(a, s);
-        case 2: return launch_chain_rl<2, 16, 2, 128>(a, s);
-        case 1: return launch_chain_rl<1, 16, 2, 128>(a, s);
+        // one workgroup per row block walks the whole band, in the shape of the per-layer kernel (8 waves,
+        // one pair each, 64-slot ring): two workgroups fit a CU, so that their load / compute / barrier
+        // phases interleave
+        case 4: return launch_chain_rl<4, 8, 2, 64>(a, s);
+        case 2: return launch_chain_rl<2, 8, 2, 64>(a, s);
+        case 1: return launch_chain_rl<1, 8, 2, 64>(a, s);
         default: return hipErrorInvalidValue;
     }
 }

@@ -145,6 +145,7 @@ struct ChainLaunch {
     int N, K, nblk, stamp0, prev_stamp, check_dead, rl, wmode;
     int unrolled;                 // every layer of the chain fits the unrolled path (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
+    int halves;                   // 1 (256-row blocks only): one workgroup per HALF row block (twice the workgroups)
     float bias, clampv;
     Publish publish;
 };

@@ -251,6 +251,7 @@ struct spdnn_net {
     // cleared when every carried block has been written again (new run, repack).
     bool blocks_skipped = false;
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
+    int chain_halves = 1;     // fused chains on half row blocks (SPDNN_CHAIN_HALVES=0: whole row blocks)
     bool fuse_pairs = true;   // fused pairs where the inspector found them (SPDNN_FUSE_PAIRS=0: never)
     int pair_seglen = 0;      // band positions per workgroup of a fused pair, 0 = heuristic (SPDNN_PAIR_SEGLEN)
     int64_t pair_min_elems = 0;  // rows x neurons below which a pair runs as two launches (SPDNN_PAIR_MIN_ELEMS)
@@ -748,6 +749,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     if (const char* e = getenv("SPDNN_FUSE_PAIRS")) n->fuse_pairs = atoi(e) != 0;
+    if (const char* e = getenv("SPDNN_CHAIN_HALVES")) n->chain_halves = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
@@ -1532,6 +1534,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
             ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = check_dead;
             ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
             ch.bias = n->bias; ch.clampv = n->clampv;
+            ch.halves = n->chain_halves;
             ch.publish = pub;
             HIPCHK(launch_band_chain(ch, n->stream));
             for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
