@@ -721,6 +721,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
                                                               plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
+    plan.failed = false;
     plan.set = true;
 }
 

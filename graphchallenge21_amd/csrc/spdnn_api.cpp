@@ -17,6 +17,8 @@
 #include <functional>
 #include <memory>
 #include <mutex>
+#include <new>
+#include <stdexcept>
 #include <string>
 #include <thread>
 #include <vector>
@@ -361,7 +363,10 @@ int alloc_feature_buffers(spdnn_net* n) {
     const char* env = getenv("SPDNN_REGION_PAIRING");
     size_t free_b = 0, total_b = 0;
     HIPCHK(hipMemGetInfo(&free_b, &total_b));
-    const size_t max_cand = std::min<size_t>(64, (size_t)((double)free_b * 0.85 / (double)half_bytes));
+    // the search never holds more than this share of the free device memory (candidates + fillers)
+    const char* budget_env = getenv("SPDNN_REGION_PAIRING_BUDGET");
+    const double budget_frac = budget_env ? std::min(0.9, std::max(0.05, atof(budget_env))) : 0.6;
+    const size_t max_cand = std::min<size_t>(64, (size_t)((double)free_b * budget_frac / (double)half_bytes));
     const char* min_env = getenv("SPDNN_REGION_PAIRING_MIN_GIB");   // smallest half-buffer worth the search
     const double min_gib = min_env ? atof(min_env) : 0.4;
     const bool search = !(env && atoi(env) == 0) && (double)half_bytes >= min_gib * 1073741824.0 && max_cand >= 12;
@@ -419,7 +424,7 @@ int alloc_feature_buffers(spdnn_net* n) {
         // every step past the first six candidates advances at least 4 GiB through the memory: small
         // half-buffers are spaced out by fillers, which are freed again below
         const size_t filler = half_bytes < ((size_t)4 << 30) ? ((size_t)4 << 30) - half_bytes : 0;
-        const size_t budget = (size_t)((double)free_b * 0.85);
+        const size_t budget = (size_t)((double)free_b * budget_frac);
         rate.assign(1, 0.0);
         bool found = false;
         int ref = 0;
@@ -711,11 +716,36 @@ int submit_layer(spdnn_net* n, int layer, std::shared_ptr<std::vector<int32_t>> 
     const int N = n->N;
     LayerPlan* plan = &n->layers[(size_t)layer];
     const bool fma_ok = n->fma_ok;
-    n->pool->submit([=] { inspect_layer(N, *rp, *col, *val, force, fma_ok, *plan); });
+    n->pool->submit([=] {
+        // a worker must not let an exception escape (std::terminate): the layer stays unset and
+        // spdnn_inspect reports it
+        try {
+            inspect_layer(N, *rp, *col, *val, force, fma_ok, *plan);
+        } catch (...) {
+            plan->set = false;
+            plan->failed = true;
+        }
+    });
     return SPDNN_OK;
 }
 
 }  // namespace
+
+// Exception barrier of the C ABI: status codes, never an exception across the boundary and never
+// std::terminate (a failed allocation inside a loader or the inspector ends here).
+template <class F> int guarded(F&& f) {
+    try {
+        return f();
+    } catch (const std::bad_alloc&) {
+        return fail(SPDNN_E_NOMEM, "out of host memory");
+    } catch (const std::length_error&) {
+        return fail(SPDNN_E_NOMEM, "out of host memory (size beyond what a container can hold)");
+    } catch (const std::exception& e) {
+        return fail(SPDNN_E_ARG, std::string("unexpected failure: ") + e.what());
+    } catch (...) {
+        return fail(SPDNN_E_ARG, "unexpected failure");
+    }
+}
 
 extern "C" {
 
@@ -723,7 +753,7 @@ int spdnn_version(void) { return 100; }
 
 const char* spdnn_last_error(void) { return g_err.c_str(); }
 
-int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp, spdnn_net** out) {
+static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, float clamp, spdnn_net** out) {
     if (!out) return fail(SPDNN_E_ARG, "out is NULL");
     *out = nullptr;
     if (neuron < 1 || neuron > (1 << 24)) return fail(SPDNN_E_ARG, "neuron must be in [1, 2^24]");
@@ -763,7 +793,7 @@ int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp,
     return SPDNN_OK;
 }
 
-int spdnn_destroy(spdnn_net* n) {
+static int spdnn_destroy_impl(spdnn_net* n) {
     if (!n) return SPDNN_OK;
     n->pool->wait_all();
     n->pool.reset();
@@ -776,7 +806,7 @@ int spdnn_destroy(spdnn_net* n) {
     return SPDNN_OK;
 }
 
-int spdnn_reference_bias(int neuron, float* bias) {
+static int spdnn_reference_bias_impl(int neuron, float* bias) {
     if (!bias) return fail(SPDNN_E_ARG, "bias is NULL");
     switch (neuron) {
         case 1024: *bias = -0.3f; return SPDNN_OK;
@@ -787,7 +817,7 @@ int spdnn_reference_bias(int neuron, float* bias) {
     }
 }
 
-int spdnn_set_force_kernel(spdnn_net* n, int kernel) {
+static int spdnn_set_force_kernel_impl(spdnn_net* n, int kernel) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (kernel != SPDNN_KERNEL_AUTO && kernel != SPDNN_KERNEL_GATHER)
         return fail(SPDNN_E_ARG, "only AUTO or GATHER can be forced");
@@ -797,7 +827,7 @@ int spdnn_set_force_kernel(spdnn_net* n, int kernel) {
     return SPDNN_OK;
 }
 
-int spdnn_set_layer_csr(spdnn_net* n, int layer, const int32_t* rowptr, const int32_t* col, const float* val) {
+static int spdnn_set_layer_csr_impl(spdnn_net* n, int layer, const int32_t* rowptr, const int32_t* col, const float* val) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     auto rp = std::make_shared<std::vector<int32_t>>();
@@ -813,7 +843,7 @@ int spdnn_set_layer_csr(spdnn_net* n, int layer, const int32_t* rowptr, const in
     return submit_layer(n, layer, rp, cc, vv);
 }
 
-int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
+static int spdnn_load_layer_tsv_impl(spdnn_net* n, int layer, const char* path) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     std::vector<int32_t> rp, cc;
@@ -823,7 +853,7 @@ int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
     return spdnn_set_layer_csr(n, layer, rp.data(), cc.data(), vv.data());
 }
 
-int spdnn_load_layers_tsv(spdnn_net* n, const char* data_dir, int first, int count) {
+static int spdnn_load_layers_tsv_impl(spdnn_net* n, const char* data_dir, int first, int count) {
     if (!n || !data_dir) return fail(SPDNN_E_ARG, "NULL argument");
     if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
     n->pool->wait_all();
@@ -866,7 +896,7 @@ int spdnn_load_layers_tsv(spdnn_net* n, const char* data_dir, int first, int cou
     return SPDNN_OK;
 }
 
-int spdnn_load_layers_bin(spdnn_net* n, const char* path, int first, int count, int64_t nnz_per_layer) {
+static int spdnn_load_layers_bin_impl(spdnn_net* n, const char* path, int first, int count, int64_t nnz_per_layer) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
     const int64_t nnz = nnz_per_layer > 0 ? nnz_per_layer : (int64_t)32 * n->N;
@@ -882,14 +912,14 @@ int spdnn_load_layers_bin(spdnn_net* n, const char* path, int first, int count, 
     return SPDNN_OK;
 }
 
-int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap) {
+static int spdnn_weight_file_name_impl(const char* data_dir, int neuron, int layer, char* out, int cap) {
     if (!data_dir || !out || cap < 1) return fail(SPDNN_E_ARG, "NULL argument");
     const int w = snprintf(out, (size_t)cap, "%s/neuron%d/n%d-l%d.tsv", data_dir, neuron, neuron, layer + 1);
     if (w < 0 || w >= cap) return fail(SPDNN_E_ARG, "buffer too small");
     return SPDNN_OK;
 }
 
-int spdnn_synth_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row, float value,
+static int spdnn_synth_layer_csr_impl(uint64_t seed, int layer, int neuron, int nnz_per_row, float value,
                           int32_t* rowptr, int32_t* col, float* val) {
     if (!rowptr || !col || !val) return fail(SPDNN_E_ARG, "NULL argument");
     std::vector<int32_t> rp, cc;
@@ -902,7 +932,7 @@ int spdnn_synth_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row,
     return SPDNN_OK;
 }
 
-int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nnz_per_row, float value) {
+static int spdnn_synth_layers_impl(spdnn_net* n, uint64_t seed, int first, int count, int nnz_per_row, float value) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (first < 0 || count < 0 || first + count > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
     if (nnz_per_row < 1 || nnz_per_row > n->N || !std::isfinite(value))
@@ -925,12 +955,15 @@ int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nn
     return SPDNN_OK;
 }
 
-int spdnn_inspect(spdnn_net* n) {
+static int spdnn_inspect_impl(spdnn_net* n) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     n->pool->wait_all();
     std::fill(n->pending.begin(), n->pending.end(), 0);
     for (int l = 0; l < n->L; ++l)
-        if (!n->layers[(size_t)l].set) return fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
+        if (!n->layers[(size_t)l].set)
+            return n->layers[(size_t)l].failed
+                       ? fail(SPDNN_E_NOMEM, "the inspection of layer " + std::to_string(l) + " ran out of host memory; hand it over again")
+                       : fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
     for (int l = 0; l < n->L; ++l) {
         LayerPlan* cur = &n->layers[(size_t)l];
         const std::vector<int32_t>* nxt = l + 1 < n->L ? &n->layers[(size_t)l + 1].in_pos : nullptr;
@@ -951,7 +984,7 @@ int spdnn_inspect(spdnn_net* n) {
     return SPDNN_OK;
 }
 
-int spdnn_set_plan_window(spdnn_net* n, int slots) {
+static int spdnn_set_plan_window_impl(spdnn_net* n, int slots) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (slots != 0 && (slots < 2 || slots > 64)) return fail(SPDNN_E_ARG, "plan window is 0 (all plans resident) or 2..64 slots");
     if (n->uploaded) return fail(SPDNN_E_STATE, "plans are on the device already: set the window before the features");
@@ -959,7 +992,7 @@ int spdnn_set_plan_window(spdnn_net* n, int slots) {
     return SPDNN_OK;
 }
 
-int spdnn_get_plan_memory(const spdnn_net* n, int* window, int64_t* device_bytes, int64_t* pinned_bytes) {
+static int spdnn_get_plan_memory_impl(const spdnn_net* n, int* window, int64_t* device_bytes, int64_t* pinned_bytes) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (!n->uploaded) return fail(SPDNN_E_STATE, "plans are not on the device yet");
     int64_t total = 0;
@@ -971,7 +1004,7 @@ int spdnn_get_plan_memory(const spdnn_net* n, int* window, int64_t* device_bytes
     return SPDNN_OK;
 }
 
-int spdnn_get_layer_plan(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
+static int spdnn_get_layer_plan_impl(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
     if (!n || !out) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     const_cast<spdnn_net*>(n)->pool->wait_all();
@@ -980,7 +1013,7 @@ int spdnn_get_layer_plan(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
     return SPDNN_OK;
 }
 
-int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel) {
+static int spdnn_get_band_plan_impl(const spdnn_net* n, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     const_cast<spdnn_net*>(n)->pool->wait_all();
@@ -992,7 +1025,7 @@ int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t*
     return SPDNN_OK;
 }
 
-int spdnn_get_band_pairs(const spdnn_net* n, int layer, int* steps, int* stride, int* padded_steps,
+static int spdnn_get_band_pairs_impl(const spdnn_net* n, int layer, int* steps, int* stride, int* padded_steps,
                          int* has_weights, uint32_t* records, float* weights) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
@@ -1008,7 +1041,7 @@ int spdnn_get_band_pairs(const spdnn_net* n, int layer, int* steps, int* stride,
     return SPDNN_OK;
 }
 
-int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
+static int spdnn_get_layer_dst_impl(const spdnn_net* n, int layer, int32_t* dst) {
     if (!n || !dst) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     if (!n->inspected) return fail(SPDNN_E_STATE, "spdnn_inspect has not been called");
@@ -1017,7 +1050,7 @@ int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
     return SPDNN_OK;
 }
 
-int spdnn_receptive_field(spdnn_net* n, int first_layer, int n_layers, const int32_t* out_neurons, int n_out,
+static int spdnn_receptive_field_impl(spdnn_net* n, int first_layer, int n_layers, const int32_t* out_neurons, int n_out,
                           int32_t* in_neurons, int64_t cap, int64_t* count) {
     if (!n || !count || (n_out > 0 && !out_neurons)) return fail(SPDNN_E_ARG, "NULL argument");
     if (first_layer < 0 || n_layers < 1 || first_layer + n_layers > n->L) return fail(SPDNN_E_ARG, "layer range out of bounds");
@@ -1034,7 +1067,7 @@ int spdnn_receptive_field(spdnn_net* n, int first_layer, int n_layers, const int
     return SPDNN_OK;
 }
 
-int spdnn_get_layer_slots(const spdnn_net* n, int layer, int* slots) {
+static int spdnn_get_layer_slots_impl(const spdnn_net* n, int layer, int* slots) {
     if (!n || !slots) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     const_cast<spdnn_net*>(n)->pool->wait_all();
@@ -1043,7 +1076,7 @@ int spdnn_get_layer_slots(const spdnn_net* n, int layer, int* slots) {
     return SPDNN_OK;
 }
 
-int spdnn_get_input_labelling(const spdnn_net* n, int layer, int32_t* phys_col) {
+static int spdnn_get_input_labelling_impl(const spdnn_net* n, int layer, int32_t* phys_col) {
     if (!n || !phys_col) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer > n->L) return fail(SPDNN_E_ARG, "layer out of range");
     const_cast<spdnn_net*>(n)->pool->wait_all();
@@ -1057,7 +1090,7 @@ int spdnn_get_input_labelling(const spdnn_net* n, int layer, int32_t* phys_col) 
     return SPDNN_OK;
 }
 
-int spdnn_hash_reorder(int v, int buckets, int domain, int* out) {
+static int spdnn_hash_reorder_impl(int v, int buckets, int domain, int* out) {
     if (!out) return fail(SPDNN_E_ARG, "out is NULL");
     if (buckets <= 0 || domain <= 0 || v < 0 || v >= domain) return fail(SPDNN_E_ARG, "ERROR: Hasing Function error!");
     const int width = domain / buckets;
@@ -1078,7 +1111,7 @@ static int begin_features(spdnn_net* n, int batch) {
     return SPDNN_OK;
 }
 
-int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
+static int spdnn_set_features_dense_impl(spdnn_net* n, const float* rowmajor, int batch) {
     if (!rowmajor) return fail(SPDNN_E_ARG, "rowmajor is NULL");
     int rc = begin_features(n, batch);
     if (rc) return rc;
@@ -1113,7 +1146,7 @@ int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
     return SPDNN_OK;
 }
 
-int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
+static int spdnn_load_features_tsv_impl(spdnn_net* n, const char* path, int batch) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
     std::vector<float> dense;
@@ -1123,7 +1156,7 @@ int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
     return spdnn_set_features_dense(n, dense.data(), batch);
 }
 
-int spdnn_read_features_tsv(const char* path, int neuron, int batch, float* rowmajor, int64_t* kept) {
+static int spdnn_read_features_tsv_impl(const char* path, int neuron, int batch, float* rowmajor, int64_t* kept) {
     if (!path || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
     if (neuron < 1 || batch < 1) return fail(SPDNN_E_ARG, "neuron and batch must be positive");
     std::string err;
@@ -1133,7 +1166,7 @@ int spdnn_read_features_tsv(const char* path, int neuron, int batch, float* rowm
     return SPDNN_OK;
 }
 
-int spdnn_load_features_bin(spdnn_net* n, const char* path, int batch) {
+static int spdnn_load_features_bin_impl(spdnn_net* n, const char* path, int batch) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     if (batch < 1 || batch > n->max_batch) return fail(SPDNN_E_ARG, "batch must be in [1, max_batch]");
     std::vector<float> dense;
@@ -1143,7 +1176,7 @@ int spdnn_load_features_bin(spdnn_net* n, const char* path, int batch) {
     return spdnn_set_features_dense(n, dense.data(), batch);
 }
 
-int spdnn_synth_features(spdnn_net* n, uint64_t seed, int batch, float dmin, float dmax) {
+static int spdnn_synth_features_impl(spdnn_net* n, uint64_t seed, int batch, float dmin, float dmax) {
     if (!(dmin >= 0.0f) || !(dmax >= dmin) || !(dmax <= 1.0f)) return fail(SPDNN_E_ARG, "need 0 <= dmin <= dmax <= 1");
     int rc = begin_features(n, batch);
     if (rc) return rc;
@@ -1164,7 +1197,7 @@ int spdnn_synth_features(spdnn_net* n, uint64_t seed, int batch, float dmin, flo
     return SPDNN_OK;
 }
 
-int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows, float dmin,
+static int spdnn_synth_features_host_impl(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows, float dmin,
                               float dmax, float* rowmajor) {
     if (!rowmajor || neuron < 1 || nrows < 0) return fail(SPDNN_E_ARG, "bad argument");
     synth_features_host(seed, neuron, row_begin, nrows, dmin, dmax, rowmajor);
@@ -1173,7 +1206,7 @@ int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int6
 
 // ---- inference -----------------------------------------------------------------------------
 
-int spdnn_default_run_options(spdnn_run_options* o) {
+static int spdnn_default_run_options_impl(spdnn_run_options* o) {
     if (!o) return fail(SPDNN_E_ARG, "opt is NULL");
     memset(o, 0, sizeof(*o));
     o->prune = 1;
@@ -1359,7 +1392,7 @@ static int wait_counts(spdnn_net* n, int l0, int c) {
     return SPDNN_OK;
 }
 
-int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
+static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     spdnn_run_options opt;
     if (opt_in) opt = *opt_in; else spdnn_default_run_options(&opt);
@@ -1656,7 +1689,7 @@ int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* r
     return SPDNN_OK;
 }
 
-int spdnn_get_active_count(const spdnn_net* n, int layer, int64_t* count) {
+static int spdnn_get_active_count_impl(const spdnn_net* n, int layer, int64_t* count) {
     if (!n || !count) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
     if (n->counts[(size_t)layer] < 0) return fail(SPDNN_E_STATE, "no count recorded for this layer");
@@ -1664,7 +1697,7 @@ int spdnn_get_active_count(const spdnn_net* n, int layer, int64_t* count) {
     return SPDNN_OK;
 }
 
-int spdnn_get_categories(spdnn_net* n, int32_t* ids, int64_t cap, int64_t* cnt) {
+static int spdnn_get_categories_impl(spdnn_net* n, int32_t* ids, int64_t cap, int64_t* cnt) {
     if (!n || !cnt) return fail(SPDNN_E_ARG, "NULL argument");
     if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
     if (n->cur_layer == 0) {  // nothing run yet: every row counts
@@ -1683,7 +1716,7 @@ int spdnn_get_categories(spdnn_net* n, int32_t* ids, int64_t cap, int64_t* cnt) 
     return SPDNN_OK;
 }
 
-int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+static int spdnn_get_activations_impl(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
     if (!n || !rows || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
     if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
     if (nrows < 0) return fail(SPDNN_E_ARG, "nrows negative");
@@ -1717,7 +1750,7 @@ int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* r
     return SPDNN_OK;
 }
 
-int spdnn_get_activations_noalloc(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+static int spdnn_get_activations_noalloc_impl(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
     if (!n || !rows || !rowmajor) return fail(SPDNN_E_ARG, "NULL argument");
     if (!n->have_features) return fail(SPDNN_E_STATE, "no features set");
     if (nrows < 0) return fail(SPDNN_E_ARG, "nrows negative");
@@ -1755,7 +1788,7 @@ int spdnn_get_activations_noalloc(spdnn_net* n, const int32_t* rows, int nrows, 
     return SPDNN_OK;
 }
 
-int spdnn_get_band_tuning(const spdnn_net* n, int index, int* row_blocks, int* shape, int* seglen) {
+static int spdnn_get_band_tuning_impl(const spdnn_net* n, int index, int* row_blocks, int* shape, int* seglen) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (index < 0 || index >= (int)n->tuned.size()) return fail(SPDNN_E_ARG, "no such tuning record");
     const spdnn_net::Tuned& t = n->tuned[(size_t)index];
@@ -1765,14 +1798,14 @@ int spdnn_get_band_tuning(const spdnn_net* n, int index, int* row_blocks, int* s
     return SPDNN_OK;
 }
 
-int spdnn_get_layer_times(const spdnn_net* n, float* ms, int cnt) {
+static int spdnn_get_layer_times_impl(const spdnn_net* n, float* ms, int cnt) {
     if (!n || !ms) return fail(SPDNN_E_ARG, "NULL argument");
     if (cnt < 0 || cnt > n->L) return fail(SPDNN_E_ARG, "n out of range");
     std::copy(n->layer_ms.begin(), n->layer_ms.begin() + cnt, ms);
     return SPDNN_OK;
 }
 
-int spdnn_write_categories(spdnn_net* n, const char* path) {
+static int spdnn_write_categories_impl(spdnn_net* n, const char* path) {
     if (!n || !path) return fail(SPDNN_E_ARG, "NULL argument");
     int64_t cnt = 0;
     int rc = spdnn_get_categories(n, nullptr, 0, &cnt);
@@ -1789,7 +1822,7 @@ int spdnn_write_categories(spdnn_net* n, const char* path) {
 
 // ---- device utilities ------------------------------------------------------------------------
 
-int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
+static int spdnn_measure_copy_bandwidth_impl(int64_t bytes, int reps, double* gbps) {
     if (!gbps || bytes < 1024 || reps < 1) return fail(SPDNN_E_ARG, "bad argument");
     bytes &= ~(int64_t)1023;
     DevTmp abuf, bbuf;
@@ -1812,7 +1845,7 @@ int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
     return SPDNN_OK;
 }
 
-int spdnn_measure_buffer_copy_bandwidth(spdnn_net* n, int reps, double* gbps) {
+static int spdnn_measure_buffer_copy_bandwidth_impl(spdnn_net* n, int reps, double* gbps) {
     if (!n || !gbps || reps < 1) return fail(SPDNN_E_ARG, "bad argument");
     if (!n->uploaded || !n->have_features) return fail(SPDNN_E_STATE, "no feature buffers yet: set features first");
     const int nblk = (n->batch + n->RB - 1) / n->RB;
@@ -1834,7 +1867,7 @@ int spdnn_measure_buffer_copy_bandwidth(spdnn_net* n, int reps, double* gbps) {
     return SPDNN_OK;
 }
 
-int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
+static int spdnn_device_info_impl(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
     int cnt = 0;
     if (hipGetDeviceCount(&cnt) != hipSuccess || cnt < 1) return fail(SPDNN_E_DEVICE, "no HIP device available");
     hipDeviceProp_t p;
@@ -1845,7 +1878,7 @@ int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_byte
     return SPDNN_OK;
 }
 
-int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates) {
+static int spdnn_get_feature_placement_impl(const spdnn_net* n, int* paired, int* candidates) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (!n->uploaded) return fail(SPDNN_E_STATE, "no feature buffers yet");
     if (paired) *paired = n->feat_paired;
@@ -1853,7 +1886,7 @@ int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates
     return SPDNN_OK;
 }
 
-int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
+static int spdnn_device_memory_impl(int64_t* free_bytes, int64_t* total_bytes) {
     size_t f = 0, t = 0;
     HIPCHK(hipMemGetInfo(&f, &t));
     if (free_bytes) *free_bytes = (int64_t)f;
@@ -1861,9 +1894,140 @@ int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
     return SPDNN_OK;
 }
 
-int spdnn_device_synchronize(void) {
+static int spdnn_device_synchronize_impl(void) {
     HIPCHK(hipDeviceSynchronize());
     return SPDNN_OK;
 }
 
+
+// ---- the entry points proper: every one behind the exception barrier ----
+int spdnn_create(int neuron, int max_batch, int layers, float bias, float clamp, spdnn_net** out) {
+    return guarded([&] { return spdnn_create_impl(neuron, max_batch, layers, bias, clamp, out); });
+}
+int spdnn_destroy(spdnn_net* n) {
+    return guarded([&] { return spdnn_destroy_impl(n); });
+}
+int spdnn_reference_bias(int neuron, float* bias) {
+    return guarded([&] { return spdnn_reference_bias_impl(neuron, bias); });
+}
+int spdnn_set_force_kernel(spdnn_net* n, int kernel) {
+    return guarded([&] { return spdnn_set_force_kernel_impl(n, kernel); });
+}
+int spdnn_set_layer_csr(spdnn_net* n, int layer, const int32_t* rowptr, const int32_t* col, const float* val) {
+    return guarded([&] { return spdnn_set_layer_csr_impl(n, layer, rowptr, col, val); });
+}
+int spdnn_load_layer_tsv(spdnn_net* n, int layer, const char* path) {
+    return guarded([&] { return spdnn_load_layer_tsv_impl(n, layer, path); });
+}
+int spdnn_load_layers_tsv(spdnn_net* n, const char* data_dir, int first, int count) {
+    return guarded([&] { return spdnn_load_layers_tsv_impl(n, data_dir, first, count); });
+}
+int spdnn_load_layers_bin(spdnn_net* n, const char* path, int first, int count, int64_t nnz_per_layer) {
+    return guarded([&] { return spdnn_load_layers_bin_impl(n, path, first, count, nnz_per_layer); });
+}
+int spdnn_weight_file_name(const char* data_dir, int neuron, int layer, char* out, int cap) {
+    return guarded([&] { return spdnn_weight_file_name_impl(data_dir, neuron, layer, out, cap); });
+}
+int spdnn_synth_layer_csr(uint64_t seed, int layer, int neuron, int nnz_per_row, float value, int32_t* rowptr, int32_t* col, float* val) {
+    return guarded([&] { return spdnn_synth_layer_csr_impl(seed, layer, neuron, nnz_per_row, value, rowptr, col, val); });
+}
+int spdnn_synth_layers(spdnn_net* n, uint64_t seed, int first, int count, int nnz_per_row, float value) {
+    return guarded([&] { return spdnn_synth_layers_impl(n, seed, first, count, nnz_per_row, value); });
+}
+int spdnn_inspect(spdnn_net* n) {
+    return guarded([&] { return spdnn_inspect_impl(n); });
+}
+int spdnn_set_plan_window(spdnn_net* n, int slots) {
+    return guarded([&] { return spdnn_set_plan_window_impl(n, slots); });
+}
+int spdnn_get_plan_memory(const spdnn_net* n, int* window, int64_t* device_bytes, int64_t* pinned_bytes) {
+    return guarded([&] { return spdnn_get_plan_memory_impl(n, window, device_bytes, pinned_bytes); });
+}
+int spdnn_get_layer_plan(const spdnn_net* n, int layer, spdnn_layer_plan* out) {
+    return guarded([&] { return spdnn_get_layer_plan_impl(n, layer, out); });
+}
+int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t* out_at, uint8_t* sel) {
+    return guarded([&] { return spdnn_get_band_plan_impl(n, layer, in_pos, out_at, sel); });
+}
+int spdnn_get_band_pairs(const spdnn_net* n, int layer, int* steps, int* stride, int* padded_steps, int* has_weights, uint32_t* records, float* weights) {
+    return guarded([&] { return spdnn_get_band_pairs_impl(n, layer, steps, stride, padded_steps, has_weights, records, weights); });
+}
+int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
+    return guarded([&] { return spdnn_get_layer_dst_impl(n, layer, dst); });
+}
+int spdnn_receptive_field(spdnn_net* n, int first_layer, int n_layers, const int32_t* out_neurons, int n_out, int32_t* in_neurons, int64_t cap, int64_t* count) {
+    return guarded([&] { return spdnn_receptive_field_impl(n, first_layer, n_layers, out_neurons, n_out, in_neurons, cap, count); });
+}
+int spdnn_get_layer_slots(const spdnn_net* n, int layer, int* slots) {
+    return guarded([&] { return spdnn_get_layer_slots_impl(n, layer, slots); });
+}
+int spdnn_get_input_labelling(const spdnn_net* n, int layer, int32_t* phys_col) {
+    return guarded([&] { return spdnn_get_input_labelling_impl(n, layer, phys_col); });
+}
+int spdnn_hash_reorder(int v, int buckets, int domain, int* out) {
+    return guarded([&] { return spdnn_hash_reorder_impl(v, buckets, domain, out); });
+}
+int spdnn_set_features_dense(spdnn_net* n, const float* rowmajor, int batch) {
+    return guarded([&] { return spdnn_set_features_dense_impl(n, rowmajor, batch); });
+}
+int spdnn_load_features_tsv(spdnn_net* n, const char* path, int batch) {
+    return guarded([&] { return spdnn_load_features_tsv_impl(n, path, batch); });
+}
+int spdnn_read_features_tsv(const char* path, int neuron, int batch, float* rowmajor, int64_t* kept) {
+    return guarded([&] { return spdnn_read_features_tsv_impl(path, neuron, batch, rowmajor, kept); });
+}
+int spdnn_load_features_bin(spdnn_net* n, const char* path, int batch) {
+    return guarded([&] { return spdnn_load_features_bin_impl(n, path, batch); });
+}
+int spdnn_synth_features(spdnn_net* n, uint64_t seed, int batch, float dmin, float dmax) {
+    return guarded([&] { return spdnn_synth_features_impl(n, seed, batch, dmin, dmax); });
+}
+int spdnn_synth_features_host(uint64_t seed, int neuron, int64_t row_begin, int64_t nrows, float dmin, float dmax, float* rowmajor) {
+    return guarded([&] { return spdnn_synth_features_host_impl(seed, neuron, row_begin, nrows, dmin, dmax, rowmajor); });
+}
+int spdnn_default_run_options(spdnn_run_options* o) {
+    return guarded([&] { return spdnn_default_run_options_impl(o); });
+}
+int spdnn_run(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
+    return guarded([&] { return spdnn_run_impl(n, opt_in, res); });
+}
+int spdnn_get_active_count(const spdnn_net* n, int layer, int64_t* count) {
+    return guarded([&] { return spdnn_get_active_count_impl(n, layer, count); });
+}
+int spdnn_get_categories(spdnn_net* n, int32_t* ids, int64_t cap, int64_t* cnt) {
+    return guarded([&] { return spdnn_get_categories_impl(n, ids, cap, cnt); });
+}
+int spdnn_get_activations(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+    return guarded([&] { return spdnn_get_activations_impl(n, rows, nrows, rowmajor); });
+}
+int spdnn_get_activations_noalloc(spdnn_net* n, const int32_t* rows, int nrows, float* rowmajor) {
+    return guarded([&] { return spdnn_get_activations_noalloc_impl(n, rows, nrows, rowmajor); });
+}
+int spdnn_get_band_tuning(const spdnn_net* n, int index, int* row_blocks, int* shape, int* seglen) {
+    return guarded([&] { return spdnn_get_band_tuning_impl(n, index, row_blocks, shape, seglen); });
+}
+int spdnn_get_layer_times(const spdnn_net* n, float* ms, int cnt) {
+    return guarded([&] { return spdnn_get_layer_times_impl(n, ms, cnt); });
+}
+int spdnn_write_categories(spdnn_net* n, const char* path) {
+    return guarded([&] { return spdnn_write_categories_impl(n, path); });
+}
+int spdnn_measure_copy_bandwidth(int64_t bytes, int reps, double* gbps) {
+    return guarded([&] { return spdnn_measure_copy_bandwidth_impl(bytes, reps, gbps); });
+}
+int spdnn_measure_buffer_copy_bandwidth(spdnn_net* n, int reps, double* gbps) {
+    return guarded([&] { return spdnn_measure_buffer_copy_bandwidth_impl(n, reps, gbps); });
+}
+int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
+    return guarded([&] { return spdnn_device_info_impl(name, cap, compute_units, hbm_bytes); });
+}
+int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates) {
+    return guarded([&] { return spdnn_get_feature_placement_impl(n, paired, candidates); });
+}
+int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
+    return guarded([&] { return spdnn_device_memory_impl(free_bytes, total_bytes); });
+}
+int spdnn_device_synchronize(void) {
+    return guarded([&] { return spdnn_device_synchronize_impl(); });
+}
 }  // extern "C"

@@ -572,3 +572,26 @@ def test_driver_usage_paths(gc):
     assert r.returncode == 0 and "Usage: exe neuron batch layer" in r.stdout      # reference network.cpp:58-61
     r = subprocess.run([exe, "1000", "10", "2"], capture_output=True, text=True)
     assert r.returncode == 2 and "neuron must be one of" in r.stderr
+
+
+def test_allocation_failure_comes_back_as_a_status(gc):
+    """No exception crosses the C ABI and nothing calls std::terminate: with the address space capped,
+    a network of 2^28 layers (tens of GB of host bookkeeping) is refused with SPDNN_E_NOMEM and the
+    process lives on."""
+    import sys
+    code = (
+        "import resource, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "import graphchallenge21_amd as gc\n"
+        "gc.load_library()\n"
+        "resource.setrlimit(resource.RLIMIT_AS, (6 << 30, 6 << 30))\n"
+        "try:\n"
+        "    gc.Network(1024, 64, 1 << 28, bias=-0.3)\n"
+        "    print('created')\n"
+        "except gc.SpdnnError as e:\n"
+        "    print('status', e.code)\n"
+        "with gc.Network(256, 4, 1, bias=-0.3) as net:\n"
+        "    print('alive', net.layers)\n" % ROOT)
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert "status 5" in out.stdout and "alive 1" in out.stdout, out.stdout + out.stderr[-500:]
