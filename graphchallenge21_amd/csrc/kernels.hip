@@ -1477,7 +1477,14 @@ bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36
 // compute / barrier phases interleave), 32 and 16 KiB and four workgroups per CU (the wave limit)
 // for 128- and 64-row blocks.  Measured at N=65536: 256-row blocks 6.0 ms per layer, 128-row blocks
 // 6.6 ms (8.8 ms with one 16-wave workgroup and a 256-slot ring per CU).
-int band_shape_count(int rl) { (void)rl; return 1; }
+// Variants of the band walk the run-time selection chooses from (BandLaunch.shape): for 256-row
+// blocks 0 = next chunk's columns straight from HBM into the LDS ring, 1 = parked in registers and
+// written to the ring after the arithmetic (the only form for smaller row blocks).
+static bool band_direct_lds_enabled() {
+    static const bool on = !(getenv("SPDNN_BAND_DIRECT_LDS") && atoi(getenv("SPDNN_BAND_DIRECT_LDS")) == 0);
+    return on;
+}
+int band_shape_count(int rl) { return rl == 4 && band_direct_lds_enabled() ? 2 : 1; }
 
 int band_chunk_outputs(int rl, int shape) {
     (void)rl; (void)shape;
@@ -1535,10 +1542,9 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
         if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);
     }
     switch (a.rl) {
-        case 4: {
-            static const bool dma = !(getenv("SPDNN_BAND_DIRECT_LDS") && atoi(getenv("SPDNN_BAND_DIRECT_LDS")) == 0);
-            return dma ? launch_band_rl<4, 8, 2, 64, 1>(b, s) : launch_band_rl<4, 8, 2, 64, 0>(b, s);
-        }
+        case 4:
+            return (band_direct_lds_enabled() && a.shape != 1) ? launch_band_rl<4, 8, 2, 64, 1>(b, s)
+                                                              : launch_band_rl<4, 8, 2, 64, 0>(b, s);
         case 2: return launch_band_rl<2, 8, 2, 64, 0>(b, s);
         case 1: return launch_band_rl<1, 8, 2, 64, 0>(b, s);
         default: return hipErrorInvalidValue;

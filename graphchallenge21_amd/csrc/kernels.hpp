@@ -53,7 +53,7 @@ struct BandLaunch {
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
     float wu, bias, clampv;
     int n_cu;
-    int shape = -1;          // tile shape (see launch_band); < 0 = default
+    int shape = -1;          // variant (see band_shape_count): 256-row blocks 0 = direct-to-LDS loads, 1 = through registers; < 0 = default
     int seglen = 0;          // band positions per workgroup; 0 = heuristic
     long long stream_min_bytes = 96ll << 20;  // launches that read + write at least this much hint their
                                               // column loads and stores as touched once
@@ -80,8 +80,9 @@ struct GatherLaunch {
 hipError_t launch_band(const BandLaunch& a, hipStream_t s);
 // 32 entries per output, at most 36 merged steps per pair, 16-dword records: the unrolled kernel path
 bool band_unrolled(int K, int steps, int stride);
-// Tuning space of the band walk: number of tile shapes for a row-block size (one at present) and
-// the candidate segment lengths for a shape (used by the run-time selection in spdnn_run).
+// Tuning space of the band walk: number of kernel variants for a row-block size (256-row blocks:
+// loads straight into LDS or through registers) and the candidate segment lengths for a variant
+// (used by the run-time selection in spdnn_run).
 int band_shape_count(int rl);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 // the occupancy / halo model's score of one candidate (higher is better), for ordering trials

@@ -365,7 +365,8 @@ int alloc_feature_buffers(spdnn_net* n) {
     HIPCHK(hipMemGetInfo(&free_b, &total_b));
     // the search never holds more than this share of the free device memory (candidates + fillers)
     const char* budget_env = getenv("SPDNN_REGION_PAIRING_BUDGET");
-    const double budget_frac = budget_env ? std::min(0.9, std::max(0.05, atof(budget_env))) : 0.6;
+    // (0.85 by default: on some boxes the second region only starts behind 180 GB of candidates)
+    const double budget_frac = budget_env ? std::min(0.9, std::max(0.05, atof(budget_env))) : 0.85;
     const size_t max_cand = std::min<size_t>(64, (size_t)((double)free_b * budget_frac / (double)half_bytes));
     const char* min_env = getenv("SPDNN_REGION_PAIRING_MIN_GIB");   // smallest half-buffer worth the search
     const double min_gib = min_env ? atof(min_env) : 0.4;

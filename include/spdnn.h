@@ -311,9 +311,10 @@ int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float*
 int spdnn_get_activations_noalloc(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
 
 /* Band-walk configuration measured at run time (record `index` = 0, 1, ...; SPDNN_E_ARG past the
- * last): row blocks it was measured for, index of the tile shape (one shape per row-block size at
- * present: 8 waves x one output pair and a 64-slot LDS ring for 256-row blocks) and band positions
- * per workgroup. */
+ * last): row blocks it was measured for, kernel variant (256-row blocks: 0 = the next chunk's columns
+ * go from HBM straight into the LDS ring, 1 = through registers; one variant for smaller row blocks;
+ * the tile is 8 waves x one output pair and a 64-slot LDS ring in every case) and band positions per
+ * workgroup. */
 int spdnn_get_band_tuning(const spdnn_net* net, int index, int* row_blocks, int* shape, int* seglen);
 
 /* Per-layer kernel milliseconds of the last run made with time_layers. */
