@@ -353,7 +353,8 @@ void free_device(spdnn_net* n);
 // are taken from two different memory regions.  Which allocation lies where only shows in a
 // measurement: candidates are allocated one after the other and each is swept by a streaming write
 // together with the first one - 6.0 TB/s when the two share a region, 7.2 TB/s when they do not
-// (MI355X) - until three candidates of either kind are there; the rest is freed again.  On a fresh
+// (MI355X) - until two candidates of the first one's kind (itself included) and three of the other
+// are there; the rest is freed again.  On a fresh
 // device the boundary comes after about a third of the memory.  SPDNN_REGION_PAIRING=0 switches
 // the search off, SPDNN_ALLOC_VERBOSE=1 prints the measurements.
 int alloc_feature_buffers(spdnn_net* n) {
@@ -420,7 +421,9 @@ int alloc_feature_buffers(spdnn_net* n) {
                 if (rate[k] > 1.10 * lowest) other.push_back((int)k);
                 else if (rate[k] < 1.05 * lowest) same.push_back((int)k);
             }
-            return same.size() >= 3 && other.size() >= 3;
+            // The two work buffers, which every layer streams through, need a half of each kind; the
+            // feature buffer (read by the first layer only) takes one if there is one.
+            return same.size() >= 2 && other.size() >= 3;
         };
         // every step past the first six candidates advances at least 4 GiB through the memory: small
         // half-buffers are spaced out by fillers, which are freed again below
@@ -466,10 +469,18 @@ int alloc_feature_buffers(spdnn_net* n) {
             fprintf(stderr, "spdnn: half-buffers of %.1f GB swept together with candidate %d, GB/s:", (double)half_bytes / 1e9, ref);
             for (size_t k = 0; k < rate.size(); ++k) if ((int)k != ref) fprintf(stderr, " %.0f", rate[k]);
             fprintf(stderr, "\nspdnn: %zu in its region, %zu elsewhere%s\n", same.size(), other.size(),
-                    found ? ": every buffer gets one half of each" : ": no pairing");
+                    found ? ": the work buffers get one half of each" : ": no pairing");
         }
         if (found) {
-            for (int b = 0; b < 3; ++b) { pick[2 * b] = same[(size_t)b]; pick[2 * b + 1] = other[(size_t)b]; }
+            for (int b = 0; b < 2; ++b) { pick[2 * b] = same[(size_t)b]; pick[2 * b + 1] = other[(size_t)b]; }
+            pick[5] = other[2];
+            pick[4] = -1;
+            if (same.size() >= 3) pick[4] = same[2];
+            for (size_t k = 0; k < c.size() && pick[4] < 0; ++k) {   // else any candidate not taken yet
+                bool taken = false;
+                for (int q = 0; q < 6; ++q) taken |= q != 4 && pick[q] == (int)k;
+                if (!taken) pick[4] = (int)k;
+            }
             n->feat_paired = 1;
         }
     }
