@@ -447,9 +447,6 @@ bool build_tiled_plan(int N, const std::vector<int32_t>& rowptr, const std::vect
     for (int t = 0; t < ntiles; ++t) {
         const int o0 = t * TO, o1 = std::min(N, o0 + TO);
         std::vector<int32_t> outs(order.begin() + o0, order.begin() + o1);
-        std::stable_sort(outs.begin(), outs.end(), [&](int32_t a, int32_t b) {
-            return rowptr[a + 1] - rowptr[a] > rowptr[b + 1] - rowptr[b];
-        });
         std::vector<int32_t> uni;
         for (int32_t j : outs) uni.insert(uni.end(), col.begin() + rowptr[j], col.begin() + rowptr[j + 1]);
         std::sort(uni.begin(), uni.end());
@@ -458,6 +455,32 @@ bool build_tiled_plan(int N, const std::vector<int32_t>& rowptr, const std::vect
         if (staged > 4 * (int64_t)N) return false;
         for (size_t k = 0; k < uni.size(); ++k) slot_of[(size_t)uni[k]] = (int32_t)k;
         const int np = (int)((uni.size() + PC - 1) / PC);
+        // The 64 outputs of a wave pad, panel by panel, to the longest among them: deal the outputs to
+        // the waves so that a wave's outputs are alike in the FIRST panel and, inside a quarter of the
+        // tile, in the rest (on 1..24 random inputs per output of 1024: 19 000 entries with padding
+        // instead of 22 700 when sorted by length alone; 13 200 are real).
+        {
+            auto first = [&](int32_t j) {
+                int c = 0;
+                for (int e = rowptr[j]; e < rowptr[j + 1] && slot_of[(size_t)col[e]] < PC; ++e) ++c;
+                return c;
+            };
+            std::vector<std::pair<int, int>> cnt(outs.size());   // (entries in the first panel, in the others)
+            std::vector<int32_t> idx(outs.size());
+            for (size_t k = 0; k < outs.size(); ++k) {
+                const int f = np > 1 ? first(outs[k]) : 0;
+                cnt[k] = {f, rowptr[outs[k] + 1] - rowptr[outs[k]] - f};
+                idx[k] = (int32_t)k;
+            }
+            std::stable_sort(idx.begin(), idx.end(), [&](int32_t a, int32_t b) { return cnt[(size_t)a].first > cnt[(size_t)b].first; });
+            const size_t quarter = ((outs.size() + 3) / 4 + WO - 1) / WO * WO;
+            for (size_t b0 = 0; b0 < idx.size(); b0 += quarter)
+                std::stable_sort(idx.begin() + (long)b0, idx.begin() + (long)std::min(idx.size(), b0 + quarter),
+                                 [&](int32_t a, int32_t b) { return cnt[(size_t)a].second > cnt[(size_t)b].second; });
+            std::vector<int32_t> dealt(outs.size());
+            for (size_t k = 0; k < outs.size(); ++k) dealt[k] = outs[(size_t)idx[k]];
+            outs.swap(dealt);
+        }
         hdr[(size_t)2 * t] = gp;
         hdr[(size_t)2 * t + 1] = np;
         for (size_t k = 0; k < outs.size(); ++k) out_at[(size_t)o0 + k] = outs[k];
