@@ -970,10 +970,11 @@ __device__ __forceinline__ void column64_to_lds(const float* gsrc_lane, unsigned
 // other half of the wave's entry ring).  The caller waits itself (wait_vector_memory).
 __device__ __forceinline__ void block_to_lds_untracked(const float* gsrc_lane, unsigned char* lds_block) {
     const uint32_t lds_off = (uint32_t)(size_t)((__attribute__((address_space(3))) unsigned char*)lds_block);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :
+    uint32_t m0_saved;   // M0 (the LDS base of such a load) is the compiler's to manage: put it back
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(m0_saved)
                  : "s"(lds_off), "v"(gsrc_lane)
-                 : "m0", "memory");
+                 : "memory");
 }
 
 template <int WMODE>
