@@ -359,13 +359,15 @@ def test_full_batch_properties_cfg1(gc, orc):
         assert same_floats(y_p[:k], ref["y"][pos])
 
 
+@pytest.mark.parametrize("halves", [1, 0])
 @pytest.mark.parametrize("prune", [True, False])
 @pytest.mark.parametrize("fuse", [4, 16])
-def test_fused_layer_chain(gc, orc, fuse, prune):
-    """The fused variant (several band layers per launch, one workgroup per row block) must give
-    what the layer-by-layer launches give: counts, categories and activations."""
+def test_fused_layer_chain(gc, orc, fuse, prune, halves, monkeypatch):
+    """The fused variant (several band layers per launch, one workgroup per half or whole row block)
+    must give what the layer-by-layer launches give: counts, categories and activations."""
+    monkeypatch.setenv("SPDNN_CHAIN_HALVES", str(halves))
     N, L, B = 1024, 24, 3000
-    print("fused chain fuse=%d prune=%s" % (fuse, prune), flush=True)
+    print("fused chain fuse=%d prune=%s halves=%d" % (fuse, prune, halves), flush=True)
     layers = [orc.gen_layer_csr(5, l, N) for l in range(L)]
     feats = orc.gen_features(5, N, 0, B, 0.10, 0.50)
     ref = orc.infer(feats, layers, -0.3, prune=True)
