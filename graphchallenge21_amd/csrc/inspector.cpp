@@ -431,7 +431,7 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
 bool build_tiled_plan(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                       const std::vector<float>& val, LayerPlan& plan) {
     constexpr int TO = kTileOutputs, PC = kPanelCols, WO = 64, NWV = TO / WO;
-    if (N < 64) return false;
+    if (N < 64 || rowptr[N] == 0) return false;   // (a layer without any entry: nothing to stage)
     const int ntiles = (N + TO - 1) / TO;
     // outputs in the order of the middle of their input lists, so that a tile's union stays small
     // where the layer has locality; empty rows last

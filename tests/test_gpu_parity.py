@@ -730,6 +730,22 @@ def test_empty_rows_and_single_layer(gc, orc):
             assert same_floats(net.activations(np.arange(B, dtype=np.int32)), y)
             assert np.array_equal(net.categories(), np.nonzero(act)[0])
             assert net.active_count(0) == int(act.sum())
+    # a layer without a single entry between two ordinary ones: every output is relu(bias)
+    N2 = 256
+    empty = (np.zeros(N2 + 1, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32))
+    layers = [orc.gen_layer_csr(1, 0, N2), empty, sort_rows(random_csr(rng, N2, rng.integers(1, 6, size=N2), "general"))]
+    f2 = orc.gen_features(1, N2, 0, B, 0.2, 0.8)
+    for bias in (-0.1, 0.2):
+        ref = orc.infer(f2, layers, bias, prune=False, keep={2})
+        with gc.Network(N2, B, 3, bias=bias) as net:
+            for l, c in enumerate(layers):
+                net.set_layer_csr(l, *c)
+            net.inspect()
+            assert net.layer_plan(1).kernel == gc.KERNEL_GATHER and net.layer_plan(2).kernel == gc.KERNEL_TILED
+            net.set_features_dense(f2)
+            net.run(prune=False, collect_counts=True)
+            assert same_floats(net.activations(np.arange(B, dtype=np.int32)), ref["kept"][2][1])
+            assert np.array_equal(net.categories(), ref["active_ids"][2])
 
 
 def test_cli_driver_on_tsv_files(gc, orc, tmp_path):
