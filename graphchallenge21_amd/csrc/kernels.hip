@@ -783,7 +783,7 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int role = wave >> 3, w = wave & 7;     // role 0: layer A, role 1: layer B
     const int loff = lane * 4;
-    if (enter_row_block<4>(active, (size_t)rb * RB + loff, prev_stamp, stamp_a, check_dead, count_prev,
+    if (enter_row_block<4>(active, (size_t)rb * RB + loff, prev_stamp, stamp_b, check_dead, count_prev,
                            blockIdx.y == 0 && threadIdx.x < 64))
         return;
     const size_t blkf = (size_t)N * RB;

@@ -465,6 +465,41 @@ def test_fused_pairs_full_batch(gc, orc):
         assert same_floats(net.activations(probe), y_fused)
 
 
+def test_fused_pairs_several_segments_per_row_block(gc, orc, monkeypatch):
+    """A pruned run in which a row block's band is cut into segments that run one after the other (more
+    workgroups than the chip holds): a workgroup that starts late finds rows already stamped by the
+    segments that have finished, and must still see them as alive."""
+    monkeypatch.setenv("SPDNN_PAIR_SEGLEN", "512")
+    N, B, L, S = 4096, 60000, 7, 512
+    print("fused pairs, segments in several rounds", flush=True)
+    rng = np.random.default_rng(78)
+    perm = rng.permutation(N)
+    # weights of both signs with gain above 1 and dense rows: every row stays alive for good (so that no row of
+    # a row block dies in a pair), at values below the clamp that differ from layer to layer
+    layers = []
+    for _ in range(L):
+        rp, c, v = common_band_csr(rng, N, perm, "general")
+        layers.append((rp, c, rng.uniform(-0.3, 0.4, size=len(v)).astype(np.float32)))
+    ref = orc.infer(orc.gen_features(10, N, 0, S, 0.30, 0.90), layers, -0.35, prune=True)
+    assert len(ref["categories"]) == S and float(np.median(ref["y"])) < 16.0
+    with gc.Network(N, B, L, bias=-0.35) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.synth_features(10, B, 0.30, 0.90)
+        net.run(prune=False, collect_counts=True, fuse_layers=1)
+        counts = [net.active_count(l) for l in range(L)]
+        cats = net.categories()
+        assert np.array_equal(cats[cats < S], ref["categories"])
+        # layer 0 alone, then the pairs (1,2), (3,4), ...: every pair runs behind a stamped layer
+        net.run(prune=True, first_layer=0, n_layers=1)
+        r = net.run(prune=True, first_layer=1, n_layers=L - 1, collect_counts=True, fuse_layers=2)
+        assert r.fused_pairs == (L - 1) // 2
+        assert [net.active_count(l) for l in range(1, L)] == counts[1:]
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(ref["categories"]), ref["y"])
+
+
 def test_fused_chain_when_everything_dies(gc, orc):
     """Literal inputs: all rows die within a few layers; workgroups leave the chain early."""
     N, L, B = 1024, 40, 2000
