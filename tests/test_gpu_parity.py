@@ -500,6 +500,57 @@ def test_fused_pairs_several_segments_per_row_block(gc, orc, monkeypatch):
         assert same_floats(net.activations(ref["categories"]), ref["y"])
 
 
+@pytest.mark.parametrize("kind", ["band", "radix", "radix-blocks", "hub", "irregular", "irregular-gather"])
+def test_pruned_run_with_rows_that_never_die(gc, orc, kind, monkeypatch):
+    """Full batch, pruning on, and every row alive for good at values below the clamp that differ from layer
+    to layer: a workgroup that wrongly takes its rows for dead (rows that the workgroups before it have
+    already stamped) leaves another layer's values behind, which this data shows."""
+    from helpers import hub_block_csr, radix_like_csr
+    N, B, L, S = 4096, 60000, 6, 256
+    print("rows that never die:", kind, flush=True)
+    if kind == "radix-blocks":
+        monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "0")
+    rng = np.random.default_rng(5)
+
+    def layer(l):
+        if kind == "band":
+            rp, c, v = orc.gen_layer_csr(3, l, N)
+        elif kind.startswith("radix"):
+            rp, c, v = radix_like_csr(rng, N, (16, 256, 2048)[l % 3], "general")
+        elif kind == "hub":
+            rp, c, v = hub_block_csr(rng, N, "general")
+        else:
+            rp, c, v = sort_rows(random_csr(rng, N, 32, "general"))   # (the oracle adds in the order given)
+        return rp, c, rng.uniform(-0.3, 0.4, size=len(v)).astype(np.float32)
+
+    layers = [layer(l) for l in range(L)]
+    ref = orc.infer(orc.gen_features(10, N, 0, S, 0.30, 0.90), layers, -0.35, prune=True, keep={2})
+    assert len(ref["active_ids"][-2]) == S and 1.0 < float(np.median(ref["y"])) < 16.0
+    want = {"band": gc.KERNEL_BAND, "radix": gc.KERNEL_BAND, "radix-blocks": gc.KERNEL_BLOCK, "hub": gc.KERNEL_BLOCK,
+            "irregular": gc.KERNEL_TILED, "irregular-gather": gc.KERNEL_GATHER}[kind]
+    force = gc.KERNEL_GATHER if kind == "irregular-gather" else gc.KERNEL_AUTO
+    with gc.Network(N, B, L, bias=-0.35, force_kernel=force) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == want for l in range(L))
+        net.synth_features(10, B, 0.30, 0.90)
+        # three layers, then the rest in a second call: both begin behind stamped rows after the first layer
+        net.run(prune=True, first_layer=0, n_layers=3, collect_counts=True)
+        ids, y = ref["kept"][2]
+        assert np.array_equal(net.categories()[: len(ids)], ids)
+        assert same_floats(net.activations(ids), y)
+        net.run(prune=True, first_layer=3, n_layers=L - 3, collect_counts=True)
+        cats = net.categories()
+        assert np.array_equal(cats[cats < S], ref["categories"])
+        assert same_floats(net.activations(ref["categories"]), ref["y"])
+        pruned = [net.active_count(l) for l in range(L)]
+        net.synth_features(10, B, 0.30, 0.90)
+        net.run(prune=False, collect_counts=True)
+        assert [net.active_count(l) for l in range(L)] == pruned
+        assert np.array_equal(net.categories(), cats)
+
+
 def test_fused_chain_when_everything_dies(gc, orc):
     """Literal inputs: all rows die within a few layers; workgroups leave the chain early."""
     N, L, B = 1024, 40, 2000
