@@ -78,10 +78,80 @@ template <> __device__ __forceinline__ float4 arr_to_vec<4>(const float* a) {
 //   WMODE 0/1: the product is exact (weight is 0 or a power of two), so a fused multiply-add
 //              rounds exactly like the reference's multiply followed by add.
 //   WMODE 2:   general weights: rounded multiply, then rounded add, as the CPU reference does.
+//   WMODE 3:   (band walk, unrolled path) the layer's ONE weight w is 0 or +-2^e: scaling by a power of
+//              two commutes with rounding (nothing here comes near the denormal range, see the
+//              inspector's fma_ok), so fl(..fl(fl(w x0) + w x1).. + w xk) = w * fl(..fl(x0 + x1).. + xk):
+//              the chain is one v_add_f32 per input - issued at twice the rate of v_fmac_f32 /
+//              v_mul_f32 on this hardware (measured: 0.95 against 1.72 ns per wave instruction and
+//              SIMD) - and the weight enters once, in the epilogue's fma(sum, w, bias), which rounds
+//              like the reference's add of the bias because w * sum is exact.
 __device__ __forceinline__ float mul_then_add(float acc, float x, float w) {
 #pragma clang fp contract(off)
     const float p = x * w;
     return acc + p;
+}
+// One step of the add-only walk for a pair of outputs: acc0[q] += x[q] if bit `bit` of mask0 is set,
+// acc1[q] += x[q] if it is set in mask1 (q = the wave's RL rows per lane).  The bit, sign-extended to 64
+// bits by one scalar instruction, becomes the execution mask of the adds (all lanes or none): no select
+// per accumulator, no branch.  Every lane of the calling wave is active, so the mask goes back to all ones.
+template <int RL> __device__ __forceinline__ void add_pair_if_used(float* acc0, float* acc1, const float* x,
+                                                                 uint64_t mask0, uint64_t mask1, int bit);
+template <> __device__ __forceinline__ void add_pair_if_used<4>(float* acc0, float* acc1, const float* x,
+                                                                uint64_t mask0, uint64_t mask1, int bit) {
+    asm volatile(
+        "s_bfe_i64 exec, %12, %14\n\t"
+        "v_add_f32 %0, %8, %0\n\tv_add_f32 %1, %9, %1\n\tv_add_f32 %2, %10, %2\n\tv_add_f32 %3, %11, %3\n\t"
+        "s_bfe_i64 exec, %13, %14\n\t"
+        "v_add_f32 %4, %8, %4\n\tv_add_f32 %5, %9, %5\n\tv_add_f32 %6, %10, %6\n\tv_add_f32 %7, %11, %7\n\t"
+        "s_mov_b64 exec, -1"
+        : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc0[2]), "+v"(acc0[3]), "+v"(acc1[0]), "+v"(acc1[1]), "+v"(acc1[2]),
+          "+v"(acc1[3])
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "s"(mask0), "s"(mask1), "n"(0x10000 | bit)
+        : "scc");
+}
+template <> __device__ __forceinline__ void add_pair_if_used<2>(float* acc0, float* acc1, const float* x,
+                                                                uint64_t mask0, uint64_t mask1, int bit) {
+    asm volatile(
+        "s_bfe_i64 exec, %6, %8\n\t"
+        "v_add_f32 %0, %4, %0\n\tv_add_f32 %1, %5, %1\n\t"
+        "s_bfe_i64 exec, %7, %8\n\t"
+        "v_add_f32 %2, %4, %2\n\tv_add_f32 %3, %5, %3\n\t"
+        "s_mov_b64 exec, -1"
+        : "+v"(acc0[0]), "+v"(acc0[1]), "+v"(acc1[0]), "+v"(acc1[1])
+        : "v"(x[0]), "v"(x[1]), "s"(mask0), "s"(mask1), "n"(0x10000 | bit)
+        : "scc");
+}
+template <> __device__ __forceinline__ void add_pair_if_used<1>(float* acc0, float* acc1, const float* x,
+                                                                uint64_t mask0, uint64_t mask1, int bit) {
+    asm volatile(
+        "s_bfe_i64 exec, %3, %5\n\t"
+        "v_add_f32 %0, %2, %0\n\t"
+        "s_bfe_i64 exec, %4, %5\n\t"
+        "v_add_f32 %1, %2, %1\n\t"
+        "s_mov_b64 exec, -1"
+        : "+v"(acc0[0]), "+v"(acc1[0])
+        : "v"(x[0]), "s"(mask0), "s"(mask1), "n"(0x10000 | bit)
+        : "scc");
+}
+// LDS address of a lane's part of ring column `slot byte b of dword`: one scalar bit-field extract and
+// one vector shift-add (written out: the compiler's own choice is shift + mask on the scalar unit, and the
+// scalar unit, one per CU, is what the add-only walk has least of).
+template <int SLOT_BITS, int COL_SHIFT>
+__device__ __forceinline__ uint32_t ring_address(uint32_t lane_base, uint32_t dword, int b) {
+    uint32_t slot, addr;
+    asm("s_bfe_u32 %0, %1, %2" : "=s"(slot) : "s"(dword), "n"((SLOT_BITS << 16) | (8 * b)) : "scc");
+    asm("v_lshl_add_u32 %0, %1, %2, %3" : "=v"(addr) : "s"(slot), "n"(COL_SHIFT), "v"(lane_base));
+    return addr;
+}
+// RL floats from an LDS byte address
+template <int RL> __device__ __forceinline__ void lds_read(uint32_t lds_address, float* x) {
+    typedef float vec_t __attribute__((ext_vector_type(RL)));
+    const vec_t v = *(const __attribute__((address_space(3))) vec_t*)(size_t)lds_address;
+#pragma unroll
+    for (int q = 0; q < RL; ++q) x[q] = v[q];
+}
+template <> __device__ __forceinline__ void lds_read<1>(uint32_t lds_address, float* x) {
+    x[0] = *(const __attribute__((address_space(3))) float*)(size_t)lds_address;
 }
 template <int WMODE> __device__ __forceinline__ float mac(float acc, float x, float w) {
     if (WMODE == 2) return mul_then_add(acc, x, w);
@@ -186,11 +256,29 @@ __device__ __forceinline__ bool enter_row_block(const int32_t* active, size_t ro
 // One input column (64 lanes x 16 bytes) straight from global memory into an LDS column slot,
 // without passing through vector registers: lane i's 16 bytes land at lds_col + 16 i, which is
 // the layout of a 256-row column.  The transfer is counted like any vector memory load.
-template <int STREAM>
+// TRACKED: through the compiler's builtin.  Once the compiler knows of a direct-to-LDS load in a kernel
+// it no longer counts LDS reads down (lgkmcnt(1), (2)) but waits for all of them (lgkmcnt(0)) wherever
+// a wave needs one, which merges the band walk's waits into one per two steps.  Measured at the headline
+// shape in one process: the multiply-add walk is faster that way (5.47 against 5.58 ms per layer), the
+// add-only walk (WMODE 3) with counted waits (5.16 against 5.22 ms).
+// Not TRACKED: as text the compiler does not look into; the callers order these loads by hand
+// (wait_vector_memory() and a barrier before any wave reads the slot).  M0 (the LDS base of such a
+// load) is the compiler's to manage and is put back.
+template <int STREAM, int TRACKED = 1>
 __device__ __forceinline__ void column_to_lds(const float* gsrc_lane, unsigned char* lds_col) {
-    __builtin_amdgcn_global_load_lds(
-        (const __attribute__((address_space(1))) void*)gsrc_lane,
-        (__attribute__((address_space(3))) void*)lds_col, 16, 0, STREAM ? 2 : 0);
+    if (TRACKED) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc_lane,
+                                         (__attribute__((address_space(3))) void*)lds_col, 16, 0, STREAM ? 2 : 0);
+        return;
+    }
+    const uint32_t lds_off = (uint32_t)(size_t)((__attribute__((address_space(3))) unsigned char*)lds_col);
+    uint32_t m0_saved;
+    if (STREAM)
+        asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off nt\n\ts_mov_b32 m0, %0"
+                     : "=&s"(m0_saved) : "s"(lds_off), "v"(gsrc_lane) : "memory");
+    else
+        asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                     : "=&s"(m0_saved) : "s"(lds_off), "v"(gsrc_lane) : "memory");
 }
 // s_waitcnt vmcnt(0) (the other counters left alone: expcnt 7, lgkmcnt 15 in the gfx9 encoding), as
 // the instruction itself rather than inline text, so that the compiler's own bookkeeping of
@@ -275,11 +363,17 @@ __device__ __forceinline__ void band_walk_body(
     static_assert((RING & (RING - 1)) == 0 && RING <= 256, "ring must be a power of two <= 256");
     static_assert(OPW % 2 == 0, "outputs are computed in pairs");
     static_assert(KT == 0 || KT == 36, "KT is 36 (up to 36 steps, unrolled, 16-dword pair records) or 0 (run-time)");
+    static_assert(WMODE != 3 || KT == 36, "sum-then-scale exists for the unrolled path only");
+    constexpr bool WSTREAM = WMODE == 1 || WMODE == 2;   // weights come per step from the plan
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int loff = lane * RL;
     const unsigned char* lane_smem = smem + loff * 4;
+    const uint32_t lane_base = (uint32_t)(size_t)((const __attribute__((address_space(3))) unsigned char*)lane_smem);
+    constexpr int SLOT_BITS = RING == 256 ? 8 : RING == 128 ? 7 : RING == 64 ? 6 : RING == 32 ? 5 : 4;
+    constexpr int COL_SHIFT = RL == 4 ? 10 : RL == 2 ? 9 : 8;
+    static_assert((1 << SLOT_BITS) == RING && (1 << COL_SHIFT) == COLB, "ring geometry");
     // the layer's one weight as scalar bits: a step's effective weight (wu or 0) is then picked by
     // integer ops on the scalar unit and feeds the multiply-add as a scalar operand
     const uint32_t wu_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(wu));
@@ -292,8 +386,8 @@ __device__ __forceinline__ void band_walk_body(
             const int g = p < 0 ? p + N : p;
             if (DMA) {
                 unsigned char* slot = smem + (size_t)(p & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1>(yin + (size_t)g * RBL + loff, slot);
-                else column_to_lds<0>(yin + (size_t)g * RBL + loff, slot);
+                if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)g * RBL + loff, slot);
+                else column_to_lds<0, WMODE != 3>(yin + (size_t)g * RBL + loff, slot);
                 continue;
             }
             float x[RL];
@@ -316,8 +410,8 @@ __device__ __forceinline__ void band_walk_body(
             const int p = min(cb + T + wave + i * NW, ve - 1);
             if (DMA) {
                 unsigned char* slot = smem + (size_t)((cb + T + wave + i * NW) & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1>(yin + (size_t)p * RBL + loff, slot);
-                else column_to_lds<0>(yin + (size_t)p * RBL + loff, slot);
+                if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)p * RBL + loff, slot);
+                else column_to_lds<0, WMODE != 3>(yin + (size_t)p * RBL + loff, slot);
             } else if (stream) load_stream<RL>(yin + (size_t)p * RBL + loff, pf[i]);
             else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RBL + loff), pf[i]);
         }
@@ -346,11 +440,17 @@ __device__ __forceinline__ void band_walk_body(
                 sa[i] = load_const_u4(rec + 4);
                 sb[i] = load_const_u4(rec + 8);
                 sc[i] = pairs[(size_t)pr[i] * 16 + 12];
-                if (WMODE) {
+                if (WSTREAM) {
                     wp[i] = pw + (size_t)pr[i] * 72;
                     w_cur[i][0] = load_const_f4(wp[i]);
                     w_cur[i][1] = load_const_f4(wp[i] + 4);
                 }
+            }
+            uint64_t use0[PPW], use1[PPW];   // the use masks of output 0 / 1 as 64-bit scalars (WMODE 3)
+#pragma unroll
+            for (int i = 0; i < PPW; ++i) {
+                use0[i] = (uint64_t)mk[i].x | ((uint64_t)mk[i].y << 32);
+                use1[i] = (uint64_t)mk[i].z | ((uint64_t)mk[i].w << 32);
             }
             float xb[3][PPW][RL];
             float4 w_nxt[PPW][2];
@@ -358,32 +458,47 @@ __device__ __forceinline__ void band_walk_body(
     (((((e) >> 2) == 0 ? sa[i].x : ((e) >> 2) == 1 ? sa[i].y : ((e) >> 2) == 2 ? sa[i].z                \
        : ((e) >> 2) == 3 ? sa[i].w : ((e) >> 2) == 4 ? sb[i].x : ((e) >> 2) == 5 ? sb[i].y              \
        : ((e) >> 2) == 6 ? sb[i].z : ((e) >> 2) == 7 ? sb[i].w : sc[i]) >> (8 * ((e) & 3))) & (RING - 1))
+#define SPDNN_SLOT_DWORD(i, e)                                                                        \
+    (((e) >> 2) == 0 ? sa[i].x : ((e) >> 2) == 1 ? sa[i].y : ((e) >> 2) == 2 ? sa[i].z                  \
+     : ((e) >> 2) == 3 ? sa[i].w : ((e) >> 2) == 4 ? sb[i].x : ((e) >> 2) == 5 ? sb[i].y                \
+     : ((e) >> 2) == 6 ? sb[i].z : ((e) >> 2) == 7 ? sb[i].w : sc[i])
+#define SPDNN_READ_COLUMN(i, e, x)                                                                    \
+    do {                                                                                              \
+        if (WMODE == 3) lds_read<RL>(ring_address<SLOT_BITS, COL_SHIFT>(lane_base, SPDNN_SLOT_DWORD(i, e), (e) & 3), x); \
+        else vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), x);     \
+    } while (0)
 #define SPDNN_USED(i, o, e) (((((e) < 32) ? ((o) ? mk[i].z : mk[i].x) : ((o) ? mk[i].w : mk[i].y)) >> ((e) & 31)) & 1u)
 #pragma unroll
             for (int e = 0; e < 2; ++e)
 #pragma unroll
                 for (int i = 0; i < PPW; ++i)
-                    vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), xb[e][i]);
+                    SPDNN_READ_COLUMN(i, e, xb[e][i]);
 #pragma unroll
             for (int st = 0; st < 36; ++st) {
                 if (st + 2 < 36 && (st + 2 < 32 || st + 2 < steps)) {
 #pragma unroll
                     for (int i = 0; i < PPW; ++i)
-                        vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, st + 2) * COLB),
-                                       xb[(st + 2) % 3][i]);
+                        SPDNN_READ_COLUMN(i, st + 2, xb[(st + 2) % 3][i]);
                 }
-                if (WMODE && (st & 3) == 0 && st + 4 < 36) {  // two weights per step, four steps per trip
+                if (WSTREAM && (st & 3) == 0 && st + 4 < 36) {  // two weights per step, four steps per trip
 #pragma unroll
                     for (int i = 0; i < PPW; ++i) {
                         w_nxt[i][0] = load_const_f4(wp[i] + 4 * ((st >> 2) * 2 + 2));
                         w_nxt[i][1] = load_const_f4(wp[i] + 4 * ((st >> 2) * 2 + 3));
                     }
                 }
-                if (st < 32 || st < steps) {
+                if (WMODE == 3) {
+                    if (st < 32 || st < steps) {
+#pragma unroll
+                        for (int i = 0; i < PPW; ++i) {
+                            add_pair_if_used<RL>(acc[i][0], acc[i][1], xb[st % 3][i], use0[i], use1[i], st);
+                        }
+                    }
+                } else if (st < 32 || st < steps) {
 #pragma unroll
                     for (int i = 0; i < PPW; ++i) {
                         float w0, w1;
-                        if (WMODE) {
+                        if (WSTREAM) {
                             const float4 wq = w_cur[i][(st >> 1) & 1];
                             w0 = (st & 1) ? wq.z : wq.x;
                             w1 = (st & 1) ? wq.w : wq.y;
@@ -398,7 +513,7 @@ __device__ __forceinline__ void band_walk_body(
                         }
                     }
                 }
-                if (WMODE && (st & 3) == 3 && st + 1 < 36) {
+                if (WSTREAM && (st & 3) == 3 && st + 1 < 36) {
 #pragma unroll
                     for (int i = 0; i < PPW; ++i) {
                         w_cur[i][0] = w_nxt[i][0];
@@ -416,6 +531,8 @@ __device__ __forceinline__ void band_walk_body(
                     }
             }
 #undef SPDNN_SLOT
+#undef SPDNN_SLOT_DWORD
+#undef SPDNN_READ_COLUMN
 #undef SPDNN_USED
         } else {
             // run-time step count: four steps per trip; the selectors (and weights) of the next
@@ -431,7 +548,7 @@ __device__ __forceinline__ void band_walk_body(
                 m0lo[i] = rec[0]; m0hi[i] = rec[1]; m1lo[i] = rec[2]; m1hi[i] = rec[3];
                 sp[i] = rec + 4;
                 s_cur[i] = sp[i][0];
-                if (WMODE) {
+                if (WSTREAM) {
                     wp[i] = pw + (size_t)pr[i] * (size_t)trips * 8;
                     w_cur[i][0] = load_const_f4(wp[i]);
                     w_cur[i][1] = load_const_f4(wp[i] + 4);
@@ -445,7 +562,7 @@ __device__ __forceinline__ void band_walk_body(
 #pragma unroll
                 for (int i = 0; i < PPW; ++i) {
                     s_nxt[i] = sp[i][mn];
-                    if (WMODE) {
+                    if (WSTREAM) {
                         w_nxt[i][0] = load_const_f4(wp[i] + 8 * mn);
                         w_nxt[i][1] = load_const_f4(wp[i] + 8 * mn + 4);
                     }
@@ -461,7 +578,7 @@ __device__ __forceinline__ void band_walk_body(
                             float x[RL];
                             vec_to_arr<RL>(xv, x);
                             float w0, w1;
-                            if (WMODE) {
+                            if (WSTREAM) {
                                 const float4 wq = w_cur[i][b >> 1];
                                 w0 = (b & 1) ? wq.z : wq.x;
                                 w1 = (b & 1) ? wq.w : wq.y;
@@ -482,7 +599,7 @@ __device__ __forceinline__ void band_walk_body(
 #pragma unroll
                 for (int i = 0; i < PPW; ++i) {
                     s_cur[i] = s_nxt[i];
-                    if (WMODE) {
+                    if (WSTREAM) {
                         w_cur[i][0] = w_nxt[i][0];
                         w_cur[i][1] = w_nxt[i][1];
                     }
@@ -514,8 +631,8 @@ __device__ __forceinline__ void band_walk_body(
                 float y0[RL], y1[RL];
 #pragma unroll
                 for (int q = 0; q < RL; ++q) {
-                    y0[q] = relu_clamp(acc[i][0][q] + bias, clampv);
-                    y1[q] = relu_clamp(acc[i][1][q] + bias, clampv);
+                    y0[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
+                    y1[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][1][q], wu, bias) : acc[i][1][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));   // one three-way maximum
                 }
                 const int d0 = dst[v0], d1 = dst[v0 + 1];
@@ -530,7 +647,7 @@ __device__ __forceinline__ void band_walk_body(
                 float y[RL];
 #pragma unroll
                 for (int q = 0; q < RL; ++q) {
-                    y[q] = relu_clamp(acc[i][0][q] + bias, clampv);
+                    y[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], y[q]);
                 }
                 *reinterpret_cast<V*>(yout + (size_t)dst[v0] * RBL + loff) = arr_to_vec<RL>(y);
@@ -1452,11 +1569,23 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     return hipGetLastError();
 }
 
+// SPDNN_BAND_SUM_THEN_SCALE=0: layers with one exact weight keep a multiply-add per input (WMODE 0)
+// instead of adding the inputs and scaling the sum (WMODE 3); read once per process.
+bool band_sum_then_scale_enabled() {
+    static const bool on = [] {
+        const char* e = getenv("SPDNN_BAND_SUM_THEN_SCALE");
+        return !(e && atoi(e) == 0);
+    }();
+    return on;
+}
+
 template <int RL, int NW, int OPW, int RING, int DMA>
 hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
     if (band_unrolled(a.K, a.steps, a.stride)) {
         switch (a.wmode) {
-            case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 36, DMA>(a, s);
+            case 0:
+                if (band_sum_then_scale_enabled()) return launch_band_inst<RL, NW, OPW, RING, 3, 36, DMA>(a, s);
+                return launch_band_inst<RL, NW, OPW, RING, 0, 36, DMA>(a, s);
             case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36, DMA>(a, s);
             default: return launch_band_inst<RL, NW, OPW, RING, 2, 36, DMA>(a, s);
         }

@@ -160,6 +160,40 @@ def test_band_kernel_weight_modes(gc, orc, values, K):
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 
 
+@pytest.mark.parametrize("structure", ["circulant", "run-chains"])
+@pytest.mark.parametrize("w", [0.0625, -0.5, 2.0 ** -24, 2.0 ** 21, 0.0])
+def test_one_power_of_two_weight_sums_then_scales(gc, orc, w, structure, monkeypatch):
+    """A layer whose entries all carry the same weight +-2^e is walked by adding the inputs and scaling the
+    sum once.  That equals the reference's multiply-then-add chain bit for bit only because scaling by a
+    power of two commutes with rounding: features of both signs over the whole accepted range (2^-100 ..
+    2^100, with cancellations down to the last bit), the smallest and largest accepted weights."""
+    from helpers import radix_like_csr
+    N, L, B = 1024, 3, 300
+    print("sum then scale w=%g %s" % (w, structure), flush=True)
+    rng = np.random.default_rng(3)
+    if structure == "run-chains":
+        monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+        monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", "0")
+        layers = []
+        for l in range(L):
+            rp, c, v = radix_like_csr(rng, N, 16 << l, "uniform")
+            layers.append((rp, c, np.full(len(v), w, np.float32)))
+    else:
+        layers = [orc.gen_layer_csr(21, l, N, 32, w) for l in range(L)]
+    mag = np.ldexp(rng.uniform(1.0, 2.0, size=(B, N)), rng.integers(-100, 100, size=(B, N)))
+    # neighbours that cancel but for the last bits, and rows of moderate values that reach the later layers
+    feats = (mag * rng.choice([-1.0, 1.0], size=(B, N)) * (rng.random((B, N)) < 0.7)).astype(np.float32)
+    feats[:, 1::2] = np.where(rng.random((B, N // 2)) < 0.5, -np.nextafter(feats[:, 0::2], np.float32(0)), feats[:, 1::2])
+    feats[B // 2:] = (rng.uniform(0, 8, size=(B - B // 2, N)) * (rng.random((B - B // 2, N)) < 0.6)).astype(np.float32)
+    with gc.Network(N, B, L, bias=-0.1) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_BAND and net.layer_plan(l).uniform_value for l in range(L))
+        net.set_features_dense(feats)
+        _layer_by_layer(gc, orc, net, layers, feats, prune=False)
+
+
 def test_forced_gather_equals_band(gc, orc):
     N, L, B = 1024, 5, 400
     print("forced gather", flush=True)
