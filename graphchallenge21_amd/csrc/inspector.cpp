@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
+#include <stdexcept>
 
 namespace spdnn {
 
@@ -676,9 +677,11 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
             }
             steps = std::max(steps, m);
         }
-        int trips = (steps + 3) / 4;
-        if (K == 32 && steps <= 36) trips = 9;  // the unrolled kernel path reads fixed 16-dword records
-        const int stride = (4 + trips + 3) / 4 * 4;
+        // A circulant pair merges to K + 1 steps, a pair inside a group of a run chain to 32: the kernel
+        // reads fixed 16-dword records (two use masks, 36 one-byte selectors) and 72 weights per pair.
+        if (steps > 36) throw std::logic_error("band pair with more than 36 merged steps");
+        const int trips = 9;
+        const int stride = 16;
         plan.pair_steps = steps;
         plan.pair_stride = stride;
         plan.pair_padded = trips * 4;

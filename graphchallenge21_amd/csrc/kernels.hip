@@ -345,7 +345,7 @@ __device__ __forceinline__ float4 load_const_f4(const __attribute__((address_spa
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA, int RBL = 64 * RL>
 __device__ __forceinline__ void band_walk_body(
     const float* __restrict__ yin, float* __restrict__ yout, const uint32_t* __restrict__ pairs_g,
-    const float* __restrict__ pw_g, const int32_t* __restrict__ dst_g, int N, int steps, int stride, int halo,
+    const float* __restrict__ pw_g, const int32_t* __restrict__ dst_g, int N, int steps, int halo,
     int vb, int ve, float wu, float bias, float clampv, unsigned char* smem, float* nz, int stream) {
     using V = typename VecOf<RL>::type;
     // The plan arrays never change while a kernel runs: read through the constant address space they
@@ -362,8 +362,7 @@ __device__ __forceinline__ void band_walk_body(
     static_assert(2 * T + 32 <= RING && T % 16 == 0, "ring too small for a halo of 32 columns");
     static_assert((RING & (RING - 1)) == 0 && RING <= 256, "ring must be a power of two <= 256");
     static_assert(OPW % 2 == 0, "outputs are computed in pairs");
-    static_assert(KT == 0 || KT == 36, "KT is 36 (up to 36 steps, unrolled, 16-dword pair records) or 0 (run-time)");
-    static_assert(WMODE != 3 || KT == 36, "sum-then-scale exists for the unrolled path only");
+    static_assert(KT == 0 || KT == 36, "KT is 36 (32 entries per output: at least 32 steps) or 0 (fewer: groups of four steps)");
     constexpr bool WSTREAM = WMODE == 1 || WMODE == 2;   // weights come per step from the plan
 
     const int lane = threadIdx.x & 63;
@@ -425,10 +424,13 @@ __device__ __forceinline__ void band_walk_body(
             for (int q = 0; q < RL; ++q) acc[i][0][q] = acc[i][1][q] = 0.0f;
         }
 
-        if (KT == 36) {
+        {
             // The whole pair record (masks + 36 selectors) sits in scalar registers up front.  The
             // LDS read of step s+2 is issued before the arithmetic of step s, so a wave always has
-            // reads in flight while its multiply-adds issue.  Steps 32..35 exist only if steps > 32.
+            // reads in flight while its multiply-adds issue.  KT = 36 (32 entries per output): the first 32
+            // steps run unconditionally, steps 32..35 only if steps > 32.  KT = 0 (fewer entries): the steps
+            // run in groups of four as far as `steps` reaches (the padding steps of the last group carry
+            // use bits and weights 0).
             uint4 mk[PPW], sa[PPW], sb[PPW];
             uint32_t sc[PPW];
             const __attribute__((address_space(4))) float* wp[PPW];
@@ -467,6 +469,7 @@ __device__ __forceinline__ void band_walk_body(
         if (WMODE == 3) lds_read<RL>(ring_address<SLOT_BITS, COL_SHIFT>(lane_base, SPDNN_SLOT_DWORD(i, e), (e) & 3), x); \
         else vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), x);     \
     } while (0)
+#define SPDNN_STEP_LIVE(e) (KT == 36 ? ((e) < 32 || (e) < steps) : (((e) & ~3) < steps))
 #define SPDNN_USED(i, o, e) (((((e) < 32) ? ((o) ? mk[i].z : mk[i].x) : ((o) ? mk[i].w : mk[i].y)) >> ((e) & 31)) & 1u)
 #pragma unroll
             for (int e = 0; e < 2; ++e)
@@ -475,7 +478,7 @@ __device__ __forceinline__ void band_walk_body(
                     SPDNN_READ_COLUMN(i, e, xb[e][i]);
 #pragma unroll
             for (int st = 0; st < 36; ++st) {
-                if (st + 2 < 36 && (st + 2 < 32 || st + 2 < steps)) {
+                if (st + 2 < 36 && SPDNN_STEP_LIVE(st + 2)) {
 #pragma unroll
                     for (int i = 0; i < PPW; ++i)
                         SPDNN_READ_COLUMN(i, st + 2, xb[(st + 2) % 3][i]);
@@ -488,13 +491,13 @@ __device__ __forceinline__ void band_walk_body(
                     }
                 }
                 if (WMODE == 3) {
-                    if (st < 32 || st < steps) {
+                    if (SPDNN_STEP_LIVE(st)) {
 #pragma unroll
                         for (int i = 0; i < PPW; ++i) {
                             add_pair_if_used<RL>(acc[i][0], acc[i][1], xb[st % 3][i], use0[i], use1[i], st);
                         }
                     }
-                } else if (st < 32 || st < steps) {
+                } else if (SPDNN_STEP_LIVE(st)) {
 #pragma unroll
                     for (int i = 0; i < PPW; ++i) {
                         float w0, w1;
@@ -534,77 +537,7 @@ __device__ __forceinline__ void band_walk_body(
 #undef SPDNN_SLOT_DWORD
 #undef SPDNN_READ_COLUMN
 #undef SPDNN_USED
-        } else {
-            // run-time step count: four steps per trip; the selectors (and weights) of the next
-            // trip are requested from the scalar cache before this trip's arithmetic starts
-            const int trips = (steps + 3) >> 2;
-            const __attribute__((address_space(4))) uint32_t* sp[PPW];
-            const __attribute__((address_space(4))) float* wp[PPW];
-            uint32_t m0lo[PPW], m0hi[PPW], m1lo[PPW], m1hi[PPW], s_cur[PPW];
-            float4 w_cur[PPW][2];
-#pragma unroll
-            for (int i = 0; i < PPW; ++i) {
-                const __attribute__((address_space(4))) uint32_t* rec = pairs + (size_t)pr[i] * stride;
-                m0lo[i] = rec[0]; m0hi[i] = rec[1]; m1lo[i] = rec[2]; m1hi[i] = rec[3];
-                sp[i] = rec + 4;
-                s_cur[i] = sp[i][0];
-                if (WSTREAM) {
-                    wp[i] = pw + (size_t)pr[i] * (size_t)trips * 8;
-                    w_cur[i][0] = load_const_f4(wp[i]);
-                    w_cur[i][1] = load_const_f4(wp[i] + 4);
-                }
-            }
-#pragma unroll 1
-            for (int m4 = 0; m4 < trips; ++m4) {
-                uint32_t s_nxt[PPW];
-                float4 w_nxt[PPW][2];
-                const int mn = min(m4 + 1, trips - 1);
-#pragma unroll
-                for (int i = 0; i < PPW; ++i) {
-                    s_nxt[i] = sp[i][mn];
-                    if (WSTREAM) {
-                        w_nxt[i][0] = load_const_f4(wp[i] + 8 * mn);
-                        w_nxt[i][1] = load_const_f4(wp[i] + 8 * mn + 4);
-                    }
-                }
-#pragma unroll
-                for (int b = 0; b < 4; ++b) {
-                    const int e = m4 * 4 + b;
-                    if (e < steps) {
-#pragma unroll
-                        for (int i = 0; i < PPW; ++i) {
-                            const uint32_t slot = (s_cur[i] >> (8 * b)) & (RING - 1);
-                            V xv = *reinterpret_cast<const V*>(lane_smem + (size_t)slot * COLB);
-                            float x[RL];
-                            vec_to_arr<RL>(xv, x);
-                            float w0, w1;
-                            if (WSTREAM) {
-                                const float4 wq = w_cur[i][b >> 1];
-                                w0 = (b & 1) ? wq.z : wq.x;
-                                w1 = (b & 1) ? wq.w : wq.y;
-                            } else {
-                                const uint32_t u0 = ((e < 32 ? m0lo[i] : m0hi[i]) >> (e & 31)) & 1u;
-                                const uint32_t u1 = ((e < 32 ? m1lo[i] : m1hi[i]) >> (e & 31)) & 1u;
-                                w0 = __uint_as_float(wu_bits & (0u - u0));
-                                w1 = __uint_as_float(wu_bits & (0u - u1));
-                            }
-#pragma unroll
-                            for (int q = 0; q < RL; ++q) {
-                                acc[i][0][q] = mac<WMODE>(acc[i][0][q], x[q], w0);
-                                acc[i][1][q] = mac<WMODE>(acc[i][1][q], x[q], w1);
-                            }
-                        }
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < PPW; ++i) {
-                    s_cur[i] = s_nxt[i];
-                    if (WSTREAM) {
-                        w_cur[i][0] = w_nxt[i][0];
-                        w_cur[i][1] = w_nxt[i][1];
-                    }
-                }
-            }
+#undef SPDNN_STEP_LIVE
         }
 
         // The parked columns go into ring slots no wave reads during this chunk - BEFORE the outputs
@@ -662,7 +595,7 @@ template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
 __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
-    int32_t* __restrict__ count_prev, int N, int steps, int stride, int halo, int seglen, int stamp, int prev_stamp,
+    int32_t* __restrict__ count_prev, int N, int steps, int halo, int seglen, int stamp, int prev_stamp,
     int check_dead, float wu, float bias, float clampv, Publish pub, int nblk, int stream) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
@@ -681,7 +614,7 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
 #pragma unroll
     for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
     band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
-                                                 pw, dst, N, steps, stride, halo, vb, ve, wu, bias, clampv, smem, nz, stream);
+                                                 pw, dst, N, steps, halo, vb, ve, wu, bias, clampv, smem, nz, stream);
     stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, nullptr);
 }
 
@@ -700,7 +633,6 @@ struct ChainLayer {
     float wu;
     int halo;
     int steps;
-    int stride;
 };
 
 template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
@@ -725,7 +657,7 @@ __global__ __launch_bounds__(NW * 64) void band_chain_kernel(
         float nz[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+        band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps,
                                                      lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
         stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
                                      count_out ? count_out + j : nullptr);
@@ -779,7 +711,7 @@ __global__ __launch_bounds__(512) void band_chain_half_kernel(
         float* out = (in == block_a) ? block_c : block_a;
         const ChainLayer lay = table[j];
         float nz[2] = {0.0f, 0.0f};
-        band_walk_body<2, 8, 2, 64, WMODE, KT, 0, RBL>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps, lay.stride,
+        band_walk_body<2, 8, 2, 64, WMODE, KT, 0, RBL>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps,
                                                        lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
         stamp_rows_workgroup<2, 8>(nz, smem, active, row0, stamp0 + j, count_out ? count_out + j : nullptr);
         // the barrier (workgroup-scope fence) makes this layer's columns visible to the other waves
@@ -1564,7 +1496,7 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     const int stream = (long long)a.nblk * (long long)block_bytes * 2 >= a.stream_min_bytes ? 1 : 0;
     dim3 grid(gx, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_prev,
-                       a.N, a.steps, a.stride, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,
+                       a.N, a.steps, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,
                        a.nblk, stream);
     return hipGetLastError();
 }
@@ -1599,7 +1531,8 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
 
 }  // namespace
 
-// 32 entries per output and at most 36 merged steps per pair in 16-dword records: the unrolled path
+// 32 entries per output (KT = 36: the first 32 steps of a pair run unconditionally); with fewer entries
+// the same walk runs its steps in groups of four as far as they reach (KT = 0)
 bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36 && stride == 16; }
 
 // Tile shape of the band walk, the same for every row-block size: 8 waves x 2 outputs (one pair) per
@@ -1660,8 +1593,7 @@ double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, in
 hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
     // host-side shape checks: what the kernel and its grid assume
     if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 ||
-        a.halo < a.K - 1 || a.halo > 32 || a.halo >= a.N || a.steps < a.K || a.steps > 2 * a.K ||
-        a.stride < 4 + (a.steps + 3) / 4 || (a.stride % 4) != 0 ||
+        a.halo < a.K - 1 || a.halo > 32 || a.halo >= a.N || a.steps < a.K || a.steps > 36 || a.stride != 16 ||
         !a.yin || !a.yout || !a.pairs || !a.dst || !a.active || (a.wmode != 0 && !a.pw))
         return hipErrorInvalidValue;
     BandLaunch b = a;

@@ -131,8 +131,7 @@ struct ChainLayerDesc {      // one entry of the device-side layer table
     const int32_t* dst;
     float wu;
     int halo;   // input columns a segment needs before its first position (K-1, or 32 for run chains)
-    int steps;  // merged steps per pair
-    int stride; // dwords per pair record
+    int steps;  // merged steps per pair (records of 16 dwords: two use masks, 36 one-byte ring selectors)
 };
 struct ChainLaunch {
     const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain
@@ -144,7 +143,7 @@ struct ChainLaunch {
     int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
     int32_t* count_prev;          // as in BandLaunch, for the layer before the chain
     int N, K, nblk, stamp0, prev_stamp, check_dead, rl, wmode;
-    int unrolled;                 // every layer of the chain fits the unrolled path (band_unrolled)
+    int unrolled;                 // every layer of the chain has 32 entries per output (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
     int halves;                   // 1 (256-row blocks only): one workgroup per HALF row block (twice the workgroups)
     float bias, clampv;

@@ -565,7 +565,6 @@ int upload_plans(spdnn_net* n) {
             table[l].pairs = n->dl[l].pairs;
             table[l].pw = n->dl[l].wv;
             table[l].steps = n->layers[l].pair_steps;
-            table[l].stride = n->layers[l].pair_stride;
             table[l].dst = n->dl[l].dst;
             table[l].wu = n->layers[l].info.value;
             table[l].halo = n->layers[l].info.band_halo;
