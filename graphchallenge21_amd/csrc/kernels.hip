@@ -1523,7 +1523,9 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
         }
     }
     switch (a.wmode) {
-        case 0: return launch_band_inst<RL, NW, OPW, RING, 0, 0, DMA>(a, s);
+        case 0:
+            if (band_sum_then_scale_enabled()) return launch_band_inst<RL, NW, OPW, RING, 3, 0, DMA>(a, s);
+            return launch_band_inst<RL, NW, OPW, RING, 0, 0, DMA>(a, s);
         case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 0, DMA>(a, s);
         default: return launch_band_inst<RL, NW, OPW, RING, 2, 0, DMA>(a, s);
     }
@@ -1629,13 +1631,16 @@ hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
 }
 template <int RL, int NW, int OPW, int RING>
 hipError_t launch_chain_rl(const ChainLaunch& a, hipStream_t s) {
+    const bool add_only = a.wmode == 0 && band_sum_then_scale_enabled();   // as in the per-layer walk
     if (a.unrolled) {
+        if (add_only) return launch_chain_inst<RL, NW, OPW, RING, 3, 36>(a, s);
         switch (a.wmode) {
             case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 36>(a, s);
             case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 36>(a, s);
             default: return launch_chain_inst<RL, NW, OPW, RING, 2, 36>(a, s);
         }
     }
+    if (add_only) return launch_chain_inst<RL, NW, OPW, RING, 3, 0>(a, s);
     switch (a.wmode) {
         case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 0>(a, s);
         case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 0>(a, s);
@@ -1661,10 +1666,11 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
                            a.active, a.count_out, a.count_prev, a.N, a.stamp0, a.prev_stamp, a.check_dead, a.bias,   \
                            a.clampv, a.publish);                                                                     \
     } while (0)
+        const bool add_only = a.wmode == 0 && band_sum_then_scale_enabled();
         if (a.unrolled) {
-            if (a.wmode == 0) SPDNN_HALF(0, 36); else if (a.wmode == 1) SPDNN_HALF(1, 36); else SPDNN_HALF(2, 36);
+            if (add_only) SPDNN_HALF(3, 36); else if (a.wmode == 0) SPDNN_HALF(0, 36); else if (a.wmode == 1) SPDNN_HALF(1, 36); else SPDNN_HALF(2, 36);
         } else {
-            if (a.wmode == 0) SPDNN_HALF(0, 0); else if (a.wmode == 1) SPDNN_HALF(1, 0); else SPDNN_HALF(2, 0);
+            if (add_only) SPDNN_HALF(3, 0); else if (a.wmode == 0) SPDNN_HALF(0, 0); else if (a.wmode == 1) SPDNN_HALF(1, 0); else SPDNN_HALF(2, 0);
         }
 #undef SPDNN_HALF
         return hipGetLastError();
