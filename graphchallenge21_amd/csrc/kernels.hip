@@ -758,7 +758,10 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
     const uint32_t sc = pairs[(size_t)pr * 16 + 12];
     const float4* wp = nullptr;
     float4 w_cur[2], w_nxt[2];
-    if (WMODE) {
+    constexpr bool WSTREAM = WMODE == 1 || WMODE == 2;   // weights come per step from the plan
+    const uint32_t lane_base = (uint32_t)(size_t)((const __attribute__((address_space(3))) unsigned char*)lane_ring);
+    const uint64_t use0 = (uint64_t)mk.x | ((uint64_t)mk.y << 32), use1 = (uint64_t)mk.z | ((uint64_t)mk.w << 32);
+    if (WSTREAM) {
         wp = reinterpret_cast<const float4*>(pw + (size_t)pr * 72);
         w_cur[0] = wp[0];
         w_cur[1] = wp[1];
@@ -769,21 +772,31 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
 #define SPDNN_PSLOT(e)                                                                                   \
     (((((e) >> 2) == 0 ? sa.x : ((e) >> 2) == 1 ? sa.y : ((e) >> 2) == 2 ? sa.z : ((e) >> 2) == 3 ? sa.w  \
        : ((e) >> 2) == 4 ? sb.x : ((e) >> 2) == 5 ? sb.y : ((e) >> 2) == 6 ? sb.z : ((e) >> 2) == 7 ? sb.w : sc) >> (8 * ((e) & 3))) & 63u)
+#define SPDNN_PSLOT_DWORD(e)                                                                             \
+    (((e) >> 2) == 0 ? sa.x : ((e) >> 2) == 1 ? sa.y : ((e) >> 2) == 2 ? sa.z : ((e) >> 2) == 3 ? sa.w    \
+     : ((e) >> 2) == 4 ? sb.x : ((e) >> 2) == 5 ? sb.y : ((e) >> 2) == 6 ? sb.z : ((e) >> 2) == 7 ? sb.w : sc)
+#define SPDNN_PREAD(e, x)                                                                                \
+    do {                                                                                                 \
+        if (WMODE == 3) lds_read<4>(ring_address<6, 10>(lane_base, SPDNN_PSLOT_DWORD(e), (e) & 3), x);      \
+        else vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(e) * 1024), x); \
+    } while (0)
 #define SPDNN_PUSED(o, e) (((((e) < 32) ? ((o) ? mk.z : mk.x) : ((o) ? mk.w : mk.y)) >> ((e) & 31)) & 1u)
 #pragma unroll
     for (int e = 0; e < 2; ++e)
-        vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(e) * 1024), xb[e]);
+        SPDNN_PREAD(e, xb[e]);
 #pragma unroll
     for (int st = 0; st < 36; ++st) {
         if (st + 2 < 36 && (st + 2 < 32 || st + 2 < steps))
-            vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(st + 2) * 1024), xb[(st + 2) % 3]);
-        if (WMODE && (st & 3) == 0 && st + 4 < 36) {
+            SPDNN_PREAD(st + 2, xb[(st + 2) % 3]);
+        if (WSTREAM && (st & 3) == 0 && st + 4 < 36) {
             w_nxt[0] = wp[(st >> 2) * 2 + 2];
             w_nxt[1] = wp[(st >> 2) * 2 + 3];
         }
-        if (st < 32 || st < steps) {
+        if (WMODE == 3) {
+            if (st < 32 || st < steps) add_pair_if_used<4>(acc[0], acc[1], xb[st % 3], use0, use1, st);
+        } else if (st < 32 || st < steps) {
             float w0, w1;
-            if (WMODE) {
+            if (WSTREAM) {
                 const float4 wq = w_cur[(st >> 1) & 1];
                 w0 = (st & 1) ? wq.z : wq.x;
                 w1 = (st & 1) ? wq.w : wq.y;
@@ -797,7 +810,7 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
                 acc[1][q] = mac<WMODE>(acc[1][q], xb[st % 3][q], w1);
             }
         }
-        if (WMODE && (st & 3) == 3 && st + 1 < 36) {
+        if (WSTREAM && (st & 3) == 3 && st + 1 < 36) {
             w_cur[0] = w_nxt[0];
             w_cur[1] = w_nxt[1];
         }
@@ -808,6 +821,8 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
         }
     }
 #undef SPDNN_PSLOT
+#undef SPDNN_PSLOT_DWORD
+#undef SPDNN_PREAD
 #undef SPDNN_PUSED
 }
 
@@ -843,6 +858,7 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
     const int va0 = vb - 32;                      // first position layer A computes (may be negative: wraps)
     float nz[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const uint32_t wu_bits = (uint32_t)__builtin_amdgcn_readfirstlane((int)__float_as_uint(role ? B.wu : A.wu));
+    const float wu = __uint_as_float(wu_bits);   // the layer's one weight (WMODE 0 and 3)
 
     if (role == 0) {
         // layer A's halo and first chunk
@@ -850,8 +866,8 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
             const int p = va0 - A.halo + c;
             const int g = p < 0 ? p + N : p;
             unsigned char* slot = ring_a + (size_t)(p & 63) * COLB;
-            if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
-            else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+            if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)g * RB + loff, slot);
+            else column_to_lds<0, WMODE != 3>(yin + (size_t)g * RB + loff, slot);
         }
         wait_vector_memory();
     }
@@ -867,8 +883,8 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
                         const int p = cb + T + w + i * 8;
                         const int g = p < 0 ? p + N : p;
                         unsigned char* slot = ring_a + (size_t)(p & 63) * COLB;
-                        if (stream) column_to_lds<1>(yin + (size_t)g * RB + loff, slot);
-                        else column_to_lds<0>(yin + (size_t)g * RB + loff, slot);
+                        if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)g * RB + loff, slot);
+                        else column_to_lds<0, WMODE != 3>(yin + (size_t)g * RB + loff, slot);
                     }
                 }
                 const int v0 = cb + 2 * w;
@@ -878,8 +894,8 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
                 float y0[4], y1[4];
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    y0[q] = relu_clamp(acc[0][q] + bias, clampv);
-                    y1[q] = relu_clamp(acc[1][q] + bias, clampv);
+                    y0[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[0][q], wu, bias) : acc[0][q] + bias, clampv);
+                    y1[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[1][q], wu, bias) : acc[1][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));
                 }
                 *reinterpret_cast<float4*>(ring_b + (size_t)(v0 & 63) * COLB + loff * 4) = arr_to_vec<4>(y0);
@@ -893,8 +909,8 @@ __global__ __launch_bounds__(1024) void band_pair_kernel(
             float y0[4], y1[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                y0[q] = relu_clamp(acc[0][q] + bias, clampv);
-                y1[q] = relu_clamp(acc[1][q] + bias, clampv);
+                y0[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[0][q], wu, bias) : acc[0][q] + bias, clampv);
+                y1[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[1][q], wu, bias) : acc[1][q] + bias, clampv);
                 nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));
             }
             const int d0 = dst[v0], d1 = dst[v0 + 1];
@@ -1727,7 +1743,7 @@ hipError_t launch_band_pair(const PairLaunch& a, hipStream_t s) {
                            a.bias, a.clampv, a.publish, a.nblk, stream);                                            \
     } while (0)
     switch (a.wmode) {
-        case 0: SPDNN_PAIR(0); break;
+        case 0: if (band_sum_then_scale_enabled()) SPDNN_PAIR(3); else SPDNN_PAIR(0); break;
         case 1: SPDNN_PAIR(1); break;
         default: SPDNN_PAIR(2); break;
     }

@@ -256,7 +256,11 @@ struct spdnn_net {
     int chain_halves = 1;     // fused chains on half row blocks (SPDNN_CHAIN_HALVES=0: whole row blocks)
     bool fuse_pairs = true;   // fused pairs where the inspector found them (SPDNN_FUSE_PAIRS=0: never)
     int pair_seglen = 0;      // band positions per workgroup of a fused pair, 0 = heuristic (SPDNN_PAIR_SEGLEN)
-    int64_t pair_min_elems = 0;  // rows x neurons below which a pair runs as two launches (SPDNN_PAIR_MIN_ELEMS)
+    // rows x neurons below which a pair runs as two launches (SPDNN_PAIR_MIN_ELEMS).  Measured, layers over one
+    // neuron order, N = 1024 ... 65536: from 2^23 elements up the fused pair takes 0.83 - 0.95 of the time of two
+    // launches (0.98 at N=4096, batch 60000), at 2^22 and below up to 2.6 times as long (a 16-wave workgroup
+    // per CU, few segments).
+    int64_t pair_min_elems = (int64_t)1 << 23;
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
@@ -1438,8 +1442,8 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
     const bool have_counts = fused_count || scan_count;
     if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
     int fuse = opt.fuse_layers ? opt.fuse_layers : n->default_fuse;
-    // fused pairs: with fused launches asked for (fuse_layers >= 2, or SPDNN_FUSE_LAYERS as the default)
-    const bool pair_mode = n->fuse_pairs && !scan_count && !plans_streamed(n) && fuse >= 2;
+    // fused pairs: by default and with fused launches asked for, not with fuse_layers = 1
+    const bool pair_mode = n->fuse_pairs && !scan_count && !plans_streamed(n) && (fuse >= 2 || opt.fuse_layers == 0);
     if (scan_count || fuse < 2 || plans_streamed(n)) fuse = 1;  // a fused launch needs all its plans resident
     if (plans_streamed(n))
         for (int l = first; l <= last && l < first + n->plan_window; ++l) HIPCHK(plan_fetch(n, l));
@@ -1489,8 +1493,10 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
         int c = 1;
         // a fused pair (intermediate tile in LDS) where the inspector found one; not while the band
         // walk's BLOCK form would run the layers (small batches of run-chain layers)
+        // (the size threshold belongs to the default; a caller that asks for fused launches gets them)
         const bool pair = pair_mode && p.fuse_next && l + 1 <= last && !use_block_form(n, p, n->carried / n->RB) &&
-                          (int64_t)(n->carried / n->RB) * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems;
+                          (opt.fuse_layers >= 2 ||
+                           (int64_t)(n->carried / n->RB) * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems);
         if (pair) c = 2;
         else if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
             while (c < fuse && l + c <= last) {

@@ -86,11 +86,13 @@ typedef struct spdnn_run_options {
     int32_t collect_counts;    /* 1: record the active-row count after every layer                 */
     int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
-    int32_t fuse_layers;       /* fused variants.  1 = every layer its own launch; 0 = default (the same, unless
-                                  SPDNN_FUSE_LAYERS says otherwise).  >1: pairs of layers the inspector marked
-                                  fuse_next run as one launch with the intermediate tile in LDS, and elsewhere up
-                                  to that many consecutive band layers share a launch (one workgroup keeps a row
-                                  block through the chain, the intermediates going through L2) */
+    int32_t fuse_layers;       /* fused variants.  1 = every layer its own launch.  0 = default: pairs of layers
+                                  the inspector marked fuse_next run as one launch with the intermediate tile in
+                                  LDS where that is the faster way (launches of 2^23 rows x neurons and more;
+                                  SPDNN_PAIR_MIN_ELEMS), every other layer as its own launch (SPDNN_FUSE_LAYERS
+                                  = n makes n the default).  >1: the pairs, and elsewhere up to that many
+                                  consecutive band layers share a launch (one workgroup keeps a row block
+                                  through the chain, the intermediates going through L2) */
     int32_t reserved[3];
 } spdnn_run_options;
 

@@ -497,6 +497,27 @@ def test_fused_pairs_full_batch(gc, orc):
         assert [net.active_count(l) for l in range(L)] == counts
         assert np.array_equal(net.categories(), cats)
         assert same_floats(net.activations(probe), y_fused)
+        # left to the library (fuse_layers = 0) a launch of this size runs the pairs fused; a pruned run only while
+        # enough rows are left (here: after the first compaction it goes on with one launch per layer)
+        net.synth_features(9, B, 0.10, 0.60)
+        r = net.run(prune=False, collect_counts=True)
+        assert (r.fused_pairs, r.launches) == (3, 3)
+        assert [net.active_count(l) for l in range(L)] == counts
+        assert same_floats(net.activations(probe), y_fused)
+        net.synth_features(9, B, 0.10, 0.60)
+        r = net.run(prune=True, collect_counts=True)
+        assert 1 <= r.fused_pairs <= 3 and r.launches == L - r.fused_pairs
+        assert [net.active_count(l) for l in range(L)] == counts
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(probe), y_fused)
+    with gc.Network(N, 512, L, bias=-0.35) as net:      # 2^21 elements: two launches are faster, and are what runs
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.synth_features(9, 512, 0.10, 0.60)
+        r = net.run(prune=False, collect_counts=True)
+        assert (r.fused_pairs, r.launches) == (0, L)
+        assert [net.active_count(l) for l in range(L)] == [len(a) for a in orc.infer(orc.gen_features(9, N, 0, 512, 0.10, 0.60), layers, -0.35, prune=False)["active_ids"]]
 
 
 def test_fused_pairs_several_segments_per_row_block(gc, orc, monkeypatch):
