@@ -143,6 +143,63 @@ __device__ __forceinline__ uint32_t ring_address(uint32_t lane_base, uint32_t dw
     asm("v_lshl_add_u32 %0, %1, %2, %3" : "=v"(addr) : "s"(slot), "n"(COL_SHIFT), "v"(lane_base));
     return addr;
 }
+// add_pair_if_used followed, in the same statement, by the LDS address of a later step's column (ring_address):
+// between two separate asm statements the compiler puts a wait state it cannot know to be unnecessary, two
+// per step of the walk; within one statement the scalar extract feeds the vector shift-add directly.
+template <int RL, int SLOT_BITS, int COL_SHIFT>
+__device__ __forceinline__ uint32_t add_pair_if_used_then_address(float* acc0, float* acc1, const float* x, uint64_t mask0,
+                                                                  uint64_t mask1, int bit, uint32_t lane_base,
+                                                                  uint32_t dword, int b);
+#define SPDNN_ADDR_TAIL "s_mov_b64 exec, -1\n\ts_bfe_u32 %[slot], %[dw], %[fld]\n\tv_lshl_add_u32 %[addr], %[slot], %[sh], %[base]"
+template <> __device__ __forceinline__ uint32_t add_pair_if_used_then_address<4, 6, 10>(
+    float* acc0, float* acc1, const float* x, uint64_t mask0, uint64_t mask1, int bit, uint32_t lane_base, uint32_t dword, int b) {
+    uint32_t addr, slot;
+    asm volatile(
+        "s_bfe_i64 exec, %[m0], %[bit]\n\t"
+        "v_add_f32 %[a0], %[x0], %[a0]\n\tv_add_f32 %[a1], %[x1], %[a1]\n\tv_add_f32 %[a2], %[x2], %[a2]\n\tv_add_f32 %[a3], %[x3], %[a3]\n\t"
+        "s_bfe_i64 exec, %[m1], %[bit]\n\t"
+        "v_add_f32 %[b0], %[x0], %[b0]\n\tv_add_f32 %[b1], %[x1], %[b1]\n\tv_add_f32 %[b2], %[x2], %[b2]\n\tv_add_f32 %[b3], %[x3], %[b3]\n\t"
+        SPDNN_ADDR_TAIL
+        : [a0] "+v"(acc0[0]), [a1] "+v"(acc0[1]), [a2] "+v"(acc0[2]), [a3] "+v"(acc0[3]), [b0] "+v"(acc1[0]),
+          [b1] "+v"(acc1[1]), [b2] "+v"(acc1[2]), [b3] "+v"(acc1[3]), [addr] "=&v"(addr), [slot] "=&s"(slot)
+        : [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [m0] "s"(mask0), [m1] "s"(mask1),
+          [bit] "n"(0x10000 | bit), [dw] "s"(dword), [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(10), [base] "v"(lane_base)
+        : "scc");
+    return addr;
+}
+template <> __device__ __forceinline__ uint32_t add_pair_if_used_then_address<2, 6, 9>(
+    float* acc0, float* acc1, const float* x, uint64_t mask0, uint64_t mask1, int bit, uint32_t lane_base, uint32_t dword, int b) {
+    uint32_t addr, slot;
+    asm volatile(
+        "s_bfe_i64 exec, %[m0], %[bit]\n\t"
+        "v_add_f32 %[a0], %[x0], %[a0]\n\tv_add_f32 %[a1], %[x1], %[a1]\n\t"
+        "s_bfe_i64 exec, %[m1], %[bit]\n\t"
+        "v_add_f32 %[b0], %[x0], %[b0]\n\tv_add_f32 %[b1], %[x1], %[b1]\n\t"
+        SPDNN_ADDR_TAIL
+        : [a0] "+v"(acc0[0]), [a1] "+v"(acc0[1]), [b0] "+v"(acc1[0]), [b1] "+v"(acc1[1]), [addr] "=&v"(addr),
+          [slot] "=&s"(slot)
+        : [x0] "v"(x[0]), [x1] "v"(x[1]), [m0] "s"(mask0), [m1] "s"(mask1), [bit] "n"(0x10000 | bit), [dw] "s"(dword),
+          [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(9), [base] "v"(lane_base)
+        : "scc");
+    return addr;
+}
+template <> __device__ __forceinline__ uint32_t add_pair_if_used_then_address<1, 6, 8>(
+    float* acc0, float* acc1, const float* x, uint64_t mask0, uint64_t mask1, int bit, uint32_t lane_base, uint32_t dword, int b) {
+    uint32_t addr, slot;
+    asm volatile(
+        "s_bfe_i64 exec, %[m0], %[bit]\n\t"
+        "v_add_f32 %[a0], %[x0], %[a0]\n\t"
+        "s_bfe_i64 exec, %[m1], %[bit]\n\t"
+        "v_add_f32 %[b0], %[x0], %[b0]\n\t"
+        SPDNN_ADDR_TAIL
+        : [a0] "+v"(acc0[0]), [b0] "+v"(acc1[0]), [addr] "=&v"(addr), [slot] "=&s"(slot)
+        : [x0] "v"(x[0]), [m0] "s"(mask0), [m1] "s"(mask1), [bit] "n"(0x10000 | bit), [dw] "s"(dword),
+          [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(8), [base] "v"(lane_base)
+        : "scc");
+    return addr;
+}
+#undef SPDNN_ADDR_TAIL
+
 // RL floats from an LDS byte address
 template <int RL> __device__ __forceinline__ void lds_read(uint32_t lds_address, float* x) {
     typedef float vec_t __attribute__((ext_vector_type(RL)));
@@ -466,9 +523,19 @@ __device__ __forceinline__ void band_walk_body(
      : ((e) >> 2) == 6 ? sb[i].z : ((e) >> 2) == 7 ? sb[i].w : sc[i])
 #define SPDNN_READ_COLUMN(i, e, x)                                                                    \
     do {                                                                                              \
-        if (WMODE == 3) lds_read<RL>(ring_address<SLOT_BITS, COL_SHIFT>(lane_base, SPDNN_SLOT_DWORD(i, e), (e) & 3), x); \
+        if (WMODE == 3) lds_read<RL>(col_addr[(e) % 3][i], x);                                         \
         else vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), x);     \
     } while (0)
+            // WMODE 3: the LDS address of step e's column, worked out one iteration before its read is issued
+            // (steps 0 .. 2 here, step s + 3 in the same statement as the adds of step s)
+            uint32_t col_addr[3][PPW];
+            if (WMODE == 3) {
+#pragma unroll
+                for (int e = 0; e < 3; ++e)
+#pragma unroll
+                    for (int i = 0; i < PPW; ++i)
+                        col_addr[e][i] = ring_address<SLOT_BITS, COL_SHIFT>(lane_base, SPDNN_SLOT_DWORD(i, e), e & 3);
+            }
 #define SPDNN_STEP_LIVE(e) (KT == 36 ? ((e) < 32 || (e) < steps) : (((e) & ~3) < steps))
 #define SPDNN_USED(i, o, e) (((((e) < 32) ? ((o) ? mk[i].z : mk[i].x) : ((o) ? mk[i].w : mk[i].y)) >> ((e) & 31)) & 1u)
 #pragma unroll
@@ -494,7 +561,12 @@ __device__ __forceinline__ void band_walk_body(
                     if (SPDNN_STEP_LIVE(st)) {
 #pragma unroll
                         for (int i = 0; i < PPW; ++i) {
-                            add_pair_if_used<RL>(acc[i][0], acc[i][1], xb[st % 3][i], use0[i], use1[i], st);
+                            if (st + 3 < 36)
+                                col_addr[st % 3][i] = add_pair_if_used_then_address<RL, SLOT_BITS, COL_SHIFT>(
+                                    acc[i][0], acc[i][1], xb[st % 3][i], use0[i], use1[i], st, lane_base,
+                                    SPDNN_SLOT_DWORD(i, st + 3), (st + 3) & 3);
+                            else
+                                add_pair_if_used<RL>(acc[i][0], acc[i][1], xb[st % 3][i], use0[i], use1[i], st);
                         }
                     }
                 } else if (SPDNN_STEP_LIVE(st)) {

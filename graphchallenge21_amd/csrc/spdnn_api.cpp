@@ -414,17 +414,26 @@ int alloc_feature_buffers(spdnn_net* n) {
             return e;
         };
         // candidates that share the reference's region (the slow ones) and candidates that do not
+        // `strong`: the two best candidates elsewhere reach the rate of two regions (7.2 against 6.0 TB/s);
+        // a candidate that straddles a boundary lies in between and makes a poor half (measured: layers of
+        // 5.23 - 5.35 ms instead of 5.16 - 5.19 at the cfg4 shape with partners that swept at 6.9 TB/s)
+        bool strong = false;
         auto classify = [&](int ref) {
             double lowest = 0.0;
             for (size_t k = 0; k < rate.size(); ++k)
                 if ((int)k != ref && (lowest == 0.0 || rate[k] < lowest)) lowest = rate[k];
-            same.assign(1, ref);
+            same.clear();
             other.clear();
             for (size_t k = 0; k < rate.size(); ++k) {
                 if ((int)k == ref) continue;
                 if (rate[k] > 1.10 * lowest) other.push_back((int)k);
                 else if (rate[k] < 1.05 * lowest) same.push_back((int)k);
             }
+            // the clearest cases first: the fastest partners elsewhere, the slowest in the reference's region
+            std::sort(other.begin(), other.end(), [&](int a, int b) { return rate[(size_t)a] > rate[(size_t)b]; });
+            std::sort(same.begin(), same.end(), [&](int a, int b) { return rate[(size_t)a] < rate[(size_t)b]; });
+            same.insert(same.begin(), ref);
+            strong = other.size() >= 2 && rate[(size_t)other[1]] >= 1.17 * lowest;
             // The two work buffers, which every layer streams through, need a half of each kind; the
             // feature buffer (read by the first layer only) takes one if there is one.
             return same.size() >= 2 && other.size() >= 3;
@@ -436,7 +445,8 @@ int alloc_feature_buffers(spdnn_net* n) {
         rate.assign(1, 0.0);
         bool found = false;
         int ref = 0;
-        for (size_t i = 1; i < max_cand && !found; ++i) {
+        int extra = 0;   // candidates tried beyond the first complete set, looking for clear partners
+        for (size_t i = 1; i < max_cand && !(found && (strong || extra >= 6)); ++i) {
             if (i >= c.size()) {
                 if ((c.size() + 1) * half_bytes + (fillers.size() + 1) * filler > budget) break;
                 if (filler) {
@@ -450,6 +460,7 @@ int alloc_feature_buffers(spdnn_net* n) {
             const hipError_t e = probe(0, i, &r);
             if (e != hipSuccess) return fail_free(SPDNN_E_DEVICE, std::string("region probe: ") + hipGetErrorString(e));
             rate.push_back(r);
+            if (found) ++extra;
             found = i >= 5 && classify(0);
         }
         if (!found && rate.size() >= 8) {
