@@ -826,8 +826,17 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
                                                 const float* __restrict__ pw, int pr, int steps, uint32_t wu_bits,
                                                 float (&acc)[2][4]) {
     const uint4* rec = reinterpret_cast<const uint4*>(pairs + (size_t)pr * 16);
-    const uint4 mk = rec[0], sa = rec[1], sb = rec[2];
-    const uint32_t sc = pairs[(size_t)pr * 16 + 12];
+    uint4 mk = rec[0], sa = rec[1], sb = rec[2];
+    uint32_t sc = pairs[(size_t)pr * 16 + 12];
+    if (WMODE == 3) {
+        // the record is the same for every lane; the add-only walk hands its words to the scalar unit as
+        // they are, so say so where the compiler has not seen it (free where it has)
+        auto uni = [](uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); };
+        mk = make_uint4(uni(mk.x), uni(mk.y), uni(mk.z), uni(mk.w));
+        sa = make_uint4(uni(sa.x), uni(sa.y), uni(sa.z), uni(sa.w));
+        sb = make_uint4(uni(sb.x), uni(sb.y), uni(sb.z), uni(sb.w));
+        sc = uni(sc);
+    }
     const float4* wp = nullptr;
     float4 w_cur[2], w_nxt[2];
     constexpr bool WSTREAM = WMODE == 1 || WMODE == 2;   // weights come per step from the plan
@@ -849,9 +858,14 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
      : ((e) >> 2) == 4 ? sb.x : ((e) >> 2) == 5 ? sb.y : ((e) >> 2) == 6 ? sb.z : ((e) >> 2) == 7 ? sb.w : sc)
 #define SPDNN_PREAD(e, x)                                                                                \
     do {                                                                                                 \
-        if (WMODE == 3) lds_read<4>(ring_address<6, 10>(lane_base, SPDNN_PSLOT_DWORD(e), (e) & 3), x);      \
+        if (WMODE == 3) lds_read<4>(col_addr[(e) % 3], x);                                                \
         else vec_to_arr<4>(*reinterpret_cast<const float4*>(lane_ring + (size_t)SPDNN_PSLOT(e) * 1024), x); \
     } while (0)
+    uint32_t col_addr[3];   // WMODE 3: LDS address of step e's column, worked out one iteration before its read
+    if (WMODE == 3) {
+#pragma unroll
+        for (int e = 0; e < 3; ++e) col_addr[e] = ring_address<6, 10>(lane_base, SPDNN_PSLOT_DWORD(e), e & 3);
+    }
 #define SPDNN_PUSED(o, e) (((((e) < 32) ? ((o) ? mk.z : mk.x) : ((o) ? mk.w : mk.y)) >> ((e) & 31)) & 1u)
 #pragma unroll
     for (int e = 0; e < 2; ++e)
@@ -865,7 +879,13 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
             w_nxt[1] = wp[(st >> 2) * 2 + 3];
         }
         if (WMODE == 3) {
-            if (st < 32 || st < steps) add_pair_if_used<4>(acc[0], acc[1], xb[st % 3], use0, use1, st);
+            if (st < 32 || st < steps) {
+                if (st + 3 < 36)
+                    col_addr[st % 3] = add_pair_if_used_then_address<4, 6, 10>(acc[0], acc[1], xb[st % 3], use0, use1, st, lane_base,
+                                                                               SPDNN_PSLOT_DWORD(st + 3), (st + 3) & 3);
+                else
+                    add_pair_if_used<4>(acc[0], acc[1], xb[st % 3], use0, use1, st);
+            }
         } else if (st < 32 || st < steps) {
             float w0, w1;
             if (WSTREAM) {
