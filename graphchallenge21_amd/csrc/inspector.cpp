@@ -562,6 +562,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
 
     plan.kmax = kmax;
     plan.self_aligned = false;
+    plan.pair_twins = false;
     plan.fuse_next = false;
     plan.info = spdnn_layer_plan{};
     plan.info.max_row_nnz = kmax;
@@ -687,6 +688,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.pair_padded = trips * 4;
         plan.pairs.assign((size_t)npairs * stride, 0u);
         if (plan.wmode != 0) plan.wv.assign((size_t)npairs * trips * 8, 0.0f); else plan.wv.clear();
+        bool twins = plan.wmode == 0;
         for (int u = 0; u < npairs; ++u) {
             const int j0 = plan.out_at[2 * u], j1 = plan.out_at[2 * u + 1];
             uint32_t* rec = &plan.pairs[(size_t)u * stride];
@@ -706,7 +708,10 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
             for (int t = m; t < trips * 4; ++t) slots[t] = slots[m - 1];
             rec[0] = (uint32_t)use0; rec[1] = (uint32_t)(use0 >> 32);
             rec[2] = (uint32_t)use1; rec[3] = (uint32_t)(use1 >> 32);
+            // every step of the record used by both outputs: under one weight the two are equal
+            if (use0 != use1 || use0 != (steps >= 64 ? ~0ull : (1ull << steps) - 1)) twins = false;
         }
+        plan.pair_twins = twins;
         plan.ell_col.clear();
         plan.rowlen.clear();
     } else if (force_kernel != SPDNN_KERNEL_GATHER && !(getenv("SPDNN_TILED") && atoi(getenv("SPDNN_TILED")) == 0) &&

@@ -62,6 +62,7 @@ struct LayerPlan {
     // the column's slot in the panel as raw bits, weight)
     int ntiles = 0;
     bool self_aligned = false;
+    bool pair_twins = false;   // BAND, one exact weight: the two outputs of every pair use the same inputs
     bool fuse_next = false;
 };
 

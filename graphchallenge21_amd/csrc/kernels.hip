@@ -85,6 +85,9 @@ template <> __device__ __forceinline__ float4 arr_to_vec<4>(const float* a) {
 //              v_mul_f32 on this hardware (measured: 0.95 against 1.72 ns per wave instruction and
 //              SIMD) - and the weight enters once, in the epilogue's fma(sum, w, bias), which rounds
 //              like the reference's add of the bias because w * sum is exact.
+//   WMODE 4:   WMODE 3 for layers in which the two outputs of every pair use the same inputs (groups of
+//              identical rows: the run chains of RadiX-Net layers): the two sums are equal, so the pair
+//              keeps one accumulator, adds every step without a mask and stores the result twice.
 __device__ __forceinline__ float mul_then_add(float acc, float x, float w) {
 #pragma clang fp contract(off)
     const float p = x * w;
@@ -199,6 +202,35 @@ template <> __device__ __forceinline__ uint32_t add_pair_if_used_then_address<1,
     return addr;
 }
 #undef SPDNN_ADDR_TAIL
+
+// twins (both outputs of a pair add every step): RL adds into the one accumulator, then the address of a
+// later step's column, in one statement as above
+template <int RL, int SLOT_BITS, int COL_SHIFT>
+__device__ __forceinline__ uint32_t add_then_address(float* acc, const float* x, uint32_t lane_base, uint32_t dword, int b) {
+    static_assert(SLOT_BITS == 6, "64-slot ring");
+    uint32_t addr, slot;
+    if (RL == 4)
+        asm volatile("v_add_f32 %[a0], %[x0], %[a0]\n\tv_add_f32 %[a1], %[x1], %[a1]\n\tv_add_f32 %[a2], %[x2], %[a2]\n\t"
+                     "v_add_f32 %[a3], %[x3], %[a3]\n\ts_bfe_u32 %[slot], %[dw], %[fld]\n\tv_lshl_add_u32 %[addr], %[slot], %[sh], %[base]"
+                     : [a0] "+v"(acc[0]), [a1] "+v"(acc[1]), [a2] "+v"(acc[2]), [a3] "+v"(acc[3]), [addr] "=&v"(addr), [slot] "=&s"(slot)
+                     : [x0] "v"(x[0]), [x1] "v"(x[1]), [x2] "v"(x[2]), [x3] "v"(x[3]), [dw] "s"(dword),
+                       [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(COL_SHIFT), [base] "v"(lane_base)
+                     : "scc");
+    else if (RL == 2)
+        asm volatile("v_add_f32 %[a0], %[x0], %[a0]\n\tv_add_f32 %[a1], %[x1], %[a1]\n\t"
+                     "s_bfe_u32 %[slot], %[dw], %[fld]\n\tv_lshl_add_u32 %[addr], %[slot], %[sh], %[base]"
+                     : [a0] "+v"(acc[0]), [a1] "+v"(acc[1]), [addr] "=&v"(addr), [slot] "=&s"(slot)
+                     : [x0] "v"(x[0]), [x1] "v"(x[1]), [dw] "s"(dword), [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(COL_SHIFT),
+                       [base] "v"(lane_base)
+                     : "scc");
+    else
+        asm volatile("v_add_f32 %[a0], %[x0], %[a0]\n\t"
+                     "s_bfe_u32 %[slot], %[dw], %[fld]\n\tv_lshl_add_u32 %[addr], %[slot], %[sh], %[base]"
+                     : [a0] "+v"(acc[0]), [addr] "=&v"(addr), [slot] "=&s"(slot)
+                     : [x0] "v"(x[0]), [dw] "s"(dword), [fld] "n"((6 << 16) | (8 * b)), [sh] "n"(COL_SHIFT), [base] "v"(lane_base)
+                     : "scc");
+    return addr;
+}
 
 // RL floats from an LDS byte address
 template <int RL> __device__ __forceinline__ void lds_read(uint32_t lds_address, float* x) {
@@ -442,8 +474,8 @@ __device__ __forceinline__ void band_walk_body(
             const int g = p < 0 ? p + N : p;
             if (DMA) {
                 unsigned char* slot = smem + (size_t)(p & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)g * RBL + loff, slot);
-                else column_to_lds<0, WMODE != 3>(yin + (size_t)g * RBL + loff, slot);
+                if (stream) column_to_lds<1, (WMODE < 3)>(yin + (size_t)g * RBL + loff, slot);
+                else column_to_lds<0, (WMODE < 3)>(yin + (size_t)g * RBL + loff, slot);
                 continue;
             }
             float x[RL];
@@ -466,8 +498,8 @@ __device__ __forceinline__ void band_walk_body(
             const int p = min(cb + T + wave + i * NW, ve - 1);
             if (DMA) {
                 unsigned char* slot = smem + (size_t)((cb + T + wave + i * NW) & (RING - 1)) * COLB;
-                if (stream) column_to_lds<1, WMODE != 3>(yin + (size_t)p * RBL + loff, slot);
-                else column_to_lds<0, WMODE != 3>(yin + (size_t)p * RBL + loff, slot);
+                if (stream) column_to_lds<1, (WMODE < 3)>(yin + (size_t)p * RBL + loff, slot);
+                else column_to_lds<0, (WMODE < 3)>(yin + (size_t)p * RBL + loff, slot);
             } else if (stream) load_stream<RL>(yin + (size_t)p * RBL + loff, pf[i]);
             else vec_to_arr<RL>(*reinterpret_cast<const V*>(yin + (size_t)p * RBL + loff), pf[i]);
         }
@@ -523,13 +555,13 @@ __device__ __forceinline__ void band_walk_body(
      : ((e) >> 2) == 6 ? sb[i].z : ((e) >> 2) == 7 ? sb[i].w : sc[i])
 #define SPDNN_READ_COLUMN(i, e, x)                                                                    \
     do {                                                                                              \
-        if (WMODE == 3) lds_read<RL>(col_addr[(e) % 3][i], x);                                         \
+        if (WMODE >= 3) lds_read<RL>(col_addr[(e) % 3][i], x);                                         \
         else vec_to_arr<RL>(*reinterpret_cast<const V*>(lane_smem + (size_t)SPDNN_SLOT(i, e) * COLB), x);     \
     } while (0)
             // WMODE 3: the LDS address of step e's column, worked out one iteration before its read is issued
             // (steps 0 .. 2 here, step s + 3 in the same statement as the adds of step s)
             uint32_t col_addr[3][PPW];
-            if (WMODE == 3) {
+            if (WMODE >= 3) {
 #pragma unroll
                 for (int e = 0; e < 3; ++e)
 #pragma unroll
@@ -557,7 +589,20 @@ __device__ __forceinline__ void band_walk_body(
                         w_nxt[i][1] = load_const_f4(wp[i] + 4 * ((st >> 2) * 2 + 3));
                     }
                 }
-                if (WMODE == 3) {
+                if (WMODE == 4) {
+                    // twins: both outputs of the pair add every step - one accumulator, no masks
+                    if (SPDNN_STEP_LIVE(st)) {
+#pragma unroll
+                        for (int i = 0; i < PPW; ++i) {
+                            if (st + 3 < 36)
+                                col_addr[st % 3][i] = add_then_address<RL, SLOT_BITS, COL_SHIFT>(
+                                    acc[i][0], xb[st % 3][i], lane_base, SPDNN_SLOT_DWORD(i, st + 3), (st + 3) & 3);
+                            else
+#pragma unroll
+                                for (int q = 0; q < RL; ++q) acc[i][0][q] += xb[st % 3][i][q];
+                        }
+                    }
+                } else if (WMODE == 3) {
                     if (SPDNN_STEP_LIVE(st)) {
 #pragma unroll
                         for (int i = 0; i < PPW; ++i) {
@@ -636,8 +681,8 @@ __device__ __forceinline__ void band_walk_body(
                 float y0[RL], y1[RL];
 #pragma unroll
                 for (int q = 0; q < RL; ++q) {
-                    y0[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
-                    y1[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][1][q], wu, bias) : acc[i][1][q] + bias, clampv);
+                    y0[q] = relu_clamp(WMODE >= 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
+                    y1[q] = WMODE == 4 ? y0[q] : relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][1][q], wu, bias) : acc[i][1][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], nz_merge(y0[q], y1[q]));   // one three-way maximum
                 }
                 const int d0 = dst[v0], d1 = dst[v0 + 1];
@@ -652,7 +697,7 @@ __device__ __forceinline__ void band_walk_body(
                 float y[RL];
 #pragma unroll
                 for (int q = 0; q < RL; ++q) {
-                    y[q] = relu_clamp(WMODE == 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
+                    y[q] = relu_clamp(WMODE >= 3 ? __builtin_fmaf(acc[i][0][q], wu, bias) : acc[i][0][q] + bias, clampv);
                     nz[q] = nz_merge(nz[q], y[q]);
                 }
                 *reinterpret_cast<V*>(yout + (size_t)dst[v0] * RBL + loff) = arr_to_vec<RL>(y);
@@ -1624,6 +1669,7 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
     if (band_unrolled(a.K, a.steps, a.stride)) {
         switch (a.wmode) {
             case 0:
+                if (band_sum_then_scale_enabled() && a.twins) return launch_band_inst<RL, NW, OPW, RING, 4, 36, DMA>(a, s);
                 if (band_sum_then_scale_enabled()) return launch_band_inst<RL, NW, OPW, RING, 3, 36, DMA>(a, s);
                 return launch_band_inst<RL, NW, OPW, RING, 0, 36, DMA>(a, s);
             case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36, DMA>(a, s);

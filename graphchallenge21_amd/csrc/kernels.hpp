@@ -46,11 +46,13 @@ struct BandLaunch {
     int32_t* active;         // [rows] row stamp: active[row] = stamp if the row has a nonzero output
     int32_t* count_prev;     // device counter of the layer that stamped prev_stamp: this launch adds the rows that layer left active (may be nullptr)
     int N, K, nblk, stamp, rl;
-    int steps, stride;       // merged steps per pair (K .. 2K); dwords per pair record (multiple of 4)
+    int steps, stride;       // merged steps per pair (K .. 36); dwords per pair record (16)
     int halo;                // input columns a segment needs before its first position: K-1 .. 32
     int prev_stamp = 0;      // stamp of the previous layer if the row slots still carry it (0 = none)
     int check_dead = 0;      // 1: row blocks the previous layer left without an active row are skipped
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
+    int twins = 0;           // 1 (wmode 0): the two outputs of every pair use the same inputs (groups of identical rows,
+                             // as in a run chain), so they are equal: one accumulator per pair, stored twice
     float wu, bias, clampv;
     int n_cu;
     int shape = -1;          // variant (see band_shape_count): 256-row blocks 0 = direct-to-LDS loads, 1 = through registers; < 0 = default

@@ -1248,7 +1248,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out
     const DevLayer& d = n->dl[(size_t)l];
     BandLaunch a{};
     a.yin = in; a.yout = out; a.pairs = d.pairs; a.pw = d.wv; a.dst = d.dst; a.active = n->d_active;
-    a.steps = p.pair_steps; a.stride = p.pair_stride;
+    a.steps = p.pair_steps; a.stride = p.pair_stride; a.twins = p.pair_twins ? 1 : 0;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
