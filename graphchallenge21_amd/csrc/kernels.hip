@@ -1155,17 +1155,15 @@ __global__ __launch_bounds__(256) void gather_kernel(
 // `rounds` rounds of 2 entries per output.  An entry is an LDS byte offset and a weight; streaming
 // 8 bytes per multiply-add through the scalar cache does not work (every access misses, and the
 // cache serves few misses at a time: measured 0.69 ms per layer of 1024 neurons where the plain
-// gather takes 0.45), so the entry blocks (1 KiB per round and wave) go through LDS too: the wave
-// sends the next block into its own two-block ring while it works on the current one and reads
-// the entries back with broadcast reads (all lanes the same address).
+// gather takes 0.45), so the entry blocks (1 KiB per round and wave) go through LDS too, into a
+// per-wave ring.  ROWBCAST = 1 (default): four reads put a round's block into registers (lane j of
+// every 16-lane row holds the entries of outputs j, 16 + j, 32 + j, 48 + j) and the DPP row
+// broadcast hands an entry's offset and weight to all lanes inside the add and the multiply that
+// use them.  ROWBCAST = 0 (SPDNN_TILED_ROW_BROADCAST=0): the entries are read back pair by pair
+// with broadcast reads (all lanes the same address) - half an LDS instruction more per entry.
 // Accumulation in ascending input index: panels ascend, entries inside a panel ascend; padding
 // entries carry weight -0 and add an exact zero.
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void column64_to_lds(const float* gsrc_lane, unsigned char* lds_col) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gsrc_lane,
-                                     (__attribute__((address_space(3))) void*)lds_col, 4, 0, 0);
-}
-
 // 64 lanes x 16 bytes from global memory into 1 KiB of LDS, issued in a form the compiler does not
 // follow: it puts a wait for ALL vector memory traffic in front of any LDS read that might touch
 // the destination of a direct-to-LDS load it knows of, which here would be the very next read (the
@@ -1179,7 +1177,20 @@ __device__ __forceinline__ void block_to_lds_untracked(const float* gsrc_lane, u
                  : "memory");
 }
 
-template <int WMODE>
+// The value lane j of every 16-lane row holds, in all lanes of that row (DPP row_newbcast: the
+// compiler folds the move into the instruction that uses it).
+__device__ __forceinline__ uint32_t row_lane(uint32_t v, int j) {
+    switch (j) {
+#define SPDNN_ROW_LANE(J) case J: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x150 + J, 0xf, 0xf, true);
+        SPDNN_ROW_LANE(0) SPDNN_ROW_LANE(1) SPDNN_ROW_LANE(2) SPDNN_ROW_LANE(3) SPDNN_ROW_LANE(4) SPDNN_ROW_LANE(5)
+        SPDNN_ROW_LANE(6) SPDNN_ROW_LANE(7) SPDNN_ROW_LANE(8) SPDNN_ROW_LANE(9) SPDNN_ROW_LANE(10) SPDNN_ROW_LANE(11)
+        SPDNN_ROW_LANE(12) SPDNN_ROW_LANE(13) SPDNN_ROW_LANE(14) SPDNN_ROW_LANE(15)
+#undef SPDNN_ROW_LANE
+    }
+    return v;
+}
+
+template <int WMODE, int ROWBCAST>
 __global__ __launch_bounds__(1024) void tiled_kernel(
     Feat yin_all, Feat yout_all, const int32_t* __restrict__ cols, const int32_t* __restrict__ hdr,
     const uint32_t* __restrict__ ent, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
@@ -1221,12 +1232,19 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
     for (int o = 0; o < 64; ++o) acc[o] = 0.0f;
 
     for (int p = 0; p < np; ++p) {
-        // the panel's columns, 32 per wave (every wave has finished the panel before: barrier below)
+        // the panel's columns, 32 per wave (every wave has finished the panel before: barrier below).  Four
+        // columns per instruction: a column is 64 rows x 4 bytes = the 16-byte parts of 16 lanes, so each
+        // quarter of the wave brings its own column and the four land in consecutive slots.
         const int32_t* pc = cols + (size_t)(gp0 + p) * 512;
-#pragma unroll 4
-        for (int i = 0; i < 32; ++i) {
-            const int sl = w + 16 * i;
-            column64_to_lds(yin + (size_t)pc[sl] * RB, smem + sl * 256);
+        {
+            const float* quarter_src = yin - lane + (lane & 15) * 4;   // (yin points at this lane's row)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int sl0 = w * 32 + i * 4;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void*)(quarter_src + (size_t)pc[sl0 + (lane >> 4)] * RB),
+                    (__attribute__((address_space(3))) void*)(smem + sl0 * 256), 16, 0, 0);
+            }
         }
         const int rounds = wave_hdr[((size_t)(gp0 + p) * 16 + w) * 2];
         const float* blk = reinterpret_cast<const float*>(ent) + (size_t)wave_hdr[((size_t)(gp0 + p) * 16 + w) * 2 + 1] * 256;
@@ -1236,6 +1254,59 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
         }
         wait_vector_memory();
         ring_barrier<1>();
+        if (ROWBCAST) {
+            // A round's entry block, [output][2](LDS offset of the column, weight), goes into registers with four
+            // reads: lane j of each of the wave's four 16-lane rows takes the 16 bytes of output 16 g + j, g = 0 .. 3
+            // (the rows read the same addresses).  An entry's offset and weight then come to all lanes of a row
+            // through the DPP row broadcast of the add and the multiply that use them: one LDS instruction per
+            // entry (the column) instead of one and a half.
+            const uint32_t ent_base = (uint32_t)(size_t)((__attribute__((address_space(3))) unsigned char*)ring) + (lane & 15) * 16;
+            const uint32_t panel_base = (uint32_t)(size_t)((__attribute__((address_space(3))) const unsigned char*)lane_panel);
+            float mg[4][4];
+            if (rounds > 0) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) lds_read<4>(ent_base + g * 256, mg[g]);
+            }
+            for (int r = 0; r < rounds; ++r) {
+                if (r + 1 < rounds) {
+                    // the block is in registers: the next round's comes into the same kilobyte
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    block_to_lds_untracked(blk + (size_t)(r + 1) * 256 + lane * 4, ring);
+                }
+                // units of two outputs (four entries), the columns of the next unit in flight during the arithmetic (two
+                // units ahead measures the same)
+                float x[2][4];
+#define SPDNN_TILE_READ(u, buf)                                                                                 \
+    do {                                                                                                        \
+        _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                                         \
+            const int o = (u) * 2 + (e >> 1);                                                                   \
+            const uint32_t off = row_lane(__float_as_uint(mg[o >> 4][(e & 1) * 2]), o & 15);                    \
+            lds_read<1>(off + panel_base, &x[buf][e]);                                                          \
+        }                                                                                                       \
+    } while (0)
+                SPDNN_TILE_READ(0, 0);
+#pragma unroll 32
+                for (int u = 0; u < 32; ++u) {
+                    if (u + 1 < 32) SPDNN_TILE_READ(u + 1, (u + 1) & 1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int o = u * 2 + (e >> 1);
+                        const float wgt = __uint_as_float(row_lane(__float_as_uint(mg[o >> 4][(e & 1) * 2 + 1]), o & 15));
+                        acc[o] = mac<WMODE>(acc[o], x[u & 1][e], wgt);
+                    }
+                    // pins the unit's arithmetic here: left alone the compiler gathers all reads of the round first
+                    asm volatile("" : "+v"(acc[u * 2]), "+v"(acc[u * 2 + 1]) : : "memory");
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+#undef SPDNN_TILE_READ
+                if (r + 1 < rounds) {
+                    wait_vector_memory();   // the next entry block has arrived
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) lds_read<4>(ent_base + g * 256, mg[g]);
+                }
+            }
+        } else
         for (int r = 0; r < rounds; ++r) {
             if (r + 1 < rounds) block_to_lds_untracked(blk + (size_t)(r + 1) * 256 + lane * 4, ring + ((r + 1) & 1) * 1024);
             const unsigned char* cur = ring + (r & 1) * 1024;
@@ -1923,16 +1994,18 @@ hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     constexpr size_t lds = 512 * 256 + 16 * 2048;   // one panel and the waves' entry rings: all 160 KiB of a CU
     dim3 grid(a.nblk * a.rl, a.ntiles), block(1024);
-#define SPDNN_TILED(WM)                                                                                          \
+#define SPDNN_TILED(WM, RBC)                                                                                     \
     do {                                                                                                         \
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM>),      \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM, RBC>), \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
         if (attr != hipSuccess) return attr;                                                                     \
-        hipLaunchKernelGGL(tiled_kernel<WM>, grid, block, lds, s, a.yin, a.yout, a.cols, a.hdr, a.ent, a.dst,    \
+        hipLaunchKernelGGL((tiled_kernel<WM, RBC>), grid, block, lds, s, a.yin, a.yout, a.cols, a.hdr, a.ent, a.dst, \
                            a.active, a.count_prev, a.N, a.ntiles, a.rl, a.stamp, a.prev_stamp, a.check_dead,     \
                            a.bias, a.clampv, a.publish);                                                         \
     } while (0)
-    if (a.wmode != 2) SPDNN_TILED(1); else SPDNN_TILED(2);
+    static const bool rowbcast = !(getenv("SPDNN_TILED_ROW_BROADCAST") && atoi(getenv("SPDNN_TILED_ROW_BROADCAST")) == 0);
+    if (rowbcast) { if (a.wmode != 2) SPDNN_TILED(1, 1); else SPDNN_TILED(2, 1); }
+    else { if (a.wmode != 2) SPDNN_TILED(1, 0); else SPDNN_TILED(2, 0); }
 #undef SPDNN_TILED
     return hipGetLastError();
 }
