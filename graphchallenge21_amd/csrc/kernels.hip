@@ -413,9 +413,11 @@ __device__ __forceinline__ float relu_clamp(float y, float clampv) {
 // feeds it to both accumulators - half the LDS reads and address arithmetic of one list per
 // output.  A step an output does not use enters it with weight 0 (adding an exact zero).
 //
-// Per pair the scalar unit streams `stride` dwords: two 64-bit use masks (output 0, output 1), then
-// the steps' one-byte ring selectors; unless the layer has one exact value also two weights per
-// step.  The output column is written to the physical column the NEXT layer wants it in (dst),
+// Per pair the scalar unit streams a record of 16 dwords: two 64-bit use masks (output 0, output 1),
+// then the steps' one-byte ring selectors; unless the layer has one exact value also two weights per
+// step (72 floats per pair).  How a step enters the accumulators depends on the weight mode (see mac
+// above): a multiply-add with the step's weight, or - one power-of-two weight per layer - a plain
+// add under the output's use bit, the weight applied once in the epilogue.  The output column is written to the physical column the NEXT layer wants it in (dst),
 // RB*4 contiguous bytes.
 // ------------------------------------------------------------------------------------------
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
