@@ -1727,23 +1727,13 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     return hipGetLastError();
 }
 
-// SPDNN_BAND_SUM_THEN_SCALE=0: layers with one exact weight keep a multiply-add per input (WMODE 0)
-// instead of adding the inputs and scaling the sum (WMODE 3); read once per process.
-bool band_sum_then_scale_enabled() {
-    static const bool on = [] {
-        const char* e = getenv("SPDNN_BAND_SUM_THEN_SCALE");
-        return !(e && atoi(e) == 0);
-    }();
-    return on;
-}
-
 template <int RL, int NW, int OPW, int RING, int DMA>
 hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
     if (band_unrolled(a.K, a.steps, a.stride)) {
         switch (a.wmode) {
             case 0:
-                if (band_sum_then_scale_enabled() && a.twins) return launch_band_inst<RL, NW, OPW, RING, 4, 36, DMA>(a, s);
-                if (band_sum_then_scale_enabled()) return launch_band_inst<RL, NW, OPW, RING, 3, 36, DMA>(a, s);
+                if (a.add_only && a.twins) return launch_band_inst<RL, NW, OPW, RING, 4, 36, DMA>(a, s);
+                if (a.add_only) return launch_band_inst<RL, NW, OPW, RING, 3, 36, DMA>(a, s);
                 return launch_band_inst<RL, NW, OPW, RING, 0, 36, DMA>(a, s);
             case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 36, DMA>(a, s);
             default: return launch_band_inst<RL, NW, OPW, RING, 2, 36, DMA>(a, s);
@@ -1751,7 +1741,7 @@ hipError_t launch_band_rl(const BandLaunch& a, hipStream_t s) {
     }
     switch (a.wmode) {
         case 0:
-            if (band_sum_then_scale_enabled()) return launch_band_inst<RL, NW, OPW, RING, 3, 0, DMA>(a, s);
+            if (a.add_only) return launch_band_inst<RL, NW, OPW, RING, 3, 0, DMA>(a, s);
             return launch_band_inst<RL, NW, OPW, RING, 0, 0, DMA>(a, s);
         case 1: return launch_band_inst<RL, NW, OPW, RING, 1, 0, DMA>(a, s);
         default: return launch_band_inst<RL, NW, OPW, RING, 2, 0, DMA>(a, s);
@@ -1858,7 +1848,7 @@ hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
 }
 template <int RL, int NW, int OPW, int RING>
 hipError_t launch_chain_rl(const ChainLaunch& a, hipStream_t s) {
-    const bool add_only = a.wmode == 0 && band_sum_then_scale_enabled();   // as in the per-layer walk
+    const bool add_only = a.wmode == 0 && a.add_only;   // as in the per-layer walk
     if (a.unrolled) {
         if (add_only) return launch_chain_inst<RL, NW, OPW, RING, 3, 36>(a, s);
         switch (a.wmode) {
@@ -1893,7 +1883,7 @@ hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
                            a.active, a.count_out, a.count_prev, a.N, a.stamp0, a.prev_stamp, a.check_dead, a.bias,   \
                            a.clampv, a.publish);                                                                     \
     } while (0)
-        const bool add_only = a.wmode == 0 && band_sum_then_scale_enabled();
+        const bool add_only = a.wmode == 0 && a.add_only;
         if (a.unrolled) {
             if (add_only) SPDNN_HALF(3, 36); else if (a.wmode == 0) SPDNN_HALF(0, 36); else if (a.wmode == 1) SPDNN_HALF(1, 36); else SPDNN_HALF(2, 36);
         } else {
@@ -1954,7 +1944,7 @@ hipError_t launch_band_pair(const PairLaunch& a, hipStream_t s) {
                            a.bias, a.clampv, a.publish, a.nblk, stream);                                            \
     } while (0)
     switch (a.wmode) {
-        case 0: if (band_sum_then_scale_enabled()) SPDNN_PAIR(3); else SPDNN_PAIR(0); break;
+        case 0: if (a.add_only) SPDNN_PAIR(3); else SPDNN_PAIR(0); break;
         case 1: SPDNN_PAIR(1); break;
         default: SPDNN_PAIR(2); break;
     }

@@ -51,6 +51,7 @@ struct BandLaunch {
     int prev_stamp = 0;      // stamp of the previous layer if the row slots still carry it (0 = none)
     int check_dead = 0;      // 1: row blocks the previous layer left without an active row are skipped
     int wmode;               // 0 uniform exact value, 1 per-entry fma (exact products), 2 mul then add
+    int add_only = 1;        // wmode 0: add the inputs and scale the sum once (0: a multiply-add per input)
     int twins = 0;           // 1 (wmode 0): the two outputs of every pair use the same inputs (groups of identical rows,
                              // as in a run chain), so they are equal: one accumulator per pair, stored twice
     float wu, bias, clampv;
@@ -148,6 +149,7 @@ struct ChainLaunch {
     int unrolled;                 // every layer of the chain has 32 entries per output (band_unrolled)
     int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
     int halves;                   // 1 (256-row blocks only): one workgroup per HALF row block (twice the workgroups)
+    int add_only = 1;             // as in BandLaunch
     float bias, clampv;
     Publish publish;
 };
@@ -170,6 +172,7 @@ struct PairLaunch {
     int32_t* active_mid;
     int32_t* count_prev;     // as in BandLaunch, for the layer before the pair
     int N, nblk, rl, wmode;
+    int add_only = 1;             // as in BandLaunch
     int halo_a, steps_a, halo_b, steps_b;
     int stamp_a, stamp_b, prev_stamp, check_dead;
     int seglen;              // band positions of the second layer per workgroup, 0 = heuristic

@@ -254,6 +254,8 @@ struct spdnn_net {
     bool blocks_skipped = false;
     int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
     int chain_halves = 1;     // fused chains on half row blocks (SPDNN_CHAIN_HALVES=0: whole row blocks)
+    int add_only = 1;         // band layers with one power-of-two weight add their inputs and scale the sum once
+                              // (SPDNN_BAND_SUM_THEN_SCALE=0: a multiply-add per input)
     bool fuse_pairs = true;   // fused pairs where the inspector found them (SPDNN_FUSE_PAIRS=0: never)
     int pair_seglen = 0;      // band positions per workgroup of a fused pair, 0 = heuristic (SPDNN_PAIR_SEGLEN)
     // rows x neurons below which a pair runs as two launches (SPDNN_PAIR_MIN_ELEMS).  Measured, layers over one
@@ -806,6 +808,7 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
     if (const char* e = getenv("SPDNN_FUSE_PAIRS")) n->fuse_pairs = atoi(e) != 0;
     if (const char* e = getenv("SPDNN_CHAIN_HALVES")) n->chain_halves = atoi(e) != 0 ? 1 : 0;
+    if (const char* e = getenv("SPDNN_BAND_SUM_THEN_SCALE")) n->add_only = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
@@ -1248,7 +1251,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out
     const DevLayer& d = n->dl[(size_t)l];
     BandLaunch a{};
     a.yin = in; a.yout = out; a.pairs = d.pairs; a.pw = d.wv; a.dst = d.dst; a.active = n->d_active;
-    a.steps = p.pair_steps; a.stride = p.pair_stride; a.twins = p.pair_twins ? 1 : 0;
+    a.steps = p.pair_steps; a.stride = p.pair_stride; a.twins = p.pair_twins ? 1 : 0; a.add_only = n->add_only;
     a.N = n->N; a.K = p.kmax; a.nblk = nblk; a.stamp = stamp; a.rl = n->rl; a.wmode = p.wmode;
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
@@ -1577,7 +1580,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
             PairLaunch pl{};
             pl.yin = in; pl.yout = out; pl.pairs_a = da.pairs; pl.pw_a = da.wv; pl.pairs_b = db.pairs; pl.pw_b = db.wv;
             pl.dst = db.dst; pl.active = n->d_active; pl.active_mid = n->d_active_mid; pl.count_prev = count_prev;
-            pl.N = n->N; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = p.wmode;
+            pl.N = n->N; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = p.wmode; pl.add_only = n->add_only;
             pl.halo_a = p.info.band_halo; pl.steps_a = p.pair_steps; pl.halo_b = q.info.band_halo; pl.steps_b = q.pair_steps;
             pl.stamp_a = stamp0; pl.stamp_b = stamp0 + 1; pl.prev_stamp = prev_stamp; pl.check_dead = check_dead;
             pl.seglen = n->pair_seglen; pl.n_cu = n->n_cu; pl.stream_min_bytes = n->stream_min_bytes;
@@ -1596,6 +1599,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
             ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
             ch.bias = n->bias; ch.clampv = n->clampv;
             ch.halves = n->chain_halves;
+            ch.add_only = n->add_only;
             ch.publish = pub;
             HIPCHK(launch_band_chain(ch, n->stream));
             for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote

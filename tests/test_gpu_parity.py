@@ -135,19 +135,22 @@ def test_gather_kernel_random_sparsity(gc, orc, values, tiled, monkeypatch):
         _layer_by_layer(gc, orc, net, [sort_rows(c) for c in layers], feats, prune=True)
 
 
-@pytest.mark.parametrize("values", ["pow2", "general"])
+@pytest.mark.parametrize("values", ["pow2", "general", "uniform", "uniform-fma"])
 @pytest.mark.parametrize("K", [32, 16, 8])
-def test_band_kernel_weight_modes(gc, orc, values, K):
-    """Band structure with per-entry weights: exact products (fma) and general (mul then add)."""
+def test_band_kernel_weight_modes(gc, orc, values, K, monkeypatch):
+    """Band structure with per-entry weights: exact products (fma) and general (mul then add); with one
+    power-of-two weight: inputs added and the sum scaled once, or (switched back) a multiply-add per input."""
     N, L, B = 1024, 3, 260
     print("band weights=%s K=%d" % (values, K), flush=True)
+    if values == "uniform-fma":
+        monkeypatch.setenv("SPDNN_BAND_SUM_THEN_SCALE", "0")
     rng = np.random.default_rng(K)
     layers = []
     for l in range(L):
         rowptr, col, val = orc.gen_layer_csr(21, l, N, K, 0.0625)
         if values == "pow2":
             val = (np.ldexp(1.0, rng.integers(-5, -1, size=len(val))) * rng.choice([-1.0, 1.0], size=len(val))).astype(np.float32)
-        else:
+        elif values == "general":
             val = rng.uniform(-0.1, 0.2, size=len(val)).astype(np.float32)
         layers.append((rowptr, col, val))
     feats = rng.uniform(0, 2, size=(B, N)).astype(np.float32)
@@ -160,16 +163,18 @@ def test_band_kernel_weight_modes(gc, orc, values, K):
         _layer_by_layer(gc, orc, net, layers, feats, prune=True)
 
 
+@pytest.mark.parametrize("add_only", [1, 0])
 @pytest.mark.parametrize("structure", ["circulant", "run-chains"])
 @pytest.mark.parametrize("w", [0.0625, -0.5, 2.0 ** -24, 2.0 ** 21, 0.0])
-def test_one_power_of_two_weight_sums_then_scales(gc, orc, w, structure, monkeypatch):
+def test_one_power_of_two_weight_sums_then_scales(gc, orc, w, structure, add_only, monkeypatch):
     """A layer whose entries all carry the same weight +-2^e is walked by adding the inputs and scaling the
     sum once.  That equals the reference's multiply-then-add chain bit for bit only because scaling by a
     power of two commutes with rounding: features of both signs over the whole accepted range (2^-100 ..
     2^100, with cancellations down to the last bit), the smallest and largest accepted weights."""
     from helpers import radix_like_csr
     N, L, B = 1024, 3, 300
-    print("sum then scale w=%g %s" % (w, structure), flush=True)
+    print("sum then scale w=%g %s add_only=%d" % (w, structure, add_only), flush=True)
+    monkeypatch.setenv("SPDNN_BAND_SUM_THEN_SCALE", str(add_only))   # 0: the same layers with a multiply-add per input
     rng = np.random.default_rng(3)
     if structure == "run-chains":
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
