@@ -137,8 +137,9 @@ template <> __device__ __forceinline__ void add_pair_if_used<1>(float* acc0, flo
         : "scc");
 }
 // LDS address of a lane's part of ring column `slot byte b of dword`: one scalar bit-field extract and
-// one vector shift-add (written out: the compiler's own choice is shift + mask on the scalar unit, and the
-// scalar unit, one per CU, is what the add-only walk has least of).
+// one vector shift-add (written out: the compiler's own choice is a shift and a mask on the scalar unit, and
+// scalar instructions are what the add-only walk can least afford: measured, each costs a SIMD as much
+// issue time as a multiply-add).
 template <int SLOT_BITS, int COL_SHIFT>
 __device__ __forceinline__ uint32_t ring_address(uint32_t lane_base, uint32_t dword, int b) {
     uint32_t slot, addr;
