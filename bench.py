@@ -326,7 +326,7 @@ def main():
                         % (args.config, N, L, "" if args.structure == "circulant" else " (%s)" % args.structure, B, bias,
                            "32 nnz/row of 0.0625" if args.structure != "irregular" else "1..24 nnz/row, random weights", seed),
             "neuron": N, "layers": L, "batch": B, "bias": bias, "seed": seed,
-            "kernel": "band_walk (rows per lane 4, LDS ring)" if n_band == L else "+".join(kernels_used),
+            "kernel": "band_walk (rows per lane 4, LDS ring, one v_add_f32 per input under one power-of-two weight)" if n_band == L else "+".join(kernels_used),
             "band_tuning_rowblocks_shape_seglen": net.band_tuning(),
             "feature_buffers_region_paired_candidates": list(net.feature_placement()),
             "plan_window_device_bytes_pinned_bytes": list(net.plan_memory()),
