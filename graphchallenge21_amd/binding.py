@@ -30,13 +30,15 @@ class LayerPlan(C.Structure):
 class RunOptions(C.Structure):
     _fields_ = [("prune", C.c_int32), ("first_layer", C.c_int32), ("n_layers", C.c_int32),
                 ("collect_counts", C.c_int32), ("time_layers", C.c_int32),
-                ("compact_threshold", C.c_float), ("fuse_layers", C.c_int32), ("reserved", C.c_int32 * 3)]
+                ("compact_threshold", C.c_float), ("fuse_layers", C.c_int32), ("persist_wait_us", C.c_int32),
+                ("reserved", C.c_int32 * 2)]
 
 
 class RunResult(C.Structure):
     _fields_ = [("layers_run", C.c_int32), ("compactions", C.c_int32), ("active_rows", C.c_int64),
                 ("carried_rows", C.c_int64), ("ms_total", C.c_float), ("ms_kernels", C.c_float),
-                ("alg_bytes", C.c_double), ("edges", C.c_double), ("launches", C.c_int32), ("fused_pairs", C.c_int32)]
+                ("alg_bytes", C.c_double), ("edges", C.c_double), ("launches", C.c_int32), ("fused_pairs", C.c_int32),
+                ("persistent_launches", C.c_int32), ("persistent_fallbacks", C.c_int32)]
 
 
 def lib_path():
@@ -101,7 +103,8 @@ def load_library():
         "spdnn_measure_copy_bandwidth": ([C.c_int64, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_measure_buffer_copy_bandwidth": ([vp, C.c_int, C.POINTER(C.c_double)], C.c_int),
         "spdnn_device_info": ([C.c_char_p, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
-        "spdnn_get_feature_placement": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
+        "spdnn_get_feature_placement": ([vp, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int64)], C.c_int),
+        "spdnn_device_alloc_calls": ([C.POINTER(C.c_int64)], C.c_int),
         "spdnn_device_memory": ([C.POINTER(C.c_int64), C.POINTER(C.c_int64)], C.c_int),
         "spdnn_device_synchronize": ([], C.c_int),
     }
@@ -169,6 +172,13 @@ def device_info():
     cu, mem = C.c_int(), C.c_int64()
     _check(load_library().spdnn_device_info(name, 256, C.byref(cu), C.byref(mem)))
     return name.value.decode(), cu.value, mem.value
+
+
+def device_alloc_calls():
+    """Device allocations the library has made in this process so far."""
+    c = C.c_int64()
+    _check(load_library().spdnn_device_alloc_calls(C.byref(c)))
+    return c.value
 
 
 def device_memory():
@@ -269,10 +279,11 @@ class Network:
         return res[:cnt.value].copy()
 
     def feature_placement(self):
-        """(paired, candidates): whether the buffer halves lie in different memory regions."""
-        paired, cand = C.c_int(), C.c_int()
-        _check(self._lib.spdnn_get_feature_placement(self._h, C.byref(paired), C.byref(cand)))
-        return bool(paired.value), cand.value
+        """(paired, candidates, search_peak_bytes): whether the buffer halves lie in different memory regions,
+        how many half-buffers the search allocated and how much device memory it held at its peak."""
+        paired, cand, peak = C.c_int(), C.c_int(), C.c_int64()
+        _check(self._lib.spdnn_get_feature_placement(self._h, C.byref(paired), C.byref(cand), C.byref(peak)))
+        return bool(paired.value), cand.value, peak.value
 
     def set_plan_window(self, slots):
         """0 = every plan resident; 2..64 = that many device slots, plans streamed from pinned memory."""
@@ -322,13 +333,14 @@ class Network:
 
     # inference
     def run(self, prune=True, first_layer=0, n_layers=-1, collect_counts=False, time_layers=False,
-            compact_threshold=0.75, fuse_layers=0):
+            compact_threshold=0.75, fuse_layers=0, persist_wait_us=0):
         opt = RunOptions()
         _check(self._lib.spdnn_default_run_options(C.byref(opt)))
         opt.prune, opt.first_layer, opt.n_layers = int(prune), first_layer, n_layers
         opt.collect_counts, opt.time_layers = int(collect_counts), int(time_layers)
         opt.compact_threshold = compact_threshold
         opt.fuse_layers = fuse_layers
+        opt.persist_wait_us = persist_wait_us
         res = RunResult()
         _check(self._lib.spdnn_run(self._h, C.byref(opt), C.byref(res)))
         return res

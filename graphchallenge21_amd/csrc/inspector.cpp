@@ -537,6 +537,25 @@ bool build_tiled_plan(int N, const std::vector<int32_t>& rowptr, const std::vect
     return true;
 }
 
+// Longest merged step list over the pairs of neighbouring band positions (2u, 2u+1): the two outputs
+// add their inputs in ascending input index, a shared input is one step.
+static int merged_pair_steps(int N, int K, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                             const std::vector<int32_t>& out_at) {
+    int steps = K;
+    for (int u = 0; u < N / 2; ++u) {
+        const int j0 = out_at[(size_t)2 * u], j1 = out_at[(size_t)2 * u + 1];
+        int a = rowptr[j0], b = rowptr[j1], m = 0;
+        while (a < rowptr[j0 + 1] || b < rowptr[j1 + 1]) {
+            const int ia = a < rowptr[j0 + 1] ? col[a] : INT32_MAX, ib = b < rowptr[j1 + 1] ? col[b] : INT32_MAX;
+            if (ia <= ib) ++a;
+            if (ib <= ia) ++b;
+            ++m;
+        }
+        steps = std::max(steps, m);
+    }
+    return steps;
+}
+
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan) {
     const int64_t nnz = rowptr[N];
@@ -595,6 +614,17 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         band = true;    // 16-output groups chained through shared 16-input runs: walked like a band
         block = false;
         halo = 32;
+    }
+
+    if (band) {
+        // A circulant pair merges to K + 1 steps, a pair inside a group of a run chain to 32; the kernel reads
+        // fixed records of at most 36 steps.  A labelling whose pairs merge to more is not walked as a band:
+        // the layer keeps its groups (BLOCK) if it has them, else it goes to the general classes.
+        if (merged_pair_steps(N, K, rowptr, col, plan.out_at) > 36) {
+            band = false;
+            block = halo == 32;
+            halo = K - 1;
+        }
     }
 
     plan.ngroups = 0;
@@ -666,21 +696,9 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         // once; per step a ring selector, a use bit per output and (unless the layer has one exact
         // value) a weight per output, 0 where the output does not use the step.
         const int npairs = N / 2;
-        int steps = K;
-        for (int u = 0; u < npairs; ++u) {
-            const int j0 = plan.out_at[2 * u], j1 = plan.out_at[2 * u + 1];
-            int a = rowptr[j0], b = rowptr[j1], m = 0;
-            while (a < rowptr[j0 + 1] || b < rowptr[j1 + 1]) {
-                const int ia = a < rowptr[j0 + 1] ? col[a] : INT32_MAX, ib = b < rowptr[j1 + 1] ? col[b] : INT32_MAX;
-                if (ia <= ib) ++a;
-                if (ib <= ia) ++b;
-                ++m;
-            }
-            steps = std::max(steps, m);
-        }
-        // A circulant pair merges to K + 1 steps, a pair inside a group of a run chain to 32: the kernel
-        // reads fixed 16-dword records (two use masks, 36 one-byte selectors) and 72 weights per pair.
-        if (steps > 36) throw std::logic_error("band pair with more than 36 merged steps");
+        // (at most 36, checked above: the kernel reads fixed 16-dword records - two use masks, 36 one-byte
+        // selectors - and 72 weights per pair)
+        const int steps = merged_pair_steps(N, K, rowptr, col, plan.out_at);
         const int trips = 9;
         const int stride = 16;
         plan.pair_steps = steps;

@@ -19,7 +19,9 @@ constexpr int kPanelCols = 512;     // TILED: input columns staged in LDS at a t
 
 struct LayerPlan {
     bool set = false;
-    bool failed = false;            // the inspection job ended in an exception (out of host memory)
+    bool failed = false;            // the inspection job ended in an exception
+    bool failed_nomem = false;      // ... which was a failed host allocation
+    std::string fail_text;          // ... what the exception said
     spdnn_layer_plan info{};
     int kernel = SPDNN_KERNEL_GATHER;
     int wmode = 2;                  // 0 uniform exact value, 1 exact products, 2 multiply then add

@@ -339,7 +339,8 @@ __device__ __forceinline__ bool enter_row_block(const int32_t* active, size_t ro
     }
     if (counts && (threadIdx.x & 63) == 0 && alive > 0) atomicAdd(count_prev, alive);
     if (!check_dead) return false;
-    return __syncthreads_or(alive) == 0;
+    // (the result is the same for every thread; said explicitly, the branch on it is a scalar one)
+    return __builtin_amdgcn_readfirstlane(__syncthreads_or(alive)) == 0;
 }
 
 
@@ -716,11 +717,14 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     Feat yin_all, Feat yout_all, const uint32_t* __restrict__ pairs,
     const float* __restrict__ pw, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
     int32_t* __restrict__ count_prev, int N, int steps, int halo, int seglen, int stamp, int prev_stamp,
-    int check_dead, float wu, float bias, float clampv, Publish pub, int nblk, int stream) {
+    int check_dead, float wu, float bias, float clampv, Publish pub, int nblk, int stream,
+    const int32_t* __restrict__ frontier, int frontier_layer) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int RB = 64 * RL;
     publish_counts(pub);
     if ((int)blockIdx.x >= nblk) return;  // padding of the grid's x extent (see the launcher)
+    // finishing a persistent launch that gave up: this row block has the layer behind it already
+    if (frontier != nullptr && frontier[blockIdx.x] > frontier_layer) return;
     // row blocks vary fastest (measured: launching the segments of one row block together
     // instead is slower on live data and reads more from HBM)
     const int rb = blockIdx.x;
@@ -736,109 +740,6 @@ __global__ __launch_bounds__(NW * 64) void band_walk_kernel(
     band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(block_base(yin_all, rb, blkf), block_base(yout_all, rb, blkf), pairs,
                                                  pw, dst, N, steps, halo, vb, ve, wu, bias, clampv, smem, nz, stream);
     stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp, nullptr);
-}
-
-// ------------------------------------------------------------------------------------------
-// Fused layer chain ("fused" variant): one workgroup keeps one row block and runs `nlayers`
-// consecutive BAND layers back to back in a single launch - whole band per layer, ping-pong
-// between the two work buffers.  The intermediate activations of a row block are private to the
-// workgroup (written and re-read by the same CU through L2), there is no launch, tail or global
-// barrier between layers, and a workgroup whose rows have all died stops: the rest of its chain
-// is all zero by definition.  Layers of one chain share K and the weight mode.
-// ------------------------------------------------------------------------------------------
-struct ChainLayer {
-    const uint32_t* pairs;
-    const float* pw;
-    const int32_t* dst;
-    float wu;
-    int halo;
-    int steps;
-};
-
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT, int DMA>
-__global__ __launch_bounds__(NW * 64) void band_chain_kernel(
-    const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int32_t* __restrict__ count_prev, int N,
-    int stamp0, int prev_stamp, int check_dead, int stop_when_dead, float bias, float clampv, Publish pub) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int RB = 64 * RL;
-    publish_counts(pub);
-    const int rb = blockIdx.x;
-    const size_t blkf = (size_t)N * RB;
-    if (enter_row_block<RL>(active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp0, check_dead, count_prev,
-                            threadIdx.x < 64))
-        return;
-    float* const block_a = block_base(buf_a, rb, blkf);
-    float* const block_c = block_base(buf_c, rb, blkf);
-    const float* in = block_base(first_in, rb, blkf);
-    for (int j = 0; j < nlayers; ++j) {
-        float* out = (in == block_a) ? block_c : block_a;
-        const ChainLayer lay = table[j];
-        float nz[RL];
-#pragma unroll
-        for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-        band_walk_body<RL, NW, OPW, RING, WMODE, KT, DMA>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps,
-                                                     lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
-        stamp_rows_workgroup<RL, NW>(nz, smem, active, (size_t)rb * RB, stamp0 + j,
-                                     count_out ? count_out + j : nullptr);
-        int any = 0;
-#pragma unroll
-        for (int q = 0; q < RL; ++q) any |= (nz[q] > 0.0f) ? 1 : 0;
-        // The barrier (with its workgroup-scope fence) makes this layer's columns visible to the
-        // other waves of the workgroup - same CU, same L1 - before the next layer reads them.  A
-        // device-scope fence here would write back and invalidate the whole L2 of the XCD.
-        const int alive = __syncthreads_or(any);
-        if (!alive && stop_when_dead) return;
-        in = out;
-    }
-}
-
-// The fused chain on HALF row blocks of the 256-row layout: a workgroup keeps 128 rows (two per
-// lane) through the chain, so that a batch gives twice as many workgroups - two per CU at the
-// challenge's batch of 60000, whose load / compute / barrier phases interleave - at half the LDS
-// each.  A half whose rows have all died keeps computing (zeros) as long as the other half of its
-// row block may be alive: the kernels of the other classes skip or run whole row blocks and expect
-// the dead rows of a live block to hold zeros.
-template <int WMODE, int KT>
-__global__ __launch_bounds__(512) void band_chain_half_kernel(
-    const ChainLayer* __restrict__ table, int nlayers, Feat first_in, Feat buf_a, Feat buf_c,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_out, int32_t* __restrict__ count_prev, int N,
-    int stamp0, int prev_stamp, int check_dead, float bias, float clampv, Publish pub) {
-    extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int RBL = 256, RBH = 128;
-    publish_counts(pub);
-    const int rb = blockIdx.x >> 1, half = blockIdx.x & 1;
-    const int lane = threadIdx.x & 63;
-    const size_t blkf = (size_t)N * RBL;
-    const size_t row0 = (size_t)rb * RBL + half * RBH;
-    if (prev_stamp != 0 && (check_dead || count_prev != nullptr)) {
-        int alive_block = 0, alive_own = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // stamps only grow: the other half's workgroup may be layers ahead already
-            const int a = active[(size_t)rb * RBL + i * 64 + lane];
-            const int c = (int)__popcll(__ballot(a >= prev_stamp ? 1 : 0));
-            alive_block += c;
-            if ((i >> 1) == half) alive_own += c;
-        }
-        if (count_prev != nullptr && threadIdx.x == 0 && alive_own > 0) atomicAdd(count_prev, alive_own);
-        if (check_dead && alive_block == 0) return;   // every wave reads the same stamps
-    }
-    float* const block_a = block_base(buf_a, rb, blkf) + half * RBH;
-    float* const block_c = block_base(buf_c, rb, blkf) + half * RBH;
-    const float* in = block_base(first_in, rb, blkf) + half * RBH;
-    for (int j = 0; j < nlayers; ++j) {
-        float* out = (in == block_a) ? block_c : block_a;
-        const ChainLayer lay = table[j];
-        float nz[2] = {0.0f, 0.0f};
-        band_walk_body<2, 8, 2, 64, WMODE, KT, 0, RBL>(in, out, lay.pairs, lay.pw, lay.dst, N, lay.steps,
-                                                       lay.halo, 0, N, lay.wu, bias, clampv, smem, nz, 0);
-        stamp_rows_workgroup<2, 8>(nz, smem, active, row0, stamp0 + j, count_out ? count_out + j : nullptr);
-        // the barrier (workgroup-scope fence) makes this layer's columns visible to the other waves
-        // of the workgroup before the next layer reads them
-        __syncthreads();
-        in = out;
-    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1193,7 +1094,7 @@ __device__ __forceinline__ uint32_t row_lane(uint32_t v, int j) {
     return v;
 }
 
-template <int WMODE, int ROWBCAST>
+template <int WMODE>
 __global__ __launch_bounds__(1024) void tiled_kernel(
     Feat yin_all, Feat yout_all, const int32_t* __restrict__ cols, const int32_t* __restrict__ hdr,
     const uint32_t* __restrict__ ent, const int32_t* __restrict__ dst, int32_t* __restrict__ active,
@@ -1257,7 +1158,7 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
         }
         wait_vector_memory();
         ring_barrier<1>();
-        if (ROWBCAST) {
+        {
             // A round's entry block, [output][2](LDS offset of the column, weight), goes into registers with four
             // reads: lane j of each of the wave's four 16-lane rows takes the 16 bytes of output 16 g + j, g = 0 .. 3
             // (the rows read the same addresses).  An entry's offset and weight then come to all lanes of a row
@@ -1309,48 +1210,6 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
                     for (int g = 0; g < 4; ++g) lds_read<4>(ent_base + g * 256, mg[g]);
                 }
             }
-        } else
-        for (int r = 0; r < rounds; ++r) {
-            if (r + 1 < rounds) block_to_lds_untracked(blk + (size_t)(r + 1) * 256 + lane * 4, ring + ((r + 1) & 1) * 1024);
-            const unsigned char* cur = ring + (r & 1) * 1024;
-            // 32 units of 2 outputs, software-pipelined three deep: while unit u does its arithmetic, the
-            // columns of unit u+1 and the entries of unit u+2 are on their way from LDS
-            float4 m[3][2];
-            float x[2][2][2];
-#pragma unroll
-            for (int o = 0; o < 2; ++o) {
-                m[0][o] = *reinterpret_cast<const float4*>(cur + o * 16);
-                m[1][o] = *reinterpret_cast<const float4*>(cur + (2 + o) * 16);
-            }
-#pragma unroll
-            for (int o = 0; o < 2; ++o) {
-                x[0][o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[0][o].x));
-                x[0][o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[0][o].z));
-            }
-#pragma unroll
-            for (int u = 0; u < 32; ++u) {
-                if (u + 2 < 32) {
-#pragma unroll
-                    for (int o = 0; o < 2; ++o)
-                        m[(u + 2) % 3][o] = *reinterpret_cast<const float4*>(cur + ((u + 2) * 2 + o) * 16);
-                }
-                __builtin_amdgcn_sched_barrier(0);   // the three stages stay in this order
-                if (u + 1 < 32) {
-#pragma unroll
-                    for (int o = 0; o < 2; ++o) {
-                        x[(u + 1) & 1][o][0] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[(u + 1) % 3][o].x));
-                        x[(u + 1) & 1][o][1] = *reinterpret_cast<const float*>(lane_panel + __float_as_uint(m[(u + 1) % 3][o].z));
-                    }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int o = 0; o < 2; ++o) {
-                    acc[u * 2 + o] = mac<WMODE>(acc[u * 2 + o], x[u & 1][o][0], m[u % 3][o].y);
-                    acc[u * 2 + o] = mac<WMODE>(acc[u * 2 + o], x[u & 1][o][1], m[u % 3][o].w);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            wait_vector_memory();   // the next entry block has arrived (nothing else is in flight)
         }
         ring_barrier<1>();          // every wave is done with the panel
     }
@@ -1383,31 +1242,14 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
 // operands only, one multiply-add per VALU instruction.  The accumulation order (ascending input
 // index) is the same for every output of a group, so the code is fully unrolled.
 // ------------------------------------------------------------------------------------------
+// groups [g0, g1) of one row block for one wave; nz collects the rows' largest outputs
 template <int RL, int WMODE, bool FULL>
-__global__ __launch_bounds__(256) void block_kernel(
-    Feat yin_all, Feat yout_all, const int32_t* __restrict__ grp_cols,
-    const int32_t* __restrict__ grp_cnt, const float* __restrict__ wv, const int32_t* __restrict__ dst,
-    int32_t* __restrict__ active, int32_t* __restrict__ count_prev, int N, int ngroups, int gpw, int stamp,
-    int prev_stamp, int check_dead, float wu, float bias, float clampv, Publish pub) {
+__device__ __forceinline__ void block_body(const float* __restrict__ yin, float* __restrict__ yout,
+                                           const int32_t* __restrict__ grp_cols, const int32_t* __restrict__ grp_cnt,
+                                           const float* __restrict__ wv, const int32_t* __restrict__ dst, int g0, int g1,
+                                           int loff, float wu, float bias, float clampv, float* nz) {
     using V = typename VecOf<RL>::type;
     constexpr int RB = 64 * RL;
-    publish_counts(pub);
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    const int rb = blockIdx.x;
-    if (enter_row_block<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp, check_dead, count_prev,
-                            blockIdx.y == 0 && wave == 0))
-        return;
-    const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
-    float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
-    const int loff = lane * RL;
-    const int g0 = (blockIdx.y * 4 + wave) * gpw;
-    const int g1 = min(ngroups, g0 + gpw);
-
-    float nz[RL];
-#pragma unroll
-    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
-
     for (int g = g0; g < g1; ++g) {
         const int S = FULL ? 32 : grp_cnt[g];
         const int32_t* cp = grp_cols + (size_t)g * 32;
@@ -1446,7 +1288,259 @@ __global__ __launch_bounds__(256) void block_kernel(
             *reinterpret_cast<V*>(yout + (size_t)d * RB + loff) = arr_to_vec<RL>(y);
         }
     }
+}
+
+template <int RL, int WMODE, bool FULL>
+__global__ __launch_bounds__(256) void block_kernel(
+    Feat yin_all, Feat yout_all, const int32_t* __restrict__ grp_cols,
+    const int32_t* __restrict__ grp_cnt, const float* __restrict__ wv, const int32_t* __restrict__ dst,
+    int32_t* __restrict__ active, int32_t* __restrict__ count_prev, int N, int ngroups, int gpw, int stamp,
+    int prev_stamp, int check_dead, float wu, float bias, float clampv, Publish pub,
+    const int32_t* __restrict__ frontier, int frontier_layer) {
+    constexpr int RB = 64 * RL;
+    publish_counts(pub);
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int rb = blockIdx.x;
+    // finishing a persistent launch that gave up: this row block has the layer behind it already
+    if (frontier != nullptr && frontier[rb] > frontier_layer) return;
+    if (enter_row_block<RL>(active, (size_t)rb * RB + lane * RL, prev_stamp, stamp, check_dead, count_prev,
+                            blockIdx.y == 0 && wave == 0))
+        return;
+    const float* __restrict__ yin = block_base(yin_all, rb, (size_t)N * RB);
+    float* __restrict__ yout = block_base(yout_all, rb, (size_t)N * RB);
+    const int loff = lane * RL;
+    const int g0 = (blockIdx.y * 4 + wave) * gpw;
+    const int g1 = min(ngroups, g0 + gpw);
+    float nz[RL];
+#pragma unroll
+    for (int q = 0; q < RL; ++q) nz[q] = 0.0f;
+    block_body<RL, WMODE, FULL>(yin, yout, grp_cols, grp_cnt, wv, dst, g0, g1, loff, wu, bias, clampv, nz);
     stamp_rows<RL>(nz, active, (size_t)rb * RB + loff, stamp);
+}
+
+// ------------------------------------------------------------------------------------------
+// Persistent launches: several layers of one kind per launch, a dependency per row block between
+// the layers (see PersistLaunch).  The reference's loop synchronises the whole device and the
+// host once per layer (src/microbenchmark/all_network.cu:333-519, the wait at :453).
+// ------------------------------------------------------------------------------------------
+struct PersistArgs {
+    const LayerDesc* table;
+    int nlayers;
+    Feat first_in, buf_a, buf_c;
+    int32_t* active;
+    int32_t* done;
+    int done_stride;
+    PersistCtl* ctl;
+    const PersistCtl* prev_ctl;
+    int prev_units;
+    int32_t* abort;
+    int32_t* host_word;
+    int N, nblk, nseg, seglen, total_units, nq, light;
+    int stamp0, prev_stamp, check_dead;
+    long long wait_limit;
+    float bias, clampv;
+    int stream;
+    Publish pub;
+};
+
+// number of the XCD (accelerator die) this wave runs on, from the hardware
+__device__ __forceinline__ int xcc_id() {
+    uint32_t x;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+    return (int)(x & 7u);
+}
+__device__ __forceinline__ int load_agent(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+// the launch gives up: every workgroup leaves at its next look at `abort`, the host sees -2
+__device__ __forceinline__ void persist_give_up(const PersistArgs& a) {
+    __hip_atomic_store(a.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(a.host_word, -2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+// Start of a persistent kernel: a launch does not start on the ruins of another (uniform result).
+__device__ __forceinline__ bool persist_may_start(const PersistArgs& a) {
+    int bad = 0;
+    if (threadIdx.x == 0) {
+        if (load_agent(a.abort) != 0) bad = 1;
+        else if (a.prev_ctl != nullptr && load_agent(&a.prev_ctl->units_done) != a.prev_units) {
+            persist_give_up(a);
+            bad = 1;
+        }
+    }
+    return __builtin_amdgcn_readfirstlane(__syncthreads_or(bad)) == 0;
+}
+
+// One thread waits until *cnt >= target; 0 = there, 1 = the launch has given up (here, after wait_limit
+// ticks of the 100 MHz clock, or elsewhere).  Then the data of the units waited for is made visible.
+__device__ __forceinline__ int persist_wait(const PersistArgs& a, const int32_t* cnt, int target) {
+    long long t0 = -1;
+    for (;;) {
+        if (load_agent(cnt) >= target) break;
+        if (load_agent(a.abort) != 0) return 1;
+        const long long now = (long long)wall_clock64();
+        if (t0 < 0) t0 = now;
+        if (now - t0 >= a.wait_limit) {
+            persist_give_up(a);
+            return 1;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
+    // the writers ran on other CUs: drop this CU's L1 (same XCD, same L2: light) or take everything that
+    // is visible at device scope
+    if (a.light) asm volatile("buffer_inv sc0" ::: "memory");
+    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return 0;
+}
+
+// End of a unit (every thread calls it after its last store): the unit's stores are made visible and
+// counted - the workgroup that finishes the launch's last unit tells the host - and the next unit is claimed,
+// all by ONE thread in ONE place: the unit loop has a single divergent region, right before the barrier at its
+// top.  (With the count at the bottom of the loop and the claim at its top, two regions of the same thread on
+// either side of the loop's back edge, the compiler let the other lanes of that wave run ahead into the next
+// iteration's barrier.)
+__device__ __forceinline__ void persist_signal_and_claim(const PersistArgs& a, int32_t* cnt, int q, int* sh_unit) {
+    wait_vector_memory();   // this wave's stores have arrived in L2
+    __syncthreads();        // (every thread has also read *sh_unit by now)
+    if (threadIdx.x == 0) {
+        if (!a.light) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");   // the XCD's L2 writes back what it holds ...
+            wait_vector_memory();   // ... and has done so before the count goes up (said explicitly: with no load or store
+                                    // of its own outstanding the compiler leaves the fence's wait out)
+        }
+        __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int fin = __hip_atomic_fetch_add(&a.ctl->units_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (fin == a.total_units - 1)
+            __hip_atomic_store(a.host_word, a.total_units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        *sh_unit = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// Entry j of the layer table through the constant address space: the table never changes while a kernel
+// runs, and read this way its words come by the scalar unit and stay in scalar registers - the band walk
+// hands them to the scalar unit as they are (pair records, selectors).
+__device__ __forceinline__ LayerDesc load_layer_desc(const LayerDesc* table, int j) {
+    constexpr int W = (int)(sizeof(LayerDesc) / 4);
+    static_assert(sizeof(LayerDesc) % 4 == 0, "layer table entries are whole dwords");
+    const __attribute__((address_space(4))) uint32_t* p = (const __attribute__((address_space(4))) uint32_t*)(table + j);
+    union { LayerDesc d; uint32_t w[W]; } u;
+#pragma unroll
+    for (int i = 0; i < W; ++i) u.w[i] = p[i];
+    return u.d;
+}
+
+// The unit loop.  body(rb, sg, lay, in, out, stamp, prev_stamp) runs one unit; the whole workgroup enters
+// it with the same arguments.
+template <int RL, class Body>
+__device__ __forceinline__ void persist_loop(const PersistArgs& a, Body body) {
+    __shared__ int sh_unit;
+    constexpr int RB = 64 * RL;
+    publish_counts(a.pub);
+    if (!persist_may_start(a)) return;
+    const int q = a.nq > 1 ? xcc_id() : 0;
+    const int nrb_q = a.nq > 1 ? (q < a.nblk ? (a.nblk - q + 7) / 8 : 0) : a.nblk;
+    const int per_layer = nrb_q * a.nseg;
+    const int total_q = per_layer * a.nlayers;
+    const size_t blkf = (size_t)a.N * RB;
+    // (pointer by pointer: a choice between whole structs would keep the kernel's arguments in scratch memory)
+    const bool in_a = a.first_in.half[0] == a.buf_a.half[0];   // the launch's first layer reads buffer A, so it writes C
+    float* const out0_h0 = in_a ? a.buf_c.half[0] : a.buf_a.half[0];
+    float* const out0_h1 = in_a ? a.buf_c.half[1] : a.buf_a.half[1];
+    float* const out1_h0 = in_a ? a.buf_a.half[0] : a.buf_c.half[0];
+    float* const out1_h1 = in_a ? a.buf_a.half[1] : a.buf_c.half[1];
+    if (threadIdx.x == 0) sh_unit = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (;;) {
+        __syncthreads();
+        const int u = __builtin_amdgcn_readfirstlane(sh_unit);
+        if (u >= total_q) break;
+        const int j = u / per_layer, rem = u - j * per_layer, ri = rem / a.nseg, sg = rem - ri * a.nseg;
+        const int rb = a.nq > 1 ? q + 8 * ri : ri;
+        int32_t* const cnt = a.done + (size_t)j * a.done_stride + rb;
+        int gone = 0;
+        if (j > 0 && threadIdx.x == 0) gone = persist_wait(a, cnt - a.done_stride, a.nseg);
+        if (__builtin_amdgcn_readfirstlane(__syncthreads_or(gone))) break;
+        const LayerDesc lay = load_layer_desc(a.table, j);
+        const int stamp = a.stamp0 + j;
+        const int prev_stamp = j > 0 ? stamp - 1 : a.prev_stamp;
+        const float* const in_h0 = j == 0 ? a.first_in.half[0] : ((j & 1) ? out0_h0 : out1_h0);
+        const float* const in_h1 = j == 0 ? a.first_in.half[1] : ((j & 1) ? out0_h1 : out1_h1);
+        float* const out_h0 = (j & 1) ? out1_h0 : out0_h0;
+        float* const out_h1 = (j & 1) ? out1_h1 : out0_h1;
+        const size_t boff = (size_t)(rb >> 1) * blkf;   // row block rb is block rb >> 1 of half rb & 1
+        body(rb, sg, lay, ((rb & 1) ? in_h1 : in_h0) + boff, ((rb & 1) ? out_h1 : out_h0) + boff, stamp, prev_stamp);
+        persist_signal_and_claim(a, cnt, q, &sh_unit);
+    }
+}
+
+template <int RL, int WMODE, int KT, int DMA>
+__global__ __launch_bounds__(512) void band_persist_kernel(PersistArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int RB = 64 * RL;
+    persist_loop<RL>(a, [&](int rb, int sg, const LayerDesc& lay, const float* yin, float* yout, int stamp, int prev_stamp) __attribute__((always_inline)) {
+        if (enter_row_block<RL>(a.active, (size_t)rb * RB + (threadIdx.x & 63) * RL, prev_stamp, stamp, a.check_dead,
+                                nullptr, false))
+            return;
+        const int vb = sg * a.seglen, ve = min(a.N, vb + a.seglen);
+        float nz[RL];
+#pragma unroll
+        for (int x = 0; x < RL; ++x) nz[x] = 0.0f;
+        band_walk_body<RL, 8, 2, 64, WMODE, KT, DMA>(yin, yout, lay.pairs, lay.pw, lay.dst, a.N, lay.steps, lay.halo, vb, ve,
+                                                     lay.wu, a.bias, a.clampv, smem, nz, a.stream);
+        stamp_rows_workgroup<RL, 8>(nz, smem, a.active, (size_t)rb * RB, stamp, nullptr);
+    });
+}
+
+// unit = 4 waves x seglen groups of one row block
+template <int RL, int WMODE, bool FULL>
+__global__ __launch_bounds__(256) void block_persist_kernel(PersistArgs a) {
+    constexpr int RB = 64 * RL;
+    persist_loop<RL>(a, [&](int rb, int sg, const LayerDesc& lay, const float* yin, float* yout, int stamp, int prev_stamp) __attribute__((always_inline)) {
+        const int lane = threadIdx.x & 63;
+        const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+        if (enter_row_block<RL>(a.active, (size_t)rb * RB + lane * RL, prev_stamp, stamp, a.check_dead, nullptr, false))
+            return;
+        const int g0 = (sg * 4 + wave) * a.seglen, g1 = min(lay.ngroups, g0 + a.seglen);
+        float nz[RL];
+#pragma unroll
+        for (int x = 0; x < RL; ++x) nz[x] = 0.0f;
+        block_body<RL, WMODE, FULL>(yin, yout, lay.blk_cols, lay.blk_cnt, lay.blk_wv, lay.blk_dst, g0, g1, lane * RL, lay.wu,
+                                    a.bias, a.clampv, nz);
+        stamp_rows<RL>(nz, a.active, (size_t)rb * RB + lane * RL, stamp);
+    });
+}
+
+// counts[i] = rows whose stamp is at least stamp_lo + i (see launch_count_stamp_range): one workgroup, a
+// histogram in LDS (per wave one atomic per distinct value), then sums from the top
+__global__ __launch_bounds__(1024) void count_stamp_range_kernel(const int32_t* __restrict__ stamps, int rows, int stamp_lo,
+                                                                 int n, int32_t* __restrict__ counts_dev,
+                                                                 int32_t* __restrict__ counts_host) {
+    extern __shared__ int hist[];
+    for (int i = threadIdx.x; i < n; i += 1024) hist[i] = 0;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    for (int r0 = 0; r0 < rows; r0 += 1024) {
+        const int r = r0 + (int)threadIdx.x;
+        int d = r < rows ? stamps[r] - stamp_lo : -1;
+        if (d >= n) d = n - 1;
+        unsigned long long todo = __ballot(d >= 0 ? 1 : 0);
+        while (todo) {
+            const int first = (int)__ffsll((long long)todo) - 1;
+            const int v = __shfl(d, first, 64);
+            const unsigned long long same = __ballot(d == v ? 1 : 0);
+            if (lane == first) atomicAdd(&hist[v], (int)__popcll(same));
+            todo &= ~same;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int i = n - 1; i >= 0; --i) { acc += hist[i]; hist[i] = acc; }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        if (counts_dev) counts_dev[i] = hist[i];
+        if (counts_host) __hip_atomic_store(counts_host + i, hist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -1724,7 +1818,7 @@ hipError_t launch_band_inst(const BandLaunch& a, hipStream_t s) {
     dim3 grid(gx, nseg), block(NW * 64);
     hipLaunchKernelGGL(kern, grid, block, lds, s, a.yin, a.yout, a.pairs, a.pw, a.dst, a.active, a.count_prev,
                        a.N, a.steps, a.halo, seglen, a.stamp, a.prev_stamp, a.check_dead, a.wu, a.bias, a.clampv, a.publish,
-                       a.nblk, stream);
+                       a.nblk, stream, a.frontier, a.frontier_layer);
     return hipGetLastError();
 }
 
@@ -1763,11 +1857,7 @@ bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36
 // Variants of the band walk the run-time selection chooses from (BandLaunch.shape): for 256-row
 // blocks 0 = next chunk's columns straight from HBM into the LDS ring, 1 = parked in registers and
 // written to the ring after the arithmetic (the only form for smaller row blocks).
-static bool band_direct_lds_enabled() {
-    static const bool on = !(getenv("SPDNN_BAND_DIRECT_LDS") && atoi(getenv("SPDNN_BAND_DIRECT_LDS")) == 0);
-    return on;
-}
-int band_shape_count(int rl) { return rl == 4 && band_direct_lds_enabled() ? 2 : 1; }
+int band_shape_count(int rl, int direct_lds) { return rl == 4 && direct_lds ? 2 : 1; }
 
 int band_chunk_outputs(int rl, int shape) {
     (void)rl; (void)shape;
@@ -1818,15 +1908,11 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     BandLaunch b = a;
     b.n_cu = (a.n_cu > 0 ? a.n_cu : 256) * band_workgroups_per_cu(a.rl, a.shape);
-    if (b.seglen <= 0) {
-        static const int env_seglen = getenv("SPDNN_BAND_SEGLEN") ? atoi(getenv("SPDNN_BAND_SEGLEN")) : 0;
-        b.seglen = env_seglen;  // tuning knob; rounded down to whole chunks, 0 = heuristic
-        if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);
-    }
+    if (b.seglen > 0) b.seglen -= b.seglen % band_chunk_outputs(a.rl, a.shape);  // whole chunks; 0 = heuristic
     switch (a.rl) {
         case 4:
-            return (band_direct_lds_enabled() && a.shape != 1) ? launch_band_rl<4, 8, 2, 64, 1>(b, s)
-                                                              : launch_band_rl<4, 8, 2, 64, 0>(b, s);
+            return (a.direct_lds && a.shape != 1) ? launch_band_rl<4, 8, 2, 64, 1>(b, s)
+                                                  : launch_band_rl<4, 8, 2, 64, 0>(b, s);
         case 2: return launch_band_rl<2, 8, 2, 64, 0>(b, s);
         case 1: return launch_band_rl<1, 8, 2, 64, 0>(b, s);
         default: return hipErrorInvalidValue;
@@ -1834,74 +1920,136 @@ hipError_t launch_band(const BandLaunch& a, hipStream_t s) {
 }
 
 namespace {
-template <int RL, int NW, int OPW, int RING, int WMODE, int KT>
-hipError_t launch_chain_inst(const ChainLaunch& a, hipStream_t s) {
-    constexpr size_t lds = (size_t)RING * 64 * RL * 4;
-    auto kern = band_chain_kernel<RL, NW, OPW, RING, WMODE, KT, RL == 4 ? 1 : 0>;
+// what a persistent launch is cut into: positions (band walk) or groups (BLOCK) per unit, units per
+// row block and layer, queues
+struct PersistShape { int seglen, nseg, nq, grid, total; };
+
+PersistShape persist_shape(const PersistLaunch& a) {
+    PersistShape p{};
+    const int slots_cu = a.block_form ? 8 : band_workgroups_per_cu(a.rl, 0);
+    const int slots = (a.n_cu > 0 ? a.n_cu : 256) * slots_cu;
+    p.nq = (a.xcd_queues && a.nblk >= 1) ? 8 : 1;
+    // row blocks that work side by side: all of them, or those of the fullest queue
+    const int nrb = p.nq > 1 ? (a.nblk + 7) / 8 : a.nblk;
+    const int slots_q = p.nq > 1 ? std::max(1, slots / 8) : slots;
+    if (a.block_form) {
+        // pieces of 4 waves x seglen groups; one group per wave where the batch is small
+        const int ngroups = a.ngroups;
+        const int pieces = (ngroups + 3) / 4;
+        int nseg = std::min(pieces, std::max(1, (slots_q + nrb - 1) / nrb));
+        int gpw = (pieces + nseg - 1) / nseg;
+        if (gpw > 8) gpw = 8;
+        if (a.seglen > 0) gpw = a.seglen;
+        p.seglen = gpw;
+        p.nseg = (pieces + gpw - 1) / gpw;
+    } else {
+        const int T = band_chunk_outputs(a.rl, 0);
+        const int nchunks = (a.N + T - 1) / T;
+        // enough units per layer to give every resident workgroup one, as long as a unit keeps a chunk;
+        // long units are cut at 64 chunks so that the launch's tail stays short
+        int nseg = std::min(nchunks, std::max(1, (slots_q + nrb - 1) / nrb));
+        int cps = (nchunks + nseg - 1) / nseg;
+        if (cps > 64) cps = 64;
+        if (a.seglen > 0) cps = std::max(1, a.seglen / T);
+        p.seglen = cps * T;
+        p.nseg = (nchunks + cps - 1) / cps;
+    }
+    p.total = a.nblk * p.nseg * a.nlayers;
+    const long long per_layer_q = (long long)nrb * p.nseg;
+    p.grid = (int)std::min<long long>(slots, per_layer_q * p.nq);
+    if (p.grid < p.nq) p.grid = p.nq;
+    return p;
+}
+
+PersistArgs persist_args(const PersistLaunch& a, const PersistShape& p) {
+    PersistArgs k{};
+    k.table = a.table; k.nlayers = a.nlayers; k.first_in = a.first_in; k.buf_a = a.buf_a; k.buf_c = a.buf_c;
+    k.active = a.active; k.done = a.done; k.done_stride = a.done_stride; k.ctl = a.ctl; k.prev_ctl = a.prev_ctl;
+    k.prev_units = a.prev_units; k.abort = a.abort; k.host_word = a.host_word;
+    k.N = a.N; k.nblk = a.nblk; k.nseg = p.nseg; k.seglen = p.seglen; k.total_units = p.total; k.nq = p.nq;
+    k.light = (a.light_sync && p.nq > 1) ? 1 : 0;
+    k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead; k.wait_limit = a.wait_limit;
+    k.bias = a.bias; k.clampv = a.clampv;
+    k.stream = (long long)a.nblk * (long long)a.N * 64 * a.rl * 4 * 2 >= a.stream_min_bytes ? 1 : 0;
+    k.pub = a.publish;
+    return k;
+}
+
+template <int RL, int WMODE, int KT>
+hipError_t launch_persist_band_inst(const PersistLaunch& a, hipStream_t s) {
+    constexpr size_t lds = (size_t)64 * 64 * RL * 4;
+    auto kern = band_persist_kernel<RL, WMODE, KT, RL == 4 ? 1 : 0>;
     // once per instantiation; a function-local static is initialised by one thread only
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (attr != hipSuccess) return attr;
-    hipLaunchKernelGGL(kern, dim3(a.nblk), dim3(NW * 64), lds, s, reinterpret_cast<const ChainLayer*>(a.table),
-                       a.nlayers, a.first_in, a.buf_a, a.buf_c, a.active, a.count_out, a.count_prev, a.N, a.stamp0,
-                       a.prev_stamp, a.check_dead, a.stop_when_dead, a.bias, a.clampv, a.publish);
+    const PersistShape p = persist_shape(a);
+    hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), lds, s, persist_args(a, p));
     return hipGetLastError();
 }
-template <int RL, int NW, int OPW, int RING>
-hipError_t launch_chain_rl(const ChainLaunch& a, hipStream_t s) {
-    const bool add_only = a.wmode == 0 && a.add_only;   // as in the per-layer walk
+template <int RL>
+hipError_t launch_persist_band_rl(const PersistLaunch& a, hipStream_t s) {
     if (a.unrolled) {
-        if (add_only) return launch_chain_inst<RL, NW, OPW, RING, 3, 36>(a, s);
         switch (a.wmode) {
-            case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 36>(a, s);
-            case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 36>(a, s);
-            default: return launch_chain_inst<RL, NW, OPW, RING, 2, 36>(a, s);
+            case 0:
+                if (a.add_only && a.twins) return launch_persist_band_inst<RL, 4, 36>(a, s);
+                if (a.add_only) return launch_persist_band_inst<RL, 3, 36>(a, s);
+                return launch_persist_band_inst<RL, 0, 36>(a, s);
+            case 1: return launch_persist_band_inst<RL, 1, 36>(a, s);
+            default: return launch_persist_band_inst<RL, 2, 36>(a, s);
         }
     }
-    if (add_only) return launch_chain_inst<RL, NW, OPW, RING, 3, 0>(a, s);
     switch (a.wmode) {
-        case 0: return launch_chain_inst<RL, NW, OPW, RING, 0, 0>(a, s);
-        case 1: return launch_chain_inst<RL, NW, OPW, RING, 1, 0>(a, s);
-        default: return launch_chain_inst<RL, NW, OPW, RING, 2, 0>(a, s);
+        case 0:
+            if (a.add_only) return launch_persist_band_inst<RL, 3, 0>(a, s);
+            return launch_persist_band_inst<RL, 0, 0>(a, s);
+        case 1: return launch_persist_band_inst<RL, 1, 0>(a, s);
+        default: return launch_persist_band_inst<RL, 2, 0>(a, s);
+    }
+}
+template <int RL, int WMODE, bool FULL>
+hipError_t launch_persist_block_inst(const PersistLaunch& a, hipStream_t s) {
+    const PersistShape p = persist_shape(a);
+    hipLaunchKernelGGL((block_persist_kernel<RL, WMODE, FULL>), dim3(p.grid), dim3(256), 0, s, persist_args(a, p));
+    return hipGetLastError();
+}
+template <int RL>
+hipError_t launch_persist_block_rl(const PersistLaunch& a, hipStream_t s) {
+    switch (a.wmode) {
+        case 0: return a.full ? launch_persist_block_inst<RL, 0, true>(a, s) : launch_persist_block_inst<RL, 0, false>(a, s);
+        case 1: return a.full ? launch_persist_block_inst<RL, 1, true>(a, s) : launch_persist_block_inst<RL, 1, false>(a, s);
+        default: return a.full ? launch_persist_block_inst<RL, 2, true>(a, s) : launch_persist_block_inst<RL, 2, false>(a, s);
     }
 }
 }  // namespace
 
-hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s) {
-    static_assert(sizeof(ChainLayer) == sizeof(ChainLayerDesc), "layer table layout");
-    if (a.N <= 0 || (a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0 || a.nblk <= 0 || a.nlayers < 1 ||
-        !a.table || !a.first_in || !a.buf_a || !a.buf_c || !a.active || a.buf_a == a.buf_c)
+int persist_units(const PersistLaunch& a) { return persist_shape(a).total; }
+
+hipError_t launch_persist(const PersistLaunch& a, hipStream_t s) {
+    // host-side shape checks: what the kernels and the unit numbering assume
+    if (a.N <= 0 || a.nblk <= 0 || a.nlayers < 1 || !a.table || !a.first_in || !a.buf_a || !a.buf_c || a.buf_a == a.buf_c ||
+        !a.active || !a.done || a.done_stride < a.nblk || !a.ctl || !a.abort || !a.host_word || a.wait_limit < 0)
         return hipErrorInvalidValue;
-    if (a.rl == 4 && a.halves) {
-        constexpr size_t lds = 64 * 128 * 4;
-#define SPDNN_HALF(WM, KTv)                                                                                          \
-    do {                                                                                                             \
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(band_chain_half_kernel<WM, KTv>), \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
-        if (attr != hipSuccess) return attr;                                                                         \
-        hipLaunchKernelGGL((band_chain_half_kernel<WM, KTv>), dim3(a.nblk * 2), dim3(512), lds, s,                   \
-                           reinterpret_cast<const ChainLayer*>(a.table), a.nlayers, a.first_in, a.buf_a, a.buf_c,    \
-                           a.active, a.count_out, a.count_prev, a.N, a.stamp0, a.prev_stamp, a.check_dead, a.bias,   \
-                           a.clampv, a.publish);                                                                     \
-    } while (0)
-        const bool add_only = a.wmode == 0 && a.add_only;
-        if (a.unrolled) {
-            if (add_only) SPDNN_HALF(3, 36); else if (a.wmode == 0) SPDNN_HALF(0, 36); else if (a.wmode == 1) SPDNN_HALF(1, 36); else SPDNN_HALF(2, 36);
-        } else {
-            if (add_only) SPDNN_HALF(3, 0); else if (a.wmode == 0) SPDNN_HALF(0, 0); else if (a.wmode == 1) SPDNN_HALF(1, 0); else SPDNN_HALF(2, 0);
-        }
-#undef SPDNN_HALF
-        return hipGetLastError();
+    if (a.block_form) {
+        if (a.ngroups <= 0) return hipErrorInvalidValue;
+    } else if ((a.N % 256) != 0 || a.K < 4 || a.K > 32 || (a.K % 4) != 0) {
+        return hipErrorInvalidValue;
     }
+    if ((long long)a.nblk * persist_shape(a).nseg * a.nlayers > (long long)INT_MAX / 2) return hipErrorInvalidValue;
     switch (a.rl) {
-        // one workgroup per row block walks the whole band, in the shape of the per-layer kernel (8 waves,
-        // one pair each, 64-slot ring): two workgroups fit a CU, so that their load / compute / barrier
-        // phases interleave
-        case 4: return launch_chain_rl<4, 8, 2, 64>(a, s);
-        case 2: return launch_chain_rl<2, 8, 2, 64>(a, s);
-        case 1: return launch_chain_rl<1, 8, 2, 64>(a, s);
+        case 4: return a.block_form ? launch_persist_block_rl<4>(a, s) : launch_persist_band_rl<4>(a, s);
+        case 2: return a.block_form ? launch_persist_block_rl<2>(a, s) : launch_persist_band_rl<2>(a, s);
+        case 1: return a.block_form ? launch_persist_block_rl<1>(a, s) : launch_persist_band_rl<1>(a, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,
+                                    int32_t* counts_host, hipStream_t s) {
+    if (!stamps || rows <= 0 || n < 1 || n > 8192 || (!counts_dev && !counts_host)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(count_stamp_range_kernel, dim3(1), dim3(1024), (size_t)n * 4, s, stamps, rows, stamp_lo, n, counts_dev,
+                       counts_host);
+    return hipGetLastError();
 }
 
 int band_pair_seglen(int N, int nblk, int n_cu) {
@@ -1987,18 +2135,16 @@ hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s) {
         return hipErrorInvalidValue;
     constexpr size_t lds = 512 * 256 + 16 * 2048;   // one panel and the waves' entry rings: all 160 KiB of a CU
     dim3 grid(a.nblk * a.rl, a.ntiles), block(1024);
-#define SPDNN_TILED(WM, RBC)                                                                                     \
+#define SPDNN_TILED(WM)                                                                                          \
     do {                                                                                                         \
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM, RBC>), \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM>),      \
                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
         if (attr != hipSuccess) return attr;                                                                     \
-        hipLaunchKernelGGL((tiled_kernel<WM, RBC>), grid, block, lds, s, a.yin, a.yout, a.cols, a.hdr, a.ent, a.dst, \
+        hipLaunchKernelGGL((tiled_kernel<WM>), grid, block, lds, s, a.yin, a.yout, a.cols, a.hdr, a.ent, a.dst,  \
                            a.active, a.count_prev, a.N, a.ntiles, a.rl, a.stamp, a.prev_stamp, a.check_dead,     \
                            a.bias, a.clampv, a.publish);                                                         \
     } while (0)
-    static const bool rowbcast = !(getenv("SPDNN_TILED_ROW_BROADCAST") && atoi(getenv("SPDNN_TILED_ROW_BROADCAST")) == 0);
-    if (rowbcast) { if (a.wmode != 2) SPDNN_TILED(1, 1); else SPDNN_TILED(2, 1); }
-    else { if (a.wmode != 2) SPDNN_TILED(1, 0); else SPDNN_TILED(2, 0); }
+    if (a.wmode != 2) SPDNN_TILED(1); else SPDNN_TILED(2);
 #undef SPDNN_TILED
     return hipGetLastError();
 }
@@ -2016,7 +2162,7 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {
 #define SPDNN_BLOCK(RLv, WM, FL)                                                                          \
     hipLaunchKernelGGL((block_kernel<RLv, WM, FL>), grid, block, 0, s, a.yin, a.yout, a.cols, a.cnt, a.wv, \
                        a.dst, a.active, a.count_prev, a.N, a.ngroups, gpw, a.stamp, a.prev_stamp, a.check_dead, a.wu, \
-                       a.bias, a.clampv, a.publish)
+                       a.bias, a.clampv, a.publish, a.frontier, a.frontier_layer)
 #define SPDNN_BLOCK_WM(RLv)                                                                 \
     switch (a.wmode) {                                                                      \
         case 0: if (a.full) SPDNN_BLOCK(RLv, 0, true); else SPDNN_BLOCK(RLv, 0, false); break; \

@@ -60,6 +60,11 @@ struct BandLaunch {
     int seglen = 0;          // band positions per workgroup; 0 = heuristic
     long long stream_min_bytes = 96ll << 20;  // launches that read + write at least this much hint their
                                               // column loads and stores as touched once
+    int direct_lds = 1;      // 256-row blocks: 0 = never load straight into LDS (shape 1 only)
+    // finishing a persistent launch that gave up: row blocks with frontier[rb] > frontier_layer have
+    // this layer behind them already and are left alone (nullptr = every row block runs)
+    const int32_t* frontier = nullptr;
+    int frontier_layer = 0;
     Publish publish;
 };
 
@@ -86,7 +91,7 @@ bool band_unrolled(int K, int steps, int stride);
 // Tuning space of the band walk: number of kernel variants for a row-block size (256-row blocks:
 // loads straight into LDS or through registers) and the candidate segment lengths for a variant
 // (used by the run-time selection in spdnn_run).
-int band_shape_count(int rl);
+int band_shape_count(int rl, int direct_lds);
 int band_seglen_candidates(int N, int K, int nblk, int rl, int shape, int n_cu, int* out, int max_out);
 // the occupancy / halo model's score of one candidate (higher is better), for ordering trials
 double band_seglen_score(int N, int K, int nblk, int rl, int shape, int n_cu, int seglen);
@@ -121,39 +126,86 @@ struct BlockLaunch {
     int N, ngroups, nblk, stamp, prev_stamp, check_dead, rl, wmode;
     int full;                // 1: every group has exactly 32 shared inputs
     float wu, bias, clampv;
+    const int32_t* frontier = nullptr;   // as in BandLaunch
+    int frontier_layer = 0;
     Publish publish;
 };
 hipError_t launch_block(const BlockLaunch& a, hipStream_t s);
 
-// Fused layer chain: `nlayers` consecutive BAND layers (same K and weight mode) in one launch,
-// one workgroup per row block.  Layer j reads what layer j-1 wrote: the first layer reads
-// first_in, every layer writes the work buffer (buf_a / buf_c) it did not read.
-struct ChainLayerDesc {      // one entry of the device-side layer table
+// ------------------------------------------------------------------------------------------
+// Several layers per launch ("persistent" launches): the per-layer decomposition - many segments
+// per row block - kept, with a dependency per ROW BLOCK where the per-layer launches have a launch
+// boundary.  The work of `nlayers` consecutive layers of one kind is cut into units (layer, row
+// block, segment) that lie in a queue in layer order; every workgroup claims the next unit with an
+// atomic add until the queue is empty.  A unit of layer j waits until all segments of its row block
+// have finished layer j-1 (a counter per layer and row block, `done`), then runs exactly what the
+// per-layer kernel's workgroup runs.  A unit only ever waits for units claimed BEFORE it by
+// workgroups that are running, so the launch cannot deadlock whatever part of its grid is resident.
+// Every wait is bounded all the same: after `wait_limit` ticks of the 100 MHz clock the waiting
+// workgroup sets `abort`, every workgroup leaves at its next look, and the host finishes the
+// layers with per-layer launches (the `frontier` of the per-layer kernels).
+//
+// With xcd_queues the queue is split in eight, one per XCD: a workgroup reads the number of the
+// XCD it runs on from the hardware and serves that queue only; row block rb belongs to queue
+// rb % 8.  Everything a row block's layers hand to each other then stays in one XCD's L2.
+// ------------------------------------------------------------------------------------------
+struct LayerDesc {           // one entry of the device-side layer table
+    // BAND form
     const uint32_t* pairs;
     const float* pw;
     const int32_t* dst;
     float wu;
-    int halo;   // input columns a segment needs before its first position (K-1, or 32 for run chains)
-    int steps;  // merged steps per pair (records of 16 dwords: two use masks, 36 one-byte ring selectors)
+    int halo;                // input columns a segment needs before its first position (K-1, or 32 for run chains)
+    int steps;               // merged steps per pair (records of 16 dwords: two use masks, 36 one-byte ring selectors)
+    // BLOCK form (BLOCK layers; run-chain BAND layers that carry one)
+    int ngroups;
+    const int32_t* blk_cols;
+    const int32_t* blk_cnt;
+    const float* blk_wv;
+    const int32_t* blk_dst;
 };
-struct ChainLaunch {
-    const ChainLayerDesc* table;  // device pointer to the entry of the first layer of the chain
+
+struct PersistCtl {          // device words of one persistent launch (zero before the launch)
+    int32_t head[8];         // next unit of each queue
+    int32_t units_done;      // units finished
+    int32_t pad[7];
+};
+
+struct PersistLaunch {
+    const LayerDesc* table;       // device pointer to the entry of the launch's first layer
     int nlayers;
-    Feat first_in;
-    Feat buf_a;
-    Feat buf_c;
+    int block_form;               // 0: band walk, 1: BLOCK kernel body
+    Feat first_in, buf_a, buf_c;  // layer j reads what layer j-1 wrote; every layer writes the work buffer it did not read
     int32_t* active;
-    int32_t* count_out;           // counter of the first layer of the chain (consecutive ints), or nullptr
-    int32_t* count_prev;          // as in BandLaunch, for the layer before the chain
-    int N, K, nblk, stamp0, prev_stamp, check_dead, rl, wmode;
-    int unrolled;                 // every layer of the chain has 32 entries per output (band_unrolled)
-    int stop_when_dead;           // 1: a workgroup whose rows have all died leaves the chain
-    int halves;                   // 1 (256-row blocks only): one workgroup per HALF row block (twice the workgroups)
-    int add_only = 1;             // as in BandLaunch
+    int32_t* done;                // [nlayers][done_stride] segments finished per layer and row block (zero before the launch)
+    int done_stride;              // >= nblk
+    int ngroups;                  // BLOCK form: groups per layer (the same for every layer of the launch)
+    PersistCtl* ctl;              // this launch's control words
+    const PersistCtl* prev_ctl;   // the persistent launch right before this one in the stream (or nullptr) ...
+    int prev_units;               // ... and the units it must have finished for this one to start
+    int32_t* abort;               // device word: nonzero = a launch gave up; sticky until the host clears it
+    int32_t* host_word;           // pinned host word: receives the unit total when the launch is complete, -2 on abort
+    int N, K, nblk, rl, wmode, stamp0, prev_stamp, check_dead;
+    int unrolled, add_only, twins, full;   // kernel variant, as in BandLaunch / BlockLaunch
+    int seglen;                   // band positions (band walk) or groups (BLOCK) per unit; 0 = heuristic
+    int xcd_queues;               // 1: one queue per XCD, row block rb in queue rb % 8
+    int light_sync;               // 1 (xcd_queues only): the hand-over between layers stays inside one L2, so the
+                                  // writer only waits for its stores and the reader only drops its CU's L1
+    long long wait_limit;         // ticks of the 100 MHz clock a unit waits for its row block at most
+    int n_cu;
+    long long stream_min_bytes;
     float bias, clampv;
     Publish publish;
 };
-hipError_t launch_band_chain(const ChainLaunch& a, hipStream_t s);
+// units the launch consists of (what ctl->units_done reaches)
+int persist_units(const PersistLaunch& a);
+hipError_t launch_persist(const PersistLaunch& a, hipStream_t s);
+
+// counts[i] = number of rows r < rows with stamps[r] >= stamp_lo + i, for i in [0, n): with bias <= 0 a
+// row that is zero stays zero, so the rows that carry the stamp of layer l or a later one are the rows
+// layer l left active.  Written to counts_dev and (system scope) to counts_host, either may be nullptr.
+hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,
+                                    int32_t* counts_host, hipStream_t s);
 
 // Fused pair: two consecutive BAND layers (32 entries per row, unrolled record form, same weight
 // mode, rows per lane 4) of which the first writes its outputs exactly where the second reads them

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <condition_variable>
@@ -34,6 +35,13 @@ using namespace spdnn;
 namespace {
 
 thread_local std::string g_err = "";
+
+// device allocations the library has made in this process (spdnn_device_alloc_calls)
+std::atomic<int64_t> g_dev_allocs{0};
+template <class T> hipError_t dev_malloc(T** p, size_t bytes) {
+    g_dev_allocs.fetch_add(1, std::memory_order_relaxed);
+    return hipMalloc(reinterpret_cast<void**>(p), bytes);
+}
 
 int fail(int code, const std::string& msg) {
     g_err = msg;
@@ -88,7 +96,7 @@ hipError_t scratch_base(unsigned char** out) {
 struct DevTmp {
     void* p = nullptr;
     ~DevTmp() { if (p) hipFree(p); }
-    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes); }
+    hipError_t alloc(size_t bytes) { return dev_malloc(&p, bytes); }
     template <class T> T* as() const { return static_cast<T*>(p); }
 };
 struct EventTmp {
@@ -136,7 +144,7 @@ class JobPool {
                 q_.pop_front();
                 cv_room_.notify_one();
             }
-            f();
+            try { f(); } catch (...) {}  // jobs report through their own state; nothing may escape a worker
             {
                 std::unique_lock<std::mutex> lk(m_);
                 if (--pending_ == 0) cv_done_.notify_all();
@@ -252,8 +260,25 @@ struct spdnn_net {
     // them; a later launch that does not look (pruning off) would.  Set by launches that may skip,
     // cleared when every carried block has been written again (new run, repack).
     bool blocks_skipped = false;
-    int default_fuse = 1;     // layers per launch when the caller leaves fuse_layers at 0
-    int chain_halves = 1;     // fused chains on half row blocks (SPDNN_CHAIN_HALVES=0: whole row blocks)
+    // Persistent launches (several layers per launch, see PersistLaunch).  SPDNN_PERSIST: 0 = never unless the
+    // caller asks (fuse_layers >= 2), 1 = where a layer's launch moves at most persist_max_bytes (default).
+    int persist_mode = 1;
+    int persist_layers = 64;          // layers per persistent launch at most (SPDNN_PERSIST_LAYERS)
+    long long persist_max_bytes = (long long)1 << 31;   // SPDNN_PERSIST_MAX_BYTES
+    int persist_xcd = -1;             // one unit queue per XCD: -1 = where the row blocks of an XCD fit its L2, 0 / 1 (SPDNN_PERSIST_XCD)
+    int persist_light = 0;            // SPDNN_PERSIST_LIGHT_SYNC: with XCD queues, hand over inside the XCD's L2 without device-scope fences
+    int persist_seglen = 0;           // band positions / groups per unit, 0 = heuristic (SPDNN_PERSIST_SEGLEN)
+    long long persist_wait_us = 2000000;   // longest wait of a unit for its row block (SPDNN_PERSIST_WAIT_US)
+    int band_seglen = 0;              // SPDNN_BAND_SEGLEN: band positions per workgroup of the per-layer walk (0 = run-time selection)
+    int band_direct_lds = 1;          // SPDNN_BAND_DIRECT_LDS=0: the per-layer walk never loads straight into LDS
+    int32_t* d_done = nullptr;        // [L][done_stride] units finished per layer and row block
+    int done_stride = 0;
+    PersistCtl* d_ctl = nullptr;      // [L] control words, one per persistent launch of a run
+    int32_t* d_abort = nullptr;
+    int32_t* d_frontier = nullptr;    // [done_stride]
+    int32_t* h_pwords = nullptr;      // pinned [L]: completion word of every persistent launch of a run
+    size_t search_peak_bytes = 0;     // device memory the placement search held at its peak
+    bool run_verbose = false;         // SPDNN_RUN_VERBOSE=1: spdnn_run reports its persistent launches on stderr
     int add_only = 1;         // band layers with one power-of-two weight add their inputs and scale the sum once
                               // (SPDNN_BAND_SUM_THEN_SCALE=0: a multiply-add per input)
     bool fuse_pairs = true;   // fused pairs where the inspector found them (SPDNN_FUSE_PAIRS=0: never)
@@ -266,7 +291,7 @@ struct spdnn_net {
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
-    ChainLayerDesc* d_chain = nullptr;
+    LayerDesc* d_table = nullptr;   // one entry per layer (resident plans only)
     std::vector<char> pending; // layer has an inspection job in flight
     std::vector<int64_t> counts;
     std::vector<float> layer_ms;
@@ -291,6 +316,11 @@ void release_device_base(spdnn_net* n) {
     hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
     hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
     hipFree(n->d_counts);
+    hipFree(n->d_done); hipFree(n->d_ctl); hipFree(n->d_abort); hipFree(n->d_frontier);
+    n->d_done = n->d_abort = n->d_frontier = nullptr;
+    n->d_ctl = nullptr;
+    if (n->h_pwords) hipHostFree(n->h_pwords);
+    n->h_pwords = nullptr;
     if (n->h_count) hipHostFree(n->h_count);
     if (n->h_counts) hipHostFree(n->h_counts);
     n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
@@ -326,20 +356,28 @@ int init_device(spdnn_net* n) {
     HIPCHK(hipEventCreate(&n->ev_start));
     HIPCHK(hipEventCreate(&n->ev_stop));
     const size_t rows = (size_t)n->rows_cap;
-    HIPCHK(hipMalloc(&n->d_active, rows * 4));
-    HIPCHK(hipMalloc(&n->d_active_mid, rows * 4));
+    HIPCHK(dev_malloc(&n->d_active, rows * 4));
+    HIPCHK(dev_malloc(&n->d_active_mid, rows * 4));
     HIPCHK(hipMemset(n->d_active_mid, 0, rows * 4));
-    HIPCHK(hipMalloc(&n->d_gid, rows * 4));
-    HIPCHK(hipMalloc(&n->d_gid_tmp, rows * 4));
-    HIPCHK(hipMalloc(&n->d_alive_src, rows * 4));
-    HIPCHK(hipMalloc(&n->d_alive_gid, rows * 4));
-    HIPCHK(hipMalloc(&n->d_count, 64));
-    HIPCHK(hipMalloc(&n->d_nonfinite, 64));
+    HIPCHK(dev_malloc(&n->d_gid, rows * 4));
+    HIPCHK(dev_malloc(&n->d_gid_tmp, rows * 4));
+    HIPCHK(dev_malloc(&n->d_alive_src, rows * 4));
+    HIPCHK(dev_malloc(&n->d_alive_gid, rows * 4));
+    HIPCHK(dev_malloc(&n->d_count, 64));
+    HIPCHK(dev_malloc(&n->d_nonfinite, 64));
     // coherent: the layer kernels store counts here and the host reads them while kernels still run
     HIPCHK(hipHostMalloc(&n->h_count, 64, hipHostMallocCoherent | hipHostMallocMapped));
-    HIPCHK(hipMalloc(&n->d_counts, (size_t)n->L * 4));
+    HIPCHK(dev_malloc(&n->d_counts, (size_t)n->L * 4));
     HIPCHK(hipHostMalloc(&n->h_counts, (size_t)n->L * 4, hipHostMallocCoherent | hipHostMallocMapped));
     HIPCHK(hipMemset(n->d_active, 0, rows * 4));
+    // persistent launches: units finished per layer and row block, control words per launch, completion words
+    n->done_stride = n->rows_cap / n->RB;
+    HIPCHK(dev_malloc(&n->d_done, (size_t)n->L * (size_t)n->done_stride * 4));
+    HIPCHK(dev_malloc(&n->d_ctl, (size_t)n->L * sizeof(PersistCtl)));
+    HIPCHK(dev_malloc(&n->d_abort, 64));
+    HIPCHK(hipMemset(n->d_abort, 0, 64));
+    HIPCHK(dev_malloc(&n->d_frontier, (size_t)n->done_stride * 4));
+    HIPCHK(hipHostMalloc(&n->h_pwords, (size_t)n->L * 4, hipHostMallocCoherent | hipHostMallocMapped));
     n->dev_ready = true;
     return SPDNN_OK;
 }
@@ -382,6 +420,7 @@ int alloc_feature_buffers(spdnn_net* n) {
     std::vector<float*>& c = n->feat_allocs;
     std::vector<double> rate;  // rate[i]: candidate i swept together with candidate 0 (rate[0] unused)
     std::vector<void*> fillers;
+    size_t filler_bytes = 0;   // size of one filler
     auto fail_free = [&](int code, const std::string& msg) {
         for (void* f : fillers) hipFree(f);
         for (float* p : c) hipFree(p);
@@ -390,7 +429,7 @@ int alloc_feature_buffers(spdnn_net* n) {
     };
     auto add = [&]() {
         float* p = nullptr;
-        if (hipMalloc(&p, half_bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
+        if (dev_malloc(&p, half_bytes) != hipSuccess) { (void)hipGetLastError(); return false; }
         c.push_back(p);
         return true;
     };
@@ -443,6 +482,7 @@ int alloc_feature_buffers(spdnn_net* n) {
         // every step past the first six candidates advances at least 4 GiB through the memory: small
         // half-buffers are spaced out by fillers, which are freed again below
         const size_t filler = half_bytes < ((size_t)4 << 30) ? ((size_t)4 << 30) - half_bytes : 0;
+        filler_bytes = filler;
         const size_t budget = (size_t)((double)free_b * budget_frac);
         rate.assign(1, 0.0);
         bool found = false;
@@ -453,7 +493,7 @@ int alloc_feature_buffers(spdnn_net* n) {
                 if ((c.size() + 1) * half_bytes + (fillers.size() + 1) * filler > budget) break;
                 if (filler) {
                     void* f = nullptr;
-                    if (hipMalloc(&f, filler) != hipSuccess) { (void)hipGetLastError(); break; }
+                    if (dev_malloc(&f, filler) != hipSuccess) { (void)hipGetLastError(); break; }
                     fillers.push_back(f);
                 }
                 if (!add()) break;
@@ -507,6 +547,8 @@ int alloc_feature_buffers(spdnn_net* n) {
         bufs[b]->half[0] = c[(size_t)pick[2 * b]];
         bufs[b]->half[1] = c[(size_t)pick[2 * b + 1]];
     }
+    // what the search held at its peak (all candidates and fillers are still allocated here)
+    n->search_peak_bytes = c.size() * half_bytes + fillers.size() * filler_bytes;
     // give back what was only a candidate
     for (void* f : fillers) hipFree(f);
     std::vector<float*> keep;
@@ -567,7 +609,7 @@ int upload_plans(spdnn_net* n) {
     n->dl.assign(L, DevLayer{});
     const bool streamed = n->plan_window >= 2 && (size_t)n->plan_window < L;
     if (!streamed) {
-        HIPCHK(hipMalloc(&n->arena, std::max<size_t>(total, 256)));
+        HIPCHK(dev_malloc(&n->arena, std::max<size_t>(total, 256)));
         std::vector<char> blob(largest);
         size_t off = 0;
         for (size_t l = 0; l < L; ++l) {
@@ -577,22 +619,40 @@ int upload_plans(spdnn_net* n) {
             n->dl[l] = plan_at(n->lay[l], (char*)n->arena + off);
             off += n->lay[l].bytes;
         }
-        std::vector<ChainLayerDesc> table(L);
+        std::vector<LayerDesc> table(L);
         for (size_t l = 0; l < L; ++l) {
-            table[l].pairs = n->dl[l].pairs;
-            table[l].pw = n->dl[l].wv;
-            table[l].steps = n->layers[l].pair_steps;
-            table[l].dst = n->dl[l].dst;
-            table[l].wu = n->layers[l].info.value;
-            table[l].halo = n->layers[l].info.band_halo;
+            const LayerPlan& p = n->layers[l];
+            LayerDesc& t = table[l];
+            t = LayerDesc{};
+            t.wu = p.info.value;
+            if (p.kernel == SPDNN_KERNEL_BAND) {
+                t.pairs = n->dl[l].pairs;
+                t.pw = n->dl[l].wv;
+                t.dst = n->dl[l].dst;
+                t.steps = p.pair_steps;
+                t.halo = p.info.band_halo;
+                if (p.alt_ngroups > 0) {   // its BLOCK form
+                    t.ngroups = p.alt_ngroups;
+                    t.blk_cols = n->dl[l].alt_cols;
+                    t.blk_cnt = n->dl[l].alt_cnt;
+                    t.blk_wv = nullptr;
+                    t.blk_dst = n->dl[l].alt_dst;
+                }
+            } else if (p.kernel == SPDNN_KERNEL_BLOCK) {
+                t.ngroups = p.ngroups;
+                t.blk_cols = n->dl[l].blk_cols;
+                t.blk_cnt = n->dl[l].blk_cnt;
+                t.blk_wv = n->dl[l].wv;
+                t.blk_dst = n->dl[l].dst;
+            }
         }
-        HIPCHK(hipMalloc(&n->d_chain, table.size() * sizeof(ChainLayerDesc)));
-        HIPCHK(hipMemcpy(n->d_chain, table.data(), table.size() * sizeof(ChainLayerDesc), hipMemcpyHostToDevice));
+        HIPCHK(dev_malloc(&n->d_table, table.size() * sizeof(LayerDesc)));
+        HIPCHK(hipMemcpy(n->d_table, table.data(), table.size() * sizeof(LayerDesc), hipMemcpyHostToDevice));
         n->slot_bytes = 0;
     } else {
         const size_t S = (size_t)n->plan_window;
         n->slot_bytes = std::max<size_t>(largest, 256);
-        HIPCHK(hipMalloc(&n->arena, S * n->slot_bytes));
+        HIPCHK(dev_malloc(&n->arena, S * n->slot_bytes));
         HIPCHK(hipHostMalloc((void**)&n->h_plans, std::max<size_t>(total, 256)));
         n->h_plan_off.assign(L, 0);
         size_t off = 0;
@@ -613,7 +673,7 @@ int upload_plans(spdnn_net* n) {
             n->ev_slot_free.push_back(e);
         }
     }
-    HIPCHK(hipMalloc(&n->d_lab, (size_t)n->N * 8));
+    HIPCHK(dev_malloc(&n->d_lab, (size_t)n->N * 8));
     HIPCHK(hipMemcpy(n->d_lab, n->layers[0].in_pos.data(), (size_t)n->N * 4, hipMemcpyHostToDevice));
     n->lab_layer = -1;
     int rc = alloc_feature_buffers(n);
@@ -650,8 +710,8 @@ void free_device(spdnn_net* n) {
     n->d_lab = nullptr;
     n->lab_layer = -1;
     if (n->arena) hipFree(n->arena);
-    if (n->d_chain) hipFree(n->d_chain);
-    n->d_chain = nullptr;
+    if (n->d_table) hipFree(n->d_table);
+    n->d_table = nullptr;
     for (float* p : n->feat_allocs) hipFree(p);
     n->feat_allocs.clear();
     n->arena = nullptr;
@@ -737,6 +797,28 @@ void reset_state(spdnn_net* n) {
     n->alive_list_valid = false;
 }
 
+// inspect_layer for a worker thread: a worker must not let an exception escape (std::terminate); the
+// layer stays unset and spdnn_inspect reports what happened
+void inspect_on_worker(int N, const std::vector<int32_t>& rp, const std::vector<int32_t>& col, const std::vector<float>& val,
+                       int force, bool fma_ok, LayerPlan* plan) {
+    try {
+        inspect_layer(N, rp, col, val, force, fma_ok, *plan);
+    } catch (const std::bad_alloc&) {
+        plan->set = false;
+        plan->failed = plan->failed_nomem = true;
+    } catch (const std::exception& e) {
+        plan->set = false;
+        plan->failed = true;
+        plan->failed_nomem = false;
+        plan->fail_text = e.what();
+    } catch (...) {
+        plan->set = false;
+        plan->failed = true;
+        plan->failed_nomem = false;
+        plan->fail_text = "unknown exception";
+    }
+}
+
 int submit_layer(spdnn_net* n, int layer, std::shared_ptr<std::vector<int32_t>> rp,
                  std::shared_ptr<std::vector<int32_t>> col, std::shared_ptr<std::vector<float>> val) {
     n->inspected = false;
@@ -744,16 +826,7 @@ int submit_layer(spdnn_net* n, int layer, std::shared_ptr<std::vector<int32_t>> 
     const int N = n->N;
     LayerPlan* plan = &n->layers[(size_t)layer];
     const bool fma_ok = n->fma_ok;
-    n->pool->submit([=] {
-        // a worker must not let an exception escape (std::terminate): the layer stays unset and
-        // spdnn_inspect reports it
-        try {
-            inspect_layer(N, *rp, *col, *val, force, fma_ok, *plan);
-        } catch (...) {
-            plan->set = false;
-            plan->failed = true;
-        }
-    });
+    n->pool->submit([=] { inspect_on_worker(N, *rp, *col, *val, force, fma_ok, plan); });
     return SPDNN_OK;
 }
 
@@ -777,7 +850,7 @@ template <class F> int guarded(F&& f) {
 
 extern "C" {
 
-int spdnn_version(void) { return 100; }
+int spdnn_version(void) { return 200; }
 
 const char* spdnn_last_error(void) { return g_err.c_str(); }
 
@@ -804,10 +877,17 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     n->layer_ms.assign((size_t)layers, 0.0f);
     n->pool.reset(new JobPool(host_threads()));
     if (const char* e = getenv("SPDNN_AUTOTUNE")) n->autotune = atoi(e) != 0;
-    if (getenv("SPDNN_BAND_SEGLEN")) n->autotune = false;  // an explicit setting wins
-    if (const char* e = getenv("SPDNN_FUSE_LAYERS")) n->default_fuse = std::max(1, atoi(e));
+    if (const char* e = getenv("SPDNN_RUN_VERBOSE")) n->run_verbose = atoi(e) != 0;
+    if (const char* e = getenv("SPDNN_PERSIST")) n->persist_mode = atoi(e) != 0 ? 1 : 0;
+    if (const char* e = getenv("SPDNN_PERSIST_LAYERS")) n->persist_layers = std::max(2, atoi(e));
+    if (const char* e = getenv("SPDNN_PERSIST_MAX_BYTES")) n->persist_max_bytes = atoll(e);
+    if (const char* e = getenv("SPDNN_PERSIST_XCD")) n->persist_xcd = atoi(e);
+    if (const char* e = getenv("SPDNN_PERSIST_LIGHT_SYNC")) n->persist_light = atoi(e) != 0 ? 1 : 0;
+    if (const char* e = getenv("SPDNN_PERSIST_SEGLEN")) n->persist_seglen = std::max(0, atoi(e));
+    if (const char* e = getenv("SPDNN_PERSIST_WAIT_US")) n->persist_wait_us = std::max(0ll, atoll(e));
+    if (const char* e = getenv("SPDNN_BAND_SEGLEN")) n->band_seglen = std::max(0, atoi(e));
+    if (const char* e = getenv("SPDNN_BAND_DIRECT_LDS")) n->band_direct_lds = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_FUSE_PAIRS")) n->fuse_pairs = atoi(e) != 0;
-    if (const char* e = getenv("SPDNN_CHAIN_HALVES")) n->chain_halves = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_BAND_SUM_THEN_SCALE")) n->add_only = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
@@ -898,6 +978,7 @@ static int spdnn_load_layers_tsv_impl(spdnn_net* n, const char* data_dir, int fi
         LayerPlan* plan = &n->layers[(size_t)l];
         const size_t k = (size_t)(l - first);
         n->pool->submit([=] {
+            plan->set = false;   // until the inspection has succeeded (whatever fails on the way)
             const std::string path = dir + "/neuron" + std::to_string(N) + "/n" + std::to_string(N) + "-l" +
                                      std::to_string(l + 1) + ".tsv";
             std::vector<int32_t> rp, cc, rp2, cc2;
@@ -916,7 +997,7 @@ static int spdnn_load_layers_tsv_impl(spdnn_net* n, const char* data_dir, int fi
                 plan->set = false;
                 return;
             }
-            inspect_layer(N, rp2, cc2, vv2, force, fma_ok, *plan);
+            inspect_on_worker(N, rp2, cc2, vv2, force, fma_ok, plan);
         });
     }
     n->pool->wait_all();
@@ -975,10 +1056,11 @@ static int spdnn_synth_layers_impl(spdnn_net* n, uint64_t seed, int first, int c
         n->pending[(size_t)l] = 1;
         LayerPlan* plan = &n->layers[(size_t)l];
         n->pool->submit([=] {
+            plan->set = false;   // until the inspection has succeeded (whatever fails on the way)
             std::vector<int32_t> rp, cc;
             std::vector<float> vv;
             synth_layer_csr(seed, l, N, nnz_per_row, value, rp, cc, vv);
-            inspect_layer(N, rp, cc, vv, force, fma_ok, *plan);
+            inspect_on_worker(N, rp, cc, vv, force, fma_ok, plan);
         });
     }
     return SPDNN_OK;
@@ -989,10 +1071,14 @@ static int spdnn_inspect_impl(spdnn_net* n) {
     n->pool->wait_all();
     std::fill(n->pending.begin(), n->pending.end(), 0);
     for (int l = 0; l < n->L; ++l)
-        if (!n->layers[(size_t)l].set)
-            return n->layers[(size_t)l].failed
-                       ? fail(SPDNN_E_NOMEM, "the inspection of layer " + std::to_string(l) + " ran out of host memory; hand it over again")
-                       : fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
+        if (!n->layers[(size_t)l].set) {
+            const LayerPlan& p = n->layers[(size_t)l];
+            if (p.failed && p.failed_nomem)
+                return fail(SPDNN_E_NOMEM, "the inspection of layer " + std::to_string(l) + " ran out of host memory; hand it over again");
+            if (p.failed)
+                return fail(SPDNN_E_UNSUPPORTED, "the inspection of layer " + std::to_string(l) + " failed: " + p.fail_text);
+            return fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
+        }
     for (int l = 0; l < n->L; ++l) {
         LayerPlan* cur = &n->layers[(size_t)l];
         const std::vector<int32_t>* nxt = l + 1 < n->L ? &n->layers[(size_t)l + 1].in_pos : nullptr;
@@ -1256,6 +1342,7 @@ static BandLaunch band_args(spdnn_net* n, int l, const Feat& in, const Feat& out
     a.halo = p.info.band_halo;
     a.wu = p.info.value; a.bias = n->bias; a.clampv = n->clampv; a.n_cu = n->n_cu;
     a.shape = -1; a.seglen = 0; a.count_prev = nullptr; a.prev_stamp = 0; a.check_dead = 0;
+    a.direct_lds = n->band_direct_lds;
     a.stream_min_bytes = n->stream_min_bytes;
     return a;
 }
@@ -1278,7 +1365,7 @@ static spdnn_net::Explore* explore_for(spdnn_net* n, int nblk, int K, int layers
         if (e.K == K && same_bucket(nblk, e.nblk)) return &e;
     spdnn_net::Explore e{nblk, K, 0, {}};
     std::vector<std::pair<double, spdnn_net::Cand>> scored;
-    for (int shape = 0; shape < band_shape_count(n->rl); ++shape) {
+    for (int shape = 0; shape < band_shape_count(n->rl, n->band_direct_lds); ++shape) {
         int lens[20];
         const int nc = band_seglen_candidates(n->N, K, nblk, n->rl, shape, n->n_cu, lens, 20);
         for (int c = 0; c < nc; ++c)
@@ -1339,7 +1426,7 @@ static bool use_block_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
 
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
                                int prev_stamp, int check_dead, int32_t* count_prev, int shape, int seglen,
-                               const Publish& pub) {
+                               const Publish& pub, const int32_t* frontier = nullptr, int frontier_layer = 0) {
     const LayerPlan& p = n->layers[(size_t)l];
     const DevLayer& d = n->dl[(size_t)l];
     if (use_block_form(n, p, nblk)) {
@@ -1348,7 +1435,7 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         b.active = n->d_active; b.count_prev = count_prev; b.check_dead = check_dead; b.N = n->N; b.ngroups = p.alt_ngroups; b.nblk = nblk;
         b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = 0; b.full = p.alt_full ? 1 : 0;
         b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
-        b.publish = pub;
+        b.publish = pub; b.frontier = frontier; b.frontier_layer = frontier_layer;
         return launch_block(b, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_BAND) {
@@ -1357,8 +1444,8 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         a.prev_stamp = prev_stamp;
         a.check_dead = check_dead;
         a.shape = shape;
-        a.seglen = seglen;
-        a.publish = pub;
+        a.seglen = seglen > 0 ? seglen : n->band_seglen;
+        a.publish = pub; a.frontier = frontier; a.frontier_layer = frontier_layer;
         return launch_band(a, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_BLOCK) {
@@ -1367,7 +1454,7 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         b.active = n->d_active; b.count_prev = count_prev; b.check_dead = check_dead; b.N = n->N; b.ngroups = p.ngroups; b.nblk = nblk;
         b.stamp = stamp; b.prev_stamp = prev_stamp; b.rl = n->rl; b.wmode = p.wmode; b.full = p.blk_full ? 1 : 0;
         b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
-        b.publish = pub;
+        b.publish = pub; b.frontier = frontier; b.frontier_layer = frontier_layer;
         return launch_block(b, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_TILED) {
@@ -1421,6 +1508,30 @@ static int wait_counts(spdnn_net* n, int l0, int c) {
     return SPDNN_OK;
 }
 
+// What layer l runs as in a launch on nblk row blocks, for grouping consecutive layers into one
+// persistent launch: layers of one signature share a kernel instantiation and a unit shape.
+struct LayerSig {
+    int form = -1;   // -1: no persistent form; 0: band walk; 1: BLOCK kernel
+    int wmode = 0, unrolled = 0, twins = 0, K = 0, full = 0, ngroups = 0;
+    bool operator==(const LayerSig& o) const {
+        return form == o.form && wmode == o.wmode && unrolled == o.unrolled && twins == o.twins && K == o.K && full == o.full &&
+               ngroups == o.ngroups;
+    }
+};
+static LayerSig layer_sig(const spdnn_net* n, int l, int nblk) {
+    const LayerPlan& p = n->layers[(size_t)l];
+    LayerSig g;
+    if (use_block_form(n, p, nblk)) {
+        g.form = 1; g.wmode = 0; g.full = p.alt_full ? 1 : 0; g.ngroups = p.alt_ngroups;
+    } else if (p.kernel == SPDNN_KERNEL_BAND) {
+        g.form = 0; g.wmode = p.wmode; g.K = p.kmax; g.twins = p.pair_twins ? 1 : 0;
+        g.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
+    } else if (p.kernel == SPDNN_KERNEL_BLOCK) {
+        g.form = 1; g.wmode = p.wmode; g.full = p.blk_full ? 1 : 0; g.ngroups = p.ngroups;
+    }
+    return g;
+}
+
 static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     spdnn_run_options opt;
@@ -1455,10 +1566,20 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
     const bool scan_count = !fused_count && opt.collect_counts;
     const bool have_counts = fused_count || scan_count;
     if (fused_count) HIPCHK(hipMemsetAsync(n->d_counts + first, 0, (size_t)nl * 4, n->stream));
-    int fuse = opt.fuse_layers ? opt.fuse_layers : n->default_fuse;
-    // fused pairs: by default and with fused launches asked for, not with fuse_layers = 1
-    const bool pair_mode = n->fuse_pairs && !scan_count && !plans_streamed(n) && (fuse >= 2 || opt.fuse_layers == 0);
-    if (scan_count || fuse < 2 || plans_streamed(n)) fuse = 1;  // a fused launch needs all its plans resident
+    // Launches that hold more than one layer need all their plans resident and count on the device:
+    // fused pairs (by default and with fused launches asked for, not with fuse_layers = 1) and persistent
+    // launches (asked for with fuse_layers >= 2 layers per launch, else by default where a layer moves
+    // little enough for the launch boundary to matter).
+    const bool no_fusion = scan_count || plans_streamed(n) || opt.fuse_layers == 1;
+    const bool pair_mode = n->fuse_pairs && !no_fusion;
+    const bool persist_asked = opt.fuse_layers >= 2;
+    bool persist_on = !no_fusion && (persist_asked || n->persist_mode == 1);
+    const int persist_cmax = persist_asked ? opt.fuse_layers : n->persist_layers;
+    const long long persist_wait_us = opt.persist_wait_us < 0 ? 0 : (opt.persist_wait_us > 0 ? opt.persist_wait_us : n->persist_wait_us);
+    if (persist_on) {
+        HIPCHK(hipMemsetAsync(n->d_done + (size_t)first * n->done_stride, 0, (size_t)nl * n->done_stride * 4, n->stream));
+        HIPCHK(hipMemsetAsync(n->d_ctl, 0, (size_t)nl * sizeof(PersistCtl), n->stream));
+    }
     if (plans_streamed(n))
         for (int l = first; l <= last && l < first + n->plan_window; ++l) HIPCHK(plan_fetch(n, l));
 
@@ -1482,213 +1603,402 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
         volatile int32_t* h = n->h_counts;
         for (int l = first; l <= last; ++l) h[l] = -1;
     }
-    Publish pub{};
-    struct Rec { int l0, c; };
-    std::vector<Rec> recs;
-    size_t processed = 0;
-    spdnn_run_result r{};
-    const int64_t alive_at_start = n->alive;
+    struct Rec { int l0, c, pl; };   // counts of layers [l0, l0+c) on their way to the host; pl: the persistent launch they come from (ordinal), or -1
     struct Timed { int l0, c; };
+    std::vector<Rec> recs;
     std::vector<Timed> timed;
-    int64_t newest_count = -1;
-    bool dead = n->carried == 0;
-    int last_launched = -1;
-    bool count_pending = false;  // the newest layer's rows have not been counted yet
+
+    // Everything the layer loop changes, so that it can go back to where a persistent launch started.
+    struct State {
+        Feat cur; int cur_layer, carried, stamp, last_stamp; bool blocks_skipped;
+        int l; bool dead, count_pending; int last_launched; int64_t newest_count; int c_prune;
+        Publish pub; size_t nrecs, processed, ntimed; spdnn_run_result r;
+    };
+    State st{};
+    st.l = first; st.dead = n->carried == 0; st.count_pending = false; st.last_launched = -1; st.newest_count = -1;
+    st.c_prune = 1; st.pub = Publish{}; st.processed = 0; st.r = spdnn_run_result{};
+    auto save = [&]() {
+        State s = st;
+        s.cur = n->cur; s.cur_layer = n->cur_layer; s.carried = n->carried; s.stamp = n->stamp; s.last_stamp = n->last_stamp;
+        s.blocks_skipped = n->blocks_skipped; s.nrecs = recs.size(); s.ntimed = timed.size();
+        return s;
+    };
+    auto restore = [&](const State& s) {
+        st = s;
+        n->cur = s.cur; n->cur_layer = s.cur_layer; n->carried = s.carried; n->stamp = s.stamp; n->last_stamp = s.last_stamp;
+        n->blocks_skipped = s.blocks_skipped;
+        recs.resize(s.nrecs);
+        timed.resize(s.ntimed);
+    };
+    // persistent launches whose completion the host has not seen yet, oldest first
+    struct PLaunch { State at; int l0, c, nblk, nseg, units, slot; };
+    std::deque<PLaunch> pending;
+    int next_slot = 0;          // control words of the run's persistent launches, in order
+    // a persistent launch that gave up is finished by per-layer launches: layers [fb_l0, fb_l0 + fb_c), each row
+    // block from the layer it had reached (d_frontier)
+    int fb_l0 = -1, fb_c = 0;
+    const int64_t alive_at_start = n->alive;
+
+    // Looks at the completion words of the pending persistent launches, oldest first, up to and including ordinal
+    // `upto`.  wait: until each word is there (bounded; the stream is asked after 100 ms as in wait_counts).
+    // *failed = index in `pending` of the first launch that did not complete (gave up, or the stream went idle
+    // without its word), -1 if none.
+    auto settle = [&](bool wait, int upto, int* failed) -> int {
+        *failed = -1;
+        volatile int32_t* h = n->h_pwords;
+        while (!pending.empty() && pending.front().slot <= upto) {
+            const PLaunch& pl = pending.front();
+            auto t_start = std::chrono::steady_clock::now(), t0 = t_start;
+            for (unsigned spins = 1; h[pl.slot] == -1; ++spins) {
+                if (!wait) return SPDNN_OK;
+                if ((spins & 255) != 0) continue;
+                auto now = std::chrono::steady_clock::now();
+                if (now - t_start < std::chrono::microseconds(300)) continue;
+                std::this_thread::sleep_for(std::chrono::microseconds(50));
+                now = std::chrono::steady_clock::now();
+                if (now - t0 < std::chrono::milliseconds(100)) continue;
+                t0 = now;
+                if (now - t_start > std::chrono::milliseconds(n->count_timeout_ms))
+                    return fail(SPDNN_E_DEVICE, "timed out waiting for the persistent launch of layers " + std::to_string(pl.l0) +
+                                                    ".." + std::to_string(pl.l0 + pl.c - 1) + " (the device did not finish it)");
+                const hipError_t q = hipStreamQuery(n->stream);
+                if (q == hipSuccess) break;   // everything queued has run: the word is final
+                if (q != hipErrorNotReady) return fail(SPDNN_E_DEVICE, std::string("hipStreamQuery: ") + hipGetErrorString(q));
+            }
+            if (n->run_verbose)
+                fprintf(stderr, "spdnn: persistent launch %d (layers %d..%d): word %d of %d units\n", pl.slot, pl.l0,
+                        pl.l0 + pl.c - 1, (int)h[pl.slot], pl.units);
+            if (h[pl.slot] != pl.units) { *failed = 0; return SPDNN_OK; }
+            pending.pop_front();
+        }
+        return SPDNN_OK;
+    };
+    // Goes back to the start of pending[idx], which did not complete: waits for the device, reads how far every row
+    // block got, and has the layer loop run that launch's layers again as per-layer launches; persistent launches
+    // are off for the rest of the run.
+    auto fall_back = [&](int idx) -> int {
+        const PLaunch pl = pending[(size_t)idx];
+        HIPCHK(hipStreamSynchronize(n->stream));
+        std::vector<int32_t> done((size_t)pl.c * (size_t)n->done_stride);
+        HIPCHK(hipMemcpy(done.data(), n->d_done + (size_t)pl.l0 * n->done_stride, done.size() * 4, hipMemcpyDeviceToHost));
+        std::vector<int32_t> frontier((size_t)n->done_stride, 0);
+        for (int rb = 0; rb < pl.nblk; ++rb) {
+            int j = 0;
+            while (j < pl.c && done[(size_t)j * n->done_stride + rb] >= pl.nseg) ++j;
+            frontier[(size_t)rb] = j;
+        }
+        HIPCHK(hipMemcpy(n->d_frontier, frontier.data(), frontier.size() * 4, hipMemcpyHostToDevice));
+        HIPCHK(hipMemset(n->d_abort, 0, 4));
+        if (n->run_verbose) {
+            fprintf(stderr, "spdnn: persistent launch %d (layers %d..%d) did not complete; layers done per row block:", pl.slot,
+                    pl.l0, pl.l0 + pl.c - 1);
+            for (int rb = 0; rb < pl.nblk; ++rb) fprintf(stderr, " %d", frontier[(size_t)rb]);
+            fprintf(stderr, "\n");
+        }
+        const int lo = pl.at.count_pending ? std::max(first, pl.l0 - 1) : pl.l0;   // counts from here on are taken again
+        if (fused_count) HIPCHK(hipMemset(n->d_counts + lo, 0, (size_t)(last - lo + 1) * 4));
+        if (polled) {
+            volatile int32_t* h = n->h_counts;
+            for (int l = lo; l <= last; ++l) h[l] = -1;
+        }
+        const int fallbacks = st.r.persistent_fallbacks + 1;
+        restore(pl.at);
+        st.r.persistent_fallbacks = fallbacks;
+        pending.clear();
+        fb_l0 = pl.l0;
+        fb_c = pl.c;
+        persist_on = false;
+        return SPDNN_OK;
+    };
 
     HIPCHK(hipEventRecord(n->ev_start, n->stream));
-    for (int l = first; l <= last;) {
-        const LayerPlan& p = n->layers[(size_t)l];
-        if (dead) {  // every row died earlier: the remaining outputs are all zero
-            r.edges += (double)n->batch * (double)p.info.nnz;
-            n->cur_layer = ++l;
-            continue;
-        }
-        // chain length: consecutive BAND layers with the same row length and weight mode
-        int c = 1;
-        // a fused pair (intermediate tile in LDS) where the inspector found one; not while the band
-        // walk's BLOCK form would run the layers (small batches of run-chain layers)
-        // (the size threshold belongs to the default; a caller that asks for fused launches gets them)
-        const bool pair = pair_mode && p.fuse_next && l + 1 <= last && !use_block_form(n, p, n->carried / n->RB) &&
-                          (opt.fuse_layers >= 2 ||
-                           (int64_t)(n->carried / n->RB) * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems);
-        if (pair) c = 2;
-        else if (fuse > 1 && p.kernel == SPDNN_KERNEL_BAND) {
-            while (c < fuse && l + c <= last) {
-                const LayerPlan& q = n->layers[(size_t)(l + c)];
-                if (q.kernel != SPDNN_KERNEL_BAND || q.kmax != p.kmax || q.wmode != p.wmode ||
-                    band_unrolled(q.kmax, q.pair_steps, q.pair_stride) != band_unrolled(p.kmax, p.pair_steps, p.pair_stride))
-                    break;
-                ++c;
+    for (;;) {   // once; again from its start after a persistent launch that did not complete
+        int failed = -1;
+        while (st.l <= last && failed < 0) {
+            const int l = st.l;
+            const LayerPlan& p = n->layers[(size_t)l];
+            if (st.dead) {  // every row died earlier: the remaining outputs are all zero
+                st.r.edges += (double)n->batch * (double)p.info.nnz;
+                n->cur_layer = ++st.l;
+                continue;
             }
-        }
-        for (int j = 0; j < c; ++j) r.edges += (double)n->batch * (double)n->layers[(size_t)(l + j)].info.nnz;
-        const int nblk = n->carried / n->RB;
-        // the layer before this launch, if the row slots still carry its stamps: its rows are
-        // counted by this launch (unless a chain or a scan has counted them already), and with
-        // pruning the row blocks it left without an active row are skipped
-        const int prev_stamp = n->last_stamp;
-        // (a run without pruning that continues a pruned one keeps skipping: the blocks skipped
-        // so far hold stale values, and with bias <= 0 a dead row stays dead, so skipping is exact)
-        const int check_dead = (opt.prune || n->blocks_skipped) ? 1 : 0;
-        if (check_dead && (prev_stamp != 0 || c > 1)) n->blocks_skipped = true;
-        int32_t* const count_prev = (fused_count && count_pending && prev_stamp != 0) ? n->d_counts + (l - 1) : nullptr;
-        const Feat in = n->cur;
-        Feat out = (n->cur == n->A) ? n->C : n->A;
-        // band tile shape and segment length: the record for this row-block count, else the next
-        // candidate of the exploration (timed), else the launcher's own heuristic
-        int shape = -1, seglen = 0;
-        bool trial = false;
-        spdnn_net::Trial tr{};
-        if (c == 1 && p.kernel == SPDNN_KERNEL_BAND && !use_block_form(n, p, nblk)) {
-            if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) {
-                shape = t->shape;
-                seglen = t->seglen;
-            } else if (n->autotune) {
-                spdnn_net::Explore* e = explore_for(n, nblk, p.kmax, last - l + 1);
-                if (e && e->issued < kTrialSamples * (int)e->cands.size()) {
-                    const int ci = e->issued++ % (int)e->cands.size();
-                    shape = e->cands[(size_t)ci].shape;
-                    seglen = e->cands[(size_t)ci].seglen;
-                    while (n->ev_free.size() < 2) {
-                        hipEvent_t ev;
-                        HIPCHK(hipEventCreate(&ev));
-                        n->ev_free.push_back(ev);
-                    }
-                    tr = {e->nblk, e->K, ci, n->ev_free[n->ev_free.size() - 1], n->ev_free[n->ev_free.size() - 2]};
-                    n->ev_free.resize(n->ev_free.size() - 2);
-                    trial = true;
+            const int nblk = n->carried / n->RB;
+            const bool fb = l == fb_l0;   // the layers of a launch that gave up, now one by one
+            // a fused pair (intermediate tile in LDS) where the inspector found one; not while the band
+            // walk's BLOCK form would run the layers (small batches of run-chain layers)
+            // (the size threshold belongs to the default; a caller that asks for fused launches gets them)
+            auto is_pair = [&](int k) {
+                const LayerPlan& pk = n->layers[(size_t)k];
+                return pair_mode && pk.fuse_next && k + 1 <= last && !use_block_form(n, pk, nblk) &&
+                       (opt.fuse_layers >= 2 || (int64_t)nblk * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems);
+            };
+            const bool pair = !fb && is_pair(l);
+            // a persistent launch: consecutive layers of one kernel form and variant
+            int c = pair ? 2 : 1;
+            bool persist = false;
+            LayerSig sig;
+            if (fb) {
+                c = fb_c;
+            } else if (!pair && persist_on) {
+                sig = layer_sig(n, l, nblk);
+                const bool small = 8ll * (long long)n->carried * (long long)n->N <= n->persist_max_bytes;
+                int cmax = std::min(persist_cmax, last - l + 1);
+                if (opt.prune && !persist_asked) cmax = std::min(cmax, st.c_prune);   // short launches while the counts still move
+                if (sig.form >= 0 && (persist_asked || small) && cmax >= 2 && next_slot < n->L) {
+                    int k = 1;
+                    while (k < cmax && !is_pair(l + k) && layer_sig(n, l + k, nblk) == sig) ++k;   // (a fused pair stays a pair)
+                    if (k >= 2) { c = k; persist = true; }
                 }
             }
-        }
-        const int stamp0 = n->stamp + 1;
-        n->stamp += c;
-        if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
-        if (c == 1) {
-            HIPCHK(plan_acquire(n, l));
-            if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
-            HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, check_dead, count_prev, shape, seglen, pub));
-            if (trial) {
-                HIPCHK(hipEventRecord(tr.e1, n->stream));
-                n->trials.push_back(tr);
-                int rc = resolve_trials(n, 3);
+            // launches of other kinds must not run on the ruins of a persistent launch: see it complete first
+            if (!persist && !pending.empty()) {
+                const int rc = settle(true, INT_MAX, &failed);
                 if (rc) return rc;
+                if (failed >= 0) break;
             }
-            HIPCHK(plan_release(n, l));
-        } else if (pair) {
-            const LayerPlan& q = n->layers[(size_t)l + 1];
-            const DevLayer &da = n->dl[(size_t)l], &db = n->dl[(size_t)l + 1];
-            PairLaunch pl{};
-            pl.yin = in; pl.yout = out; pl.pairs_a = da.pairs; pl.pw_a = da.wv; pl.pairs_b = db.pairs; pl.pw_b = db.wv;
-            pl.dst = db.dst; pl.active = n->d_active; pl.active_mid = n->d_active_mid; pl.count_prev = count_prev;
-            pl.N = n->N; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = p.wmode; pl.add_only = n->add_only;
-            pl.halo_a = p.info.band_halo; pl.steps_a = p.pair_steps; pl.halo_b = q.info.band_halo; pl.steps_b = q.pair_steps;
-            pl.stamp_a = stamp0; pl.stamp_b = stamp0 + 1; pl.prev_stamp = prev_stamp; pl.check_dead = check_dead;
-            pl.seglen = n->pair_seglen; pl.n_cu = n->n_cu; pl.stream_min_bytes = n->stream_min_bytes;
-            pl.wu_a = p.info.value; pl.wu_b = q.info.value; pl.bias = n->bias; pl.clampv = n->clampv;
-            pl.publish = pub;
-            HIPCHK(launch_band_pair(pl, n->stream));
-            // the first layer's rows: nobody looks at active_mid again, so they are counted here
-            if (fused_count) HIPCHK(launch_count_stamped(n->d_active_mid, n->carried, stamp0, n->d_counts + l, n->stream));
-        } else {
-            ChainLaunch ch{};
-            ch.table = n->d_chain + l; ch.nlayers = c; ch.first_in = in; ch.buf_a = n->A; ch.buf_c = n->C;
-            ch.active = n->d_active; ch.count_out = fused_count ? n->d_counts + l : nullptr;
-            ch.count_prev = count_prev; ch.check_dead = check_dead;
-            ch.N = n->N; ch.K = p.kmax; ch.nblk = nblk; ch.stamp0 = stamp0; ch.prev_stamp = prev_stamp;
-            ch.rl = n->rl; ch.wmode = p.wmode; ch.stop_when_dead = check_dead;
-            ch.unrolled = band_unrolled(p.kmax, p.pair_steps, p.pair_stride) ? 1 : 0;
-            ch.bias = n->bias; ch.clampv = n->clampv;
-            ch.halves = n->chain_halves;
-            ch.add_only = n->add_only;
-            ch.publish = pub;
-            HIPCHK(launch_band_chain(ch, n->stream));
-            for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
-        }
-        if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back({l, c}); }
-        r.layers_run += c;
-        r.launches += 1;
-        if (pair) r.fused_pairs += 1;
-        last_launched = l + c - 1;
-        n->last_stamp = stamp0 + c - 1;
-        n->cur = out;
-        n->cur_layer = l + c;
-        if (scan_count) {
-            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
-                                      n->d_alive_gid, n->stream));
-            HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
-        }
-        if (fused_count) {
-            // Counts that are final once this launch has finished: the previous layer's (counted at
-            // this launch's start) and, of a fused launch, its own layers'.  The next launch hands
-            // them to the host; this launch handed over the ones before (pub).
-            if (polled && pub.n > 0) recs.push_back({(int)(pub.src - n->d_counts), pub.n});
-            // (a chain counts all its layers itself; of a pair the first layer is counted behind the
-            // launch and the second, like a single layer, by whatever comes next)
-            const int lo = count_prev ? l - 1 : l, hi = c == 1 ? l : (pair ? l + 1 : l + c);
-            pub = Publish{};
-            if (polled && hi > lo) { pub.src = n->d_counts + lo; pub.dst = n->h_counts + lo; pub.n = hi - lo; }
-            count_pending = c == 1 || pair;
-        }
-        l += c;
-        if (!opt.prune) continue;
-
-        // a record is pushed when the launch that hands it over is queued, i.e. one launch late
-        const size_t lookahead = lookahead_for(n->carried) - 1;
-        while (recs.size() - processed > lookahead && !dead) {
-            const Rec rc = recs[processed++];
-            const int wrc = wait_counts(n, rc.l0, rc.c);
-            if (wrc) return wrc;
-            for (int j = rc.l0; j < rc.l0 + rc.c && !dead; ++j) {
-                newest_count = n->h_counts[j];
-                if (newest_count == 0) dead = true;
-            }
-        }
-        if (dead) { n->carried = 0; continue; }
-        if (newest_count > 0 && (double)newest_count <= (double)thr * (double)n->carried && l < n->L) {
-            const int nb = (int)((newest_count + n->RB - 1) / n->RB);  // upper bound of what is alive now
-            if (nb * n->RB < n->carried) {
-                const Feat dstbuf = (n->cur == n->A) ? n->C : n->A;
-                HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count,
-                                          n->d_alive_src, n->d_alive_gid, n->stream));
-                if (count_pending) {  // the scan has just counted the newest layer's rows
-                    HIPCHK(hipMemcpyAsync(n->d_counts + (l - 1), n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
-                    count_pending = false;
+            for (int j = 0; j < c; ++j) st.r.edges += (double)n->batch * (double)n->layers[(size_t)(l + j)].info.nnz;
+            // the layer before this launch, if the row slots still carry its stamps: its rows are
+            // counted by this launch (unless a scan has counted them already), and with
+            // pruning the row blocks it left without an active row are skipped
+            const int prev_stamp = n->last_stamp;
+            // (a run without pruning that continues a pruned one keeps skipping: the blocks skipped
+            // so far hold stale values, and with bias <= 0 a dead row stays dead, so skipping is exact)
+            const int check_dead = (opt.prune || n->blocks_skipped) ? 1 : 0;
+            State at_start{};
+            if (persist) at_start = save();
+            if (check_dead && (prev_stamp != 0 || c > 1)) n->blocks_skipped = true;
+            const bool group = persist || fb;   // c layers whose rows are counted behind them, from the stamps
+            int32_t* const count_prev = (fused_count && st.count_pending && prev_stamp != 0 && !group) ? n->d_counts + (l - 1) : nullptr;
+            const Feat in = n->cur;
+            Feat out = (n->cur == n->A) ? n->C : n->A;
+            // band tile shape and segment length: the record for this row-block count, else the next
+            // candidate of the exploration (timed), else the launcher's own heuristic
+            int shape = -1, seglen = 0;
+            bool trial = false;
+            spdnn_net::Trial tr{};
+            if (c == 1 && p.kernel == SPDNN_KERNEL_BAND && !use_block_form(n, p, nblk)) {
+                if (const spdnn_net::Tuned* t = find_tuned(n, nblk, p.kmax)) {
+                    shape = t->shape;
+                    seglen = t->seglen;
+                } else if (n->autotune && n->band_seglen == 0) {
+                    spdnn_net::Explore* e = explore_for(n, nblk, p.kmax, last - l + 1);
+                    if (e && e->issued < kTrialSamples * (int)e->cands.size()) {
+                        const int ci = e->issued++ % (int)e->cands.size();
+                        shape = e->cands[(size_t)ci].shape;
+                        seglen = e->cands[(size_t)ci].seglen;
+                        while (n->ev_free.size() < 2) {
+                            hipEvent_t ev;
+                            HIPCHK(hipEventCreate(&ev));
+                            n->ev_free.push_back(ev);
+                        }
+                        tr = {e->nblk, e->K, ci, n->ev_free[n->ev_free.size() - 1], n->ev_free[n->ev_free.size() - 2]};
+                        n->ev_free.resize(n->ev_free.size() - 2);
+                        trial = true;
+                    }
                 }
-                HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
-                                     n->N, n->rl, nb, n->stream));
-                std::swap(n->d_gid, n->d_gid_tmp);
-                n->gid_dirty = true;
-                n->cur = dstbuf;
-                n->carried = nb * n->RB;
-                n->last_stamp = 0;  // the row slots moved: the stamps no longer describe them
-                n->blocks_skipped = false;  // every carried block has just been written
-                r.compactions++;
+            }
+            const int stamp0 = n->stamp + 1;
+            n->stamp += c;
+            if (opt.time_layers) HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l)], n->stream));
+            if (persist) {
+                PersistLaunch pl{};
+                pl.table = n->d_table + l; pl.nlayers = c; pl.block_form = sig.form; pl.first_in = in; pl.buf_a = n->A; pl.buf_c = n->C;
+                pl.active = n->d_active; pl.done = n->d_done + (size_t)l * n->done_stride; pl.done_stride = n->done_stride;
+                pl.ngroups = sig.ngroups; pl.ctl = n->d_ctl + next_slot;
+                pl.prev_ctl = pending.empty() ? nullptr : n->d_ctl + pending.back().slot;
+                pl.prev_units = pending.empty() ? 0 : pending.back().units;
+                pl.abort = n->d_abort; pl.host_word = n->h_pwords + next_slot;
+                pl.N = n->N; pl.K = sig.K; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = sig.wmode; pl.stamp0 = stamp0;
+                pl.prev_stamp = prev_stamp; pl.check_dead = check_dead; pl.unrolled = sig.unrolled; pl.add_only = n->add_only;
+                pl.twins = sig.twins; pl.full = sig.full; pl.seglen = n->persist_seglen;
+                // one queue per XCD where the row blocks of an XCD keep their input and output in its L2 (4 MiB)
+                const size_t block_bytes = (size_t)n->N * (size_t)n->RB * 4;
+                pl.xcd_queues = n->persist_xcd >= 0 ? (n->persist_xcd ? 1 : 0)
+                                                    : (nblk >= 3 && (size_t)((nblk + 7) / 8) * block_bytes * 2 <= ((size_t)4 << 20) ? 1 : 0);
+                pl.light_sync = n->persist_light;
+                pl.wait_limit = persist_wait_us * 100;
+                pl.n_cu = n->n_cu; pl.stream_min_bytes = n->stream_min_bytes; pl.bias = n->bias; pl.clampv = n->clampv;
+                pl.publish = st.pub;
+                volatile int32_t* hw = n->h_pwords;
+                hw[next_slot] = -1;
+                HIPCHK(launch_persist(pl, n->stream));
+                PLaunch rec{};
+                rec.at = at_start; rec.l0 = l; rec.c = c; rec.nblk = nblk; rec.units = persist_units(pl);
+                rec.nseg = rec.units / (nblk * c); rec.slot = next_slot++;
+                pending.push_back(rec);
+                if (n->run_verbose)
+                    fprintf(stderr, "spdnn: persistent launch %d: layers %d..%d, %d row blocks, form %d, %d units/row block, %d units, "
+                                    "xcd queues %d, light %d\n", rec.slot, l, l + c - 1, nblk, sig.form, rec.nseg, rec.units,
+                            pl.xcd_queues, pl.light_sync);
+                for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
+                st.r.persistent_launches += 1;
+            } else if (fb) {
+                Feat fin = in, fout = out;
+                for (int j = 0; j < c; ++j) {
+                    int sh = -1, sl = 0;
+                    const LayerPlan& pj = n->layers[(size_t)(l + j)];
+                    if (const spdnn_net::Tuned* t = find_tuned(n, nblk, pj.kmax)) { sh = t->shape; sl = t->seglen; }
+                    HIPCHK(launch_layer(n, l + j, fin, fout, nblk, stamp0 + j, j == 0 ? prev_stamp : stamp0 + j - 1, check_dead,
+                                        nullptr, sh, sl, j == 0 ? st.pub : Publish{}, n->d_frontier, j));
+                    out = fout;
+                    fin = fout;
+                    fout = (fout == n->A) ? n->C : n->A;
+                }
+                fb_l0 = -1;
+            } else if (c == 1) {
+                HIPCHK(plan_acquire(n, l));
+                if (trial) HIPCHK(hipEventRecord(tr.e0, n->stream));
+                HIPCHK(launch_layer(n, l, in, out, nblk, stamp0, prev_stamp, check_dead, count_prev, shape, seglen, st.pub));
+                if (trial) {
+                    HIPCHK(hipEventRecord(tr.e1, n->stream));
+                    n->trials.push_back(tr);
+                    int rc = resolve_trials(n, 3);
+                    if (rc) return rc;
+                }
+                HIPCHK(plan_release(n, l));
+            } else {
+                const LayerPlan& q = n->layers[(size_t)l + 1];
+                const DevLayer &da = n->dl[(size_t)l], &db = n->dl[(size_t)l + 1];
+                PairLaunch pl{};
+                pl.yin = in; pl.yout = out; pl.pairs_a = da.pairs; pl.pw_a = da.wv; pl.pairs_b = db.pairs; pl.pw_b = db.wv;
+                pl.dst = db.dst; pl.active = n->d_active; pl.active_mid = n->d_active_mid; pl.count_prev = count_prev;
+                pl.N = n->N; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = p.wmode; pl.add_only = n->add_only;
+                pl.halo_a = p.info.band_halo; pl.steps_a = p.pair_steps; pl.halo_b = q.info.band_halo; pl.steps_b = q.pair_steps;
+                pl.stamp_a = stamp0; pl.stamp_b = stamp0 + 1; pl.prev_stamp = prev_stamp; pl.check_dead = check_dead;
+                pl.seglen = n->pair_seglen; pl.n_cu = n->n_cu; pl.stream_min_bytes = n->stream_min_bytes;
+                pl.wu_a = p.info.value; pl.wu_b = q.info.value; pl.bias = n->bias; pl.clampv = n->clampv;
+                pl.publish = st.pub;
+                HIPCHK(launch_band_pair(pl, n->stream));
+                // the first layer's rows: nobody looks at active_mid again, so they are counted here
+                if (fused_count) HIPCHK(launch_count_stamped(n->d_active_mid, n->carried, stamp0, n->d_counts + l, n->stream));
+            }
+            if (opt.time_layers) { HIPCHK(hipEventRecord(n->ev_layer[(size_t)(2 * l + 1)], n->stream)); timed.push_back({l, c}); }
+            st.r.layers_run += c;
+            st.r.launches += (fb ? c : 1);
+            if (pair) st.r.fused_pairs += 1;
+            st.last_launched = l + c - 1;
+            n->last_stamp = stamp0 + c - 1;
+            n->cur = out;
+            n->cur_layer = l + c;
+            if (scan_count) {
+                HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
+                                          n->d_alive_gid, n->stream));
+                HIPCHK(hipMemcpyAsync(n->d_counts + l, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
+            }
+            if (fused_count && group) {
+                // The rows the layers of the launch left active, from the stamps behind it: a row that carries the
+                // stamp of layer j or of a later one was active after layer j (bias <= 0: a zero row stays zero).
+                // The layer before the launch is counted the same way if nobody has counted it yet.  The kernel
+                // hands its counts to the host itself.
+                const bool with_prev = st.count_pending && prev_stamp != 0 && prev_stamp == stamp0 - 1;
+                const int lo = with_prev ? l - 1 : l, cnt = c + (with_prev ? 1 : 0);
+                HIPCHK(launch_count_stamp_range(n->d_active, n->carried, with_prev ? prev_stamp : stamp0, cnt, n->d_counts + lo,
+                                                polled ? n->h_counts + lo : nullptr, n->stream));
+                if (polled) {
+                    if (st.pub.n > 0) recs.push_back({(int)(st.pub.src - n->d_counts), st.pub.n, -1});
+                    recs.push_back({lo, cnt, persist ? next_slot - 1 : -1});
+                }
+                st.pub = Publish{};
+                st.count_pending = false;
+            } else if (fused_count) {
+                // Counts that are final once this launch has finished: the previous layer's (counted at
+                // this launch's start) and, of a fused pair, its first layer's.  The next launch hands
+                // them to the host; this launch handed over the ones before (pub).
+                if (polled && st.pub.n > 0) recs.push_back({(int)(st.pub.src - n->d_counts), st.pub.n, -1});
+                // (of a pair the first layer is counted behind the launch and the second, like a single
+                // layer, by whatever comes next)
+                const int lo = count_prev ? l - 1 : l, hi = pair ? l + 1 : l;
+                st.pub = Publish{};
+                if (polled && hi > lo) { st.pub.src = n->d_counts + lo; st.pub.dst = n->h_counts + lo; st.pub.n = hi - lo; }
+                st.count_pending = true;
+            }
+            st.l = l + c;
+            if (!opt.prune) continue;
+
+            // a record is pushed when the launch that hands it over is queued, i.e. one launch late
+            const size_t lookahead = lookahead_for(n->carried) - 1;
+            while (recs.size() - st.processed > lookahead && !st.dead && failed < 0) {
+                const Rec rc = recs[st.processed++];
+                const int wrc = wait_counts(n, rc.l0, rc.c);
+                if (wrc) return wrc;
+                if (rc.pl >= 0) {   // counts taken behind a persistent launch mean something only if it completed
+                    const int src = settle(true, rc.pl, &failed);
+                    if (src) return src;
+                    if (failed >= 0) break;
+                }
+                const int64_t before = st.newest_count;
+                for (int j = rc.l0; j < rc.l0 + rc.c && !st.dead; ++j) {
+                    st.newest_count = n->h_counts[j];
+                    if (st.newest_count == 0) st.dead = true;
+                }
+                // layers per persistent launch while pruning: doubled while the counts hold still (within 3 % from
+                // one record to the next), one layer per launch again when they move
+                if (before > 0 && st.newest_count * 100 >= before * 97) st.c_prune = std::min(persist_cmax, std::max(2, st.c_prune * 2));
+                else st.c_prune = 1;
+            }
+            if (failed >= 0) break;
+            if (st.dead) { n->carried = 0; continue; }
+            if (st.newest_count > 0 && (double)st.newest_count <= (double)thr * (double)n->carried && st.l < n->L) {
+                const int nb = (int)((st.newest_count + n->RB - 1) / n->RB);  // upper bound of what is alive now
+                if (nb * n->RB < n->carried) {
+                    if (!pending.empty()) {   // the repack overwrites a work buffer: not on the ruins of a persistent launch
+                        const int rc = settle(true, INT_MAX, &failed);
+                        if (rc) return rc;
+                        if (failed >= 0) break;
+                    }
+                    const Feat dstbuf = (n->cur == n->A) ? n->C : n->A;
+                    HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count,
+                                              n->d_alive_src, n->d_alive_gid, n->stream));
+                    if (st.count_pending) {  // the scan has just counted the newest layer's rows
+                        HIPCHK(hipMemcpyAsync(n->d_counts + (st.l - 1), n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
+                        st.count_pending = false;
+                    }
+                    HIPCHK(launch_repack(n->cur, dstbuf, n->d_count, n->d_alive_src, n->d_alive_gid, n->d_gid_tmp,
+                                         n->N, n->rl, nb, n->stream));
+                    std::swap(n->d_gid, n->d_gid_tmp);
+                    n->gid_dirty = true;
+                    n->cur = dstbuf;
+                    n->carried = nb * n->RB;
+                    n->last_stamp = 0;  // the row slots moved: the stamps no longer describe them
+                    n->blocks_skipped = false;  // every carried block has just been written
+                    st.r.compactions++;
+                }
             }
         }
-    }
-    // categories of the last layer: survivor list by the scan.  After a final repack the list
-    // produced for the repack is that list already.
-    n->alive_list_valid = false;
-    if (!dead && last_launched == last) {
-        if (n->last_stamp != 0) {
-            HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
-                                      n->d_alive_gid, n->stream));
+        if (failed < 0) {
+            // categories of the last layer: survivor list by the scan.  After a final repack the list
+            // produced for the repack is that list already.
+            n->alive_list_valid = false;
+            if (!st.dead && st.last_launched == last) {
+                if (n->last_stamp != 0) {
+                    HIPCHK(launch_scan_active(n->d_active, n->d_gid, n->carried, n->last_stamp, n->d_count, n->d_alive_src,
+                                              n->d_alive_gid, n->stream));
+                }
+                HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
+                if (st.count_pending)  // no launch follows the last layer: the scan's count is its count
+                    HIPCHK(hipMemcpyAsync(n->d_counts + last, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
+                n->alive_list_valid = true;
+            }
+            HIPCHK(hipEventRecord(n->ev_stop, n->stream));
+            if (have_counts && st.last_launched >= first)   // all of them once more (the last launch's have no launch after it)
+                HIPCHK(hipMemcpyAsync(n->h_counts + first, n->d_counts + first, (size_t)(st.last_launched - first + 1) * 4,
+                                      hipMemcpyDeviceToHost, n->stream));
+            HIPCHK(hipStreamSynchronize(n->stream));
+            if (plans_streamed(n)) HIPCHK(hipStreamSynchronize(n->copy_stream));
+            // everything has run: the completion words are final
+            const int rc = settle(false, INT_MAX, &failed);
+            if (rc) return rc;
+            if (failed < 0 && !pending.empty()) failed = 0;   // a word still missing: that launch never finished its units
+            if (failed < 0) break;
         }
-        HIPCHK(hipMemcpyAsync(n->h_count, n->d_count, 4, hipMemcpyDeviceToHost, n->stream));
-        if (count_pending)  // no launch follows the last layer: the scan's count is its count
-            HIPCHK(hipMemcpyAsync(n->d_counts + last, n->d_count, 4, hipMemcpyDeviceToDevice, n->stream));
-        n->alive_list_valid = true;
+        const int rc = fall_back(failed);
+        if (rc) return rc;
     }
-    HIPCHK(hipEventRecord(n->ev_stop, n->stream));
-    if (have_counts && last_launched >= first)   // all of them once more (the last launch's have no launch after it)
-        HIPCHK(hipMemcpyAsync(n->h_counts + first, n->d_counts + first, (size_t)(last_launched - first + 1) * 4,
-                              hipMemcpyDeviceToHost, n->stream));
-    HIPCHK(hipStreamSynchronize(n->stream));
-    if (plans_streamed(n)) HIPCHK(hipStreamSynchronize(n->copy_stream));
     {
         int rc = resolve_trials(n, 0);
         if (rc) return rc;
     }
+    spdnn_run_result& r = st.r;
     HIPCHK(hipEventElapsedTime(&r.ms_total, n->ev_start, n->ev_stop));
     for (const Timed& t : timed) {
         float ms = 0.0f;
@@ -1697,6 +2007,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
         r.ms_kernels += ms;
     }
     // per-layer counts: everything that was launched has finished now
+    const int last_launched = st.last_launched;
     bool zero_seen = false;
     for (int l = first; l <= last; ++l) {
         if (zero_seen) { n->counts[(size_t)l] = 0; continue; }
@@ -1704,7 +2015,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
         else if (l > last_launched) n->counts[(size_t)l] = (last_launched >= first || n->carried == 0) ? 0 : -1;
         if (n->counts[(size_t)l] == 0) zero_seen = true;
     }
-    if (dead || zero_seen) { if (opt.prune) n->carried = 0; n->alive = 0; }
+    if (st.dead || zero_seen) { if (opt.prune) n->carried = 0; n->alive = 0; }
     else if (n->alive_list_valid) n->alive = n->h_count[0];
     if (n->alive == 0) n->alive_list_valid = true;  // the empty list
     // byte model: rows entering each launched layer
@@ -1910,11 +2221,18 @@ static int spdnn_device_info_impl(char* name, int cap, int* compute_units, int64
     return SPDNN_OK;
 }
 
-static int spdnn_get_feature_placement_impl(const spdnn_net* n, int* paired, int* candidates) {
+static int spdnn_get_feature_placement_impl(const spdnn_net* n, int* paired, int* candidates, int64_t* search_peak_bytes) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     if (!n->uploaded) return fail(SPDNN_E_STATE, "no feature buffers yet");
     if (paired) *paired = n->feat_paired;
     if (candidates) *candidates = n->feat_candidates;
+    if (search_peak_bytes) *search_peak_bytes = (int64_t)n->search_peak_bytes;
+    return SPDNN_OK;
+}
+
+static int spdnn_device_alloc_calls_impl(int64_t* calls) {
+    if (!calls) return fail(SPDNN_E_ARG, "calls is NULL");
+    *calls = g_dev_allocs.load(std::memory_order_relaxed);
     return SPDNN_OK;
 }
 
@@ -2053,8 +2371,11 @@ int spdnn_measure_buffer_copy_bandwidth(spdnn_net* n, int reps, double* gbps) {
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes) {
     return guarded([&] { return spdnn_device_info_impl(name, cap, compute_units, hbm_bytes); });
 }
-int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates) {
-    return guarded([&] { return spdnn_get_feature_placement_impl(n, paired, candidates); });
+int spdnn_get_feature_placement(const spdnn_net* n, int* paired, int* candidates, int64_t* search_peak_bytes) {
+    return guarded([&] { return spdnn_get_feature_placement_impl(n, paired, candidates, search_peak_bytes); });
+}
+int spdnn_device_alloc_calls(int64_t* calls) {
+    return guarded([&] { return spdnn_device_alloc_calls_impl(calls); });
 }
 int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes) {
     return guarded([&] { return spdnn_device_memory_impl(free_bytes, total_bytes); });

@@ -93,7 +93,10 @@ typedef struct spdnn_run_options {
                                   = n makes n the default).  >1: the pairs, and elsewhere up to that many
                                   consecutive band layers share a launch (one workgroup keeps a row block
                                   through the chain, the intermediates going through L2) */
-    int32_t reserved[3];
+    int32_t persist_wait_us;   /* persistent launches: longest wait of a unit for its row block in microseconds; 0 = default
+                                  (2 s, SPDNN_PERSIST_WAIT_US), negative = give up at the first look that finds the row
+                                  block not ready (exercises the fall-back to per-layer launches)                     */
+    int32_t reserved[2];
 } spdnn_run_options;
 
 typedef struct spdnn_run_result {
@@ -107,6 +110,8 @@ typedef struct spdnn_run_result {
     double  edges;           /* batch * nnz summed over the layers requested                      */
     int32_t launches;        /* layer-kernel launches made (a fused launch counts once)           */
     int32_t fused_pairs;     /* of them, fused pairs of layers (intermediate tile in LDS)         */
+    int32_t persistent_launches;   /* of them, persistent launches (several layers, a dependency per row block)   */
+    int32_t persistent_fallbacks;  /* persistent launches that gave up and were finished by per-layer launches     */
 } spdnn_run_result;
 
 /* ---- life cycle ------------------------------------------------------------------------- */
@@ -299,9 +304,10 @@ int spdnn_get_categories(spdnn_net* net, int32_t* ids, int64_t cap, int64_t* n);
  * (all_network.cu:521). */
 int spdnn_get_activations(spdnn_net* net, const int32_t* rows, int nrows, float* rowmajor);
 
-/* spdnn_get_activations for callers that cannot allocate device memory (code under HIP graph
- * capture around it, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
- * reference.  Same arguments and results as spdnn_get_activations, but where that call allocates
+/* spdnn_get_activations for callers that cannot allocate device memory (tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  It allocates nothing, but it
+ * is not a call for inside a HIP graph capture: it synchronises its stream once per pass and copies
+ * to and from pageable host memory.  Same arguments and results as spdnn_get_activations, but where that call allocates
  * its row list and its row-major staging rows for every call, this one calls no hipMalloc / hipFree:
  * it works in a 12.1 MiB scratch array that is part of the library's device code (one copy per GPU,
  * held until the process ends): a row table (global id -> physical row, filled by two small
@@ -341,9 +347,12 @@ int spdnn_measure_buffer_copy_bandwidth(spdnn_net* net, int reps, double* gbps);
 int spdnn_device_info(char* name, int cap, int* compute_units, int64_t* hbm_bytes);
 
 /* How the feature buffers were placed (after features were set): *paired = 1 if the two halves of
- * every buffer lie in different memory regions (searched for buffers of 8 GiB and more, see
- * SPDNN_REGION_PAIRING), *candidates = half-buffers allocated during the search (6 = no search). */
-int spdnn_get_feature_placement(const spdnn_net* net, int* paired, int* candidates);
+ * every buffer lie in different memory regions (searched for half-buffers of 0.4 GiB and more, see
+ * SPDNN_REGION_PAIRING), *candidates = half-buffers allocated during the search (6 = no search),
+ * *search_peak_bytes = device memory the search held at its peak (candidates and the fillers between
+ * them; everything beyond the six half-buffers kept was freed again before the call returned).  Any
+ * pointer may be NULL. */
+int spdnn_get_feature_placement(const spdnn_net* net, int* paired, int* candidates, int64_t* search_peak_bytes);
 
 /* Free and total device memory of device 0 in bytes (what hipMemGetInfo reports); either pointer
  * may be NULL.  Sizing aid: a network holds three feature buffers of rows*neuron*4 bytes plus the
@@ -351,6 +360,10 @@ int spdnn_get_feature_placement(const spdnn_net* net, int* paired, int* candidat
 int spdnn_device_memory(int64_t* free_bytes, int64_t* total_bytes);
 
 int spdnn_device_synchronize(void);
+
+/* Number of device allocations (hipMalloc) the library has made in this process so far: a diagnostic for
+ * callers that must know that a call allocates nothing (spdnn_get_activations_noalloc leaves it unchanged). */
+int spdnn_device_alloc_calls(int64_t* calls);
 
 #ifdef __cplusplus
 }

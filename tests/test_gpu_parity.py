@@ -86,6 +86,19 @@ def test_full_chain_cfg0_shape(gc, orc, prune):
             assert r.layers_run < L and r.compactions >= 1
         else:
             assert r.layers_run == L
+        # layer by layer at the real batch: the id set and every row's activations after each layer, until
+        # everything has died (counts alone would not tell which rows survive)
+        ref_u = orc.infer(feats, layers[:12], -0.3, prune=False, keep=set(range(12)))
+        rows = np.arange(B, dtype=np.int32)
+        checked = 0
+        for l in range(12):
+            net.run(prune=prune, first_layer=l, n_layers=1, collect_counts=True)
+            assert np.array_equal(net.categories(), ref["active_ids"][l]), "layer %d" % l
+            assert same_floats(net.activations(rows), ref_u["kept"][l][1]), "layer %d" % l
+            checked += 1
+            if len(ref["active_ids"][l]) == 0:
+                break
+        assert checked >= 3 and len(ref["active_ids"][0]) > 1000
 
 
 def test_survivor_chain_with_compaction(gc, orc):
@@ -398,15 +411,25 @@ def test_full_batch_properties_cfg1(gc, orc):
         assert same_floats(y_p[:k], ref["y"][pos])
 
 
-@pytest.mark.parametrize("halves", [1, 0])
+PERSIST_MODES = {   # how the units of a persistent launch are queued and handed over (environment, read at creation)
+    "default": {},
+    "one-queue": {"SPDNN_PERSIST_XCD": "0"},
+    "xcd-queues": {"SPDNN_PERSIST_XCD": "1"},
+    "xcd-queues-light": {"SPDNN_PERSIST_XCD": "1", "SPDNN_PERSIST_LIGHT_SYNC": "1"},
+}
+
+
+@pytest.mark.parametrize("mode", sorted(PERSIST_MODES))
 @pytest.mark.parametrize("prune", [True, False])
 @pytest.mark.parametrize("fuse", [4, 16])
-def test_fused_layer_chain(gc, orc, fuse, prune, halves, monkeypatch):
-    """The fused variant (several band layers per launch, one workgroup per half or whole row block)
-    must give what the layer-by-layer launches give: counts, categories and activations."""
-    monkeypatch.setenv("SPDNN_CHAIN_HALVES", str(halves))
+def test_persistent_launches(gc, orc, fuse, prune, mode, monkeypatch):
+    """Several band layers per launch with a dependency per row block between the layers must give what the
+    layer-by-layer launches give: counts, categories and activations - with one unit queue or one per XCD,
+    with device-scope fences or the hand-over inside one XCD's L2."""
+    for k, v in PERSIST_MODES[mode].items():
+        monkeypatch.setenv(k, v)
     N, L, B = 1024, 24, 3000
-    print("fused chain fuse=%d prune=%s halves=%d" % (fuse, prune, halves), flush=True)
+    print("persistent launches fuse=%d prune=%s %s" % (fuse, prune, mode), flush=True)
     layers = [orc.gen_layer_csr(5, l, N) for l in range(L)]
     feats = orc.gen_features(5, N, 0, B, 0.10, 0.50)
     ref = orc.infer(feats, layers, -0.3, prune=True)
@@ -416,15 +439,90 @@ def test_fused_layer_chain(gc, orc, fuse, prune, halves, monkeypatch):
         net.set_features_dense(feats)
         r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
         assert r.layers_run == L
+        assert r.persistent_launches >= L // fuse and r.persistent_fallbacks == 0 and r.launches < L
         assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
         cats = net.categories()
         assert np.array_equal(cats, ref["categories"])
         assert same_floats(net.activations(cats), ref["y"])
         dead = np.setdiff1d(np.arange(B), cats)[:64].astype(np.int32)
         assert not net.activations(dead).any()
-        # a chain that stops in the middle of the network and is continued layer by layer
+        # a persistent launch that stops in the middle of the network, continued layer by layer and by another one
         net.run(prune=prune, first_layer=0, n_layers=10, fuse_layers=fuse)
-        net.run(prune=prune, first_layer=10, n_layers=L - 10, fuse_layers=1)
+        net.run(prune=prune, first_layer=10, n_layers=4, fuse_layers=1)
+        net.run(prune=prune, first_layer=14, n_layers=L - 14, fuse_layers=fuse)
+        assert np.array_equal(net.categories(), ref["categories"])
+        assert same_floats(net.activations(cats), ref["y"])
+        # left to the library (fuse_layers = 0): launches of this size are persistent by default
+        r = net.run(prune=False, collect_counts=True)
+        assert r.persistent_launches >= 1 and r.persistent_fallbacks == 0
+        assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+        assert same_floats(net.activations(cats), ref["y"])
+
+
+@pytest.mark.parametrize("mode", ["one-queue", "xcd-queues"])
+@pytest.mark.parametrize("prune", [True, False])
+def test_persistent_launch_that_gives_up(gc, orc, prune, mode, monkeypatch):
+    """A unit of a persistent launch waits for its row block for a bounded time only.  With the limit at zero the
+    launch gives up at the first look that finds a row block not ready: every workgroup leaves, the host reads how
+    far each row block got and finishes the layers with per-layer launches.  Results must not change."""
+    for k, v in PERSIST_MODES[mode].items():
+        monkeypatch.setenv(k, v)
+    N, L, B = 1024, 20, 2600
+    print("persistent launch gives up prune=%s %s" % (prune, mode), flush=True)
+    layers = [orc.gen_layer_csr(6, l, N) for l in range(L)]
+    feats = orc.gen_features(6, N, 0, B, 0.10, 0.55)
+    ref = orc.infer(feats, layers, -0.3, prune=True)
+    with gc.Network(N, B, L) as net:
+        net.synth_layers(6)
+        net.inspect()
+        net.set_features_dense(feats)
+        gave_up = 0
+        for attempt in range(3):
+            r = net.run(prune=prune, collect_counts=True, fuse_layers=8, persist_wait_us=-1)
+            gave_up += r.persistent_fallbacks
+            assert r.layers_run == L
+            assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+            cats = net.categories()
+            assert np.array_equal(cats, ref["categories"])
+            assert same_floats(net.activations(cats), ref["y"])
+        assert gave_up >= 1
+        # and the next run, with the default limit, is persistent again
+        r = net.run(prune=prune, collect_counts=True, fuse_layers=8)
+        assert r.persistent_launches >= 2 and r.persistent_fallbacks == 0
+        assert np.array_equal(net.categories(), ref["categories"])
+        assert same_floats(net.activations(cats), ref["y"])
+
+
+@pytest.mark.parametrize("mode", ["one-queue", "xcd-queues-light"])
+@pytest.mark.parametrize("N,B,values", [(1024, 2100, "uniform"), (1024, 900, "general"), (4096, 1300, "uniform")])
+def test_persistent_launches_block_kernel(gc, orc, N, B, values, mode, monkeypatch):
+    """RadiX-Net-like layers on the BLOCK kernel (narrow layers, and the BLOCK form of run chains on small batches),
+    several layers per launch: bit-equal to the oracle, pruned and unpruned, and to one launch per layer."""
+    for k, v in PERSIST_MODES[mode].items():
+        monkeypatch.setenv(k, v)
+    print("persistent BLOCK launches N=%d B=%d %s %s" % (N, B, values, mode), flush=True)
+    rng = np.random.default_rng(N + B)
+    nst = int(np.log2(N)) - 4
+    base = [radix_like_csr(rng, N, 16 << k, values) for k in range(nst)]
+    L = 2 * nst + 1
+    layers = [base[l % nst] for l in range(L)]
+    dens = np.where(rng.random(B) < 0.3, 0.7, 0.08).astype(np.float32)
+    feats = (rng.random((B, N), dtype=np.float32) < dens[:, None]).astype(np.float32)
+    bias = -0.3 if N == 1024 else -0.35
+    ref = orc.infer(feats, layers, bias, prune=True)
+    with gc.Network(N, B, L, bias=bias) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.set_features_dense(feats)
+        for prune in (True, False):
+            r = net.run(prune=prune, collect_counts=True, fuse_layers=6)
+            assert r.persistent_launches >= 1 and r.persistent_fallbacks == 0
+            assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
+            cats = net.categories()
+            assert np.array_equal(cats, ref["categories"])
+            assert same_floats(net.activations(cats), ref["y"])
+        r = net.run(prune=True, collect_counts=True, fuse_layers=6, persist_wait_us=-1)
         assert np.array_equal(net.categories(), ref["categories"])
         assert same_floats(net.activations(cats), ref["y"])
 
@@ -611,10 +709,10 @@ def test_pruned_run_with_rows_that_never_die(gc, orc, kind, monkeypatch):
         assert np.array_equal(net.categories(), cats)
 
 
-def test_fused_chain_when_everything_dies(gc, orc):
-    """Literal inputs: all rows die within a few layers; workgroups leave the chain early."""
+def test_persistent_launches_when_everything_dies(gc, orc):
+    """Literal inputs: all rows die within a few layers; the units of dead row blocks are skipped."""
     N, L, B = 1024, 40, 2000
-    print("fused chain, all rows die", flush=True)
+    print("persistent launches, all rows die", flush=True)
     layers = [orc.gen_layer_csr(0, l, N) for l in range(12)]
     ref = orc.infer(orc.gen_features(0, N, 0, B), layers, -0.3, prune=True)
     want = [len(a) for a in ref["active_ids"]] + [0] * (L - 12)
@@ -713,8 +811,9 @@ def test_headline_widths_against_oracle_sample(gc, orc, N, B, L, bias):
             assert np.array_equal(cats[cats < S], ref["active_ids"][l]), "layer %d" % l
             assert same_floats(net.activations(rows), ref["kept"][l][1]), "layer %d" % l
         full = net.run(prune=False, collect_counts=True)
-        paired, candidates = net.feature_placement()
-        print("feature buffers paired over two memory regions:", paired, "candidates", candidates, flush=True)
+        paired, candidates, peak = net.feature_placement()
+        print("feature buffers paired over two memory regions:", paired, "candidates", candidates, "search peak GiB %.1f" % (peak / 2**30), flush=True)
+        assert peak >= 6 * ((B + 255) // 256 * 256 // 2) * N * 4
         assert candidates >= 6      # three buffers of two halves; more candidates = the two-region search ran (N >= 4096 here)
         assert np.array_equal(net.categories()[net.categories() < S], ref["active_ids"][-1])
         assert same_floats(net.activations(rows), ref["kept"][L - 1][1])
@@ -1070,13 +1169,21 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         window = int(rng.choice([0, 0, 2, 3]))
         minchain = int(rng.choice([256, 4096]))
         values = str(rng.choice(["uniform", "pow2", "general"]))
+        # a third of the cases: every layer of one kind and row length, so that consecutive layers can share a
+        # persistent launch (switched on and off, queued per XCD or not, with a wait limit of zero now and then)
+        same_kind = str(rng.choice(["circ", "radix", "hub"])) if rng.random() < 0.35 else None
+        same_nnz = int(rng.choice([4, 16, 32]))
+        persist = dict(SPDNN_PERSIST=str(int(rng.integers(0, 2))), SPDNN_PERSIST_XCD=str(int(rng.choice([-1, 0, 1]))),
+                       SPDNN_PERSIST_LIGHT_SYNC=str(int(rng.integers(0, 2))))
+        wait_us = int(rng.choice([0, 0, -1]))
         layers, kinds = [], []
         for l in range(L):
-            kind = str(rng.choice(["circ", "circ", "gather", "radix", "hub"]))
+            kind = same_kind or str(rng.choice(["circ", "circ", "gather", "radix", "hub"]))
             if kind in ("radix", "hub") and (N % 32 or N < 64):
                 kind = "circ"
             if kind == "circ":
-                rp, c, v = orc.gen_layer_csr(int(rng.integers(0, 1000)), l, N, int(min(N, rng.integers(1, 41))))
+                nnz = same_nnz if same_kind else int(rng.integers(1, 41))
+                rp, c, v = orc.gen_layer_csr(int(rng.integers(0, 1000)), l, N, int(min(N, nnz)))
                 if values == "pow2":
                     v = np.ldexp(1.0, rng.integers(-6, -2, size=len(v))).astype(np.float32)
                 elif values == "general":
@@ -1092,9 +1199,11 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         dens = float(rng.choice([0.05, 0.3, 0.8]))
         feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < dens)).astype(np.float32)
         what = dict(case=case, N=N, B=B, L=L, rl=rl, bias=bias, prune=prune, fuse=fuse, window=window,
-                    minchain=minchain, values=values, kinds=kinds, dens=dens)
+                    minchain=minchain, values=values, kinds=kinds, dens=dens, persist=persist, wait_us=wait_us)
         if case % 50 == 0:
             print("random case", what, flush=True)
+        for k, v in persist.items():
+            monkeypatch.setenv(k, v)
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
         monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))   # run chains: band walk or BLOCK form
@@ -1108,7 +1217,7 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
             net.inspect()
             net.set_features_dense(feats)
             for rep in range(2):
-                net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                net.run(prune=prune, collect_counts=True, fuse_layers=fuse, persist_wait_us=wait_us)
                 assert np.array_equal(net.categories(), ref["active_ids"][L - 1]), what
                 assert same_floats(net.activations(np.arange(B, dtype=np.int32)), ref["kept"][L - 1][1]), what
                 if bias <= 0:
@@ -1148,7 +1257,13 @@ def test_randomized_call_sequences(gc, orc, monkeypatch):
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(int(rng.choice([1, 2, 4]))))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(int(rng.choice([256, 4096]))))
         monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))
-        layers = [make_layer(rng, N, l, values) for l in range(L)]
+        monkeypatch.setenv("SPDNN_PERSIST_XCD", str(int(rng.choice([-1, 0, 1]))))
+        monkeypatch.setenv("SPDNN_PERSIST_LIGHT_SYNC", str(int(rng.integers(0, 2))))
+        if rng.random() < 0.4:   # every layer the same band layer: runs of them share persistent launches
+            one = make_layer(np.random.default_rng(case), N, 0, values)
+            layers = [one for l in range(L)]
+        else:
+            layers = [make_layer(rng, N, l, values) for l in range(L)]
         what = dict(case=case, N=N, maxB=maxB, L=L, bias=bias, values=values, window=window)
         if case % 25 == 0:
             print("random sequence", what, flush=True)
@@ -1174,7 +1289,7 @@ def test_randomized_call_sequences(gc, orc, monkeypatch):
                 elif op in ("run_all", "threshold"):
                     thr = float(rng.choice([0.0, 0.3, 1.0])) if op == "threshold" else 0.0
                     net.run(prune=bool(rng.integers(0, 2)), collect_counts=True, fuse_layers=int(rng.choice([0, 2, 4])),
-                            compact_threshold=thr)
+                            compact_threshold=thr, persist_wait_us=int(rng.choice([0, 0, 0, -1])))
                     ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
                     y, done = ref["kept"][L - 1][1], L
                     assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]], (what, log)

@@ -25,8 +25,11 @@ def test_activations_without_allocation(gc, orc):
             r = net.run(prune=True, collect_counts=True)
             ref = orc.infer(feats, layers, -0.3, prune=False, keep={L - 1})
             rows = rng.permutation(B)[:nreq].astype(np.int32)
+            calls0 = gc.device_alloc_calls()
             got = net.activations_noalloc(rows)
+            assert gc.device_alloc_calls() == calls0          # the library allocated nothing during the call ...
             want = net.activations(rows)
+            assert gc.device_alloc_calls() > calls0           # ... which the counter would have seen
             assert same_floats(got, want)
             assert same_floats(got, ref["kept"][L - 1][1][rows])
             assert got.any() and not got.all(axis=1).all()        # survivors and dead rows both present
