@@ -79,6 +79,82 @@ def irregular_layer(rng, n, kmax=24):
     return rowptr, col, val
 
 
+def sustained_block(gc, name, seed, log, per_layer_too):
+    """One BASELINE configuration other than the headline one, sustained (pruning off, full batch at every layer): ms per
+    layer and fraction of the HBM roofline on the configured features (all-zero activations from layer 2 on) and on live
+    data (densities up to 0.7: rows survive every layer), two timed passes each after one warm-up pass; for the narrow
+    configurations also with every layer as its own launch (the default shares persistent launches where it pays)."""
+    N, L, B, bias = CONFIGS[name]
+    t0 = time.time()
+    net = gc.Network(N, B, L, bias=bias)
+    net.synth_layers(seed)
+    net.inspect()
+    alg = 8.0 * B * N + 8.0 * 32 * N + 4.0 * (N + 1)
+    out = {"neuron": N, "layers": L, "batch": B, "alg_bytes_per_layer": alg}
+
+    def timed(fuse):
+        net.run(prune=False, fuse_layers=fuse)
+        best, r = None, None
+        for _ in range(2):
+            r = net.run(prune=False, fuse_layers=fuse)
+            best = r.ms_total if best is None else min(best, r.ms_total)
+        ms = best / L
+        return {"ms_per_layer": ms, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "launches_per_pass": int(r.launches),
+                "persistent_launches_per_pass": int(r.persistent_launches), "persistent_fallbacks": int(r.persistent_fallbacks),
+                "rows_nonzero_at_end": int(r.active_rows)}
+
+    net.synth_features(seed, B, 0.10, 0.25)
+    out["zeros"] = timed(0)
+    net.synth_features(seed, B, 0.10, 0.70)
+    out["live"] = timed(0)
+    if per_layer_too:
+        out["live_one_launch_per_layer"] = timed(1)
+    lit = net.run(prune=True, collect_counts=True)
+    out["literal_live_pruned_ms"] = lit.ms_total
+    out["band_tuning_rowblocks_shape_seglen"] = net.band_tuning()
+    out["feature_buffers_region_paired_candidates_peak_bytes"] = list(net.feature_placement())
+    net.close()
+    out["wall_s"] = time.time() - t0
+    log("other config %s: zeros %.4f ms/layer (frac %.3f), live %.4f ms/layer (frac %.3f), %.1f s"
+        % (name, out["zeros"]["ms_per_layer"], out["zeros"]["frac"], out["live"]["ms_per_layer"], out["live"]["frac"], out["wall_s"]))
+    return out
+
+
+def challenge_like_block(gc, N, L, B, bias, log):
+    """A run shaped like the challenge's own (the official files are not available offline): RadiX-Net-like layers of
+    strides 16, 32, ... N/2 in turn behind random relabellings, batch B of which 3 % are dense rows that survive every
+    layer and the rest dies within two layers, pruning on: the whole run's milliseconds."""
+    rng = np.random.default_rng(N)
+    t0 = time.time()
+    kinds = [radix_layer(rng, N, 16 << k) for k in range(int(np.log2(N // 16)))]
+    net = gc.Network(N, B, L, bias=bias)
+    for l in range(L):
+        net.set_layer_csr(l, *kinds[l % len(kinds)])
+    net.inspect()
+    t_inspect = time.time() - t0
+    blk = 3000
+    dens = np.where(rng.random(blk) < 0.03, 0.7, 0.05).astype(np.float32)
+    part = (rng.random((blk, N), dtype=np.float32) < dens[:, None]).astype(np.float32)
+    feats = np.tile(part, (B // blk, 1))
+    del part
+    net.set_features_dense(feats)
+    del feats
+    best, r = None, None
+    for _ in range(3):
+        r = net.run(prune=True, collect_counts=True)
+        best = r.ms_total if best is None else min(best, r.ms_total)
+    counts = [int(net.active_count(l)) for l in (0, 1, 2, L - 1)]
+    plans = sorted({net.layer_plan(l).kernel for l in range(0, L, max(1, L // 16))})
+    net.close()
+    out = {"neuron": N, "layers": L, "batch": B, "ms": best, "edges_per_s": float(B) * 32.0 * N * L / (best * 1e-3),
+           "us_per_layer": best * 1e3 / L, "compactions": int(r.compactions), "carried_rows_at_end": int(r.carried_rows),
+           "active_rows_after_layers_0_1_2_last": counts, "launches": int(r.launches),
+           "persistent_launches": int(r.persistent_launches), "kernel_classes": plans, "setup_s": time.time() - t0,
+           "inspect_s": t_inspect}
+    log("challenge-like N=%d x %d layers: %.3f ms, %d rows at the end, setup %.1f s" % (N, L, best, counts[-1], out["setup_s"]))
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,6 +172,9 @@ def main():
     ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
     ap.add_argument("--no-live", action="store_true", help="skip the sustained pass on live data")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the blocks beside the headline run: the other BASELINE configurations, the challenge-like "
+                         "pruned runs and the CPU's literal run of the headline configuration")
     ap.add_argument("--survivor-check", type=int, default=0, metavar="ROWS",
                     help="extra (slow): features with densities up to 0.7 so that rows survive every layer; "
                          "the category set of the first ROWS rows after ALL layers is compared with the oracle")
@@ -260,6 +339,32 @@ def main():
             cpu["cfg0_full"] = {"cores": cores, "edges": e0, "pruned_s": tp, "pruned_edges_per_s": e0 / tp,
                                 "unpruned_s": tu, "unpruned_edges_per_s": e0 / tu,
                                 "categories": int(len(res_p["active_ids"][-1]))}
+            if not args.no_extras:
+                # the literal run of THIS configuration on the CPU (pruning on, every row of the batch, all cores), in row
+                # chunks to bound the memory: the run the GPU's `literal` block makes, its per-layer counts compared
+                chunk, t_lit = 4096, 0.0
+                cpu_counts = np.zeros(L, np.int64)
+                layers_cache = {}
+                for r0 in range(0, B, chunk):
+                    y = orc.gen_features(seed, N, r0, min(chunk, B - r0), 0.10, 0.25)
+                    gid = np.arange(len(y), dtype=np.int32)
+                    for l in range(L):
+                        if l not in layers_cache:
+                            layers_cache[l] = layer_csr(l)
+                        t0 = time.perf_counter()
+                        y, act = orc.layer(y, layers_cache[l], bias)
+                        y, gid = orc.compact(y, act, gid)
+                        t_lit += time.perf_counter() - t0
+                        cpu_counts[l] += len(gid)
+                        if len(gid) == 0:
+                            break
+                ran = int(np.count_nonzero(cpu_counts)) + 1
+                cpu["literal"] = {"workload": "%s literal: pruning on, batch %d, all %d layers (rows of chunk after chunk of %d)"
+                                              % (args.config, B, L, chunk),
+                                  "cores": cores, "seconds": t_lit, "edges_per_s": edges / t_lit,
+                                  "layers_with_work": min(ran, L), "active_rows_first_layers": [int(c) for c in cpu_counts[:8]],
+                                  "categories": int(cpu_counts[L - 1]),
+                                  "counts_equal_gpu": [int(c) for c in cpu_counts[:len(lit_counts)]] == lit_counts}
         ok_ids, ok_y, max_abs = True, True, 0.0
         sample = np.arange(rows, dtype=np.int32)
         for l in range(n_check):
@@ -307,6 +412,21 @@ def main():
                 traffic_source = ("profiles/band_walk_cfg4_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
                                   "command, kept as text; not measured by this process")
 
+    band_tuning = net.band_tuning()
+    placement = list(net.feature_placement())
+    plan_memory = list(net.plan_memory())
+    net.close()
+
+    # ---- beside the headline run: the other BASELINE configurations and challenge-like pruned runs -----------
+    other, challenge = None, None
+    if not args.no_extras and args.structure == "circulant":
+        other = {name: sustained_block(gc, name, seed, log, per_layer_too=name in ("cfg0", "cfg1", "cfg2"))
+                 for name in ("cfg0", "cfg1", "cfg2", "cfg3") if name != args.config}
+        challenge = {"workload": "RadiX-Net-like layers (strides 16 .. N/2 in turn, random relabellings), batch 60000 with 3 % "
+                                 "dense rows that survive, pruning on, whole run; best of three",
+                     "runs": [challenge_like_block(gc, n_, l_, 60000, b_, log)
+                              for n_, l_, b_ in ((1024, 120, -0.30), (4096, 480, -0.35), (16384, 1920, -0.40), (65536, 1920, -0.45))]}
+
     out = {
         "metric": METRIC,
         "value": value,
@@ -327,11 +447,13 @@ def main():
                            "32 nnz/row of 0.0625" if args.structure != "irregular" else "1..24 nnz/row, random weights", seed),
             "neuron": N, "layers": L, "batch": B, "bias": bias, "seed": seed,
             "kernel": "band_walk (rows per lane 4, LDS ring, one v_add_f32 per input under one power-of-two weight)" if n_band == L else "+".join(kernels_used),
-            "band_tuning_rowblocks_shape_seglen": net.band_tuning(),
-            "feature_buffers_region_paired_candidates": list(net.feature_placement()),
-            "plan_window_device_bytes_pinned_bytes": list(net.plan_memory()),
+            "band_tuning_rowblocks_shape_seglen": band_tuning,
+            "feature_buffers_region_paired_candidates_peak_bytes": placement,
+            "feature_buffers_region_paired_candidates": placement[:2],
+            "plan_window_device_bytes_pinned_bytes": plan_memory,
             "final_active_rows": sustained_final_active,
             "launches_per_pass": int(r.launches), "fused_pairs_per_pass": int(r.fused_pairs),
+            "persistent_launches_per_pass": int(r.persistent_launches),
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
@@ -341,7 +463,10 @@ def main():
                              "see roofline_live for the same run on live data",
                      "copy_kernel_gbps_plain_allocations": copy_gbps,
                      "copy_kernel_gbps_work_buffers": buffer_copy_gbps,
-                     "frac_of_work_buffer_copy": achieved / buffer_copy_gbps if buffer_copy_gbps else None},
+                     "frac_of_work_buffer_copy": achieved / buffer_copy_gbps if buffer_copy_gbps else None,
+                     # (the names these two had before)
+                     "measured_copy_peak_gbps": copy_gbps,
+                     "frac_of_measured_copy": achieved / copy_gbps if copy_gbps else None},
         "roofline_live": live,
         "cpu_baseline": cpu,
         "literal": {"workload": "same inputs, pruning on", "edges_per_s": edges / (lit.ms_total * 1e-3),
@@ -353,9 +478,10 @@ def main():
         "survivor_check": survivor,
         "setup_s": {"inspector": t_inspect, "upload_and_features": t_features},
         "events_ms_per_step": ms_events / args.steps,
+        "other_configs": other,
+        "challenge_like": challenge,
     }
     print(json.dumps(out))
-    net.close()
     return 0
 
 

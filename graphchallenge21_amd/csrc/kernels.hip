@@ -96,7 +96,9 @@ __device__ __forceinline__ float mul_then_add(float acc, float x, float w) {
 // One step of the add-only walk for a pair of outputs: acc0[q] += x[q] if bit `bit` of mask0 is set,
 // acc1[q] += x[q] if it is set in mask1 (q = the wave's RL rows per lane).  The bit, sign-extended to 64
 // bits by one scalar instruction, becomes the execution mask of the adds (all lanes or none): no select
-// per accumulator, no branch.  Every lane of the calling wave is active, so the mask goes back to all ones.
+// per accumulator, no branch.  CALLERS: every lane of the calling wave must be active (wave-uniform control
+// flow around the call): the statement ends by setting the mask to all ones, it does not restore what it found
+// (saving and restoring would cost two more scalar instructions per step, which the walk cannot afford).
 template <int RL> __device__ __forceinline__ void add_pair_if_used(float* acc0, float* acc1, const float* x,
                                                                  uint64_t mask0, uint64_t mask1, int bit);
 template <> __device__ __forceinline__ void add_pair_if_used<4>(float* acc0, float* acc1, const float* x,
@@ -607,6 +609,8 @@ __device__ __forceinline__ void band_walk_body(
                         }
                     }
                 } else if (WMODE == 3) {
+                    // (add_pair_if_used* set the execution mask and put it back to ALL ONES: every lane of the wave
+                    // is active here - the walk's control flow is wave-uniform - and it must stay that way)
                     if (SPDNN_STEP_LIVE(st)) {
 #pragma unroll
                         for (int i = 0; i < PPW; ++i) {
@@ -828,6 +832,8 @@ __device__ __forceinline__ void pair_accumulate(const unsigned char* lane_ring, 
             w_nxt[1] = wp[(st >> 2) * 2 + 3];
         }
         if (WMODE == 3) {
+            // (as in the band walk: the callee leaves the execution mask at all ones, which is what it is here - the
+            // branches around this code are wave-uniform - and must stay)
             if (st < 32 || st < steps) {
                 if (st + 3 < 36)
                     col_addr[st % 3] = add_pair_if_used_then_address<4, 6, 10>(acc[0], acc[1], xb[st % 3], use0, use1, st, lane_base,
@@ -1352,10 +1358,9 @@ __device__ __forceinline__ int xcc_id() {
 }
 __device__ __forceinline__ int load_agent(const int32_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-// the launch gives up: every workgroup leaves at its next look at `abort`, the host sees -2
+// the launch gives up: every workgroup leaves at its next look at `abort`
 __device__ __forceinline__ void persist_give_up(const PersistArgs& a) {
     __hip_atomic_store(a.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(a.host_word, -2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
 // Start of a persistent kernel: a launch does not start on the ruins of another (uniform result).
@@ -1372,7 +1377,7 @@ __device__ __forceinline__ bool persist_may_start(const PersistArgs& a) {
 }
 
 // One thread waits until *cnt >= target; 0 = there, 1 = the launch has given up (here, after wait_limit
-// ticks of the 100 MHz clock, or elsewhere).  Then the data of the units waited for is made visible.
+// ticks of the 100 MHz clock, or elsewhere).
 __device__ __forceinline__ int persist_wait(const PersistArgs& a, const int32_t* cnt, int target) {
     long long t0 = -1;
     for (;;) {
@@ -1386,34 +1391,15 @@ __device__ __forceinline__ int persist_wait(const PersistArgs& a, const int32_t*
         }
         __builtin_amdgcn_s_sleep(1);
     }
-    // the writers ran on other CUs: drop this CU's L1 (same XCD, same L2: light) or take everything that
-    // is visible at device scope
-    if (a.light) asm volatile("buffer_inv sc0" ::: "memory");
-    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     return 0;
 }
 
-// End of a unit (every thread calls it after its last store): the unit's stores are made visible and
-// counted - the workgroup that finishes the launch's last unit tells the host - and the next unit is claimed,
-// all by ONE thread in ONE place: the unit loop has a single divergent region, right before the barrier at its
-// top.  (With the count at the bottom of the loop and the claim at its top, two regions of the same thread on
-// either side of the loop's back edge, the compiler let the other lanes of that wave run ahead into the next
-// iteration's barrier.)
-__device__ __forceinline__ void persist_signal_and_claim(const PersistArgs& a, int32_t* cnt, int q, int* sh_unit) {
-    wait_vector_memory();   // this wave's stores have arrived in L2
-    __syncthreads();        // (every thread has also read *sh_unit by now)
-    if (threadIdx.x == 0) {
-        if (!a.light) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");   // the XCD's L2 writes back what it holds ...
-            wait_vector_memory();   // ... and has done so before the count goes up (said explicitly: with no load or store
-                                    // of its own outstanding the compiler leaves the fence's wait out)
-        }
-        __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int fin = __hip_atomic_fetch_add(&a.ctl->units_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (fin == a.total_units - 1)
-            __hip_atomic_store(a.host_word, a.total_units, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-        *sh_unit = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+// After the wait (every wave, behind the barrier that follows it): the writers ran on other CUs, so this CU's L1
+// is dropped (same XCD, same L2: light) or everything visible at device scope is taken.  Every wave does it
+// for itself, in front of its own loads: an invalidate issued by one wave orders that wave's loads only.
+__device__ __forceinline__ void persist_acquire(const PersistArgs& a) {
+    if (a.light & 1) asm volatile("buffer_inv sc0" ::: "memory");
+    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
 // Entry j of the layer table through the constant address space: the table never changes while a kernel
@@ -1431,12 +1417,19 @@ __device__ __forceinline__ LayerDesc load_layer_desc(const LayerDesc* table, int
 
 // The unit loop.  body(rb, sg, lay, in, out, stamp, prev_stamp) runs one unit; the whole workgroup enters
 // it with the same arguments.
+//
+// One thread (thread 0) does everything between two units in ONE place, right before the barrier at the top of
+// the loop: it counts the unit that has just finished, claims the next one and waits for that unit's row block.  (With a single-thread region at the bottom of the loop and another at its top - two regions of
+// the same thread on either side of the back edge - the compiler let the other lanes of that wave run ahead into
+// the next iteration's barrier.)  The wait for the wave's LDS traffic in front of that barrier is written out
+// (ring_barrier): the barrier alone does not order thread 0's LDS writes before the other waves' reads, and the
+// compiler leaves the wait of __syncthreads() out there (seen in the generated code, and in rare units whose
+// waves disagreed on the unit).
 template <int RL, class Body>
 __device__ __forceinline__ void persist_loop(const PersistArgs& a, Body body) {
-    __shared__ int sh_unit;
+    __shared__ int sh_unit, sh_gone;
     constexpr int RB = 64 * RL;
     publish_counts(a.pub);
-    if (!persist_may_start(a)) return;
     const int q = a.nq > 1 ? xcc_id() : 0;
     const int nrb_q = a.nq > 1 ? (q < a.nblk ? (a.nblk - q + 7) / 8 : 0) : a.nblk;
     const int per_layer = nrb_q * a.nseg;
@@ -1448,27 +1441,64 @@ __device__ __forceinline__ void persist_loop(const PersistArgs& a, Body body) {
     float* const out0_h1 = in_a ? a.buf_c.half[1] : a.buf_a.half[1];
     float* const out1_h0 = in_a ? a.buf_a.half[0] : a.buf_c.half[0];
     float* const out1_h1 = in_a ? a.buf_a.half[1] : a.buf_c.half[1];
-    if (threadIdx.x == 0) sh_unit = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    for (;;) {
-        __syncthreads();
-        const int u = __builtin_amdgcn_readfirstlane(sh_unit);
-        if (u >= total_q) break;
-        const int j = u / per_layer, rem = u - j * per_layer, ri = rem / a.nseg, sg = rem - ri * a.nseg;
-        const int rb = a.nq > 1 ? q + 8 * ri : ri;
-        int32_t* const cnt = a.done + (size_t)j * a.done_stride + rb;
-        int gone = 0;
-        if (j > 0 && threadIdx.x == 0) gone = persist_wait(a, cnt - a.done_stride, a.nseg);
-        if (__builtin_amdgcn_readfirstlane(__syncthreads_or(gone))) break;
-        const LayerDesc lay = load_layer_desc(a.table, j);
-        const int stamp = a.stamp0 + j;
-        const int prev_stamp = j > 0 ? stamp - 1 : a.prev_stamp;
-        const float* const in_h0 = j == 0 ? a.first_in.half[0] : ((j & 1) ? out0_h0 : out1_h0);
-        const float* const in_h1 = j == 0 ? a.first_in.half[1] : ((j & 1) ? out0_h1 : out1_h1);
-        float* const out_h0 = (j & 1) ? out1_h0 : out0_h0;
-        float* const out_h1 = (j & 1) ? out1_h1 : out0_h1;
-        const size_t boff = (size_t)(rb >> 1) * blkf;   // row block rb is block rb >> 1 of half rb & 1
-        body(rb, sg, lay, ((rb & 1) ? in_h1 : in_h0) + boff, ((rb & 1) ? out_h1 : out_h0) + boff, stamp, prev_stamp);
-        persist_signal_and_claim(a, cnt, q, &sh_unit);
+    // where unit u's row block counts its finished units, and what unit u waits for (thread 0)
+    auto counter_of = [&](int u) -> int32_t* {
+        const int j = u / per_layer, rem = u - j * per_layer, ri = rem / a.nseg;
+        return a.done + (size_t)j * a.done_stride + (a.nq > 1 ? q + 8 * ri : ri);
+    };
+    auto wait_for = [&](int u) -> int {
+        if (u >= total_q || u < per_layer) return 0;   // no such unit, or a unit of the launch's first layer
+        return persist_wait(a, counter_of(u) - a.done_stride, a.nseg);
+    };
+    if (persist_may_start(a)) {
+        if (threadIdx.x == 0) {
+            const int first = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sh_unit = first;
+            sh_gone = wait_for(first);
+        }
+        for (;;) {
+            ring_barrier<1>();
+            const int u = __builtin_amdgcn_readfirstlane(sh_unit);
+            if (u >= total_q || __builtin_amdgcn_readfirstlane(sh_gone) != 0) break;
+            const int j = u / per_layer, rem = u - j * per_layer, ri = rem / a.nseg, sg = rem - ri * a.nseg;
+            const int rb = a.nq > 1 ? q + 8 * ri : ri;
+            if (j > 0) persist_acquire(a);
+            const LayerDesc lay = load_layer_desc(a.table, j);
+            const int stamp = a.stamp0 + j;
+            const int prev_stamp = j > 0 ? stamp - 1 : a.prev_stamp;
+            const float* const in_h0 = j == 0 ? a.first_in.half[0] : ((j & 1) ? out0_h0 : out1_h0);
+            const float* const in_h1 = j == 0 ? a.first_in.half[1] : ((j & 1) ? out0_h1 : out1_h1);
+            float* const out_h0 = (j & 1) ? out1_h0 : out0_h0;
+            float* const out_h1 = (j & 1) ? out1_h1 : out0_h1;
+            const size_t boff = (size_t)(rb >> 1) * blkf;   // row block rb is block rb >> 1 of half rb & 1
+            body(rb, sg, lay, ((rb & 1) ? in_h1 : in_h0) + boff, ((rb & 1) ? out_h1 : out_h0) + boff, stamp, prev_stamp);
+            wait_vector_memory();   // this wave's stores have arrived in L2
+            ring_barrier<1>();      // ... every wave's have, and every thread has read sh_unit / sh_gone
+            if (threadIdx.x == 0) {
+                if (!(a.light & 2)) {
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");   // the XCD's L2 writes back what it holds ...
+                    wait_vector_memory();   // ... and has done so before the count goes up (said explicitly: with no load or
+                                            // store of its own outstanding the compiler leaves the fence's wait out)
+                }
+                __hip_atomic_fetch_add(counter_of(u), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_fetch_add(&a.ctl->units_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // (claimed here, not a unit ahead under the arithmetic: a unit held by a busy workgroup while others
+                // idle costs more than the atomic's round trip - 21.8 against 18.2 us per layer at N=1024, batch 6000)
+                const int next = __hip_atomic_fetch_add(&a.ctl->head[q], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                sh_unit = next;
+                sh_gone = wait_for(next);
+            }
+        }
+    }
+    // The last workgroup to leave tells the host: the unit total if every unit was run, -2 if the launch gave up.
+    if (threadIdx.x == 0) {
+        wait_vector_memory();   // this thread's counts have been made
+        const int left = __hip_atomic_fetch_add(&a.ctl->exited, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {
+            const int done = load_agent(&a.ctl->units_done);
+            __hip_atomic_store(a.host_word, (done == a.total_units && load_agent(a.abort) == 0) ? done : -2, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
+        }
     }
 }
 
@@ -1486,6 +1516,8 @@ __global__ __launch_bounds__(512) void band_persist_kernel(PersistArgs a) {
         for (int x = 0; x < RL; ++x) nz[x] = 0.0f;
         band_walk_body<RL, 8, 2, 64, WMODE, KT, DMA>(yin, yout, lay.pairs, lay.pw, lay.dst, a.N, lay.steps, lay.halo, vb, ve,
                                                      lay.wu, a.bias, a.clampv, smem, nz, a.stream);
+        // (one store per row through LDS: with every wave stamping its rows itself - 8 times the stores on the
+        // row block's 1 KiB of stamps from every unit of the block - a small layer took 0.5 - 1.5 us longer)
         stamp_rows_workgroup<RL, 8>(nz, smem, a.active, (size_t)rb * RB, stamp, nullptr);
     });
 }
@@ -1967,7 +1999,8 @@ PersistArgs persist_args(const PersistLaunch& a, const PersistShape& p) {
     k.active = a.active; k.done = a.done; k.done_stride = a.done_stride; k.ctl = a.ctl; k.prev_ctl = a.prev_ctl;
     k.prev_units = a.prev_units; k.abort = a.abort; k.host_word = a.host_word;
     k.N = a.N; k.nblk = a.nblk; k.nseg = p.nseg; k.seglen = p.seglen; k.total_units = p.total; k.nq = p.nq;
-    k.light = (a.light_sync && p.nq > 1) ? 1 : 0;
+    // light_sync 1: both sides light; for measurements 2 = the writer's side only, 4 = the reader's side only
+    k.light = p.nq > 1 ? (a.light_sync == 1 ? 3 : a.light_sync == 2 ? 2 : a.light_sync == 4 ? 1 : 0) : 0;
     k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead; k.wait_limit = a.wait_limit;
     k.bias = a.bias; k.clampv = a.clampv;
     k.stream = (long long)a.nblk * (long long)a.N * 64 * a.rl * 4 * 2 >= a.stream_min_bytes ? 1 : 0;
@@ -1978,7 +2011,7 @@ PersistArgs persist_args(const PersistLaunch& a, const PersistShape& p) {
 template <int RL, int WMODE, int KT>
 hipError_t launch_persist_band_inst(const PersistLaunch& a, hipStream_t s) {
     constexpr size_t lds = (size_t)64 * 64 * RL * 4;
-    auto kern = band_persist_kernel<RL, WMODE, KT, RL == 4 ? 1 : 0>;
+    auto kern = band_persist_kernel<RL, WMODE, KT, 0>;
     // once per instantiation; a function-local static is initialised by one thread only
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -168,7 +168,8 @@ struct LayerDesc {           // one entry of the device-side layer table
 struct PersistCtl {          // device words of one persistent launch (zero before the launch)
     int32_t head[8];         // next unit of each queue
     int32_t units_done;      // units finished
-    int32_t pad[7];
+    int32_t exited;          // workgroups that have left the kernel
+    int32_t pad[6];
 };
 
 struct PersistLaunch {

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from helpers import random_csr, same_floats, sort_rows
-from helpers import common_band_csr
+from helpers import common_band_csr, radix_like_csr
 
 pytestmark = pytest.mark.gpu
 
@@ -414,7 +414,7 @@ def test_full_batch_properties_cfg1(gc, orc):
 PERSIST_MODES = {   # how the units of a persistent launch are queued and handed over (environment, read at creation)
     "default": {},
     "one-queue": {"SPDNN_PERSIST_XCD": "0"},
-    "xcd-queues": {"SPDNN_PERSIST_XCD": "1"},
+    "xcd-queues": {"SPDNN_PERSIST_XCD": "1", "SPDNN_PERSIST_LIGHT_SYNC": "0"},
     "xcd-queues-light": {"SPDNN_PERSIST_XCD": "1", "SPDNN_PERSIST_LIGHT_SYNC": "1"},
 }
 
@@ -452,11 +452,45 @@ def test_persistent_launches(gc, orc, fuse, prune, mode, monkeypatch):
         net.run(prune=prune, first_layer=14, n_layers=L - 14, fuse_layers=fuse)
         assert np.array_equal(net.categories(), ref["categories"])
         assert same_floats(net.activations(cats), ref["y"])
-        # left to the library (fuse_layers = 0): launches of this size are persistent by default
+        # left to the library (fuse_layers = 0): launches this small stay one per layer
         r = net.run(prune=False, collect_counts=True)
-        assert r.persistent_launches >= 1 and r.persistent_fallbacks == 0
+        assert r.persistent_launches == 0 and r.launches == L
         assert [net.active_count(l) for l in range(L)] == [len(a) for a in ref["active_ids"]]
         assert same_floats(net.activations(cats), ref["y"])
+
+
+@pytest.mark.parametrize("N,L,bias", [(1024, 120, -0.3), (4096, 40, -0.35)])
+def test_persistent_by_default_at_full_batch(gc, orc, N, L, bias):
+    """Batch 60000: left to the library (fuse_layers = 0) the layers of these widths share persistent launches (one unit
+    queue per XCD, the hand-over between layers inside the XCD's L2).  Every activation of every row after the last
+    layer, the per-layer counts and the categories must equal those of one launch per layer bit for bit, on live data
+    (rows that survive every layer), pruned and unpruned; an oracle row sample pins both."""
+    B, S = 60000, 256
+    print("persistent by default N=%d L=%d" % (N, L), flush=True)
+    layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
+    ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.70), layers, bias, prune=False, keep={L - 1})
+    rows = np.arange(B, dtype=np.int32)
+    with gc.Network(N, B, L, bias=bias) as net:
+        net.synth_layers(0)
+        net.inspect()
+        net.synth_features(0, B, 0.10, 0.70)
+
+        def state():
+            acts = np.concatenate([net.activations(rows[i:i + 8192]) for i in range(0, B, 8192)])
+            return acts, [net.active_count(l) for l in range(L)], net.categories()
+
+        r1 = net.run(prune=False, collect_counts=True, fuse_layers=1)
+        want = state()
+        assert r1.persistent_launches == 0 and len(want[2]) > 1000
+        assert same_floats(want[0][:S], ref["kept"][L - 1][1])
+        for attempt in range(3):
+            r = net.run(prune=False, collect_counts=True)
+            assert r.persistent_launches >= 1 and r.persistent_fallbacks == 0 and r.launches < L
+            got = state()
+            assert np.array_equal(got[0], want[0]) and got[1] == want[1] and np.array_equal(got[2], want[2]), attempt
+        r = net.run(prune=True, collect_counts=True)
+        got = state()
+        assert np.array_equal(got[0], want[0]) and got[1] == want[1] and np.array_equal(got[2], want[2])
 
 
 @pytest.mark.parametrize("mode", ["one-queue", "xcd-queues"])
