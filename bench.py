@@ -45,11 +45,12 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def radix_layer(rng, n, stride):
+def radix_layer(rng, n, stride, perm=None):
     """A layer with the structure of the challenge's RadiX-Net files: the 16 outputs of group g read the
     two 16-wide input runs [16g, 16g+16) and [16g+stride, 16g+stride+16) (mod n), hidden behind random
-    relabellings of inputs and outputs; 32 entries of 1/16 per row.  CSR with row = output neuron."""
-    pin, pout = rng.permutation(n).astype(np.int32), rng.permutation(n)
+    relabellings of inputs and outputs (perm: behind that one relabelling for both, the network's common
+    neuron numbering); 32 entries of 1/16 per row.  CSR with row = output neuron."""
+    pin, pout = (perm, perm) if perm is not None else (rng.permutation(n).astype(np.int32), rng.permutation(n))
     base = (np.arange(n) // 16 * 16)[:, None]
     run = np.arange(16)[None, :]
     ins = np.concatenate([base + run, (base + stride + run) % n], axis=1)
@@ -165,9 +166,11 @@ def main():
     ap.add_argument("--batch", type=int, default=0, help="override the batch (quick runs)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--fuse", type=int, default=0, help="spdnn_run_options.fuse_layers for the timed runs (1 = no fused launches)")
-    ap.add_argument("--structure", default="circulant", choices=["circulant", "radix", "irregular", "common-band"],
+    ap.add_argument("--structure", default="circulant", choices=["circulant", "radix", "radix-common", "irregular", "common-band"],
                     help="layers: the seeded permuted-stride generator (default, the configured workload), RadiX-Net-like "
-                         "layers (one per stride 16, 32, ... n/2, repeated), or layers without structure (n <= 4096)")
+                         "layers (one per stride 16, 32, ... n/2, repeated; radix-common: all of them behind one hidden "
+                         "neuron numbering, as the layer files of one challenge network), bands over one common order, "
+                         "or layers without structure (n <= 4096)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
     ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
@@ -208,6 +211,9 @@ def main():
         rng = np.random.default_rng(seed)
         if args.structure == "radix":
             kinds = [radix_layer(rng, N, 16 << k) for k in range(max(1, int(np.log2(N // 16))))]
+        elif args.structure == "radix-common":
+            perm = rng.permutation(N).astype(np.int32)
+            kinds = [radix_layer(rng, N, 16 << k, perm) for k in range(max(1, int(np.log2(N // 16))))]
         elif args.structure == "common-band":
             kinds = [common_band_layer(rng.permutation(N).astype(np.int32))]
         else:
@@ -233,16 +239,18 @@ def main():
         % (t_inspect, n_band, L, "+".join(kernels_used), t_features))
 
     # ---- sustained run: the timed steps ---------------------------------------------------
-    for _ in range(args.warmup):
-        net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
+    for i in range(args.warmup):
+        r = net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
+        log("warmup %d/%d: %.0f ms" % (i + 1, args.warmup, r.ms_total))
     gc.load_library().spdnn_device_synchronize()
     layer_ms = []
     t0 = time.perf_counter()
     ms_events = 0.0
-    for _ in range(args.steps):
+    for i in range(args.steps):
         r = net.run(prune=False, time_layers=True, fuse_layers=args.fuse)
         ms_events += r.ms_total
         layer_ms.append(net.layer_times().copy())
+        log("step %d/%d: %.0f ms" % (i + 1, args.steps, r.ms_total))   # between steps, the GPU idle: a progress line
     gc.load_library().spdnn_device_synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     ms_per_step = wall_ms / args.steps

@@ -24,7 +24,7 @@ class LayerPlan(C.Structure):
     _fields_ = [("kernel", C.c_int32), ("max_row_nnz", C.c_int32), ("regular", C.c_int32),
                 ("uniform_value", C.c_int32), ("value", C.c_float), ("exact_products", C.c_int32),
                 ("band_halo", C.c_int32), ("nnz", C.c_int64), ("plan_bytes", C.c_int64),
-                ("block_form", C.c_int32), ("fuse_next", C.c_int32)]
+                ("block_form", C.c_int32), ("fuse_next", C.c_int32), ("common_order", C.c_int32)]
 
 
 class RunOptions(C.Structure):

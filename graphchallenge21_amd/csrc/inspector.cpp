@@ -298,8 +298,9 @@ bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vecto
 
 bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                          const std::vector<std::vector<int32_t>>& groups, std::vector<int32_t>& in_pos,
-                         std::vector<int32_t>& out_at) {
+                         std::vector<int32_t>& out_at, int* cycles) {
     const int G = 16, K = 32, R = 16;
+    int ncycles = 0;
     if (N % 256 != 0 || (int)groups.size() * G != N) return false;
     const int ng = N / G;
     for (const auto& g : groups)
@@ -400,8 +401,10 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
             }
         }
         base += c;
+        ++ncycles;
     }
     if (base != ng) return false;
+    if (cycles) *cycles = ncycles;
     // full check of what the kernel assumes: every entry of the output at position v lies in
     // [16*floor(v/16) - 32, 16*floor(v/16) + 15] (mod N)
     for (int v = 0; v < N; ++v) {
@@ -416,6 +419,68 @@ bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::v
         }
     }
     return true;
+}
+
+bool common_run_order(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                      std::vector<int32_t>& pos) {
+    const int G = 16;
+    if (N % 256 != 0) return false;
+    std::vector<std::vector<int32_t>> groups;
+    if (!discover_blocks(N, rowptr, col, groups) || (int)groups.size() * G != N) return false;
+    const int ng = N / G;
+    std::vector<int32_t> group_of((size_t)N, -1);
+    for (int g = 0; g < ng; ++g) {
+        if ((int)groups[(size_t)g].size() != G) return false;
+        for (int32_t j : groups[(size_t)g]) group_of[(size_t)j] = g;
+    }
+    // every group reads its own 16 neurons and the 16 neurons of one other group
+    std::vector<int32_t> other((size_t)ng, -1);
+    for (int g = 0; g < ng; ++g) {
+        const int j0 = groups[(size_t)g][0];
+        if (rowptr[j0 + 1] - rowptr[j0] != 2 * G) return false;
+        int own = 0, far = 0;
+        for (int e = rowptr[j0]; e < rowptr[j0 + 1]; ++e) {
+            const int h = group_of[(size_t)col[e]];
+            if (h == g) ++own;
+            else if (other[(size_t)g] < 0 || other[(size_t)g] == h) { other[(size_t)g] = h; ++far; }
+            else return false;
+        }
+        if (own != G || far != G) return false;
+    }
+    // one cycle through all groups; the group a slot reads lies one slot back
+    std::vector<int32_t> slot((size_t)ng, -1);
+    int g = 0;
+    for (int t = 0; t < ng; ++t) {
+        if (slot[(size_t)g] >= 0) return false;
+        slot[(size_t)g] = (ng - t) % ng;
+        g = other[(size_t)g];
+    }
+    if (g != 0) return false;
+    pos.assign((size_t)N, -1);
+    for (int h = 0; h < ng; ++h)
+        for (int o = 0; o < G; ++o) pos[(size_t)groups[(size_t)h][(size_t)o]] = slot[(size_t)h] * G + o;
+    return true;
+}
+
+int common_order_offset(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                        const std::vector<int32_t>& pos) {
+    const int G = 16;
+    if (N % 256 != 0 || (int)pos.size() != N) return 0;
+    const int ng = N / G;
+    int d = 0;
+    for (int j = 0; j < N; ++j) {
+        if (rowptr[j + 1] - rowptr[j] != 2 * G) return 0;
+        const int t = pos[(size_t)j] / G;
+        int own = 0, far = 0;
+        for (int e = rowptr[j]; e < rowptr[j + 1]; ++e) {
+            const int back = ((t - pos[(size_t)col[e]] / G) % ng + ng) % ng;
+            if (back == 0) ++own;
+            else if ((back == 1 || back == 2) && (d == 0 || d == back)) { d = back; ++far; }
+            else return 0;
+        }
+        if (own != G || far != G) return 0;
+    }
+    return d;
 }
 
 // TILED plan (layers that are neither a band nor groups of identical rows).  Outputs are cut into
@@ -557,7 +622,8 @@ static int merged_pair_steps(int N, int K, const std::vector<int32_t>& rowptr, c
 }
 
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
-                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan) {
+                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan,
+                   const std::vector<int32_t>* common_pos) {
     const int64_t nnz = rowptr[N];
     int kmax = 0;
     bool rows_regular = true, dup = false;
@@ -610,7 +676,18 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     // below that a row block's whole input sits in L2 and the BLOCK kernel's independent waves win.
     const char* chain_env = getenv("SPDNN_RUN_CHAINS_MIN_N");
     const int chain_min_n = chain_env ? atoi(chain_env) : 4096;   // 0 or negative: never
-    if (block && chain_min_n > 0 && N >= chain_min_n && plan.info.regular && K == 32 && discover_run_chains(N, rowptr, col, groups, plan.in_pos, plan.out_at)) {
+    const bool chains_ok = block && chain_min_n > 0 && N >= chain_min_n && plan.info.regular && K == 32;
+    plan.info.common_order = 0;
+    if (chains_ok && common_pos && uniform && exact && (plan.info.common_order = common_order_offset(N, rowptr, col, *common_pos)) > 0) {
+        // the network's common neuron order is a run-chain labelling of this layer: inputs and outputs
+        // both take it, so a neighbour laid out the same way finds the columns where it reads them
+        plan.in_pos = *common_pos;
+        plan.out_at.assign((size_t)N, 0);
+        for (int i = 0; i < N; ++i) plan.out_at[(size_t)plan.in_pos[(size_t)i]] = i;
+        band = true;
+        block = false;
+        halo = 32;
+    } else if (chains_ok && discover_run_chains(N, rowptr, col, groups, plan.in_pos, plan.out_at, &plan.rc_cycles)) {
         band = true;    // 16-output groups chained through shared 16-input runs: walked like a band
         block = false;
         halo = 32;

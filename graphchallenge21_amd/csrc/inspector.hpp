@@ -63,6 +63,7 @@ struct LayerPlan {
     // panel and wave; wv the entry blocks of 1 KiB: per round 64 outputs x 2 entries x (byte offset of
     // the column's slot in the panel as raw bits, weight)
     int ntiles = 0;
+    int rc_cycles = 0;         // run chains: cycles of groups the layer's own labelling found
     bool self_aligned = false;
     bool pair_twins = false;   // BAND, one exact weight: the two outputs of every pair use the same inputs
     bool fuse_next = false;
@@ -92,14 +93,33 @@ bool discover_blocks(int N, const std::vector<int32_t>& rowptr, const std::vecto
 // The result is a BAND labelling (in_pos, out_at) for a halo of 32.
 bool discover_run_chains(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                          const std::vector<std::vector<int32_t>>& groups, std::vector<int32_t>& in_pos,
-                         std::vector<int32_t>& out_at);
+                         std::vector<int32_t>& out_at, int* cycles = nullptr);
+
+// One neuron order for the RadiX-Net layers of a network whose files share a (hidden) neuron
+// numbering - layer l's output j and layer l+1's input j are the same neuron, and under the hidden
+// numbering group g of every such layer reads neuron blocks g and g + m_l (mod N/16).  From a layer
+// whose blocks form a single cycle (m coprime to N/16, e.g. stride 16): pos[neuron] = 16 * slot of
+// its block along the cycle + rank inside the block, oriented so that the block a slot reads besides
+// its own lies one slot back.  False when the layer has no such structure (groups that are not also
+// the runs they read, several cycles).
+bool common_run_order(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                      std::vector<int32_t>& pos);
+
+// Whether `pos` is a run-chain labelling of this layer too: every output at slot t reads all of
+// slot t and all of slot t - d with the same d for the whole layer.  Returns d (1 or 2: inside the
+// band kernel's halo of 32), 0 otherwise.
+int common_order_offset(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                        const std::vector<int32_t>& pos);
 
 // Full per-layer inspection (everything except dst, which needs the next layer's labelling).
 // fma_ok: nonzero activations stay far above the denormal range, so that a product with a
 // power-of-two weight is exact and a fused multiply-add rounds like multiply-then-add; when false
-// every layer uses the unfused pair.
+// every layer uses the unfused pair.  common_pos: the network's common neuron order (common_run_order);
+// a run-chain layer with one exact weight that it fits (common_order_offset) takes it for inputs and
+// outputs instead of a labelling of its own.
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
-                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan);
+                   const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan,
+                   const std::vector<int32_t>* common_pos = nullptr);
 
 // The layer's structure back from its plan: rowptr[N+1] / col[] with row = output neuron and the
 // input neurons of every row ascending.

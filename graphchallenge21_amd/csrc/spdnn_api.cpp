@@ -803,9 +803,9 @@ void reset_state(spdnn_net* n) {
 // inspect_layer for a worker thread: a worker must not let an exception escape (std::terminate); the
 // layer stays unset and spdnn_inspect reports what happened
 void inspect_on_worker(int N, const std::vector<int32_t>& rp, const std::vector<int32_t>& col, const std::vector<float>& val,
-                       int force, bool fma_ok, LayerPlan* plan) {
+                       int force, bool fma_ok, LayerPlan* plan, const std::vector<int32_t>* common_pos = nullptr) {
     try {
-        inspect_layer(N, rp, col, val, force, fma_ok, *plan);
+        inspect_layer(N, rp, col, val, force, fma_ok, *plan, common_pos);
     } catch (const std::bad_alloc&) {
         plan->set = false;
         plan->failed = plan->failed_nomem = true;
@@ -1070,10 +1070,8 @@ static int spdnn_synth_layers_impl(spdnn_net* n, uint64_t seed, int first, int c
     return SPDNN_OK;
 }
 
-static int spdnn_inspect_impl(spdnn_net* n) {
-    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
-    n->pool->wait_all();
-    std::fill(n->pending.begin(), n->pending.end(), 0);
+// Every layer inspected?  Otherwise the status that says what happened to the first one that is not.
+static int layers_all_set(spdnn_net* n) {
     for (int l = 0; l < n->L; ++l)
         if (!n->layers[(size_t)l].set) {
             const LayerPlan& p = n->layers[(size_t)l];
@@ -1083,6 +1081,57 @@ static int spdnn_inspect_impl(spdnn_net* n) {
                 return fail(SPDNN_E_UNSUPPORTED, "the inspection of layer " + std::to_string(l) + " failed: " + p.fail_text);
             return fail(SPDNN_E_STATE, "layer " + std::to_string(l) + " has not been set");
         }
+    return SPDNN_OK;
+}
+
+// Second pass over the run-chain layers with one exact weight.  Each of them chose a labelling of its
+// own, so no two agree on where a neuron sits and none can hand its outputs to the next one in LDS.
+// When the network's files share one neuron numbering there is an order that serves several of them at
+// once (common_run_order, taken from the first such layer whose groups form a single cycle): every
+// layer it fits (common_order_offset: the stride of that layer and twice it) is laid out again in that
+// order, and neighbours among them then pass pair_fusable.
+static void adopt_common_order(spdnn_net* n) {
+    if (getenv("SPDNN_COMMON_ORDER") && atoi(getenv("SPDNN_COMMON_ORDER")) == 0) return;
+    const int N = n->N;
+    auto pos = std::make_shared<std::vector<int32_t>>();
+    std::vector<int32_t> rp, cc;
+    int tried = 0;
+    for (int l = 0; l < n->L && pos->empty() && tried < 4; ++l) {
+        const LayerPlan& p = n->layers[(size_t)l];
+        if (p.kernel != SPDNN_KERNEL_BAND || p.alt_ngroups == 0 || p.rc_cycles != 1) continue;
+        ++tried;
+        plan_adjacency(p, N, rp, cc);
+        if (!common_run_order(N, rp, cc, *pos)) pos->clear();
+    }
+    if (pos->empty()) return;
+    const int force = n->force_kernel;
+    const bool fma_ok = n->fma_ok;
+    for (int l = 0; l < n->L; ++l) {
+        LayerPlan* p = &n->layers[(size_t)l];
+        if (p->kernel != SPDNN_KERNEL_BAND || p->alt_ngroups == 0 || p->rc_cycles > 2) continue;
+        if (p->info.common_order > 0 && p->in_pos == *pos) continue;   // laid out that way by an earlier call
+        n->pool->submit([=] {
+            try {
+                std::vector<int32_t> rowptr, col;
+                plan_adjacency(*p, N, rowptr, col);
+                if (common_order_offset(N, rowptr, col, *pos) == 0) return;
+                const std::vector<float> val(col.size(), p->info.value);
+                inspect_on_worker(N, rowptr, col, val, force, fma_ok, p, pos.get());
+            } catch (...) {
+                // out of memory before the layer was touched: it keeps the labelling it has
+            }
+        });
+    }
+    n->pool->wait_all();
+}
+
+static int spdnn_inspect_impl(spdnn_net* n) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    n->pool->wait_all();
+    std::fill(n->pending.begin(), n->pending.end(), 0);
+    if (int rc = layers_all_set(n)) return rc;
+    adopt_common_order(n);
+    if (int rc = layers_all_set(n)) return rc;
     for (int l = 0; l < n->L; ++l) {
         LayerPlan* cur = &n->layers[(size_t)l];
         const std::vector<int32_t>* nxt = l + 1 < n->L ? &n->layers[(size_t)l + 1].in_pos : nullptr;

@@ -77,6 +77,9 @@ typedef struct spdnn_layer_plan {
                                 spdnn_run uses on small batches                                   */
     int32_t fuse_next;       /* 1 (after spdnn_inspect): this layer and the next can run as one fused launch, the
                                 activations between them kept in LDS (see spdnn_run_options.fuse_layers)  */
+    int32_t common_order;    /* run chains, after spdnn_inspect: 0 = the layer has a labelling of its own; 1 or 2 = it is
+                                laid out in the neuron order its network's RadiX-Net layers share, the second run of
+                                every group that many 16-neuron slots behind the group (what lets neighbours fuse)  */
 } spdnn_layer_plan;
 
 typedef struct spdnn_run_options {

@@ -43,13 +43,15 @@ def same_floats(a, b):
     return a.shape == b.shape and bool(np.all((a == b) | (np.isnan(a) & np.isnan(b))))
 
 
-def radix_like_csr(rng, n, stride, values="uniform", relabel=True, run=16):
+def radix_like_csr(rng, n, stride, values="uniform", relabel=True, run=16, perm=None):
     """RadiX-Net-like layer: the outputs of group g (16 consecutive outputs) all read the two
     16-wide input runs [16g, 16g+16) and [16g+stride, 16g+stride+16) (mod n) - the structure the
     reference's kernels assume after its hash reorder - optionally hidden behind random
-    relabellings of inputs and outputs, as in the raw challenge files."""
-    pin = rng.permutation(n) if relabel else np.arange(n)
-    pout = rng.permutation(n) if relabel else np.arange(n)
+    relabellings of inputs and outputs, as in the raw challenge files.  perm: one relabelling for
+    inputs and outputs alike (the layers of a network built with the same perm share a neuron
+    numbering, as consecutive layer files of the challenge do)."""
+    pin = perm if perm is not None else rng.permutation(n) if relabel else np.arange(n)
+    pout = perm if perm is not None else rng.permutation(n) if relabel else np.arange(n)
     rows = [None] * n
     for j in range(n):
         g = j // run

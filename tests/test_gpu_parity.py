@@ -607,6 +607,70 @@ def test_fused_pairs_in_lds(gc, orc, N, B, values):
             assert same_floats(net.activations(cats), ref["y"])
 
 
+def test_fused_pairs_radix_common(gc, orc, monkeypatch):
+    """RadiX-Net layers behind one hidden neuron numbering (strides 16, 32, 64, ...): the layers of stride
+    16 and 32 take the network's common order and neighbours among them run as one launch with the
+    activations in LDS.  Counts of every layer, categories and activations against the oracle, pruned
+    and not, fused and one launch per layer; then the full batch: an oracle row sample, and the whole
+    batch against the run with one launch per layer."""
+    N, B = 4096, 700
+    print("fused pairs, radix layers of one numbering N=%d B=%d" % (N, B), flush=True)
+    rng = np.random.default_rng(N + B)
+    perm = rng.permutation(N)
+    strides = [16, 32, 64, 16, 32, 32, 16, 128]
+    L = len(strides)
+    layers = [radix_like_csr(rng, N, s, perm=perm) for s in strides]
+    feats = orc.gen_features(8, N, 0, B, 0.10, 0.60)
+    ref = orc.infer(feats, layers, -0.4, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    assert 0 < want_counts[-1] < B
+    monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", "0")   # a batch this small would run the layers' BLOCK form
+    with gc.Network(N, B, L, bias=-0.4) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert [net.layer_plan(l).common_order for l in range(L)] == [1, 2, 0, 1, 2, 2, 1, 0]
+        assert [net.layer_plan(l).fuse_next for l in range(L)] == [1, 0, 0, 1, 1, 1, 0, 0]
+        net.set_features_dense(feats)
+        cats = ref["categories"]
+        for prune in (True, False):
+            for fuse in (2, 1):
+                r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert r.layers_run == L
+                assert (r.fused_pairs, r.launches) == ((3, 5) if fuse == 2 else (0, L))
+                assert [net.active_count(l) for l in range(L)] == want_counts
+                assert np.array_equal(net.categories(), cats)
+                assert same_floats(net.activations(cats), ref["y"])
+        for l in range(L):    # every layer's survivors and their activations, the layer inside a pair included
+            net.run(prune=True, first_layer=0, n_layers=l + 1, fuse_layers=2)
+            gid, y = ref["kept"][l]
+            assert np.array_equal(net.categories(), ref["active_ids"][l])
+            assert same_floats(net.activations(gid), y)
+    monkeypatch.delenv("SPDNN_BLOCK_FORM_MAX_ELEMS")
+    B, S = 60000, 768
+    print("fused pairs, radix layers of one numbering N=%d B=%d" % (N, B), flush=True)
+    ref = orc.infer(orc.gen_features(9, N, 0, S, 0.10, 0.60), layers, -0.4, prune=True)
+    with gc.Network(N, B, L, bias=-0.4) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.synth_features(9, B, 0.10, 0.60)
+        r = net.run(prune=False, collect_counts=True)     # left to the library, launches of this size run the pairs fused
+        assert r.fused_pairs == 3 and r.launches == 5
+        counts = [net.active_count(l) for l in range(L)]
+        cats = net.categories()
+        assert np.array_equal(cats[cats < S], ref["categories"])
+        assert same_floats(net.activations(ref["categories"]), ref["y"])
+        probe = cats[:: max(1, len(cats) // 512)].astype(np.int32)
+        y_fused = net.activations(probe)
+        net.synth_features(9, B, 0.10, 0.60)
+        r = net.run(prune=False, collect_counts=True, fuse_layers=1)
+        assert r.fused_pairs == 0
+        assert [net.active_count(l) for l in range(L)] == counts
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(probe), y_fused)
+
+
 def test_fused_pairs_full_batch(gc, orc):
     """The fused pair on a batch of 60000 (235 row blocks, several segments per row block, streaming
     loads and stores): an oracle row sample through 6 layers, and the whole batch against the run

@@ -320,6 +320,43 @@ def test_fusable_pairs_are_found_by_the_inspector(gc, orc):
         assert len(net.receptive_field(4, 2, out_at[:64])) > 0.95 * n
 
 
+def test_radix_layers_of_one_numbering_share_an_order(gc, orc):
+    """RadiX-Net layers whose files share a hidden neuron numbering: the inspector lays the layers of
+    stride 16 and 32 out in one common order (the cycle of the stride-16 layer), so that neighbours
+    among them write where the next one reads and are marked for the fused launch; wider strides and
+    layers with a numbering of their own keep their own labelling.  The structure the plans describe
+    stays the layer's."""
+    rng = np.random.default_rng(31)
+    n = 4096
+    perm = rng.permutation(n)
+    strides = [16, 32, 64, 2048, 16, 32, 32, 16, None, 16]
+    layers = [radix_like_csr(rng, n, s, perm=perm) if s else radix_like_csr(rng, n, 16) for s in strides]
+    with gc.Network(n, 4, len(layers), bias=-0.3) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        plans = [net.layer_plan(l) for l in range(len(layers))]
+        assert [p.kernel for p in plans] == [gc.KERNEL_BAND] * len(layers)
+        assert [p.common_order for p in plans] == [1, 2, 0, 0, 1, 2, 2, 1, 0, 1]
+        assert [p.fuse_next for p in plans] == [1, 0, 0, 0, 1, 1, 1, 0, 0, 0]
+        in0, out0, _ = net.band_plan(0)
+        assert np.array_equal(in0[out0], np.arange(n))           # one place per neuron, as input and as output
+        for l in (1, 4, 5, 6, 7, 9):
+            in_pos, out_at, _ = net.band_plan(l)
+            assert np.array_equal(in_pos, in0) and np.array_equal(out_at, out0)
+        for l in (0, 4, 5, 6):
+            assert np.array_equal(net.layer_dst(l), np.arange(n))
+        # the neurons of a 16-wide slot are one block of the hidden numbering
+        inv = np.argsort(perm)
+        assert all(len(set(inv[out0[16 * t:16 * t + 16]] // 16)) == 1 for t in range(n // 16))
+        for l in (0, 1, 5, 8):
+            assert np.array_equal(net.receptive_field(l, 1, np.arange(n)), np.arange(n))
+            some = np.arange(40, 56)
+            assert np.array_equal(net.receptive_field(l, 1, some), orc.receptive_field(layers[l:l + 1], some))
+        net.inspect()    # a second call finds the order again and leaves the layers as they are
+        assert [net.layer_plan(l).common_order for l in range(len(layers))] == [1, 2, 0, 0, 1, 2, 2, 1, 0, 1]
+
+
 def test_forced_gather(gc, orc):
     with gc.Network(256, 4, 2, bias=-0.3, force_kernel=gc.KERNEL_GATHER) as net:
         net.synth_layers(0, nnz_per_row=8)
