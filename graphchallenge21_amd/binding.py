@@ -38,7 +38,8 @@ class RunResult(C.Structure):
     _fields_ = [("layers_run", C.c_int32), ("compactions", C.c_int32), ("active_rows", C.c_int64),
                 ("carried_rows", C.c_int64), ("ms_total", C.c_float), ("ms_kernels", C.c_float),
                 ("alg_bytes", C.c_double), ("edges", C.c_double), ("launches", C.c_int32), ("fused_pairs", C.c_int32),
-                ("persistent_launches", C.c_int32), ("persistent_fallbacks", C.c_int32)]
+                ("persistent_launches", C.c_int32), ("persistent_fallbacks", C.c_int32),
+                ("resident_launches", C.c_int32), ("reserved", C.c_int32)]
 
 
 def lib_path():

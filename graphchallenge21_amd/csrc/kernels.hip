@@ -1541,6 +1541,179 @@ __global__ __launch_bounds__(256) void block_persist_kernel(PersistArgs a) {
     });
 }
 
+// ------------------------------------------------------------------------------------------
+// Resident launch: rows never interact, so a workgroup can keep a handful of feature rows in LDS and
+// take them through many layers with no other workgroup to wait for - the only traffic to memory is
+// the rows coming in, the rows going out and the layers' index lists (from L2).  What makes it pay
+// is the BLOCK structure (RadiX-Net layers): the 16 outputs of a group read the same 32 columns and,
+// under the layer's one exact weight, are equal, so a (group, row) item costs 32 LDS reads and 16
+// LDS writes; a layer without that structure would need 32 reads per output, and LDS would then be no
+// faster than the per-layer kernels' memory.  (The reference fuses two layers this way for one tile,
+// src/microbenchmark/fuse.cu:16-110; its loop over the other layers goes through memory and the
+// host, all_network.cu:333-519.)
+//
+// A workgroup of 1024 threads owns R consecutive rows of one row block (R = 16 for up to 1024 neurons,
+// 4 for up to 4096: two buffers of N x R floats in LDS, laid out [column][row]) and
+// thread t the item (group t / R, row t % R).  The R lanes of a group hold the group's 32 column
+// offsets and 16 output columns between them (32/R and 16/R registers each, read from memory in one
+// coalesced piece, a layer ahead) and hand them round by DPP (16-lane row broadcast for R = 16, quad
+// broadcast for R = 4).  Accumulation as in block_body: ascending input index, multiply-add by the one exact
+// weight, bias last.  One barrier per layer.  Rows are stamped with the last layer that left them
+// nonzero (the per-layer counts are taken from the stamps behind the launch); once all R rows are
+// zero and the bias is not positive the workgroup stops and stores zeros.
+// ------------------------------------------------------------------------------------------
+struct ResidentArgs {
+    const LayerDesc* table;
+    int nlayers;
+    Feat first_in, buf_a, buf_c;
+    int32_t* active;
+    int N, ngroups, rl;
+    int stamp0, prev_stamp, check_dead;
+    float bias, clampv;
+    Publish pub;
+};
+
+// the value register k / R of the lane with row index k % R of this lane's group holds (k a constant after unrolling)
+template <int R, int NREG> __device__ __forceinline__ uint32_t group_lane(const uint32_t (&v)[NREG], int k) {
+    if constexpr (R == 16) {
+        return row_lane(v[k >> 4], k & 15);
+    } else if constexpr (R == 4) {
+        const int x = (int)v[k >> 2];
+        switch (k & 3) {
+            case 0: return (uint32_t)__builtin_amdgcn_update_dpp(0, x, 0x00, 0xf, 0xf, true);
+            case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, x, 0x55, 0xf, 0xf, true);
+            case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, x, 0xaa, 0xf, 0xf, true);
+            default: return (uint32_t)__builtin_amdgcn_update_dpp(0, x, 0xff, 0xf, 0xf, true);
+        }
+    } else {
+        static_assert(R == 16 || R == 4, "rows per workgroup: 16 or 4");
+        return 0;
+    }
+}
+
+template <int R, bool FULL>
+__global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int sh_alive[3];
+    constexpr int LOG_R = R == 16 ? 4 : 2;
+    constexpr int NC = 32 / R, ND = 16 / R;    // index registers per lane
+    constexpr int VW = 4;                      // floats per memory access of a column's rows
+    constexpr int PARTS = R / VW;
+    using V = typename VecOf<VW>::type;
+    publish_counts(a.pub);
+    const int t = (int)threadIdx.x, lane = t & 63;
+    const int RB = 64 * a.rl;
+    // Workgroups go to the 8 XCDs round robin by number; a 64-byte piece of a column holds the rows of 16 / R
+    // workgroups, which should find it in ONE L2: every XCD takes a contiguous eighth of the rows.
+    const unsigned nwg = gridDim.x;
+    const unsigned wg = (nwg % 8u) == 0u ? (blockIdx.x % 8u) * (nwg / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const size_t row0 = (size_t)wg * R;
+    const int rb = (int)(row0 / (size_t)RB), rin = (int)(row0 - (size_t)rb * RB);
+    if (a.check_dead && a.prev_stamp != 0) {   // a row block without an active row is skipped, as by the per-layer kernels
+        int alive = 0;
+        for (int i = t; i < RB; i += 1024) alive |= (a.active[(size_t)rb * RB + i] == a.prev_stamp) ? 1 : 0;
+        if (__syncthreads_or(alive) == 0) return;
+    }
+    const size_t blkf = (size_t)a.N * RB;
+    // two buffers of N + 1 columns x R rows; column N takes the stores of lanes without an output
+    const uint32_t buf_bytes = (uint32_t)(a.N + 1) * R * 4;
+    unsigned char* const buf0 = smem;
+    unsigned char* const buf1 = smem + buf_bytes;
+    {
+        // (four loads in flight per thread: a workgroup has nothing else to do while its rows come in)
+        const float* __restrict__ gin = block_base(a.first_in, rb, blkf) + rin;
+        const int total = a.N * PARTS;
+        for (int base = t; base < total; base += 4096) {
+            V v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * 1024;
+                const int col = idx / PARTS, part = idx - col * PARTS;
+                if (idx < total) v[u] = *reinterpret_cast<const V*>(gin + (size_t)col * RB + part * VW);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * 1024;
+                const int col = idx / PARTS, part = idx - col * PARTS;
+                if (idx < total) *reinterpret_cast<V*>(buf0 + ((size_t)col * R + part * VW) * 4) = v[u];
+            }
+        }
+    }
+    if (t < 3) sh_alive[t] = 0;
+    const int g = t >> LOG_R, r = t & (R - 1);
+    const bool item = g < a.ngroups;
+    const int gq = item ? g : 0;               // (lanes without an item go through the motions of group 0 and store to column N)
+    // byte offsets of the group's input columns and of its outputs' columns inside a buffer, spread over the group's lanes
+    uint32_t cb[NC], db[ND], cb_next[NC], db_next[ND];
+    int cnt = 32, cnt_next = 32;
+    auto load_indices = [&](int j, uint32_t (&c)[NC], uint32_t (&d)[ND], int& n_in) {
+        const LayerDesc lay = load_layer_desc(a.table, j);
+        // (the pointers come out of the table: said to be global memory, or the loads become flat ones)
+        using GI = const __attribute__((address_space(1))) int32_t*;
+        const GI cols = (GI)lay.blk_cols, dsts = (GI)lay.blk_dst, cnts = (GI)lay.blk_cnt;
+#pragma unroll
+        for (int i = 0; i < NC; ++i) c[i] = (uint32_t)cols[(size_t)gq * 32 + i * R + r] * (uint32_t)(R * 4);
+#pragma unroll
+        for (int i = 0; i < ND; ++i) {
+            const int dcol = dsts[(size_t)gq * 16 + i * R + r];
+            d[i] = (uint32_t)((item && dcol >= 0) ? dcol : a.N) * (uint32_t)(R * 4);
+        }
+        if (!FULL) n_in = cnts[gq];
+    };
+    load_indices(0, cb, db, cnt);
+    int last_alive = -1;
+    bool all_dead = false;
+    int done_layers = 0;
+    ring_barrier<1>();
+    for (int j = 0; j < a.nlayers; ++j) {
+        const unsigned char* const in = ((j & 1) ? buf1 : buf0) + r * 4;
+        unsigned char* const out = ((j & 1) ? buf0 : buf1) + r * 4;
+        const float wu = load_layer_desc(a.table, j).wu;
+        if (j + 1 < a.nlayers) load_indices(j + 1, cb_next, db_next, cnt_next);   // in flight under this layer's arithmetic
+        float x[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k) x[k] = *reinterpret_cast<const float*>(in + group_lane<R, NC>(cb, k));
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            if (FULL || k < cnt) acc = mac<0>(acc, x[k], wu);
+        const float y = relu_clamp(acc + a.bias, a.clampv);
+#pragma unroll
+        for (int o = 0; o < 16; ++o) *reinterpret_cast<float*>(out + group_lane<R, ND>(db, o)) = y;
+        unsigned long long m = __ballot((item && y > 0.0f) ? 1 : 0);
+#pragma unroll
+        for (int sft = R; sft < 64; sft <<= 1) m |= m >> sft;
+        const int bits = (int)(m & ((1ull << R) - 1ull));
+        if (lane == 0 && bits != 0) atomicOr(&sh_alive[j % 3], bits);
+        ring_barrier<1>();
+        const int mask = sh_alive[j % 3];
+        if (t == 0) sh_alive[(j + 2) % 3] = 0;
+        if (t < R && ((mask >> t) & 1)) last_alive = j;
+        done_layers = j + 1;
+        if (mask == 0 && a.bias <= 0.0f) { all_dead = true; break; }   // zero rows stay zero
+#pragma unroll
+        for (int i = 0; i < NC; ++i) cb[i] = cb_next[i];
+#pragma unroll
+        for (int i = 0; i < ND; ++i) db[i] = db_next[i];
+        cnt = cnt_next;
+    }
+    // the launch's last layer writes the work buffer the layer before it did not (layer 0: the one it did not read)
+    const bool in_a = a.first_in.half[0] == a.buf_a.half[0];
+    const bool to_c = in_a == ((a.nlayers & 1) != 0);
+    float* const o_h0 = to_c ? a.buf_c.half[0] : a.buf_a.half[0];
+    float* const o_h1 = to_c ? a.buf_c.half[1] : a.buf_a.half[1];
+    float* __restrict__ gout = ((rb & 1) ? o_h1 : o_h0) + (size_t)(rb >> 1) * blkf + rin;
+    const unsigned char* const fin = (done_layers & 1) ? buf1 : buf0;
+    for (int idx = t; idx < a.N * PARTS; idx += 1024) {
+        const int col = idx / PARTS, part = idx - col * PARTS;
+        V v;
+        if (all_dead) v = V{};
+        else v = *reinterpret_cast<const V*>(fin + ((size_t)col * R + part * VW) * 4);
+        *reinterpret_cast<V*>(gout + (size_t)col * RB + part * VW) = v;
+    }
+    if (t < R && last_alive >= 0) a.active[row0 + t] = a.stamp0 + last_alive;
+}
+
 // counts[i] = rows whose stamp is at least stamp_lo + i (see launch_count_stamp_range): one workgroup, a
 // histogram in LDS (per wave one atomic per distinct value), then sums from the top
 __global__ __launch_bounds__(1024) void count_stamp_range_kernel(const int32_t* __restrict__ stamps, int rows, int stamp_lo,
@@ -2075,6 +2248,45 @@ hipError_t launch_persist(const PersistLaunch& a, hipStream_t s) {
         case 1: return a.block_form ? launch_persist_block_rl<1>(a, s) : launch_persist_band_rl<1>(a, s);
         default: return hipErrorInvalidValue;
     }
+}
+
+int resident_rows_per_workgroup(int N, int ngroups) {
+    if (N <= 0 || ngroups <= 0) return 0;
+    // (2 and 1 rows per workgroup - 8192 and 16384 neurons - run, but every workgroup then reads a layer's whole
+    // index lists for very few rows: measured half as fast as the per-layer kernels, so they are not offered)
+    for (int R : {16, 4})
+        if ((long long)(N + 1) * R * 8 <= 136 * 1024 && (long long)ngroups * R <= 1024) return R;
+    return 0;
+}
+
+template <int R>
+static hipError_t launch_block_resident_r(const ResidentLaunch& a, hipStream_t s) {
+    ResidentArgs k{};
+    k.table = a.table; k.nlayers = a.nlayers; k.first_in = a.first_in; k.buf_a = a.buf_a; k.buf_c = a.buf_c; k.active = a.active;
+    k.N = a.N; k.ngroups = a.ngroups; k.rl = a.rl; k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
+    k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
+    const size_t lds = (size_t)(a.N + 1) * R * 8;
+    dim3 grid((unsigned)(a.rows / R)), block(1024);
+#define SPDNN_RESIDENT(FULL)                                                                                              \
+    do {                                                                                                                  \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(block_resident_kernel<R, FULL>), \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024);       \
+        if (attr != hipSuccess) return attr;                                                                              \
+        hipLaunchKernelGGL((block_resident_kernel<R, FULL>), grid, block, lds, s, k);                                     \
+    } while (0)
+    if (a.full) SPDNN_RESIDENT(true); else SPDNN_RESIDENT(false);
+#undef SPDNN_RESIDENT
+    return hipGetLastError();
+}
+
+hipError_t launch_block_resident(const ResidentLaunch& a, hipStream_t s) {
+    // host-side shape checks: what the kernel's item numbering and its two LDS buffers assume
+    if (a.N <= 0 || a.nlayers < 1 || !a.table || !a.first_in || !a.buf_a || !a.buf_c || a.buf_a == a.buf_c || !a.active ||
+        a.ngroups <= 0 || a.rows <= 0 || (a.rl != 1 && a.rl != 2 && a.rl != 4) || (a.rows % (64 * a.rl)) != 0)
+        return hipErrorInvalidValue;
+    const int R = resident_rows_per_workgroup(a.N, a.ngroups);
+    if (R == 0 || (64 * a.rl) % R != 0 || (long long)a.rows / R > 0x7fffffffll) return hipErrorInvalidValue;
+    return R == 16 ? launch_block_resident_r<16>(a, s) : launch_block_resident_r<4>(a, s);
 }
 
 hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,

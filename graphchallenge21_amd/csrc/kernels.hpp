@@ -202,6 +202,26 @@ struct PersistLaunch {
 int persist_units(const PersistLaunch& a);
 hipError_t launch_persist(const PersistLaunch& a, hipStream_t s);
 
+// Resident launch: `nlayers` consecutive layers that all have a BLOCK form with one exact weight (BLOCK layers of
+// weight mode 0, run-chain BAND layers that carry their BLOCK form) and the same group count, run by workgroups
+// that keep R rows each in LDS from the first layer to the last (block_resident_kernel); no workgroup waits for
+// another, so such a launch cannot give up.  Buffers as in PersistLaunch.  Rows get the stamp of the last layer
+// that left them nonzero (stamp0 + j), none if no layer did; count with launch_count_stamp_range.
+struct ResidentLaunch {
+    const LayerDesc* table;       // device pointer to the entry of the launch's first layer
+    int nlayers;
+    Feat first_in, buf_a, buf_c;
+    int32_t* active;
+    int N, ngroups, rows, rl, full;   // rows: carried rows (whole row blocks); full: every group has 32 inputs
+    int stamp0, prev_stamp, check_dead;
+    float bias, clampv;
+    Publish publish;
+};
+// rows a workgroup keeps (16 or 4), 0 if the shape does not fit: two buffers of (N + 1) x R floats in LDS
+// (N <= 1024: 16 rows, N <= 4096: 4) and one (group, row) item per thread of 1024
+int resident_rows_per_workgroup(int N, int ngroups);
+hipError_t launch_block_resident(const ResidentLaunch& a, hipStream_t s);
+
 // counts[i] = number of rows r < rows with stamps[r] >= stamp_lo + i, for i in [0, n): with bias <= 0 a
 // row that is zero stays zero, so the rows that carry the stamp of layer l or a later one are the rows
 // layer l left active.  Written to counts_dev and (system scope) to counts_host, either may be nullptr.

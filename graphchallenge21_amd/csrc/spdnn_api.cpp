@@ -268,9 +268,12 @@ struct spdnn_net {
     // SPDNN_PERSIST_MAX_BYTES).  Measured, batch 60000, sustained, per layer: N=1024 102.7 -> 99.1 us, N=4096 344 -> 325 us,
     // N=16384 1285 -> 1280 us (beyond the upper bound: left alone); N=1024 with batch 6000 15.9 -> 18.2 us (below the lower).
     long long persist_min_bytes = (long long)1 << 28, persist_max_bytes = (long long)1 << 31;
+    int persist_min_blocks = 64;      // fewest row blocks a persistent launch is made for by default (SPDNN_PERSIST_MIN_BLOCKS)
     int persist_xcd = -1;             // one unit queue per XCD: -1 = from 8 row blocks up, 0 / 1 (SPDNN_PERSIST_XCD)
     int persist_light = 1;            // SPDNN_PERSIST_LIGHT_SYNC=0: device-scope fences also with XCD queues (3 times slower)
     int persist_seglen = 0;           // band positions / groups per unit, 0 = heuristic (SPDNN_PERSIST_SEGLEN)
+    int resident_mode = 1;            // 1: layers with a BLOCK form of one exact weight run as resident launches where the
+                                      // shape fits (rows kept in LDS through the layers; SPDNN_RESIDENT=0: never)
     long long persist_wait_us = 2000000;   // longest wait of a unit for its row block (SPDNN_PERSIST_WAIT_US)
     int band_seglen = 0;              // SPDNN_BAND_SEGLEN: band positions per workgroup of the per-layer walk (0 = run-time selection)
     int band_direct_lds = 1;          // SPDNN_BAND_DIRECT_LDS=0: the per-layer walk never loads straight into LDS
@@ -886,8 +889,10 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_PERSIST_MAX_BYTES")) n->persist_max_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_PERSIST_MIN_BYTES")) n->persist_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_PERSIST_XCD")) n->persist_xcd = atoi(e);
+    if (const char* e = getenv("SPDNN_PERSIST_MIN_BLOCKS")) n->persist_min_blocks = std::max(1, atoi(e));
     if (const char* e = getenv("SPDNN_PERSIST_LIGHT_SYNC")) n->persist_light = atoi(e);
     if (const char* e = getenv("SPDNN_PERSIST_SEGLEN")) n->persist_seglen = std::max(0, atoi(e));
+    if (const char* e = getenv("SPDNN_RESIDENT")) n->resident_mode = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PERSIST_WAIT_US")) n->persist_wait_us = std::max(0ll, atoll(e));
     if (const char* e = getenv("SPDNN_BAND_SEGLEN")) n->band_seglen = std::max(0, atoi(e));
     if (const char* e = getenv("SPDNN_BAND_DIRECT_LDS")) n->band_direct_lds = atoi(e) != 0 ? 1 : 0;
@@ -1585,6 +1590,25 @@ static LayerSig layer_sig(const spdnn_net* n, int l, int nblk) {
     return g;
 }
 
+// Whether layer l can be part of a resident launch (rows kept in LDS through the layers): it needs a BLOCK form
+// with one exact weight - a BLOCK layer of weight mode 0, or a run-chain BAND layer that carries its BLOCK form -
+// and a shape the kernel's LDS buffers and item numbering hold.
+struct ResidentSig {
+    int ok = 0, full = 0, ngroups = 0;
+    bool operator==(const ResidentSig& o) const { return ok == o.ok && full == o.full && ngroups == o.ngroups; }
+};
+static ResidentSig resident_sig(const spdnn_net* n, int l) {
+    const LayerPlan& p = n->layers[(size_t)l];
+    ResidentSig g;
+    if (p.kernel == SPDNN_KERNEL_BAND && p.alt_ngroups > 0) { g.ok = 1; g.full = p.alt_full ? 1 : 0; g.ngroups = p.alt_ngroups; }
+    else if (p.kernel == SPDNN_KERNEL_BLOCK && p.wmode == 0) { g.ok = 1; g.full = p.blk_full ? 1 : 0; g.ngroups = p.ngroups; }
+    if (g.ok) {
+        const int R = resident_rows_per_workgroup(n->N, g.ngroups);
+        if (R == 0 || n->RB % R != 0) g.ok = 0;
+    }
+    return g;
+}
+
 static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
     if (!n) return fail(SPDNN_E_ARG, "net is NULL");
     spdnn_run_options opt;
@@ -1785,19 +1809,36 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 return pair_mode && pk.fuse_next && k + 1 <= last && !use_block_form(n, pk, nblk) &&
                        (opt.fuse_layers >= 2 || (int64_t)nblk * (int64_t)n->RB * (int64_t)n->N >= n->pair_min_elems);
             };
-            const bool pair = !fb && is_pair(l);
+            // a resident launch (rows kept in LDS through the layers) where consecutive layers have the structure for it:
+            // no launch, fused or not, that goes through memory between the layers comes near it
+            int c = 1;
+            bool resident = false, persist = false;
+            ResidentSig rsig;
+            int cmax = std::min(persist_cmax, last - l + 1);
+            if (opt.prune && !persist_asked) cmax = std::min(cmax, st.c_prune);   // short launches while the counts still move
+            if (!fb && persist_on && n->resident_mode && n->d_table && (rsig = resident_sig(n, l)).ok) {
+                // Bringing the rows in and out costs such a launch as much as two layers save it with 16 rows per workgroup
+                // (64-byte pieces of a column) and as much as eight save it with 4 rows (16-byte pieces): measured
+                // at 2048 and at 60000 rows.  So left to the library: from 2 layers (even while the counts still move -
+                // workgroups whose rows have all died leave early) and from 8; a caller that asks for launches of a
+                // given length gets them.
+                const bool wide_rows = resident_rows_per_workgroup(n->N, rsig.ngroups) >= 16;
+                const int rmin = (persist_asked || wide_rows) ? 2 : 8;
+                const int rmax = std::min(wide_rows ? std::max(cmax, 2) : cmax, last - l + 1);
+                int k = 1;
+                while (k < rmax && resident_sig(n, l + k) == rsig) ++k;
+                if (k >= rmin) { c = k; resident = true; }
+            }
+            const bool pair = !fb && !resident && is_pair(l);
+            if (pair) c = 2;
             // a persistent launch: consecutive layers of one kernel form and variant
-            int c = pair ? 2 : 1;
-            bool persist = false;
             LayerSig sig;
             if (fb) {
                 c = fb_c;
-            } else if (!pair && persist_on) {
+            } else if (!pair && !resident && persist_on) {
                 sig = layer_sig(n, l, nblk);
                 const long long layer_bytes = 8ll * (long long)n->carried * (long long)n->N;
-                const bool small = layer_bytes >= n->persist_min_bytes && layer_bytes <= n->persist_max_bytes && nblk >= 8;
-                int cmax = std::min(persist_cmax, last - l + 1);
-                if (opt.prune && !persist_asked) cmax = std::min(cmax, st.c_prune);   // short launches while the counts still move
+                const bool small = layer_bytes >= n->persist_min_bytes && layer_bytes <= n->persist_max_bytes && nblk >= n->persist_min_blocks;
                 if (sig.form >= 0 && (persist_asked || small) && cmax >= 2 && next_slot < n->L) {
                     int k = 1;
                     while (k < cmax && !is_pair(l + k) && layer_sig(n, l + k, nblk) == sig) ++k;   // (a fused pair stays a pair)
@@ -1821,7 +1862,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
             State at_start{};
             if (persist) at_start = save();
             if (check_dead && (prev_stamp != 0 || c > 1)) n->blocks_skipped = true;
-            const bool group = persist || fb;   // c layers whose rows are counted behind them, from the stamps
+            const bool group = persist || fb || resident;   // c layers whose rows are counted behind them, from the stamps
             int32_t* const count_prev = (fused_count && st.count_pending && prev_stamp != 0 && !group) ? n->d_counts + (l - 1) : nullptr;
             const Feat in = n->cur;
             Feat out = (n->cur == n->A) ? n->C : n->A;
@@ -1886,6 +1927,18 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                             pl.xcd_queues, pl.light_sync);
                 for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
                 st.r.persistent_launches += 1;
+            } else if (resident) {
+                ResidentLaunch rl{};
+                rl.table = n->d_table + l; rl.nlayers = c; rl.first_in = in; rl.buf_a = n->A; rl.buf_c = n->C; rl.active = n->d_active;
+                rl.N = n->N; rl.ngroups = rsig.ngroups; rl.rows = n->carried; rl.rl = n->rl; rl.full = rsig.full;
+                rl.stamp0 = stamp0; rl.prev_stamp = prev_stamp; rl.check_dead = check_dead; rl.bias = n->bias; rl.clampv = n->clampv;
+                rl.publish = st.pub;
+                HIPCHK(launch_block_resident(rl, n->stream));
+                if (n->run_verbose)
+                    fprintf(stderr, "spdnn: resident launch: layers %d..%d, %d rows, %d rows per workgroup\n", l, l + c - 1, n->carried,
+                            resident_rows_per_workgroup(n->N, rsig.ngroups));
+                for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
+                st.r.resident_launches += 1;
             } else if (fb) {
                 Feat fin = in, fout = out;
                 for (int j = 0; j < c; ++j) {
@@ -1970,7 +2023,9 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
             if (!opt.prune) continue;
 
             // a record is pushed when the launch that hands it over is queued, i.e. one launch late
-            const size_t lookahead = lookahead_for(n->carried) - 1;
+            // (while the counts are unknown or still moving the host waits for each launch's counts: a launch made on rows
+            // that have died since costs more than the round trip)
+            const size_t lookahead = st.c_prune <= 1 ? 0 : lookahead_for(n->carried) - 1;
             while (recs.size() - st.processed > lookahead && !st.dead && failed < 0) {
                 const Rec rc = recs[st.processed++];
                 const int wrc = wait_counts(n, rc.l0, rc.c);
@@ -1981,13 +2036,17 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                     if (failed >= 0) break;
                 }
                 const int64_t before = st.newest_count;
+                int64_t layer_before = before;
                 for (int j = rc.l0; j < rc.l0 + rc.c && !st.dead; ++j) {
+                    layer_before = st.newest_count;
                     st.newest_count = n->h_counts[j];
                     if (st.newest_count == 0) st.dead = true;
                 }
-                // layers per persistent launch while pruning: doubled while the counts hold still (within 3 % from
-                // one record to the next), one layer per launch again when they move
-                if (before > 0 && st.newest_count * 100 >= before * 97) st.c_prune = std::min(persist_cmax, std::max(2, st.c_prune * 2));
+                // layers per multi-layer launch while pruning: all that are allowed once a layer has left the count as it
+                // was, doubled while the counts hold still (within 3 % from one record to the next), one layer per
+                // launch again when they move
+                if (layer_before > 0 && st.newest_count == layer_before) st.c_prune = std::max(2, persist_cmax);
+                else if (before > 0 && st.newest_count * 100 >= before * 97) st.c_prune = std::min(persist_cmax, std::max(2, st.c_prune * 2));
                 else st.c_prune = 1;
             }
             if (failed >= 0) break;

@@ -115,6 +115,8 @@ typedef struct spdnn_run_result {
     int32_t fused_pairs;     /* of them, fused pairs of layers (intermediate tile in LDS)         */
     int32_t persistent_launches;   /* of them, persistent launches (several layers, a dependency per row block)   */
     int32_t persistent_fallbacks;  /* persistent launches that gave up and were finished by per-layer launches     */
+    int32_t resident_launches;     /* of the launches, resident ones (several layers, the rows kept in LDS throughout) */
+    int32_t reserved;
 } spdnn_run_result;
 
 /* ---- life cycle ------------------------------------------------------------------------- */

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 from helpers import random_csr, same_floats, sort_rows
-from helpers import common_band_csr, radix_like_csr
+from helpers import common_band_csr, hub_block_csr, radix_like_csr
 
 pytestmark = pytest.mark.gpu
 
@@ -527,6 +527,94 @@ def test_persistent_launch_that_gives_up(gc, orc, prune, mode, monkeypatch):
         assert same_floats(net.activations(cats), ref["y"])
 
 
+@pytest.mark.parametrize("N,B,kind", [(256, 300, "radix"), (1024, 2100, "radix"), (1024, 700, "hub"), (4096, 1300, "radix")])
+def test_resident_launches(gc, orc, N, B, kind):
+    """RadiX-Net-like layers of one exact weight, up to 4096 neurons wide, run as resident launches: a workgroup keeps
+    16 or 4 rows (by the width) in LDS through all layers of the launch.  Per-layer counts, categories and activations against
+    the oracle, pruned and unpruned, whole and cut into calls, and the state after every layer; `hub` layers have
+    groups of fewer than 32 inputs."""
+    print("resident launches N=%d B=%d %s" % (N, B, kind), flush=True)
+    rng = np.random.default_rng(N + B)
+    nst = int(np.log2(N)) - 4
+    if kind == "hub":
+        base = [hub_block_csr(rng, N) for _ in range(3)]
+    else:
+        base = [radix_like_csr(rng, N, 16 << k) for k in range(nst)]
+    L = 2 * len(base) + 1
+    layers = [base[l % len(base)] for l in range(L)]
+    dens = np.where(rng.random(B) < 0.3, 0.7, 0.08).astype(np.float32)
+    feats = (rng.random((B, N), dtype=np.float32) < dens[:, None]).astype(np.float32)
+    bias = -0.3 if N <= 1024 else -0.35 if N <= 4096 else -0.4
+    ref = orc.infer(feats, layers, bias, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    assert 0 < want_counts[-1] < B
+    with gc.Network(N, B, L, bias=bias) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.set_features_dense(feats)
+        cats = ref["categories"]
+        for prune in (True, False):
+            for fuse in (0, 5, 1):
+                r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert r.layers_run == L
+                assert r.persistent_launches == 0 and (r.resident_launches == 0) == (fuse == 1) or (fuse == 0 and prune)
+                if fuse == 5:
+                    assert r.resident_launches == L // 5 + (1 if L % 5 >= 2 else 0) and r.launches == (L + 4) // 5
+                assert [net.active_count(l) for l in range(L)] == want_counts
+                assert np.array_equal(net.categories(), cats)
+                assert same_floats(net.activations(cats), ref["y"])
+                dead = np.setdiff1d(np.arange(B), cats)[:64].astype(np.int32)
+                assert not net.activations(dead).any()
+        for l in range(1, L, 2):    # the state after layer l, from a resident launch that ends there
+            net.run(prune=True, first_layer=0, n_layers=l + 1, fuse_layers=L)
+            gid, y = ref["kept"][l]
+            assert np.array_equal(net.categories(), ref["active_ids"][l])
+            assert same_floats(net.activations(gid), y)
+        # cut into calls: resident, layer by layer, resident again (odd and even layer counts)
+        net.run(prune=True, first_layer=0, n_layers=3, fuse_layers=3)
+        net.run(prune=True, first_layer=3, n_layers=1, fuse_layers=1)
+        r = net.run(prune=False, first_layer=4, n_layers=L - 4, collect_counts=True, fuse_layers=L)
+        assert r.resident_launches == 1
+        assert [net.active_count(l) for l in range(4, L)] == want_counts[4:]
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(cats), ref["y"])
+
+
+def test_resident_launches_full_batch(gc, orc):
+    """Batch 60000 of RadiX-Net-like layers, N=1024: every activation of every row, the per-layer counts and the
+    categories of the default run (resident launches) equal those of one launch per layer bit for bit, on live
+    data, pruned and unpruned; an oracle row sample pins both."""
+    N, L, B, S, bias = 1024, 30, 60000, 256, -0.3
+    print("resident launches, full batch", flush=True)
+    rng = np.random.default_rng(5)
+    base = [radix_like_csr(rng, N, 16 << k) for k in range(6)]
+    layers = [base[l % 6] for l in range(L)]
+    dens = np.where(rng.random(B) < 0.3, 0.7, 0.08).astype(np.float32)
+    feats = (rng.random((B, N), dtype=np.float32) < dens[:, None]).astype(np.float32)
+    ref = orc.infer(feats[:S], layers, bias, prune=False, keep={L - 1})
+    rows = np.arange(B, dtype=np.int32)
+    with gc.Network(N, B, L, bias=bias) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        net.set_features_dense(feats)
+
+        def state():
+            acts = np.concatenate([net.activations(rows[i:i + 8192]) for i in range(0, B, 8192)])
+            return acts, [net.active_count(l) for l in range(L)], net.categories()
+
+        r1 = net.run(prune=False, collect_counts=True, fuse_layers=1)
+        want = state()
+        assert r1.resident_launches == 0 and len(want[2]) > 1000
+        assert same_floats(want[0][:S], ref["kept"][L - 1][1])
+        for prune in (False, True):
+            r = net.run(prune=prune, collect_counts=True)
+            assert r.resident_launches >= 1
+            got = state()
+            assert np.array_equal(got[0], want[0]) and got[1] == want[1] and np.array_equal(got[2], want[2]), prune
+
+
 @pytest.mark.parametrize("mode", ["one-queue", "xcd-queues-light"])
 @pytest.mark.parametrize("N,B,values", [(1024, 2100, "uniform"), (1024, 900, "general"), (4096, 1300, "uniform")])
 def test_persistent_launches_block_kernel(gc, orc, N, B, values, mode, monkeypatch):
@@ -534,6 +622,7 @@ def test_persistent_launches_block_kernel(gc, orc, N, B, values, mode, monkeypat
     several layers per launch: bit-equal to the oracle, pruned and unpruned, and to one launch per layer."""
     for k, v in PERSIST_MODES[mode].items():
         monkeypatch.setenv(k, v)
+    monkeypatch.setenv("SPDNN_RESIDENT", "0")    # (layers of one exact weight would otherwise run as resident launches)
     print("persistent BLOCK launches N=%d B=%d %s %s" % (N, B, values, mode), flush=True)
     rng = np.random.default_rng(N + B)
     nst = int(np.log2(N)) - 4
@@ -625,6 +714,7 @@ def test_fused_pairs_radix_common(gc, orc, monkeypatch):
     want_counts = [len(a) for a in ref["active_ids"]]
     assert 0 < want_counts[-1] < B
     monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", "0")   # a batch this small would run the layers' BLOCK form
+    monkeypatch.setenv("SPDNN_RESIDENT", "0")   # and layers this narrow as resident launches (the pairs are for wider ones)
     with gc.Network(N, B, L, bias=-0.4) as net:
         for l, csr in enumerate(layers):
             net.set_layer_csr(l, *csr)
