@@ -171,6 +171,9 @@ def main():
                          "layers (one per stride 16, 32, ... n/2, repeated; radix-common: all of them behind one hidden "
                          "neuron numbering, as the layer files of one challenge network), bands over one common order, "
                          "or layers without structure (n <= 4096)")
+    ap.add_argument("--density-hi", type=float, default=0.25,
+                    help="features: every row's density is drawn from U[0.10, this] (0.25 = the configured workload, whose rows "
+                         "all die within two layers; 0.7 = live data: rows survive every layer)")
     ap.add_argument("--cpu-rows", type=int, default=0, help="rows of the CPU sample (0 = auto)")
     ap.add_argument("--cpu-layers", type=int, default=6, help="layers the CPU baseline is timed on")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and the parity gate")
@@ -233,7 +236,7 @@ def main():
     kernels_used = sorted({kernel_names[p.kernel] for p in plans})
     nnz_layer = float(sum(p.nnz for p in plans)) / L     # the same for every layer except with --structure irregular
     t0 = time.time()
-    net.synth_features(seed, B, 0.10, 0.25)
+    net.synth_features(seed, B, 0.10, args.density_hi)
     t_features = time.time() - t0
     log("setup: inspector %.1f s (%d/%d layers BAND, kernels %s), plan upload + features %.1f s"
         % (t_inspect, n_band, L, "+".join(kernels_used), t_features))
@@ -277,7 +280,7 @@ def main():
         buffer_copy_gbps = net.buffer_copy_bandwidth(3)            # the work buffers where they lie
     except gc.SpdnnError:
         buffer_copy_gbps = None
-    net.synth_features(seed, B, 0.10, 0.25)                    # the probe resets the state
+    net.synth_features(seed, B, 0.10, args.density_hi)                    # the probe resets the state
 
     # ---- live data: the same sustained run on features whose rows survive (densities up to 0.7) --
     live = None
@@ -292,7 +295,7 @@ def main():
                 "frac": alg_bytes_launch / (live_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "unit": "GB/s",
                 "launches_timed": int(lms.size), "rows_nonzero_at_end": int(rl.active_rows),
                 "edges_per_s": edges / (rl.ms_total * 1e-3)}
-        net.synth_features(seed, B, 0.10, 0.25)
+        net.synth_features(seed, B, 0.10, args.density_hi)
 
     # ---- CPU baseline + parity gate on a row sample ---------------------------------------------
     cpu = None
@@ -302,7 +305,7 @@ def main():
         cores = orc.get_threads()
         rows = args.cpu_rows or max(256, min(B, int(7.0e10 * max(cores, 1) / 16 / (N * 32.0))) // 256 * 256)
         rows = min(rows, B)
-        feats = orc.gen_features(seed, N, 0, rows, 0.10, 0.25)
+        feats = orc.gen_features(seed, N, 0, rows, 0.10, args.density_hi)
         # timed: the first layers of the same workload, chained, on the sample rows (every row kept,
         # as in the sustained run); the first three of them are the parity reference below
         n_cpu = min(L, args.cpu_layers)
@@ -354,7 +357,7 @@ def main():
                 cpu_counts = np.zeros(L, np.int64)
                 layers_cache = {}
                 for r0 in range(0, B, chunk):
-                    y = orc.gen_features(seed, N, r0, min(chunk, B - r0), 0.10, 0.25)
+                    y = orc.gen_features(seed, N, r0, min(chunk, B - r0), 0.10, args.density_hi)
                     gid = np.arange(len(y), dtype=np.int32)
                     for l in range(L):
                         if l not in layers_cache:
@@ -462,13 +465,19 @@ def main():
             "final_active_rows": sustained_final_active,
             "launches_per_pass": int(r.launches), "fused_pairs_per_pass": int(r.fused_pairs),
             "persistent_launches_per_pass": int(r.persistent_launches),
+            "resident_launches_per_pass": int(r.resident_launches),
+            "feature_density": [0.10, args.density_hi],
         },
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
                      "kernel": "+".join(kernels_used), "alg_bytes_per_launch": alg_bytes_launch,
                      "avg_launch_ms": avg_launch_ms, "launches_timed": int(layer_ms.size),
-                     "data": "all-zero activations from layer 2 on (bias -0.45 kills every row of the configured features); "
-                             "see roofline_live for the same run on live data",
+                     "note": ("resident launches: the rows stay in LDS between the layers of a launch, so the algorithmic bytes of a "
+                              "layer never reach HBM and `frac` (algorithmic bytes over time, against the HBM peak) is not a bound "
+                              "here - the kernel is bound by LDS") if r.resident_launches else None,
+                     "data": ("all-zero activations from layer 2 on (bias -0.45 kills every row of the configured features); "
+                              "see roofline_live for the same run on live data") if args.density_hi <= 0.25 else
+                             "live data: feature densities U[0.10, %g]" % args.density_hi,
                      "copy_kernel_gbps_plain_allocations": copy_gbps,
                      "copy_kernel_gbps_work_buffers": buffer_copy_gbps,
                      "frac_of_work_buffer_copy": achieved / buffer_copy_gbps if buffer_copy_gbps else None,

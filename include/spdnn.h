@@ -89,13 +89,18 @@ typedef struct spdnn_run_options {
     int32_t collect_counts;    /* 1: record the active-row count after every layer                 */
     int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
-    int32_t fuse_layers;       /* fused variants.  1 = every layer its own launch.  0 = default: pairs of layers
-                                  the inspector marked fuse_next run as one launch with the intermediate tile in
-                                  LDS where that is the faster way (launches of 2^23 rows x neurons and more;
-                                  SPDNN_PAIR_MIN_ELEMS), every other layer as its own launch (SPDNN_FUSE_LAYERS
-                                  = n makes n the default).  >1: the pairs, and elsewhere up to that many
-                                  consecutive band layers share a launch (one workgroup keeps a row block
-                                  through the chain, the intermediates going through L2) */
+    int32_t fuse_layers;       /* launches that hold more than one layer.  1 = every layer its own launch.  0 = default:
+                                  - resident launches where consecutive layers have a BLOCK form with one exact weight and
+                                    at most 4096 neurons (RadiX-Net layers): a workgroup keeps 16 or 4 rows in LDS through
+                                    up to 64 layers (SPDNN_RESIDENT=0: never);
+                                  - pairs of layers the inspector marked fuse_next as one launch with the intermediate tile
+                                    in LDS, on launches of 2^23 rows x neurons and more (SPDNN_PAIR_MIN_ELEMS);
+                                  - persistent launches (up to 64 layers of one kernel form, a dependency per row block
+                                    between the layers) where a layer moves 256 MiB - 2 GiB on 64 row blocks or more
+                                    (SPDNN_PERSIST=0: never);
+                                  - every other layer as its own launch.
+                                  n >= 2: the pairs, and elsewhere resident or persistent launches of up to n layers
+                                  whatever the size.  Results are the same bit for bit in every mode. */
     int32_t persist_wait_us;   /* persistent launches: longest wait of a unit for its row block in microseconds; 0 = default
                                   (2 s, SPDNN_PERSIST_WAIT_US), negative = give up at the first look that finds the row
                                   block not ready (exercises the fall-back to per-layer launches)                     */
