@@ -713,6 +713,8 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.alt_cnt.clear();
     plan.alt_out_at.clear();
     plan.alt_dst.clear();
+    plan.alt_wv.clear();
+    plan.alt_kmax = 0;
     if (band && halo == 32 && uniform && exact) {
         // the BLOCK form of a run-chain layer, its columns in the band's input labelling
         plan.alt_ngroups = (int)groups.size();
@@ -817,6 +819,22 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
         plan.sel.clear();
         plan.pairs.clear();
+        // its GATHER form, for launches too small to fill the chip with tiles
+        const int kw = std::max(kmax, 1);
+        plan.alt_kmax = kw;
+        plan.alt_cols.assign((size_t)N * kw, 0);
+        plan.alt_wv.assign((size_t)N * kw, 0.0f);
+        plan.alt_cnt.resize((size_t)N);
+        plan.alt_out_at.resize((size_t)N);
+        std::iota(plan.alt_out_at.begin(), plan.alt_out_at.end(), 0);
+        for (int j = 0; j < N; ++j) {
+            const int len = rowptr[j + 1] - rowptr[j];
+            plan.alt_cnt[(size_t)j] = len;
+            for (int k = 0; k < len; ++k) {
+                plan.alt_cols[(size_t)j * kw + k] = col[rowptr[j] + k];
+                plan.alt_wv[(size_t)j * kw + k] = val[rowptr[j] + k];
+            }
+        }
     } else {
         plan.kernel = SPDNN_KERNEL_GATHER;
         plan.wmode = exact ? 1 : 2;
@@ -841,10 +859,10 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.pairs.clear();
     }
     plan.info.kernel = plan.kernel;
-    plan.info.block_form = plan.alt_ngroups > 0 ? 1 : 0;
+    plan.info.block_form = plan.alt_ngroups > 0 ? 1 : (plan.alt_kmax > 0 ? 2 : 0);
     plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
                                                               plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
-                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() +
+                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() + plan.alt_wv.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.failed = false;

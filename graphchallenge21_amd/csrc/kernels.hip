@@ -2059,10 +2059,14 @@ bool band_unrolled(int K, int steps, int stride) { return K == 32 && steps <= 36
 // compute / barrier phases interleave), 32 and 16 KiB and four workgroups per CU (the wave limit)
 // for 128- and 64-row blocks.  Measured at N=65536: 256-row blocks 6.0 ms per layer, 128-row blocks
 // 6.6 ms (8.8 ms with one 16-wave workgroup and a 256-slot ring per CU).
-// Variants of the band walk the run-time selection chooses from (BandLaunch.shape): for 256-row
-// blocks 0 = next chunk's columns straight from HBM into the LDS ring, 1 = parked in registers and
-// written to the ring after the arithmetic (the only form for smaller row blocks).
-int band_shape_count(int rl, int direct_lds) { return rl == 4 && direct_lds ? 2 : 1; }
+// Variants of the band walk (BandLaunch.shape, BandLaunch.direct_lds): for 256-row blocks the next chunk's
+// columns go straight from HBM into the LDS ring (shape 0 with direct_lds), or are parked in registers and
+// written to the ring after the arithmetic (shape 1, or direct_lds off; the only form for smaller row
+// blocks).  The run-time selection used to try both; measured one after the other on live data, per layer:
+// N=1024 102.9 against 107.0 us, N=4096 337.9 against 352 - 380, N=16384 1280 against 1291, N=65536 and batch
+// 6000 within the noise - straight into LDS is never the slower one, so it is the one form the selection
+// uses and only the segment length is left to it.
+int band_shape_count(int rl, int direct_lds) { (void)rl; (void)direct_lds; return 1; }
 
 int band_chunk_outputs(int rl, int shape) {
     (void)rl; (void)shape;
@@ -2181,10 +2185,10 @@ PersistArgs persist_args(const PersistLaunch& a, const PersistShape& p) {
     return k;
 }
 
-template <int RL, int WMODE, int KT>
-hipError_t launch_persist_band_inst(const PersistLaunch& a, hipStream_t s) {
+template <int RL, int WMODE, int KT, int DMA>
+hipError_t launch_persist_band_dma(const PersistLaunch& a, hipStream_t s) {
     constexpr size_t lds = (size_t)64 * 64 * RL * 4;
-    auto kern = band_persist_kernel<RL, WMODE, KT, 0>;
+    auto kern = band_persist_kernel<RL, WMODE, KT, DMA>;
     // once per instantiation; a function-local static is initialised by one thread only
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -2192,6 +2196,14 @@ hipError_t launch_persist_band_inst(const PersistLaunch& a, hipStream_t s) {
     const PersistShape p = persist_shape(a);
     hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), lds, s, persist_args(a, p));
     return hipGetLastError();
+}
+// (256-row blocks: the next chunk's columns straight into the LDS ring, as in the per-layer launches)
+template <int RL, int WMODE, int KT>
+hipError_t launch_persist_band_inst(const PersistLaunch& a, hipStream_t s) {
+    if constexpr (RL == 4) {
+        if (a.direct_lds) return launch_persist_band_dma<RL, WMODE, KT, 1>(a, s);
+    }
+    return launch_persist_band_dma<RL, WMODE, KT, 0>(a, s);
 }
 template <int RL>
 hipError_t launch_persist_band_rl(const PersistLaunch& a, hipStream_t s) {

@@ -188,6 +188,7 @@ struct PersistLaunch {
     int32_t* host_word;           // pinned host word: receives the unit total when the launch is complete, -2 on abort
     int N, K, nblk, rl, wmode, stamp0, prev_stamp, check_dead;
     int unrolled, add_only, twins, full;   // kernel variant, as in BandLaunch / BlockLaunch
+    int direct_lds;               // band walk on 256-row blocks: columns straight into the LDS ring (as BandLaunch.direct_lds)
     int seglen;                   // band positions (band walk) or groups (BLOCK) per unit; 0 = heuristic
     int xcd_queues;               // 1: one queue per XCD, row block rb in queue rb % 8
     int light_sync;               // 1 (xcd_queues only): the hand-over between layers stays inside one L2, so the

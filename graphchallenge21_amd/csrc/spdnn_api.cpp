@@ -181,12 +181,13 @@ struct DevLayer {
     int32_t* alt_cols = nullptr;   // the BLOCK form of a run-chain BAND layer (see LayerPlan)
     int32_t* alt_cnt = nullptr;
     int32_t* alt_dst = nullptr;
+    float* alt_wv = nullptr;       // (with alt_cols / alt_cnt / alt_dst: the GATHER form of a TILED layer)
 };
 
 // Where the arrays of one layer's plan lie inside its block of device memory (and inside the
 // pinned host copy of that block when plans are streamed): pairs, ell, rowlen, wv, dst, blk_cols,
-// blk_cnt, alt_cols, alt_cnt, alt_dst, each aligned to 256 bytes.
-constexpr int kPlanArrays = 10;
+// blk_cnt, alt_cols, alt_cnt, alt_dst, alt_wv, each aligned to 256 bytes.
+constexpr int kPlanArrays = 11;
 struct PlanLayout {
     size_t off[kPlanArrays] = {};
     size_t len[kPlanArrays] = {};
@@ -295,6 +296,7 @@ struct spdnn_net {
     // per CU, few segments).
     int64_t pair_min_elems = (int64_t)1 << 23;
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
+    int64_t tiled_min_rows = 8192;                    // see use_gather_form (SPDNN_TILED_MIN_ROWS)
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
     LayerDesc* d_table = nullptr;   // one entry per layer (resident plans only)
@@ -571,7 +573,7 @@ PlanLayout plan_layout(const LayerPlan& p) {
     PlanLayout y;
     const size_t len[kPlanArrays] = {p.pairs.size() * 4,    p.ell_col.size() * 4,  p.rowlen.size() * 4,   p.wv.size() * 4,
                                      p.dst.size() * 4,      p.blk_cols.size() * 4, p.blk_cnt.size() * 4,  p.alt_cols.size() * 4,
-                                     p.alt_cnt.size() * 4,  p.alt_dst.size() * 4};
+                                     p.alt_cnt.size() * 4,  p.alt_dst.size() * 4,  p.alt_wv.size() * 4};
     for (int k = 0; k < kPlanArrays; ++k) {
         y.off[k] = y.bytes;
         y.len[k] = len[k];
@@ -582,7 +584,8 @@ PlanLayout plan_layout(const LayerPlan& p) {
 
 void pack_plan(const LayerPlan& p, const PlanLayout& y, char* dst) {
     const void* src[kPlanArrays] = {p.pairs.data(),   p.ell_col.data(),  p.rowlen.data(),  p.wv.data(),      p.dst.data(),
-                                    p.blk_cols.data(), p.blk_cnt.data(), p.alt_cols.data(), p.alt_cnt.data(), p.alt_dst.data()};
+                                    p.blk_cols.data(), p.blk_cnt.data(), p.alt_cols.data(), p.alt_cnt.data(), p.alt_dst.data(),
+                                    p.alt_wv.data()};
     for (int k = 0; k < kPlanArrays; ++k)
         if (y.len[k]) memcpy(dst + y.off[k], src[k], y.len[k]);
 }
@@ -600,6 +603,7 @@ DevLayer plan_at(const PlanLayout& y, char* base) {
     d.alt_cols = (int32_t*)at(7);
     d.alt_cnt = (int32_t*)at(8);
     d.alt_dst = (int32_t*)at(9);
+    d.alt_wv = (float*)at(10);
     return d;
 }
 
@@ -901,6 +905,7 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
+    if (const char* e = getenv("SPDNN_TILED_MIN_ROWS")) n->tiled_min_rows = atoll(e);
     if (const char* e = getenv("SPDNN_STREAM_MIN_BYTES")) n->stream_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_COUNT_TIMEOUT_MS")) n->count_timeout_ms = std::max(1ll, atoll(e));
     if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
@@ -1482,6 +1487,17 @@ static bool use_block_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
            (int64_t)nblk * (int64_t)n->RB * (int64_t)n->N < n->block_form_max_elems;
 }
 
+// A TILED layer also carries its GATHER form.  A tile's workgroup takes 64 rows x 1024 outputs with all of a CU's
+// LDS, so a launch has rows / 64 x tiles workgroups, each of them tens of microseconds long; where that does not fill
+// the chip the gather kernel (8 outputs per wave, no LDS) is the faster one.  Measured cross-over on layers of 1..24
+// random inputs per output, per layer: N=1024 4096 rows 46 against 31 us, 16384 rows 55 against 77; N=2048 67 against
+// 46 and 162 against 190; N=4096 98 against 79 and 465 against 431 (60000 rows: 1641 against 1900); N <= 512: the
+// tiles are never slower.  So: the gather form below 8192 rows on layers of 1024 neurons and more.
+static bool use_gather_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
+    return p.kernel == SPDNN_KERNEL_TILED && p.alt_kmax > 0 && n->N >= 1024 &&
+           (int64_t)nblk * (int64_t)n->RB < n->tiled_min_rows;
+}
+
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,
                                int prev_stamp, int check_dead, int32_t* count_prev, int shape, int seglen,
                                const Publish& pub, const int32_t* frontier = nullptr, int frontier_layer = 0) {
@@ -1514,6 +1530,13 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         b.wu = p.info.value; b.bias = n->bias; b.clampv = n->clampv;
         b.publish = pub; b.frontier = frontier; b.frontier_layer = frontier_layer;
         return launch_block(b, n->stream);
+    }
+    if (use_gather_form(n, p, nblk)) {
+        GatherLaunch g{};
+        g.yin = in; g.yout = out; g.cols = d.alt_cols; g.rowlen = d.alt_cnt; g.wv = d.alt_wv; g.dst = d.alt_dst;
+        g.active = n->d_active; g.count_prev = count_prev; g.check_dead = check_dead; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.alt_kmax;
+        g.nblk = nblk; g.stamp = stamp; g.rl = n->rl; g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv; g.publish = pub;
+        return launch_gather(g, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_TILED) {
         TiledLaunch t{};
@@ -1905,7 +1928,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 pl.abort = n->d_abort; pl.host_word = n->h_pwords + next_slot;
                 pl.N = n->N; pl.K = sig.K; pl.nblk = nblk; pl.rl = n->rl; pl.wmode = sig.wmode; pl.stamp0 = stamp0;
                 pl.prev_stamp = prev_stamp; pl.check_dead = check_dead; pl.unrolled = sig.unrolled; pl.add_only = n->add_only;
-                pl.twins = sig.twins; pl.full = sig.full; pl.seglen = n->persist_seglen;
+                pl.twins = sig.twins; pl.full = sig.full; pl.seglen = n->persist_seglen; pl.direct_lds = n->band_direct_lds;
                 // one queue per XCD where every XCD gets a row block: what the layers of a row block hand to each other
                 // then stays in one XCD's L2 and needs no device-scope fences (measured at N=1024, batch 6000, per layer:
                 // 17 us, against 55 - 64 us with the fences, of which the writer's 12 and the readers' 24)

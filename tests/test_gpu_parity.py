@@ -148,6 +148,45 @@ def test_gather_kernel_random_sparsity(gc, orc, values, tiled, monkeypatch):
         _layer_by_layer(gc, orc, net, [sort_rows(c) for c in layers], feats, prune=True)
 
 
+@pytest.mark.parametrize("min_rows", [0, 8192])
+@pytest.mark.parametrize("N", [1024, 2048])
+def test_tiled_layers_carry_their_gather_form(gc, orc, N, min_rows, monkeypatch):
+    """A TILED layer of 1024 neurons or more also holds its GATHER form, and launches below 8192 rows use it (a tile's
+    workgroup takes 64 rows x 1024 outputs to itself: too few workgroups on small batches).  Either way the results
+    are the oracle's; a run that starts above the threshold and is compacted below it switches form on the way."""
+    monkeypatch.setenv("SPDNN_TILED_MIN_ROWS", str(min_rows))
+    L, B = 9, 9000
+    print("tiled / gather form N=%d min_rows=%d" % (N, min_rows), flush=True)
+    rng = np.random.default_rng(N + min_rows)
+    base = [random_csr(rng, N, rng.integers(1, 25, size=N), "general") for _ in range(5)]
+    layers = [base[l] if l < 5 else base[2 + l % 3] for l in range(L)]
+    dens = np.where(rng.random(B) < 0.25, 0.9, 0.02).astype(np.float32)
+    feats = ((rng.random((B, N), dtype=np.float32) < dens[:, None]) * rng.uniform(0.5, 2.0, size=(B, N))).astype(np.float32)
+    ref = orc.infer(feats, [sort_rows(c) for c in layers], -0.15, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    assert 0 < want_counts[4] < 0.5 * B and want_counts[-1] == 0    # (the rows left after layer 4 die in layer 5)
+    with gc.Network(N, B, L, bias=-0.15) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_TILED and net.layer_plan(l).block_form == 2 for l in range(L))
+        net.set_features_dense(feats)
+        for prune in (True, False):
+            r = net.run(prune=prune, collect_counts=True)
+            assert (r.compactions >= 1) == prune    # (compacted below 8192 rows on the way)
+            assert [net.active_count(l) for l in range(L)] == want_counts
+            assert len(net.categories()) == 0
+        for l in range(5):
+            net.run(prune=True, first_layer=0, n_layers=l + 1)
+            gid, y = ref["kept"][l]
+            assert np.array_equal(net.categories(), ref["active_ids"][l])
+            assert same_floats(net.activations(gid), y)
+        net.run(prune=True, first_layer=0, n_layers=3)
+        net.run(prune=True, first_layer=3, n_layers=2)     # continued after the compaction
+        assert np.array_equal(net.categories(), ref["active_ids"][4])
+        assert same_floats(net.activations(ref["kept"][4][0]), ref["kept"][4][1])
+
+
 @pytest.mark.parametrize("values", ["pow2", "general", "uniform", "uniform-fma"])
 @pytest.mark.parametrize("K", [32, 16, 8])
 def test_band_kernel_weight_modes(gc, orc, values, K, monkeypatch):
@@ -280,7 +319,7 @@ def test_streamed_plans(gc, orc, window, monkeypatch):
             assert kernels == {gc.KERNEL_BAND, gc.KERNEL_BLOCK, gc.KERNEL_TILED}
             net.set_features_dense(feats)
             w, dev_bytes, pinned = net.plan_memory()
-            assert w == window and pinned > dev_bytes > 0
+            assert w == window and pinned > 0 and dev_bytes > 0   # (window slots of the largest plan's size; all plans pinned)
             with pytest.raises(gc.SpdnnError):
                 net.set_plan_window(0)       # too late: the plans are uploaded
             for attempt in range(2):         # the second run starts with the slots as the first left them
@@ -1395,6 +1434,7 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
         monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))   # run chains: band walk or BLOCK form
+        monkeypatch.setenv("SPDNN_TILED_MIN_ROWS", str(int(rng.choice([0, 8192]))))            # unstructured layers: tiles or their gather form
         monkeypatch.setenv("SPDNN_STREAM_MIN_BYTES", str(int(rng.choice([0, 96 << 20]))))      # band walk with or without streaming hints
         ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
         with gc.Network(N, B, L, bias=bias) as net:
