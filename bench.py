@@ -150,7 +150,8 @@ def challenge_like_block(gc, N, L, B, bias, log):
     out = {"neuron": N, "layers": L, "batch": B, "ms": best, "edges_per_s": float(B) * 32.0 * N * L / (best * 1e-3),
            "us_per_layer": best * 1e3 / L, "compactions": int(r.compactions), "carried_rows_at_end": int(r.carried_rows),
            "active_rows_after_layers_0_1_2_last": counts, "launches": int(r.launches),
-           "persistent_launches": int(r.persistent_launches), "kernel_classes": plans, "setup_s": time.time() - t0,
+           "persistent_launches": int(r.persistent_launches), "resident_launches": int(r.resident_launches),
+           "kernel_classes": plans, "setup_s": time.time() - t0,
            "inspect_s": t_inspect}
     log("challenge-like N=%d x %d layers: %.3f ms, %d rows at the end, setup %.1f s" % (N, L, best, counts[-1], out["setup_s"]))
     return out
@@ -376,6 +377,7 @@ def main():
                                   "layers_with_work": min(ran, L), "active_rows_first_layers": [int(c) for c in cpu_counts[:8]],
                                   "categories": int(cpu_counts[L - 1]),
                                   "counts_equal_gpu": [int(c) for c in cpu_counts[:len(lit_counts)]] == lit_counts}
+                cpu["literal_%s" % args.config] = cpu["literal"]    # (the same block under the configuration's name)
         ok_ids, ok_y, max_abs = True, True, 0.0
         sample = np.arange(rows, dtype=np.int32)
         for l in range(n_check):

@@ -1066,11 +1066,11 @@ __global__ __launch_bounds__(256) void gather_kernel(
 // 8 bytes per multiply-add through the scalar cache does not work (every access misses, and the
 // cache serves few misses at a time: measured 0.69 ms per layer of 1024 neurons where the plain
 // gather takes 0.45), so the entry blocks (1 KiB per round and wave) go through LDS too, into a
-// per-wave ring.  ROWBCAST = 1 (default): four reads put a round's block into registers (lane j of
-// every 16-lane row holds the entries of outputs j, 16 + j, 32 + j, 48 + j) and the DPP row
-// broadcast hands an entry's offset and weight to all lanes inside the add and the multiply that
-// use them.  ROWBCAST = 0 (SPDNN_TILED_ROW_BROADCAST=0): the entries are read back pair by pair
-// with broadcast reads (all lanes the same address) - half an LDS instruction more per entry.
+// per-wave ring.  Four reads put a round's block into registers (lane j of every 16-lane row holds
+// the entries of outputs j, 16 + j, 32 + j, 48 + j) and the DPP row broadcast hands an entry's offset
+// and weight to all lanes inside the add and the multiply that use them.  (Reading the entries back
+// pair by pair with broadcast LDS reads - all lanes the same address - took half an LDS instruction
+// more per entry: 0.266 against 0.239 ms per layer of 1024 neurons.)
 // Accumulation in ascending input index: panels ascend, entries inside a panel ascend; padding
 // entries carry weight -0 and add an exact zero.
 // ------------------------------------------------------------------------------------------
@@ -1112,8 +1112,23 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int RB = 64 * rl;
-    const int sb = blockIdx.x, rb = sb / rl, q = sb - rb * rl;
-    const int t = blockIdx.y;
+    // Which (64 rows, tile) this workgroup takes.  The tiles of one set of rows read much the same input columns
+    // (for layers without structure: all of them), so they should run at the same time behind the same L2:
+    // workgroups go to the 8 XCDs round robin by number, so the tiles of row set sb get the numbers
+    // sb % 8 + 8 * (tile + ntiles * (sb / 8)) - consecutive workgroups of one XCD.  (Row sets beyond the last
+    // whole eight: tile after tile.)
+    const int nsb = (int)gridDim.x / ntiles, nsb8 = nsb / 8 * 8;
+    int sb, t;
+    if ((int)blockIdx.x < nsb8 * ntiles) {
+        const int x = (int)blockIdx.x % 8, k = (int)blockIdx.x / 8;
+        t = k % ntiles;
+        sb = (k / ntiles) * 8 + x;
+    } else {
+        const int rem = (int)blockIdx.x - nsb8 * ntiles;
+        sb = nsb8 + rem / ntiles;
+        t = rem % ntiles;
+    }
+    const int rb = sb / rl, q = sb - rb * rl;
     const size_t row = (size_t)rb * RB + q * 64 + lane;
     if (prev_stamp != 0 && (check_dead || (count_prev != nullptr && t == 0))) {
         // Only a row block without ANY active row may be skipped (the kernels of the other classes
@@ -2391,7 +2406,8 @@ hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s) {
         !a.cols || !a.hdr || !a.ent || !a.dst || !a.active)
         return hipErrorInvalidValue;
     constexpr size_t lds = 512 * 256 + 16 * 2048;   // one panel and the waves' entry rings: all 160 KiB of a CU
-    dim3 grid(a.nblk * a.rl, a.ntiles), block(1024);
+    if ((long long)a.nblk * a.rl * a.ntiles > 0x7fffffffll) return hipErrorInvalidValue;
+    dim3 grid((unsigned)(a.nblk * a.rl * a.ntiles)), block(1024);
 #define SPDNN_TILED(WM)                                                                                          \
     do {                                                                                                         \
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(tiled_kernel<WM>),      \
