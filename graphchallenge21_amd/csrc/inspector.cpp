@@ -714,6 +714,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.alt_out_at.clear();
     plan.alt_dst.clear();
     plan.alt_wv.clear();
+    plan.rt_ent.clear();
     plan.alt_kmax = 0;
     if (band && halo == 32 && uniform && exact) {
         // the BLOCK form of a run-chain layer, its columns in the band's input labelling
@@ -819,7 +820,8 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
         plan.sel.clear();
         plan.pairs.clear();
-        // its GATHER form, for launches too small to fill the chip with tiles
+        // its GATHER form, for launches too small to fill the chip with tiles, and its ROWTILE form; both over
+        // the outputs ordered by length, longest first
         const int kw = std::max(kmax, 1);
         plan.alt_kmax = kw;
         plan.alt_cols.assign((size_t)N * kw, 0);
@@ -827,12 +829,24 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.alt_cnt.resize((size_t)N);
         plan.alt_out_at.resize((size_t)N);
         std::iota(plan.alt_out_at.begin(), plan.alt_out_at.end(), 0);
-        for (int j = 0; j < N; ++j) {
+        std::stable_sort(plan.alt_out_at.begin(), plan.alt_out_at.end(), [&](int32_t x, int32_t y) {
+            return rowptr[x + 1] - rowptr[x] > rowptr[y + 1] - rowptr[y];
+        });
+        const int kpad = (kw + 3) / 4 * 4;   // the kernel requests entries four at a time
+        plan.rt_ent.assign((size_t)kpad * N * 2, 0u);
+        for (int slot = 0; slot < N; ++slot) {
+            const int j = plan.alt_out_at[(size_t)slot];
             const int len = rowptr[j + 1] - rowptr[j];
-            plan.alt_cnt[(size_t)j] = len;
+            plan.alt_cnt[(size_t)slot] = len;
             for (int k = 0; k < len; ++k) {
-                plan.alt_cols[(size_t)j * kw + k] = col[rowptr[j] + k];
-                plan.alt_wv[(size_t)j * kw + k] = val[rowptr[j] + k];
+                const int32_t c = col[rowptr[j] + k];
+                const float w = val[rowptr[j] + k];
+                plan.alt_cols[(size_t)slot * kw + k] = c;
+                plan.alt_wv[(size_t)slot * kw + k] = w;
+                uint32_t wb;
+                memcpy(&wb, &w, 4);
+                plan.rt_ent[((size_t)k * N + slot) * 2] = (uint32_t)c;
+                plan.rt_ent[((size_t)k * N + slot) * 2 + 1] = wb;
             }
         }
     } else {
@@ -862,7 +876,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.info.block_form = plan.alt_ngroups > 0 ? 1 : (plan.alt_kmax > 0 ? 2 : 0);
     plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
                                                               plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
-                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() + plan.alt_wv.size() +
+                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() + plan.alt_wv.size() + plan.rt_ent.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.failed = false;

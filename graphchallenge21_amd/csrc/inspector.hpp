@@ -56,11 +56,15 @@ struct LayerPlan {
     std::vector<int32_t> alt_out_at; // [alt_ngroups*16] output neuron of the slot, -1 = unused
     std::vector<int32_t> alt_dst;    // [alt_ngroups*16] physical column in the next buffer
     // A TILED layer carries its GATHER form in the same arrays (alt_ngroups stays 0): alt_cols [N][alt_kmax] input
-    // columns in accumulation order, alt_cnt [N] row lengths, alt_wv [N][alt_kmax] weights, alt_out_at = the neurons
-    // 0 .. N-1, alt_dst [N].  A tile's workgroup needs 64 rows x 1024 outputs to itself: on small batches of wide
+    // columns in accumulation order, alt_cnt [N] row lengths, alt_wv [N][alt_kmax] weights, alt_out_at [N] = the output
+    // neuron of every slot, alt_dst [N].  A tile's workgroup needs 64 rows x 1024 outputs to itself: on small batches of wide
     // layers that leaves most of the chip idle, and the gather kernel, which spreads over 8 outputs per wave, is faster.
     std::vector<float> alt_wv;
     int alt_kmax = 0;
+    // ... and its ROWTILE form over the same slots (outputs ordered by length, longest first, so that the 64 lanes of a
+    // wave have about the same number of entries): rt_ent [alt_kmax rounded up to 4][N][2] = (input column, weight bits)
+    // of the slot's k-th entry, zeros behind a list, entry-major so that the lanes of a wave read neighbouring words.
+    std::vector<uint32_t> rt_ent;
     // BAND: neuron j sits at the same band position as an input and as an output (see
     // canonicalize_self_aligned_band); fuse_next: this layer writes its outputs exactly where the
     // next layer's band reads them (dst = identity) and both fit the fused pair kernel

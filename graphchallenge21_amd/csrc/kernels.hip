@@ -1256,6 +1256,211 @@ __global__ __launch_bounds__(1024) void tiled_kernel(
     }
 }
 
+// Lanes in groups of P (4, 2 or 1) neighbours.  group_turn: the value of the lane i places down in the group (lane j
+// takes from lane (j - i) mod P); group_lane_value: the value of lane r of the group.  i and r are constants after
+// unrolling (DPP quad permutations).
+template <int P> __device__ __forceinline__ uint32_t group_turn_u32(uint32_t v, int i) {
+    if constexpr (P == 4) {
+        switch (i & 3) {
+            case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x93, 0xf, 0xf, true);   // quad_perm [3,0,1,2]
+            case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4e, 0xf, 0xf, true);   // quad_perm [2,3,0,1]
+            case 3: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x39, 0xf, 0xf, true);   // quad_perm [1,2,3,0]
+            default: return v;
+        }
+    } else if constexpr (P == 2) {
+        return (i & 1) ? (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xb1, 0xf, 0xf, true) : v;  // quad_perm [1,0,3,2]
+    } else {
+        return v;
+    }
+}
+template <int P> __device__ __forceinline__ float4 group_turn(const float4& v, int i) {
+    float4 o;
+    o.x = __uint_as_float(group_turn_u32<P>(__float_as_uint(v.x), i));
+    o.y = __uint_as_float(group_turn_u32<P>(__float_as_uint(v.y), i));
+    o.z = __uint_as_float(group_turn_u32<P>(__float_as_uint(v.z), i));
+    o.w = __uint_as_float(group_turn_u32<P>(__float_as_uint(v.w), i));
+    return o;
+}
+template <int P> __device__ __forceinline__ uint32_t group_lane_value(uint32_t v, int r) {
+    if constexpr (P == 4) {
+        switch (r & 3) {
+            case 0: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x00, 0xf, 0xf, true);
+            case 1: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x55, 0xf, 0xf, true);
+            case 2: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xaa, 0xf, 0xf, true);
+            default: return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xff, 0xf, 0xf, true);
+        }
+    } else if constexpr (P == 2) {
+        return (r & 1) ? (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xf5, 0xf, 0xf, true)    // quad_perm [1,1,3,3]
+                       : (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xa0, 0xf, 0xf, true);   // quad_perm [0,0,2,2]
+    } else {
+        return v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// ROWTILE kernel (the other form of a TILED layer): the transposed assignment.  A workgroup of 1024
+// threads stages R feature rows - all N columns of them - in LDS, laid out [column][row], and thread
+// t computes whole outputs (slots t, t + 1024, ...) for those R rows, the rows in registers.  A lane
+// walks its own entry list (input column, weight: 8 bytes from memory, entry-major so that the lanes
+// of a wave read neighbouring words, the next entry requested under the arithmetic) and reads the
+// column's R rows with R/4 16-byte LDS reads, so an LDS instruction serves four multiply-adds
+// instead of one; lanes of a wave differ only in the number of entries, and the slots are ordered by
+// length.  No panels, so no padding per panel: with the tiles two fifths of the entry slots are
+// padding on layers of 1..24 random inputs, here a fourteenth.  Lane l reads the four-row parts of
+// a column in the order l, l + 1, ... (mod R/4) - all lanes at the same part would meet in the same
+// banks - and so holds the rows in a rotated order, which only its stores and its alive bits need to
+// know.  Accumulation: ascending input index per output, as everywhere.
+//
+// Measured at N=1024, batch 60000, 1..24 random inputs per output, per layer: 156 us where the tiles take 228
+// (166 before the lanes traded parts for the stores); with parts of the kernel switched off, then: nothing but
+// the launch 25 us, rows in 40, arithmetic (with its entry reads: 105 KB per row set from L2) 51, rows out 55 -
+// the phases add up.  Two other forms were built and
+// measured no faster, and are gone: one workgroup per CU that stays and takes row set after row set with two LDS
+// buffers, its entries requested a group ahead (192 us), and the same with the entry lists held in registers
+// for the whole launch and the rows brought straight into LDS (169 us: its arithmetic is hidden entirely, and
+// rows in and out alone take those 169 us - 64-byte pieces both ways, a third of the memory's rate).
+// ------------------------------------------------------------------------------------------
+struct RowtileArgs {
+    Feat yin, yout;
+    const uint32_t* ent;
+    const int32_t* len;
+    const int32_t* dst;
+    int32_t* active;
+    int32_t* count_prev;
+    int N, kmax, rl, stamp, prev_stamp, check_dead;
+    float bias, clampv;
+    Publish pub;
+};
+
+template <int R, int WMODE>
+__global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int sh_alive;
+    constexpr int PARTS = R / 4;
+    publish_counts(a.pub);
+    const int t = (int)threadIdx.x, lane = t & 63;
+    const int RB = 64 * a.rl;
+    // every XCD takes a contiguous eighth of the rows (see block_resident_kernel)
+    const unsigned nwg = gridDim.x;
+    const unsigned wg = (nwg % 8u) == 0u ? (blockIdx.x % 8u) * (nwg / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const size_t row0 = (size_t)wg * R;
+    const int rb = (int)(row0 / (size_t)RB), rin = (int)(row0 - (size_t)rb * RB);
+    if (a.prev_stamp != 0 && (a.check_dead || (a.count_prev != nullptr && rin == 0))) {
+        // the rows the layer before left active in this row block: counted by the block's first workgroup; a row
+        // block without any is skipped (as by the other per-layer kernels)
+        const int st = t < RB ? a.active[(size_t)rb * RB + t] : 0;
+        const bool alive = t < RB && (st == a.prev_stamp || st == a.stamp);
+        const int n_alive = (int)__popcll(__ballot(alive ? 1 : 0));
+        if (a.count_prev != nullptr && rin == 0 && lane == 0 && n_alive > 0) atomicAdd(a.count_prev, n_alive);
+        if (a.check_dead && __builtin_amdgcn_readfirstlane(__syncthreads_or(alive ? 1 : 0)) == 0) return;
+    }
+    const size_t blkf = (size_t)a.N * RB;
+    {
+        // (half by half: indexing the halves of a Feat inside the argument struct would put the struct into scratch memory)
+        const float* __restrict__ gin = ((rb & 1) ? a.yin.half[1] : a.yin.half[0]) + (size_t)(rb >> 1) * blkf + rin;
+        const int total = a.N * PARTS;
+        for (int base = t; base < total; base += 4096) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = min(base + u * 1024, total - 1);   // (a lane past the end reads the last piece again and drops it)
+                const int col = idx / PARTS, part = idx - col * PARTS;
+                v[u] = *reinterpret_cast<const float4*>(gin + (size_t)col * RB + part * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * 1024;
+                if (idx < total) *reinterpret_cast<float4*>(smem + (size_t)idx * 16) = v[u];
+            }
+        }
+    }
+    if (t == 0) sh_alive = 0;
+    __syncthreads();
+    float* __restrict__ gout = ((rb & 1) ? a.yout.half[1] : a.yout.half[0]) + (size_t)(rb >> 1) * blkf + rin;
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    using GB = const __attribute__((address_space(1))) unsigned char*;
+    const GB entb = (GB)a.ent;
+    const uint32_t estride = (uint32_t)a.N * 8u;   // bytes from a slot's entry k to its entry k + 1
+    // this lane's order of the four-row parts of a column, as byte offsets
+    uint32_t poff[PARTS];
+#pragma unroll
+    for (int i = 0; i < PARTS; ++i) poff[i] = (uint32_t)(((i + lane) & (PARTS - 1)) * 16);
+    unsigned bits = 0;   // rows of this workgroup that one of this lane's outputs left nonzero
+    for (int slot0 = 0; slot0 < a.N; slot0 += 1024) {
+        const int slot = slot0 + t;
+        const bool have = slot < a.N;
+        const int n_in = have ? a.len[slot] : 0;
+        // the slots are ordered by length, longest first: the wave's first lane has the most entries
+        const int n_wave = __builtin_amdgcn_readfirstlane(n_in);
+        float acc[R];
+#pragma unroll
+        for (int i = 0; i < R; ++i) acc[i] = 0.0f;
+        uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
+        u32x2 e = {0u, 0u};
+        if (n_wave > 0) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+        for (int k = 0; k < n_wave; ++k) {
+            const u32x2 cur = e;
+            eoff += estride;
+            // (lanes with fewer entries read the zero padding behind their lists: the array has kmax rows)
+            if (k + 1 < n_wave) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+            if (k < n_in) {
+                const float w = __uint_as_float(cur.y);
+                const uint32_t colb = cur.x * (uint32_t)(R * 4);
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) {
+                    const float4 x = *reinterpret_cast<const float4*>(smem + (colb + poff[i]));
+                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x.x, w);
+                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x.y, w);
+                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x.z, w);
+                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x.w, w);
+                }
+            }
+        }
+        const int d = have ? a.dst[slot] : -1;
+        float4 y[PARTS];
+#pragma unroll
+        for (int i = 0; i < PARTS; ++i) {
+            y[i].x = relu_clamp(acc[i * 4 + 0] + a.bias, a.clampv);
+            y[i].y = relu_clamp(acc[i * 4 + 1] + a.bias, a.clampv);
+            y[i].z = relu_clamp(acc[i * 4 + 2] + a.bias, a.clampv);
+            y[i].w = relu_clamp(acc[i * 4 + 3] + a.bias, a.clampv);
+            const unsigned nzb = (y[i].x > 0.0f ? 1u : 0u) | (y[i].y > 0.0f ? 2u : 0u) | (y[i].z > 0.0f ? 4u : 0u) | (y[i].w > 0.0f ? 8u : 0u);
+            if (d >= 0) bits |= nzb << (poff[i] >> 2);
+        }
+        // Stores.  A lane has the R rows of ITS output: written as they are, every 16 bytes are a request of their own
+        // to L2 (neighbouring lanes write columns a KiB apart), and the requests, not the bytes, bound the stores
+        // (N=1024, batch 60000: 15.4 million write requests per layer, 55 us).  So the PARTS lanes of a group trade
+        // parts first - lane j of the group ends up with part j of every output of the group - and each store
+        // instruction writes, group by group, one output's R rows as one contiguous piece.
+        // y[i] of lane s is part (i + s) mod PARTS of output s; turned by i lanes it arrives at lane j = (s + i) mod
+        // PARTS as part j of output s = (j - i) mod PARTS.
+        const int j = lane & (PARTS - 1);
+        float4 z[PARTS];
+#pragma unroll
+        for (int r = 0; r < PARTS; ++r) z[r] = y[0];
+#pragma unroll
+        for (int i = 0; i < PARTS; ++i) {
+            const float4 c = group_turn<PARTS>(y[i], i);
+#pragma unroll
+            for (int r = 0; r < PARTS; ++r)
+                if (j == ((r + i) & (PARTS - 1))) z[r] = c;
+        }
+#pragma unroll
+        for (int r = 0; r < PARTS; ++r) {
+            const int dr = (int)group_lane_value<PARTS>((uint32_t)d, r);
+            // (plain stores and loads: with the non-temporal hint on both the layer takes the same time)
+            if (dr >= 0) *reinterpret_cast<float4*>(reinterpret_cast<unsigned char*>(gout + (size_t)dr * RB) + j * 16) = z[r];
+        }
+    }
+    unsigned wave_bits = 0;
+#pragma unroll
+    for (int b = 0; b < R; ++b)
+        if (__ballot((bits >> b) & 1u) != 0ull) wave_bits |= 1u << b;
+    if (lane == 0 && wave_bits != 0) atomicOr(&sh_alive, (int)wave_bits);
+    __syncthreads();
+    if (t < R && ((sh_alive >> t) & 1)) a.active[row0 + t] = a.stamp;
+}
+
 // ------------------------------------------------------------------------------------------
 // BLOCK kernel: groups of up to 16 outputs that read the same (up to 32) input columns - the
 // structure of the challenge's RadiX-Net layers.  A wave loads the shared columns of a group once
@@ -2420,6 +2625,48 @@ hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s) {
     if (a.wmode != 2) SPDNN_TILED(1); else SPDNN_TILED(2);
 #undef SPDNN_TILED
     return hipGetLastError();
+}
+
+int rowtile_rows_per_workgroup(int N) {
+    if (N <= 0) return 0;
+    if (N <= 2048) return 16;   // N x 64 bytes of LDS: up to 128 KiB
+    if (N <= 4096) return 8;
+    if (N <= 8192) return 4;
+    return 0;
+}
+
+template <int R>
+static hipError_t launch_rowtile_r(const RowtileLaunch& a, hipStream_t s) {
+    RowtileArgs k{};
+    k.yin = a.yin; k.yout = a.yout; k.ent = a.ent; k.len = a.len; k.dst = a.dst; k.active = a.active; k.count_prev = a.count_prev;
+    k.N = a.N; k.kmax = a.kpad; k.rl = a.rl; k.stamp = a.stamp; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
+    k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
+    const size_t lds = (size_t)a.N * R * 4;
+    dim3 grid((unsigned)(a.rows / R)), block(1024);
+#define SPDNN_ROWTILE(WM)                                                                                        \
+    do {                                                                                                         \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rowtile_kernel<R, WM>), \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
+        if (attr != hipSuccess) return attr;                                                                     \
+        hipLaunchKernelGGL((rowtile_kernel<R, WM>), grid, block, lds, s, k);                                     \
+    } while (0)
+    if (a.wmode != 2) SPDNN_ROWTILE(1); else SPDNN_ROWTILE(2);
+#undef SPDNN_ROWTILE
+    return hipGetLastError();
+}
+
+hipError_t launch_rowtile(const RowtileLaunch& a, hipStream_t s) {
+    // host-side shape checks: what the kernel's LDS buffer and its row numbering assume
+    if (a.N <= 0 || a.kpad < 1 || !a.yin || !a.yout || !a.ent || !a.len || !a.dst || !a.active || a.rows <= 0 ||
+        (a.rl != 1 && a.rl != 2 && a.rl != 4) || (a.rows % (64 * a.rl)) != 0)
+        return hipErrorInvalidValue;
+    const int R = rowtile_rows_per_workgroup(a.N);
+    if (R == 0 || (64 * a.rl) % R != 0 || (size_t)a.N * R * 4 > 128 * 1024) return hipErrorInvalidValue;
+    switch (R) {
+        case 16: return launch_rowtile_r<16>(a, s);
+        case 8: return launch_rowtile_r<8>(a, s);
+        default: return launch_rowtile_r<4>(a, s);
+    }
 }
 
 hipError_t launch_block(const BlockLaunch& a, hipStream_t s) {

@@ -113,6 +113,26 @@ struct TiledLaunch {
 };
 hipError_t launch_tiled(const TiledLaunch& a, hipStream_t s);
 
+// TILED layers, ROWTILE form: a workgroup stages R feature rows (all N columns) in LDS, laid out [column][row], and
+// every thread computes whole outputs for those rows - its own entry list, the rows in registers.  Every lane has its
+// own number of entries, so the only padding is the spread of lengths inside a wave (the slots are ordered by
+// length), whatever the number of columns.
+struct RowtileLaunch {
+    Feat yin;
+    Feat yout;
+    const uint32_t* ent;     // [kpad][N][2] (input column, weight bits) of every slot's k-th entry, zeros behind a list
+    const int32_t* len;      // [N] entries per slot
+    const int32_t* dst;      // [N] physical output column of the slot
+    int32_t* active;
+    int32_t* count_prev;     // as in BandLaunch
+    int N, kpad, rows, rl, wmode, stamp, prev_stamp, check_dead;   // kpad: rows of `ent`, a multiple of 4; rows: carried rows (whole row blocks)
+    float bias, clampv;
+    Publish publish;
+};
+// rows a workgroup stages (16, 8 or 4 by the width), 0 = the width does not fit (more than 8192 neurons)
+int rowtile_rows_per_workgroup(int N);
+hipError_t launch_rowtile(const RowtileLaunch& a, hipStream_t s);
+
 // BLOCK layers: groups of up to 16 outputs sharing up to 32 input columns.
 struct BlockLaunch {
     Feat yin;

@@ -182,12 +182,13 @@ struct DevLayer {
     int32_t* alt_cnt = nullptr;
     int32_t* alt_dst = nullptr;
     float* alt_wv = nullptr;       // (with alt_cols / alt_cnt / alt_dst: the GATHER form of a TILED layer)
+    uint32_t* rt_ent = nullptr;    // (with alt_cnt / alt_dst: its ROWTILE form)
 };
 
 // Where the arrays of one layer's plan lie inside its block of device memory (and inside the
 // pinned host copy of that block when plans are streamed): pairs, ell, rowlen, wv, dst, blk_cols,
-// blk_cnt, alt_cols, alt_cnt, alt_dst, alt_wv, each aligned to 256 bytes.
-constexpr int kPlanArrays = 11;
+// blk_cnt, alt_cols, alt_cnt, alt_dst, alt_wv, rt_ent, each aligned to 256 bytes.
+constexpr int kPlanArrays = 12;
 struct PlanLayout {
     size_t off[kPlanArrays] = {};
     size_t len[kPlanArrays] = {};
@@ -297,6 +298,7 @@ struct spdnn_net {
     int64_t pair_min_elems = (int64_t)1 << 23;
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     int64_t tiled_min_rows = 8192;                    // see use_gather_form (SPDNN_TILED_MIN_ROWS)
+    int rowtile_mode = 1;                             // TILED layers up to 8192 neurons wide run their ROWTILE form (SPDNN_ROWTILE=0: the tiles)
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
     LayerDesc* d_table = nullptr;   // one entry per layer (resident plans only)
@@ -573,7 +575,8 @@ PlanLayout plan_layout(const LayerPlan& p) {
     PlanLayout y;
     const size_t len[kPlanArrays] = {p.pairs.size() * 4,    p.ell_col.size() * 4,  p.rowlen.size() * 4,   p.wv.size() * 4,
                                      p.dst.size() * 4,      p.blk_cols.size() * 4, p.blk_cnt.size() * 4,  p.alt_cols.size() * 4,
-                                     p.alt_cnt.size() * 4,  p.alt_dst.size() * 4,  p.alt_wv.size() * 4};
+                                     p.alt_cnt.size() * 4,  p.alt_dst.size() * 4,  p.alt_wv.size() * 4,
+                                     p.rt_ent.size() * 4};
     for (int k = 0; k < kPlanArrays; ++k) {
         y.off[k] = y.bytes;
         y.len[k] = len[k];
@@ -585,7 +588,7 @@ PlanLayout plan_layout(const LayerPlan& p) {
 void pack_plan(const LayerPlan& p, const PlanLayout& y, char* dst) {
     const void* src[kPlanArrays] = {p.pairs.data(),   p.ell_col.data(),  p.rowlen.data(),  p.wv.data(),      p.dst.data(),
                                     p.blk_cols.data(), p.blk_cnt.data(), p.alt_cols.data(), p.alt_cnt.data(), p.alt_dst.data(),
-                                    p.alt_wv.data()};
+                                    p.alt_wv.data(),   p.rt_ent.data()};
     for (int k = 0; k < kPlanArrays; ++k)
         if (y.len[k]) memcpy(dst + y.off[k], src[k], y.len[k]);
 }
@@ -604,6 +607,7 @@ DevLayer plan_at(const PlanLayout& y, char* base) {
     d.alt_cnt = (int32_t*)at(8);
     d.alt_dst = (int32_t*)at(9);
     d.alt_wv = (float*)at(10);
+    d.rt_ent = (uint32_t*)at(11);
     return d;
 }
 
@@ -906,6 +910,7 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
     if (const char* e = getenv("SPDNN_TILED_MIN_ROWS")) n->tiled_min_rows = atoll(e);
+    if (const char* e = getenv("SPDNN_ROWTILE")) n->rowtile_mode = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_STREAM_MIN_BYTES")) n->stream_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_COUNT_TIMEOUT_MS")) n->count_timeout_ms = std::max(1ll, atoll(e));
     if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
@@ -1537,6 +1542,14 @@ static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& 
         g.active = n->d_active; g.count_prev = count_prev; g.check_dead = check_dead; g.prev_stamp = prev_stamp; g.N = n->N; g.kmax = p.alt_kmax;
         g.nblk = nblk; g.stamp = stamp; g.rl = n->rl; g.wmode = p.wmode; g.bias = n->bias; g.clampv = n->clampv; g.publish = pub;
         return launch_gather(g, n->stream);
+    }
+    if (p.kernel == SPDNN_KERNEL_TILED && n->rowtile_mode && !p.rt_ent.empty() && rowtile_rows_per_workgroup(n->N) > 0 &&
+        n->RB % rowtile_rows_per_workgroup(n->N) == 0) {
+        RowtileLaunch t{};
+        t.yin = in; t.yout = out; t.ent = d.rt_ent; t.len = d.alt_cnt; t.dst = d.alt_dst; t.active = n->d_active;
+        t.count_prev = count_prev; t.check_dead = check_dead; t.prev_stamp = prev_stamp; t.N = n->N; t.kpad = (p.alt_kmax + 3) / 4 * 4;
+        t.rows = nblk * n->RB; t.rl = n->rl; t.wmode = p.wmode; t.stamp = stamp; t.bias = n->bias; t.clampv = n->clampv; t.publish = pub;
+        return launch_rowtile(t, n->stream);
     }
     if (p.kernel == SPDNN_KERNEL_TILED) {
         TiledLaunch t{};

@@ -58,8 +58,9 @@ enum spdnn_kernel {
     SPDNN_KERNEL_BAND = 2,   /* row-succ / tiled: relabelled circulant band walked through an LDS ring */
     SPDNN_KERNEL_BLOCK = 3,  /* groups of outputs that read the same inputs (RadiX-Net style): the shared
                                 input columns are held in registers and reused by every output of the group */
-    SPDNN_KERNEL_TILED = 4   /* any sparsity pattern: tiles of 1024 outputs whose input columns are staged in
-                                LDS panel by panel, every column read once per tile                          */
+    SPDNN_KERNEL_TILED = 4   /* any sparsity pattern, staged through LDS: up to 8192 neurons a workgroup keeps 16, 8 or 4
+                                feature rows (all columns) and every thread computes whole outputs for them; beyond,
+                                tiles of 1024 outputs whose input columns are staged panel by panel                */
 };
 
 typedef struct spdnn_layer_plan {

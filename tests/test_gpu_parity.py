@@ -127,14 +127,16 @@ def test_survivor_chain_with_compaction(gc, orc):
             assert not net.activations(dead).any()
 
 
-@pytest.mark.parametrize("tiled", [1, 0])
+@pytest.mark.parametrize("tiled,rowtile", [(1, 1), (1, 0), (0, 1)])
 @pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
-def test_gather_kernel_random_sparsity(gc, orc, values, tiled, monkeypatch):
-    """Irregular rows (0..40 entries), unsorted columns: the general classes - tiles of outputs with
-    their input columns staged in LDS, and the plain gather."""
+def test_gather_kernel_random_sparsity(gc, orc, values, tiled, rowtile, monkeypatch):
+    """Irregular rows (0..40 entries), unsorted columns: the general classes - the TILED class in its two forms
+    (rows of a workgroup staged in LDS and whole outputs per thread; tiles of outputs with their input columns
+    staged in LDS panel by panel) and the plain gather."""
     monkeypatch.setenv("SPDNN_TILED", str(tiled))
+    monkeypatch.setenv("SPDNN_ROWTILE", str(rowtile))
     N, L, B = 512, 3, 300
-    print("general class tiled=%d values=%s" % (tiled, values), flush=True)
+    print("general class tiled=%d rowtile=%d values=%s" % (tiled, rowtile, values), flush=True)
     rng = np.random.default_rng(11)
     layers = [random_csr(rng, N, rng.integers(0, 41, size=N), values) for _ in range(L)]
     feats = rng.uniform(0, 4, size=(B, N)).astype(np.float32) * (rng.random((B, N)) < 0.3)
@@ -148,13 +150,15 @@ def test_gather_kernel_random_sparsity(gc, orc, values, tiled, monkeypatch):
         _layer_by_layer(gc, orc, net, [sort_rows(c) for c in layers], feats, prune=True)
 
 
+@pytest.mark.parametrize("rowtile", [1, 0])
 @pytest.mark.parametrize("min_rows", [0, 8192])
 @pytest.mark.parametrize("N", [1024, 2048])
-def test_tiled_layers_carry_their_gather_form(gc, orc, N, min_rows, monkeypatch):
+def test_tiled_layers_carry_their_gather_form(gc, orc, N, min_rows, rowtile, monkeypatch):
     """A TILED layer of 1024 neurons or more also holds its GATHER form, and launches below 8192 rows use it (a tile's
     workgroup takes 64 rows x 1024 outputs to itself: too few workgroups on small batches).  Either way the results
     are the oracle's; a run that starts above the threshold and is compacted below it switches form on the way."""
     monkeypatch.setenv("SPDNN_TILED_MIN_ROWS", str(min_rows))
+    monkeypatch.setenv("SPDNN_ROWTILE", str(rowtile))     # above the threshold: whole outputs per thread, or the tiles
     L, B = 9, 9000
     print("tiled / gather form N=%d min_rows=%d" % (N, min_rows), flush=True)
     rng = np.random.default_rng(N + min_rows)
@@ -1435,6 +1439,7 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", str(minchain))
         monkeypatch.setenv("SPDNN_BLOCK_FORM_MAX_ELEMS", str(int(rng.choice([0, 1 << 26]))))   # run chains: band walk or BLOCK form
         monkeypatch.setenv("SPDNN_TILED_MIN_ROWS", str(int(rng.choice([0, 8192]))))            # unstructured layers: tiles or their gather form
+        monkeypatch.setenv("SPDNN_ROWTILE", str(int(rng.integers(0, 2))))                      # ... and which of the two forms with LDS staging
         monkeypatch.setenv("SPDNN_STREAM_MIN_BYTES", str(int(rng.choice([0, 96 << 20]))))      # band walk with or without streaming hints
         ref = orc.infer(feats, layers, bias, prune=False, keep={L - 1})
         with gc.Network(N, B, L, bias=bias) as net:
