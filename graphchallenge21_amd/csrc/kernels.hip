@@ -1332,7 +1332,7 @@ struct RowtileArgs {
     Publish pub;
 };
 
-template <int R, int WMODE>
+template <int R, int WMODE, bool PAIRS>
 __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int sh_alive;
@@ -1395,24 +1395,67 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
         float acc[R];
 #pragma unroll
         for (int i = 0; i < R; ++i) acc[i] = 0.0f;
-        uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
-        u32x2 e = {0u, 0u};
-        if (n_wave > 0) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
-        for (int k = 0; k < n_wave; ++k) {
-            const u32x2 cur = e;
-            eoff += estride;
-            // (lanes with fewer entries read the zero padding behind their lists: the array has kmax rows)
-            if (k + 1 < n_wave) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
-            if (k < n_in) {
-                const float w = __uint_as_float(cur.y);
-                const uint32_t colb = cur.x * (uint32_t)(R * 4);
+        if constexpr (!PAIRS) {
+            // (one entry at a time where two workgroups fit a CU - 16 rows of up to 1280 neurons: with two entries the
+            // sixteen more registers for the second column leave it one - N=1024, batch 60000: 170 against 156 us per layer)
+            uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
+            u32x2 e = {0u, 0u};
+            if (n_wave > 0) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+            for (int k = 0; k < n_wave; ++k) {
+                const u32x2 cur = e;
+                eoff += estride;
+                // (lanes with fewer entries read the zero padding behind their lists: the array has kmax rows)
+                if (k + 1 < n_wave) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+                if (k < n_in) {
+                    const float w = __uint_as_float(cur.y);
+                    const uint32_t colb = cur.x * (uint32_t)(R * 4);
+#pragma unroll
+                    for (int i = 0; i < PARTS; ++i) {
+                        const float4 x = *reinterpret_cast<const float4*>(smem + (colb + poff[i]));
+                        acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x.x, w);
+                        acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x.y, w);
+                        acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x.z, w);
+                        acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x.w, w);
+                    }
+                }
+            }
+        } else {
+            // Two entries at a time, the next two requested under the arithmetic.  No test of k against the lane's own
+            // length: behind a list the array holds (column 0, weight +0), and adding x * (+0) to an accumulator that
+            // started at +0 changes nothing (it can never be -0).
+            uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
+            u32x2 e0 = {0u, 0u}, e1 = {0u, 0u};
+            if (n_wave > 0) {
+                e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+                e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
+            }
+            for (int k = 0; k < n_wave; k += 2) {
+                const u32x2 c0 = e0, c1 = e1;
+                eoff += 2u * estride;
+                if (k + 2 < n_wave) {
+                    e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+                    e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
+                }
+                const float w0 = __uint_as_float(c0.y), w1 = __uint_as_float(c1.y);
+                const uint32_t colb0 = c0.x * (uint32_t)(R * 4), colb1 = c1.x * (uint32_t)(R * 4);
+                float4 x0[PARTS], x1[PARTS];
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) x0[i] = *reinterpret_cast<const float4*>(smem + (colb0 + poff[i]));
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) x1[i] = *reinterpret_cast<const float4*>(smem + (colb1 + poff[i]));
 #pragma unroll
                 for (int i = 0; i < PARTS; ++i) {
-                    const float4 x = *reinterpret_cast<const float4*>(smem + (colb + poff[i]));
-                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x.x, w);
-                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x.y, w);
-                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x.z, w);
-                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x.w, w);
+                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x0[i].x, w0);
+                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x0[i].y, w0);
+                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x0[i].z, w0);
+                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x0[i].w, w0);
+                }
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) {
+                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x1[i].x, w1);
+                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x1[i].y, w1);
+                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x1[i].z, w1);
+                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x1[i].w, w1);
                 }
             }
         }
@@ -1930,6 +1973,159 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
         if (all_dead) v = V{};
         else v = *reinterpret_cast<const V*>(fin + ((size_t)col * R + part * VW) * 4);
         *reinterpret_cast<V*>(gout + (size_t)col * RB + part * VW) = v;
+    }
+    if (t < R && last_alive >= 0) a.active[row0 + t] = a.stamp0 + last_alive;
+}
+
+// The resident launch of TILED layers: block_resident_kernel's frame (R rows of a workgroup in LDS through all layers
+// of the launch, two buffers, one barrier per layer, rows stamped with the last layer that left them nonzero, a
+// workgroup whose rows are all zero stops) around rowtile_kernel's arithmetic (thread t computes whole outputs - slots
+// t, t + 1024, ... - from its own entry list, 16-byte LDS reads of a column's rows in a lane-rotated order).  The
+// outputs go to the other LDS buffer as they are (a lane writes its parts where they belong), so of a layer's time
+// in rowtile_kernel - the launch, the rows in, the rows out - only the arithmetic is left.
+template <int R, int WMODE>
+__global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int sh_alive[3];
+    constexpr int PARTS = R / 4;
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    using GB = const __attribute__((address_space(1))) unsigned char*;
+    using GI = const __attribute__((address_space(1))) int32_t*;
+    publish_counts(a.pub);
+    const int t = (int)threadIdx.x, lane = t & 63;
+    const int RB = 64 * a.rl;
+    const unsigned nwg = gridDim.x;
+    const unsigned wg = (nwg % 8u) == 0u ? (blockIdx.x % 8u) * (nwg / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const size_t row0 = (size_t)wg * R;
+    const int rb = (int)(row0 / (size_t)RB), rin = (int)(row0 - (size_t)rb * RB);
+    if (a.check_dead && a.prev_stamp != 0) {   // a row block without an active row is skipped, as by the per-layer kernels
+        int alive = 0;
+        for (int i = t; i < RB; i += 1024) alive |= (a.active[(size_t)rb * RB + i] == a.prev_stamp) ? 1 : 0;
+        if (__syncthreads_or(alive) == 0) return;
+    }
+    const size_t blkf = (size_t)a.N * RB;
+    const uint32_t buf_bytes = (uint32_t)a.N * R * 4;
+    const int total = a.N * PARTS;
+    {
+        const float* __restrict__ gin = ((rb & 1) ? a.first_in.half[1] : a.first_in.half[0]) + (size_t)(rb >> 1) * blkf + rin;
+        for (int base = t; base < total; base += 4096) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = min(base + u * 1024, total - 1);   // (a lane past the end reads the last piece again and drops it)
+                const int col = idx / PARTS, part = idx - col * PARTS;
+                v[u] = *reinterpret_cast<const float4*>(gin + (size_t)col * RB + part * 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int idx = base + u * 1024;
+                if (idx < total) *reinterpret_cast<float4*>(smem + (size_t)idx * 16) = v[u];
+            }
+        }
+    }
+    if (t < 3) sh_alive[t] = 0;
+    uint32_t poff[PARTS];   // this lane's order of the four-row parts of a column, as byte offsets
+#pragma unroll
+    for (int i = 0; i < PARTS; ++i) poff[i] = (uint32_t)(((i + lane) & (PARTS - 1)) * 16);
+    const uint32_t estride = (uint32_t)a.N * 8u;
+    int last_alive = -1;
+    bool all_dead = false;
+    int done_layers = 0;
+    __syncthreads();
+    for (int j = 0; j < a.nlayers; ++j) {
+        const unsigned char* const in = smem + ((j & 1) ? buf_bytes : 0u);
+        unsigned char* const out = smem + ((j & 1) ? 0u : buf_bytes);
+        const LayerDesc lay = load_layer_desc(a.table, j);
+        const GB entb = (GB)lay.rt_ent;
+        const GI lens = (GI)lay.rt_len, dsts = (GI)lay.rt_dst;
+        unsigned bits = 0;   // rows that one of this lane's outputs left nonzero
+        for (int slot0 = 0; slot0 < a.N; slot0 += 1024) {
+            const int slot = slot0 + t;
+            const bool have = slot < a.N;
+            const int n_in = have ? lens[slot] : 0;
+            const int n_wave = __builtin_amdgcn_readfirstlane(n_in);   // slots are ordered by length: the wave's first lane has the most
+            float acc[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) acc[i] = 0.0f;
+            // Two entries at a time, the next two requested under the arithmetic: one workgroup per CU leaves a SIMD
+            // four waves, so a wave has to keep eight LDS reads of its own in flight.  No test of k against the lane's
+            // own length: behind a list the array holds (column 0, weight +0), and adding x * (+0) to an accumulator
+            // that started at +0 changes nothing (it can never be -0).
+            uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
+            u32x2 e0 = {0u, 0u}, e1 = {0u, 0u};
+            if (n_wave > 0) {
+                e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+                e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
+            }
+            for (int k = 0; k < n_wave; k += 2) {
+                const u32x2 c0 = e0, c1 = e1;
+                eoff += 2u * estride;
+                if (k + 2 < n_wave) {
+                    e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+                    e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
+                }
+                const float w0 = __uint_as_float(c0.y), w1 = __uint_as_float(c1.y);
+                const uint32_t colb0 = c0.x * (uint32_t)(R * 4), colb1 = c1.x * (uint32_t)(R * 4);
+                float4 x0[PARTS], x1[PARTS];
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) x0[i] = *reinterpret_cast<const float4*>(in + (colb0 + poff[i]));
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) x1[i] = *reinterpret_cast<const float4*>(in + (colb1 + poff[i]));
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) {
+                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x0[i].x, w0);
+                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x0[i].y, w0);
+                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x0[i].z, w0);
+                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x0[i].w, w0);
+                }
+#pragma unroll
+                for (int i = 0; i < PARTS; ++i) {
+                    acc[i * 4 + 0] = mac<WMODE>(acc[i * 4 + 0], x1[i].x, w1);
+                    acc[i * 4 + 1] = mac<WMODE>(acc[i * 4 + 1], x1[i].y, w1);
+                    acc[i * 4 + 2] = mac<WMODE>(acc[i * 4 + 2], x1[i].z, w1);
+                    acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x1[i].w, w1);
+                }
+            }
+            const int d = have ? dsts[slot] : -1;
+#pragma unroll
+            for (int i = 0; i < PARTS; ++i) {
+                float4 y;
+                y.x = relu_clamp(acc[i * 4 + 0] + a.bias, a.clampv);
+                y.y = relu_clamp(acc[i * 4 + 1] + a.bias, a.clampv);
+                y.z = relu_clamp(acc[i * 4 + 2] + a.bias, a.clampv);
+                y.w = relu_clamp(acc[i * 4 + 3] + a.bias, a.clampv);
+                const unsigned nzb = (y.x > 0.0f ? 1u : 0u) | (y.y > 0.0f ? 2u : 0u) | (y.z > 0.0f ? 4u : 0u) | (y.w > 0.0f ? 8u : 0u);
+                if (d >= 0) {
+                    bits |= nzb << (poff[i] >> 2);
+                    *reinterpret_cast<float4*>(out + ((uint32_t)d * (uint32_t)(R * 4) + poff[i])) = y;
+                }
+            }
+        }
+        unsigned wave_bits = 0;
+#pragma unroll
+        for (int b = 0; b < R; ++b)
+            if (__ballot((bits >> b) & 1u) != 0ull) wave_bits |= 1u << b;
+        if (lane == 0 && wave_bits != 0) atomicOr(&sh_alive[j % 3], (int)wave_bits);
+        __syncthreads();
+        const int mask = sh_alive[j % 3];
+        if (t == 0) sh_alive[(j + 2) % 3] = 0;
+        if (t < R && ((mask >> t) & 1)) last_alive = j;
+        done_layers = j + 1;
+        if (mask == 0 && a.bias <= 0.0f) { all_dead = true; break; }   // zero rows stay zero
+    }
+    // the launch's last layer writes the work buffer the layer before it did not (layer 0: the one it did not read)
+    const bool in_a = a.first_in.half[0] == a.buf_a.half[0];
+    const bool to_c = in_a == ((a.nlayers & 1) != 0);
+    float* const o_h0 = to_c ? a.buf_c.half[0] : a.buf_a.half[0];
+    float* const o_h1 = to_c ? a.buf_c.half[1] : a.buf_a.half[1];
+    float* __restrict__ gout = ((rb & 1) ? o_h1 : o_h0) + (size_t)(rb >> 1) * blkf + rin;
+    const unsigned char* const fin = smem + ((done_layers & 1) ? buf_bytes : 0u);
+    for (int idx = t; idx < total; idx += 1024) {
+        const int col = idx / PARTS, part = idx - col * PARTS;
+        float4 v;
+        if (all_dead) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        else v = *reinterpret_cast<const float4*>(fin + (size_t)idx * 16);
+        *reinterpret_cast<float4*>(gout + (size_t)col * RB + part * 4) = v;
     }
     if (t < R && last_alive >= 0) a.active[row0 + t] = a.stamp0 + last_alive;
 }
@@ -2521,6 +2717,48 @@ hipError_t launch_block_resident(const ResidentLaunch& a, hipStream_t s) {
     return R == 16 ? launch_block_resident_r<16>(a, s) : launch_block_resident_r<4>(a, s);
 }
 
+int rowtile_resident_rows(int N) {
+    if (N <= 0) return 0;
+    if (N <= 1024) return 16;   // two buffers of N x R floats: up to 128 KiB
+    if (N <= 2048) return 8;
+    if (N <= 4096) return 4;
+    return 0;
+}
+
+template <int R>
+static hipError_t launch_rowtile_resident_r(const ResidentLaunch& a, int wmode, hipStream_t s) {
+    ResidentArgs k{};
+    k.table = a.table; k.nlayers = a.nlayers; k.first_in = a.first_in; k.buf_a = a.buf_a; k.buf_c = a.buf_c; k.active = a.active;
+    k.N = a.N; k.ngroups = 0; k.rl = a.rl; k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
+    k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
+    const size_t lds = (size_t)a.N * R * 8;
+    dim3 grid((unsigned)(a.rows / R)), block(1024);
+#define SPDNN_RT_RESIDENT(WM)                                                                                               \
+    do {                                                                                                                    \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rowtile_resident_kernel<R, WM>),   \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);        \
+        if (attr != hipSuccess) return attr;                                                                                \
+        hipLaunchKernelGGL((rowtile_resident_kernel<R, WM>), grid, block, lds, s, k);                                       \
+    } while (0)
+    if (wmode != 2) SPDNN_RT_RESIDENT(1); else SPDNN_RT_RESIDENT(2);
+#undef SPDNN_RT_RESIDENT
+    return hipGetLastError();
+}
+
+hipError_t launch_rowtile_resident(const ResidentLaunch& a, int wmode, hipStream_t s) {
+    // host-side shape checks: what the kernel's two LDS buffers and its row numbering assume
+    if (a.N <= 0 || a.nlayers < 1 || !a.table || !a.first_in || !a.buf_a || !a.buf_c || a.buf_a == a.buf_c || !a.active ||
+        a.rows <= 0 || (a.rl != 1 && a.rl != 2 && a.rl != 4) || (a.rows % (64 * a.rl)) != 0)
+        return hipErrorInvalidValue;
+    const int R = rowtile_resident_rows(a.N);
+    if (R == 0 || (64 * a.rl) % R != 0 || (size_t)a.N * R * 8 > 128 * 1024 || (long long)a.rows / R > 0x7fffffffll) return hipErrorInvalidValue;
+    switch (R) {
+        case 16: return launch_rowtile_resident_r<16>(a, wmode, s);
+        case 8: return launch_rowtile_resident_r<8>(a, wmode, s);
+        default: return launch_rowtile_resident_r<4>(a, wmode, s);
+    }
+}
+
 hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,
                                     int32_t* counts_host, hipStream_t s) {
     if (!stamps || rows <= 0 || n < 1 || n > 8192 || (!counts_dev && !counts_host)) return hipErrorInvalidValue;
@@ -2643,14 +2881,19 @@ static hipError_t launch_rowtile_r(const RowtileLaunch& a, hipStream_t s) {
     k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
     const size_t lds = (size_t)a.N * R * 4;
     dim3 grid((unsigned)(a.rows / R)), block(1024);
-#define SPDNN_ROWTILE(WM)                                                                                        \
-    do {                                                                                                         \
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rowtile_kernel<R, WM>), \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-        if (attr != hipSuccess) return attr;                                                                     \
-        hipLaunchKernelGGL((rowtile_kernel<R, WM>), grid, block, lds, s, k);                                     \
+#define SPDNN_ROWTILE(WM, PAIRS)                                                                                        \
+    do {                                                                                                                \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(rowtile_kernel<R, WM, PAIRS>), \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);    \
+        if (attr != hipSuccess) return attr;                                                                            \
+        hipLaunchKernelGGL((rowtile_kernel<R, WM, PAIRS>), grid, block, lds, s, k);                                     \
     } while (0)
-    if (a.wmode != 2) SPDNN_ROWTILE(1); else SPDNN_ROWTILE(2);
+    // two entries per step where a CU holds one workgroup anyway (more than half of its LDS)
+    if (R == 16 && lds <= 80 * 1024) {
+        if (a.wmode != 2) SPDNN_ROWTILE(1, false); else SPDNN_ROWTILE(2, false);
+    } else {
+        if (a.wmode != 2) SPDNN_ROWTILE(1, true); else SPDNN_ROWTILE(2, true);
+    }
 #undef SPDNN_ROWTILE
     return hipGetLastError();
 }

@@ -183,6 +183,12 @@ struct LayerDesc {           // one entry of the device-side layer table
     const int32_t* blk_cnt;
     const float* blk_wv;
     const int32_t* blk_dst;
+    // ROWTILE form (TILED layers up to 8192 neurons wide)
+    const uint32_t* rt_ent;
+    const int32_t* rt_len;
+    const int32_t* rt_dst;
+    int rt_kpad;
+    int pad_;
 };
 
 struct PersistCtl {          // device words of one persistent launch (zero before the launch)
@@ -238,6 +244,13 @@ struct ResidentLaunch {
     float bias, clampv;
     Publish publish;
 };
+// The same for TILED layers in their ROWTILE form (any sparsity pattern): `nlayers` consecutive such layers of one
+// weight mode, the R rows of a workgroup in LDS from the first layer to the last, every thread computing whole outputs
+// from its own entry list (rowtile_resident_kernel).  ngroups and full are not used.
+hipError_t launch_rowtile_resident(const ResidentLaunch& a, int wmode, hipStream_t s);
+// rows such a workgroup keeps (16, 8 or 4 for up to 1024, 2048, 4096 neurons: two buffers of N x R floats), 0 = too wide
+int rowtile_resident_rows(int N);
+
 // rows a workgroup keeps (16 or 4), 0 if the shape does not fit: two buffers of (N + 1) x R floats in LDS
 // (N <= 1024: 16 rows, N <= 4096: 4) and one (group, row) item per thread of 1024
 int resident_rows_per_workgroup(int N, int ngroups);

@@ -658,6 +658,11 @@ int upload_plans(spdnn_net* n) {
                 t.blk_cnt = n->dl[l].blk_cnt;
                 t.blk_wv = n->dl[l].wv;
                 t.blk_dst = n->dl[l].dst;
+            } else if (p.kernel == SPDNN_KERNEL_TILED && !p.rt_ent.empty()) {   // its ROWTILE form
+                t.rt_ent = n->dl[l].rt_ent;
+                t.rt_len = n->dl[l].alt_cnt;
+                t.rt_dst = n->dl[l].alt_dst;
+                t.rt_kpad = (p.alt_kmax + 3) / 4 * 4;
             }
         }
         HIPCHK(dev_malloc(&n->d_table, table.size() * sizeof(LayerDesc)));
@@ -1626,21 +1631,24 @@ static LayerSig layer_sig(const spdnn_net* n, int l, int nblk) {
     return g;
 }
 
-// Whether layer l can be part of a resident launch (rows kept in LDS through the layers): it needs a BLOCK form
-// with one exact weight - a BLOCK layer of weight mode 0, or a run-chain BAND layer that carries its BLOCK form -
-// and a shape the kernel's LDS buffers and item numbering hold.
+// Whether layer l can be part of a resident launch (rows kept in LDS through the layers), and in which form: its
+// BLOCK form with one exact weight - a BLOCK layer of weight mode 0, or a run-chain BAND layer that carries its
+// BLOCK form - or the ROWTILE form of a TILED layer; and a shape the kernel's LDS buffers and numbering hold.
 struct ResidentSig {
-    int ok = 0, full = 0, ngroups = 0;
-    bool operator==(const ResidentSig& o) const { return ok == o.ok && full == o.full && ngroups == o.ngroups; }
+    int ok = 0;      // 0 no resident form; 1 BLOCK form of one exact weight; 2 ROWTILE form (TILED layers)
+    int full = 0, ngroups = 0, wmode = 0;
+    int rows = 0;    // rows a workgroup keeps
+    bool operator==(const ResidentSig& o) const { return ok == o.ok && full == o.full && ngroups == o.ngroups && wmode == o.wmode; }
 };
 static ResidentSig resident_sig(const spdnn_net* n, int l) {
     const LayerPlan& p = n->layers[(size_t)l];
     ResidentSig g;
     if (p.kernel == SPDNN_KERNEL_BAND && p.alt_ngroups > 0) { g.ok = 1; g.full = p.alt_full ? 1 : 0; g.ngroups = p.alt_ngroups; }
     else if (p.kernel == SPDNN_KERNEL_BLOCK && p.wmode == 0) { g.ok = 1; g.full = p.blk_full ? 1 : 0; g.ngroups = p.ngroups; }
+    else if (p.kernel == SPDNN_KERNEL_TILED && !p.rt_ent.empty() && n->rowtile_mode) { g.ok = 2; g.wmode = p.wmode; }
     if (g.ok) {
-        const int R = resident_rows_per_workgroup(n->N, g.ngroups);
-        if (R == 0 || n->RB % R != 0) g.ok = 0;
+        g.rows = g.ok == 1 ? resident_rows_per_workgroup(n->N, g.ngroups) : rowtile_resident_rows(n->N);
+        if (g.rows == 0 || n->RB % g.rows != 0) g.ok = 0;
     }
     return g;
 }
@@ -1858,12 +1866,16 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 // at 2048 and at 60000 rows.  So left to the library: from 2 layers (even while the counts still move -
                 // workgroups whose rows have all died leave early) and from 8; a caller that asks for launches of a
                 // given length gets them.
-                const bool wide_rows = resident_rows_per_workgroup(n->N, rsig.ngroups) >= 16;
+                const bool wide_rows = rsig.rows >= 16;
                 const int rmin = (persist_asked || wide_rows) ? 2 : 8;
                 const int rmax = std::min(wide_rows ? std::max(cmax, 2) : cmax, last - l + 1);
                 int k = 1;
                 while (k < rmax && resident_sig(n, l + k) == rsig) ++k;
-                if (k >= rmin) { c = k; resident = true; }
+                // (entry lists for 8 or 4 rows at a time: on large launches the per-layer kernel, which reads them for 16, is the
+                // faster one - measured per layer at batch 60000: N=2048 376 against 337 us, N=4096 1232 against 948; at 2048
+                // rows 13 against 38 and 42 against 57)
+                const bool too_large = !persist_asked && rsig.ok == 2 && !wide_rows && n->carried >= n->tiled_min_rows;
+                if (k >= rmin && !too_large) { c = k; resident = true; }
             }
             const bool pair = !fb && !resident && is_pair(l);
             if (pair) c = 2;
@@ -1969,10 +1981,10 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 rl.N = n->N; rl.ngroups = rsig.ngroups; rl.rows = n->carried; rl.rl = n->rl; rl.full = rsig.full;
                 rl.stamp0 = stamp0; rl.prev_stamp = prev_stamp; rl.check_dead = check_dead; rl.bias = n->bias; rl.clampv = n->clampv;
                 rl.publish = st.pub;
-                HIPCHK(launch_block_resident(rl, n->stream));
+                HIPCHK(rsig.ok == 1 ? launch_block_resident(rl, n->stream) : launch_rowtile_resident(rl, rsig.wmode, n->stream));
                 if (n->run_verbose)
-                    fprintf(stderr, "spdnn: resident launch: layers %d..%d, %d rows, %d rows per workgroup\n", l, l + c - 1, n->carried,
-                            resident_rows_per_workgroup(n->N, rsig.ngroups));
+                    fprintf(stderr, "spdnn: resident launch (%s): layers %d..%d, %d rows, %d rows per workgroup\n",
+                            rsig.ok == 1 ? "groups" : "entry lists", l, l + c - 1, n->carried, rsig.rows);
                 for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
                 st.r.resident_launches += 1;
             } else if (fb) {

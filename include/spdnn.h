@@ -92,9 +92,9 @@ typedef struct spdnn_run_options {
     int32_t time_layers;       /* 1: bracket every layer with HIP events                           */
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
     int32_t fuse_layers;       /* launches that hold more than one layer.  1 = every layer its own launch.  0 = default:
-                                  - resident launches where consecutive layers have a BLOCK form with one exact weight and
-                                    at most 4096 neurons (RadiX-Net layers): a workgroup keeps 16 or 4 rows in LDS through
-                                    up to 64 layers (SPDNN_RESIDENT=0: never);
+                                  - resident launches where consecutive layers have a BLOCK form with one exact weight
+                                    (RadiX-Net layers) or are TILED layers, at most 4096 neurons wide: a workgroup keeps
+                                    16, 8 or 4 rows in LDS through up to 64 layers (SPDNN_RESIDENT=0: never);
                                   - pairs of layers the inspector marked fuse_next as one launch with the intermediate tile
                                     in LDS, on launches of 2^23 rows x neurons and more (SPDNN_PAIR_MIN_ELEMS);
                                   - persistent launches (up to 64 layers of one kernel form, a dependency per row block

@@ -624,6 +624,54 @@ def test_resident_launches(gc, orc, N, B, kind):
         assert same_floats(net.activations(cats), ref["y"])
 
 
+@pytest.mark.parametrize("N,B,values", [(512, 900, "general"), (1024, 1500, "general"), (1024, 700, "pow2"), (2048, 600, "general"),
+                                        (4096, 400, "general")])
+def test_resident_launches_of_unstructured_layers(gc, orc, N, B, values):
+    """Layers without structure (TILED class) up to 4096 neurons wide run as resident launches too: the 16, 8 or 4 rows of
+    a workgroup stay in LDS through the layers, every thread computing whole outputs from its entry list.  Per-layer
+    counts, categories and activations against the oracle, pruned and unpruned, whole and cut into calls, and the
+    state after every layer."""
+    print("resident launches, unstructured layers N=%d B=%d %s" % (N, B, values), flush=True)
+    rng = np.random.default_rng(N + B)
+    L = 7
+    base = [random_csr(rng, N, rng.integers(0, 25, size=N), values) for _ in range(3)]
+    layers = [base[l % 3] for l in range(L)]
+    dens = np.where(rng.random(B) < 0.3, 0.9, 0.05).astype(np.float32)
+    feats = ((rng.random((B, N), dtype=np.float32) < dens[:, None]) * rng.uniform(0.5, 2.0, size=(B, N))).astype(np.float32)
+    bias = -0.05
+    ref = orc.infer(feats, [sort_rows(c) for c in layers], bias, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    with gc.Network(N, B, L, bias=bias) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_TILED for l in range(L))
+        net.set_features_dense(feats)
+        cats = ref["categories"]
+        for prune in (True, False):
+            for fuse in (0, 3, 1):
+                r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert r.layers_run == L and r.persistent_launches == 0
+                if fuse == 1:
+                    assert r.resident_launches == 0
+                elif fuse == 3 or (N <= 1024 and not prune):   # (left to the library, 8- and 4-row workgroups want 8 layers and more)
+                    assert r.resident_launches >= 1
+                assert [net.active_count(l) for l in range(L)] == want_counts
+                assert np.array_equal(net.categories(), cats)
+                assert same_floats(net.activations(cats), ref["y"])
+        for l in range(L):    # the state after layer l, from a resident launch that ends there
+            net.run(prune=True, first_layer=0, n_layers=l + 1, fuse_layers=L)
+            gid, y = ref["kept"][l]
+            assert np.array_equal(net.categories(), ref["active_ids"][l])
+            assert same_floats(net.activations(gid), y)
+        net.run(prune=True, first_layer=0, n_layers=3, fuse_layers=3)
+        r = net.run(prune=False, first_layer=3, n_layers=L - 3, collect_counts=True, fuse_layers=L)
+        assert r.resident_launches == 1
+        assert [net.active_count(l) for l in range(3, L)] == want_counts[3:]
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(cats), ref["y"])
+
+
 def test_resident_launches_full_batch(gc, orc):
     """Batch 60000 of RadiX-Net-like layers, N=1024: every activation of every row, the per-layer counts and the
     categories of the default run (resident launches) equal those of one launch per layer bit for bit, on live
