@@ -80,7 +80,29 @@ def irregular_layer(rng, n, kmax=24):
     return rowptr, col, val
 
 
-def sustained_block(gc, name, seed, log, per_layer_too):
+def cpu_literal_run(orc, layer_csr, N, L, B, bias, seed, dens_hi, chunk=4096):
+    """The literal run of a configuration on the CPU oracle (pruning on, every row of the batch, all cores), in row
+    chunks to bound the memory: seconds and the per-layer active-row counts."""
+    t_lit = 0.0
+    counts = np.zeros(L, np.int64)
+    layers_cache = {}
+    for r0 in range(0, B, chunk):
+        y = orc.gen_features(seed, N, r0, min(chunk, B - r0), 0.10, dens_hi)
+        gid = np.arange(len(y), dtype=np.int32)
+        for l in range(L):
+            if l not in layers_cache:
+                layers_cache[l] = layer_csr(l)
+            t0 = time.perf_counter()
+            y, act = orc.layer(y, layers_cache[l], bias)
+            y, gid = orc.compact(y, act, gid)
+            t_lit += time.perf_counter() - t0
+            counts[l] += len(gid)
+            if len(gid) == 0:
+                break
+    return t_lit, counts
+
+
+def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
     """One BASELINE configuration other than the headline one, sustained (pruning off, full batch at every layer): ms per
     layer and fraction of the HBM roofline on the configured features (all-zero activations from layer 2 on) and on live
     data (densities up to 0.7: rows survive every layer), two timed passes each after one warm-up pass; for the narrow
@@ -112,6 +134,16 @@ def sustained_block(gc, name, seed, log, per_layer_too):
         out["live_one_launch_per_layer"] = timed(1)
     lit = net.run(prune=True, collect_counts=True)
     out["literal_live_pruned_ms"] = lit.ms_total
+    # the literal run of the configuration as BASELINE defines it (densities up to 0.25, pruning on), GPU and CPU side by side
+    net.synth_features(seed, B, 0.10, 0.25)
+    lit = net.run(prune=True, collect_counts=True)
+    gpu_counts = [int(net.active_count(l)) for l in range(min(L, 8))]
+    out["literal"] = {"gpu_ms": lit.ms_total, "active_rows_first_layers": gpu_counts, "categories": int(lit.active_rows)}
+    if with_cpu:
+        from oracle import oracle as orc
+        t_cpu, cpu_counts = cpu_literal_run(orc, lambda l: orc.gen_layer_csr(seed, l, N), N, L, B, bias, seed, 0.25)
+        out["literal"].update({"cpu_s": t_cpu, "cpu_cores": orc.get_threads(),
+                               "counts_equal": [int(c) for c in cpu_counts[:len(gpu_counts)]] == gpu_counts})
     out["band_tuning_rowblocks_shape_seglen"] = net.band_tuning()
     out["feature_buffers_region_paired_candidates_peak_bytes"] = list(net.feature_placement())
     net.close()
@@ -354,22 +386,8 @@ def main():
             if not args.no_extras:
                 # the literal run of THIS configuration on the CPU (pruning on, every row of the batch, all cores), in row
                 # chunks to bound the memory: the run the GPU's `literal` block makes, its per-layer counts compared
-                chunk, t_lit = 4096, 0.0
-                cpu_counts = np.zeros(L, np.int64)
-                layers_cache = {}
-                for r0 in range(0, B, chunk):
-                    y = orc.gen_features(seed, N, r0, min(chunk, B - r0), 0.10, args.density_hi)
-                    gid = np.arange(len(y), dtype=np.int32)
-                    for l in range(L):
-                        if l not in layers_cache:
-                            layers_cache[l] = layer_csr(l)
-                        t0 = time.perf_counter()
-                        y, act = orc.layer(y, layers_cache[l], bias)
-                        y, gid = orc.compact(y, act, gid)
-                        t_lit += time.perf_counter() - t0
-                        cpu_counts[l] += len(gid)
-                        if len(gid) == 0:
-                            break
+                chunk = 4096
+                t_lit, cpu_counts = cpu_literal_run(orc, layer_csr, N, L, B, bias, seed, args.density_hi, chunk)
                 ran = int(np.count_nonzero(cpu_counts)) + 1
                 cpu["literal"] = {"workload": "%s literal: pruning on, batch %d, all %d layers (rows of chunk after chunk of %d)"
                                               % (args.config, B, L, chunk),
@@ -433,7 +451,7 @@ def main():
     # ---- beside the headline run: the other BASELINE configurations and challenge-like pruned runs -----------
     other, challenge = None, None
     if not args.no_extras and args.structure == "circulant":
-        other = {name: sustained_block(gc, name, seed, log, per_layer_too=name in ("cfg0", "cfg1", "cfg2"))
+        other = {name: sustained_block(gc, name, seed, log, per_layer_too=name in ("cfg0", "cfg1", "cfg2"), with_cpu=not args.no_cpu)
                  for name in ("cfg0", "cfg1", "cfg2", "cfg3") if name != args.config}
         challenge = {"workload": "RadiX-Net-like layers (strides 16 .. N/2 in turn, random relabellings), batch 60000 with 3 % "
                                  "dense rows that survive, pruning on, whole run; best of three",
