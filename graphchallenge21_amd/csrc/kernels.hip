@@ -1657,12 +1657,16 @@ __device__ __forceinline__ int persist_wait(const PersistArgs& a, const int32_t*
     return 0;
 }
 
-// After the wait (every wave, behind the barrier that follows it): the writers ran on other CUs, so this CU's L1
-// is dropped (same XCD, same L2: light) or everything visible at device scope is taken.  Every wave does it
-// for itself, in front of its own loads: an invalidate issued by one wave orders that wave's loads only.
-__device__ __forceinline__ void persist_acquire(const PersistArgs& a) {
-    if (a.light & 1) asm volatile("buffer_inv sc0" ::: "memory");
-    else __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+// After the wait (every wave, behind the barrier that follows it): the writers ran on other CUs, so what this CU's
+// L1 holds of the buffer is stale - it may have read the same lines two layers earlier.  Every wave invalidates for
+// itself, in front of its own loads: an invalidate issued by one wave orders that wave's loads only.  At device
+// scope (buffer_inv sc1), also where writer and reader share an XCD and its L2: the workgroup-scope form (buffer_inv
+// sc0) leaves the L1 as it is outside threadgroup-split mode - seen as wrong results (different from run to run) on
+// a network of 256 neurons in 64-row blocks, three layers per launch, whose buffers stay in L1 from layer to layer;
+// wider layers push their lines out of the 32 KiB by themselves and never showed it.  The invalidate costs the
+// launches that are persistent by default nothing measurable (N=1024, batch 60000: 99.5 against 99.8 us per layer).
+__device__ __forceinline__ void persist_acquire(const PersistArgs&) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
 // Entry j of the layer table through the constant address space: the table never changes while a kernel
@@ -2592,8 +2596,8 @@ PersistArgs persist_args(const PersistLaunch& a, const PersistShape& p) {
     k.active = a.active; k.done = a.done; k.done_stride = a.done_stride; k.ctl = a.ctl; k.prev_ctl = a.prev_ctl;
     k.prev_units = a.prev_units; k.abort = a.abort; k.host_word = a.host_word;
     k.N = a.N; k.nblk = a.nblk; k.nseg = p.nseg; k.seglen = p.seglen; k.total_units = p.total; k.nq = p.nq;
-    // light_sync 1: both sides light; for measurements 2 = the writer's side only, 4 = the reader's side only
-    k.light = p.nq > 1 ? (a.light_sync == 1 ? 3 : a.light_sync == 2 ? 2 : a.light_sync == 4 ? 1 : 0) : 0;
+    // light_sync (per-XCD queues only): the writer waits for its stores and leaves the L2 write-back out (bit 1)
+    k.light = (p.nq > 1 && a.light_sync) ? 2 : 0;
     k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead; k.wait_limit = a.wait_limit;
     k.bias = a.bias; k.clampv = a.clampv;
     k.stream = (long long)a.nblk * (long long)a.N * 64 * a.rl * 4 * 2 >= a.stream_min_bytes ? 1 : 0;

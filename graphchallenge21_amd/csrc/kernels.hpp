@@ -167,7 +167,8 @@ hipError_t launch_block(const BlockLaunch& a, hipStream_t s);
 //
 // With xcd_queues the queue is split in eight, one per XCD: a workgroup reads the number of the
 // XCD it runs on from the hardware and serves that queue only; row block rb belongs to queue
-// rb % 8.  Everything a row block's layers hand to each other then stays in one XCD's L2.
+// rb % 8.  Everything a row block's layers hand to each other then stays in one XCD's L2, which saves the writer
+// the write-back of that L2.
 // ------------------------------------------------------------------------------------------
 struct LayerDesc {           // one entry of the device-side layer table
     // BAND form
@@ -218,7 +219,8 @@ struct PersistLaunch {
     int seglen;                   // band positions (band walk) or groups (BLOCK) per unit; 0 = heuristic
     int xcd_queues;               // 1: one queue per XCD, row block rb in queue rb % 8
     int light_sync;               // 1 (xcd_queues only): the hand-over between layers stays inside one L2, so the
-                                  // writer only waits for its stores and the reader only drops its CU's L1
+                                  // writer only waits for its stores (no L2 write-back); the reader invalidates at
+                                  // device scope either way
     long long wait_limit;         // ticks of the 100 MHz clock a unit waits for its row block at most
     int n_cu;
     long long stream_min_bytes;

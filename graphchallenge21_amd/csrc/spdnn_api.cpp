@@ -272,7 +272,7 @@ struct spdnn_net {
     long long persist_min_bytes = (long long)1 << 28, persist_max_bytes = (long long)1 << 31;
     int persist_min_blocks = 64;      // fewest row blocks a persistent launch is made for by default (SPDNN_PERSIST_MIN_BLOCKS)
     int persist_xcd = -1;             // one unit queue per XCD: -1 = from 8 row blocks up, 0 / 1 (SPDNN_PERSIST_XCD)
-    int persist_light = 1;            // SPDNN_PERSIST_LIGHT_SYNC=0: device-scope fences also with XCD queues (3 times slower)
+    int persist_light = 1;            // SPDNN_PERSIST_LIGHT_SYNC=0: the writer's L2 write-back also with XCD queues
     int persist_seglen = 0;           // band positions / groups per unit, 0 = heuristic (SPDNN_PERSIST_SEGLEN)
     int resident_mode = 1;            // 1: layers with a BLOCK form of one exact weight run as resident launches where the
                                       // shape fits (rows kept in LDS through the layers; SPDNN_RESIDENT=0: never)
@@ -903,7 +903,7 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_PERSIST_MIN_BYTES")) n->persist_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_PERSIST_XCD")) n->persist_xcd = atoi(e);
     if (const char* e = getenv("SPDNN_PERSIST_MIN_BLOCKS")) n->persist_min_blocks = std::max(1, atoi(e));
-    if (const char* e = getenv("SPDNN_PERSIST_LIGHT_SYNC")) n->persist_light = atoi(e);
+    if (const char* e = getenv("SPDNN_PERSIST_LIGHT_SYNC")) n->persist_light = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PERSIST_SEGLEN")) n->persist_seglen = std::max(0, atoi(e));
     if (const char* e = getenv("SPDNN_RESIDENT")) n->resident_mode = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_PERSIST_WAIT_US")) n->persist_wait_us = std::max(0ll, atoll(e));
@@ -1955,8 +1955,8 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 pl.prev_stamp = prev_stamp; pl.check_dead = check_dead; pl.unrolled = sig.unrolled; pl.add_only = n->add_only;
                 pl.twins = sig.twins; pl.full = sig.full; pl.seglen = n->persist_seglen; pl.direct_lds = n->band_direct_lds;
                 // one queue per XCD where every XCD gets a row block: what the layers of a row block hand to each other
-                // then stays in one XCD's L2 and needs no device-scope fences (measured at N=1024, batch 6000, per layer:
-                // 17 us, against 55 - 64 us with the fences, of which the writer's 12 and the readers' 24)
+                // then stays in one XCD's L2 and the writer need not write that L2 back (measured at N=1024, batch 6000, per
+                // layer: the write-back 12 us of a 17 us layer)
                 pl.xcd_queues = n->persist_xcd >= 0 ? (n->persist_xcd ? 1 : 0) : (nblk >= 8 ? 1 : 0);
                 pl.light_sync = n->persist_light;
                 pl.wait_limit = persist_wait_us * 100;

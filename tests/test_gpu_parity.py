@@ -454,7 +454,8 @@ def test_full_batch_properties_cfg1(gc, orc):
         assert same_floats(y_p[:k], ref["y"][pos])
 
 
-PERSIST_MODES = {   # how the units of a persistent launch are queued and handed over (environment, read at creation)
+PERSIST_MODES = {   # how the units of a persistent launch are queued and handed over (environment, read at creation);
+                    # light = the writer leaves the write-back of its XCD's L2 out
     "default": {},
     "one-queue": {"SPDNN_PERSIST_XCD": "0"},
     "xcd-queues": {"SPDNN_PERSIST_XCD": "1", "SPDNN_PERSIST_LIGHT_SYNC": "0"},
@@ -704,6 +705,39 @@ def test_resident_launches_full_batch(gc, orc):
             assert r.resident_launches >= 1
             got = state()
             assert np.array_equal(got[0], want[0]) and got[1] == want[1] and np.array_equal(got[2], want[2]), prune
+
+
+@pytest.mark.parametrize("rl", [1, 2])
+def test_persistent_launches_on_buffers_that_stay_in_l1(gc, orc, rl, monkeypatch):
+    """Narrow layers in small row blocks: the buffers of a persistent launch stay in the CUs' L1 from layer to layer, so a
+    unit that does not really invalidate its L1 reads what the buffer held two layers earlier (found by a random case:
+    the workgroup-scope invalidate is no invalidate outside threadgroup-split mode).  Three and four layers per launch,
+    one unit queue per XCD, pruned: counts, categories and activations against the oracle, several networks, each run
+    three times."""
+    monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
+    monkeypatch.setenv("SPDNN_PERSIST_XCD", "1")
+    N, B = 256, 1500
+    for seed in range(8):
+        rng = np.random.default_rng(9100 + seed)
+        L = 3 + seed % 2
+        layers = []
+        for l in range(L):
+            rp, c, v = orc.gen_layer_csr(int(rng.integers(0, 1000)), l, N, 4)
+            layers.append((rp, c, rng.uniform(-0.1, 0.2, size=len(v)).astype(np.float32)))
+        feats = (rng.uniform(0, 3, size=(B, N)) * (rng.random((B, N)) < 0.8)).astype(np.float32)
+        ref = orc.infer(feats, layers, -0.05, prune=True)
+        want_counts = [len(a) for a in ref["active_ids"]]
+        with gc.Network(N, B, L, bias=-0.05) as net:
+            for l, csr in enumerate(layers):
+                net.set_layer_csr(l, *csr)
+            net.inspect()
+            net.set_features_dense(feats)
+            for rep in range(3):
+                r = net.run(prune=True, collect_counts=True, fuse_layers=L)
+                assert r.persistent_launches == 1 and r.persistent_fallbacks == 0
+                assert [net.active_count(l) for l in range(L)] == want_counts, (seed, rep)
+                assert np.array_equal(net.categories(), ref["categories"]), (seed, rep)
+                assert same_floats(net.activations(ref["categories"]), ref["y"]), (seed, rep)
 
 
 @pytest.mark.parametrize("mode", ["one-queue", "xcd-queues-light"])
@@ -1450,15 +1484,17 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         values = str(rng.choice(["uniform", "pow2", "general"]))
         # a third of the cases: every layer of one kind and row length, so that consecutive layers can share a
         # persistent launch (switched on and off, queued per XCD or not, with a wait limit of zero now and then)
-        same_kind = str(rng.choice(["circ", "radix", "hub"])) if rng.random() < 0.35 else None
+        same_kind = str(rng.choice(["circ", "radix", "hub", "gather", "radix-common"])) if rng.random() < 0.45 else None
         same_nnz = int(rng.choice([4, 16, 32]))
         persist = dict(SPDNN_PERSIST=str(int(rng.integers(0, 2))), SPDNN_PERSIST_XCD=str(int(rng.choice([-1, 0, 1]))),
-                       SPDNN_PERSIST_LIGHT_SYNC=str(int(rng.integers(0, 2))))
+                       SPDNN_PERSIST_LIGHT_SYNC=str(int(rng.integers(0, 2))), SPDNN_RESIDENT=str(int(rng.choice([1, 1, 0]))),
+                       SPDNN_COMMON_ORDER=str(int(rng.choice([1, 1, 0]))))
+        common_perm = rng.permutation(N)
         wait_us = int(rng.choice([0, 0, -1]))
         layers, kinds = [], []
         for l in range(L):
             kind = same_kind or str(rng.choice(["circ", "circ", "gather", "radix", "hub"]))
-            if kind in ("radix", "hub") and (N % 32 or N < 64):
+            if kind in ("radix", "hub", "radix-common") and (N % 32 or N < 64):
                 kind = "circ"
             if kind == "circ":
                 nnz = same_nnz if same_kind else int(rng.integers(1, 41))
@@ -1472,6 +1508,8 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
                 layers.append(sort_rows(random_csr(rng, N, rng.integers(0, min(N, 24), size=N), values)))
             elif kind == "radix":
                 layers.append(radix_like_csr(rng, N, int(16 * rng.integers(1, N // 16)), values))
+            elif kind == "radix-common":   # one hidden numbering for all such layers, strides 16 and 32 mostly
+                layers.append(radix_like_csr(rng, N, int(rng.choice([16, 16, 32, 32, 64])) % N or 16, values, perm=common_perm))
             else:
                 layers.append(hub_block_csr(rng, N, values))
             kinds.append(kind)
