@@ -106,7 +106,7 @@ def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
     """One BASELINE configuration other than the headline one, sustained (pruning off, full batch at every layer): ms per
     layer and fraction of the HBM roofline on the configured features (all-zero activations from layer 2 on) and on live
     data (densities up to 0.7: rows survive every layer), two timed passes each after one warm-up pass; for the narrow
-    configurations also with every layer as its own launch (the default shares persistent launches where it pays)."""
+    configurations also with every layer as its own launch (the default shares resident or persistent launches where it pays)."""
     N, L, B, bias = CONFIGS[name]
     t0 = time.time()
     net = gc.Network(N, B, L, bias=bias)
@@ -124,10 +124,13 @@ def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
         ms = best / L
         return {"ms_per_layer": ms, "frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "launches_per_pass": int(r.launches),
                 "persistent_launches_per_pass": int(r.persistent_launches), "persistent_fallbacks": int(r.persistent_fallbacks),
-                "rows_nonzero_at_end": int(r.active_rows)}
+                "resident_launches_per_pass": int(r.resident_launches), "rows_nonzero_at_end": int(r.active_rows)}
 
     net.synth_features(seed, B, 0.10, 0.25)
     out["zeros"] = timed(0)
+    if out["zeros"]["resident_launches_per_pass"]:
+        out["zeros"]["note"] = ("resident launches: a workgroup whose 16 rows are all zero leaves at once, so this figure is no "
+                                "measure of the kernels - the live figures are")
     net.synth_features(seed, B, 0.10, 0.70)
     out["live"] = timed(0)
     if per_layer_too:
@@ -494,7 +497,10 @@ def main():
                      "avg_launch_ms": avg_launch_ms, "launches_timed": int(layer_ms.size),
                      "note": ("resident launches: the rows stay in LDS between the layers of a launch, so the algorithmic bytes of a "
                               "layer never reach HBM and `frac` (algorithmic bytes over time, against the HBM peak) is not a bound "
-                              "here - the kernel is bound by LDS") if r.resident_launches else None,
+                              "here - the kernel is bound by LDS and the vector ALUs"
+                              + ("; on the all-zero activations of this run a workgroup leaves the launch as soon as its rows are zero, so "
+                                 "`value` is no measure of the kernels either: run with --density-hi 0.7" if args.density_hi <= 0.25 else ""))
+                     if r.resident_launches else None,
                      "data": ("all-zero activations from layer 2 on (bias -0.45 kills every row of the configured features); "
                               "see roofline_live for the same run on live data") if args.density_hi <= 0.25 else
                              "live data: feature densities U[0.10, %g]" % args.density_hi,

@@ -621,6 +621,61 @@ static int merged_pair_steps(int N, int K, const std::vector<int32_t>& rowptr, c
     return steps;
 }
 
+// The QUAD form of a BAND layer (see LayerPlan::quad_col): a four-way merge of the outputs' entry lists, which are
+// sorted by input index.  Left empty when some quad merges to more than 36 steps.
+static void build_quad_form(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
+                            const std::vector<float>& val, LayerPlan& plan) {
+    const int nq = N / 4;
+    int steps = 0;
+    std::vector<int32_t> merged;
+    auto merge_quad = [&](int c) {
+        merged.clear();
+        int at[4];
+        for (int j = 0; j < 4; ++j) at[j] = rowptr[plan.out_at[(size_t)4 * c + j]];
+        for (;;) {
+            int32_t in = INT32_MAX;
+            for (int j = 0; j < 4; ++j) {
+                const int row = plan.out_at[(size_t)4 * c + j];
+                if (at[j] < rowptr[row + 1]) in = std::min(in, col[at[j]]);
+            }
+            if (in == INT32_MAX) break;
+            merged.push_back(in);
+            for (int j = 0; j < 4; ++j) {
+                const int row = plan.out_at[(size_t)4 * c + j];
+                if (at[j] < rowptr[row + 1] && col[at[j]] == in) ++at[j];
+            }
+        }
+    };
+    for (int c = 0; c < nq; ++c) {
+        merge_quad(c);
+        steps = std::max(steps, (int)merged.size());
+    }
+    if (steps < 1 || steps > 36) return;
+    const int ng = (steps + 3) / 4;
+    plan.quad_groups = ng;
+    plan.quad_col.assign((size_t)nq * ng * 4, 0u);
+    plan.quad_w.assign((size_t)nq * ng * 16, 0.0f);
+    for (int c = 0; c < nq; ++c) {
+        merge_quad(c);
+        int at[4];
+        for (int j = 0; j < 4; ++j) at[j] = rowptr[plan.out_at[(size_t)4 * c + j]];
+        const int m_used = (int)merged.size();
+        for (int m = 0; m < ng * 4; ++m) {
+            const size_t grp = (size_t)c * ng + (size_t)(m >> 2);
+            const int32_t in = merged[(size_t)std::min(m, m_used - 1)];   // padding steps: the last column again, weights 0
+            plan.quad_col[grp * 4 + (size_t)(m & 3)] = (uint32_t)plan.in_pos[(size_t)in] * (uint32_t)kQuadColumnBytes;
+            if (m >= m_used) continue;
+            for (int j = 0; j < 4; ++j) {
+                const int row = plan.out_at[(size_t)4 * c + j];
+                if (at[j] < rowptr[row + 1] && col[at[j]] == in) {
+                    plan.quad_w[(grp * 4 + (size_t)j) * 4 + (size_t)(m & 3)] = val[at[j]];
+                    ++at[j];
+                }
+            }
+        }
+    }
+}
+
 void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<int32_t>& col,
                    const std::vector<float>& val, int force_kernel, bool fma_ok, LayerPlan& plan,
                    const std::vector<int32_t>* common_pos) {
@@ -716,6 +771,9 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.alt_wv.clear();
     plan.rt_ent.clear();
     plan.alt_kmax = 0;
+    plan.quad_col.clear();
+    plan.quad_w.clear();
+    plan.quad_groups = 0;
     if (band && halo == 32 && uniform && exact) {
         // the BLOCK form of a run-chain layer, its columns in the band's input labelling
         plan.alt_ngroups = (int)groups.size();
@@ -812,6 +870,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.pair_twins = twins;
         plan.ell_col.clear();
         plan.rowlen.clear();
+        if (N <= kQuadMaxNeurons) build_quad_form(N, rowptr, col, val, plan);
     } else if (force_kernel != SPDNN_KERNEL_GATHER && !(getenv("SPDNN_TILED") && atoi(getenv("SPDNN_TILED")) == 0) &&
                build_tiled_plan(N, rowptr, col, val, plan)) {
         plan.kernel = SPDNN_KERNEL_TILED;
@@ -876,7 +935,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
     plan.info.block_form = plan.alt_ngroups > 0 ? 1 : (plan.alt_kmax > 0 ? 2 : 0);
     plan.info.plan_bytes = (int64_t)(4 * (plan.ell_col.size() + plan.rowlen.size() + plan.wv.size() +
                                                               plan.blk_cols.size() + plan.blk_cnt.size() + plan.pairs.size() +
-                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() + plan.alt_wv.size() + plan.rt_ent.size() +
+                                                              plan.alt_cols.size() + plan.alt_cnt.size() + plan.alt_out_at.size() + plan.alt_wv.size() + plan.rt_ent.size() + plan.quad_col.size() + plan.quad_w.size() +
                                                               plan.out_at.size() + (size_t)N));
     plan.dst.clear();
     plan.failed = false;

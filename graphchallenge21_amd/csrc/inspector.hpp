@@ -16,6 +16,8 @@ namespace spdnn {
 
 constexpr int kTileOutputs = 1024;  // TILED: outputs per tile (16 waves x 64)
 constexpr int kPanelCols = 512;     // TILED: input columns staged in LDS at a time
+constexpr int kQuadMaxNeurons = 1024;  // BAND: widest layer that carries its QUAD form (two buffers of N x 16 rows in LDS)
+constexpr int kQuadColumnBytes = 64;   // ... whose columns are 16 rows of 4 bytes: the form holds byte offsets
 
 struct LayerPlan {
     bool set = false;
@@ -65,6 +67,15 @@ struct LayerPlan {
     // wave have about the same number of entries): rt_ent [alt_kmax rounded up to 4][N][2] = (input column, weight bits)
     // of the slot's k-th entry, zeros behind a list, entry-major so that the lanes of a wave read neighbouring words.
     std::vector<uint32_t> rt_ent;
+    // A BAND layer of up to 1024 neurons also carries its QUAD form, for launches that keep 16 rows of a workgroup in
+    // LDS through the layers: the four outputs at band positions 4c .. 4c+3 add their inputs in ascending input index,
+    // so their lists merge into one list of steps (K + 3 for a circulant band), padded to quad_groups groups of four.
+    // quad_col [N/4][quad_groups][4] = input column of each step, as the byte offset of the column in a buffer of 16 rows per
+    // column; quad_w [N/4][quad_groups][4 outputs][4 steps] = the
+    // weight of the step in each output, 0 where the output does not use it (padding steps repeat the last column).
+    std::vector<uint32_t> quad_col;
+    std::vector<float> quad_w;
+    int quad_groups = 0;
     // BAND: neuron j sits at the same band position as an input and as an output (see
     // canonicalize_self_aligned_band); fuse_next: this layer writes its outputs exactly where the
     // next layer's band reads them (dst = identity) and both fit the fused pair kernel

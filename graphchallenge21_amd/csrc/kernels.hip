@@ -1838,6 +1838,11 @@ struct ResidentArgs {
     int stamp0, prev_stamp, check_dead;
     float bias, clampv;
     Publish pub;
+    // QUAD form: the arrays of the launch's first layer; those of layer j lie j * quad_stride bytes further on
+    const uint32_t* quad_col;
+    const float* quad_w;
+    const int32_t* quad_dst;
+    long long quad_stride;
 };
 
 // the value register k / R of the lane with row index k % R of this lane's group holds (k a constant after unrolling)
@@ -2125,6 +2130,207 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
     float* __restrict__ gout = ((rb & 1) ? o_h1 : o_h0) + (size_t)(rb >> 1) * blkf + rin;
     const unsigned char* const fin = smem + ((done_layers & 1) ? buf_bytes : 0u);
     for (int idx = t; idx < total; idx += 1024) {
+        const int col = idx / PARTS, part = idx - col * PARTS;
+        float4 v;
+        if (all_dead) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        else v = *reinterpret_cast<const float4*>(fin + (size_t)idx * 16);
+        *reinterpret_cast<float4*>(gout + (size_t)col * RB + part * 4) = v;
+    }
+    if (t < R && last_alive >= 0) a.active[row0 + t] = a.stamp0 + last_alive;
+}
+
+// The resident launch of BAND layers in their QUAD form (up to 1024 neurons, any weights): the frame of the two kernels
+// above - 16 rows of a workgroup in LDS through all layers of the launch, two buffers laid out [column][row], one barrier per
+// layer, rows stamped with the last layer that left them nonzero, a workgroup whose rows are all zero stops - around an
+// arithmetic that shares LDS reads between neighbouring outputs of the band.  The workgroup has N threads; thread t
+// belongs to quad t / 4 (band positions 4c .. 4c+3) and computes those four outputs for rows 4 (t % 4) .. + 3.  The four
+// outputs add their inputs in ascending input index, so their lists are one merged list of steps (K + 3 for a
+// circulant band of K entries): per step ONE 16-byte LDS read - the column's four rows - feeds 16 multiply-adds, a
+// step an output does not use entering it with weight 0 (an exact zero added).  The plan stream of a quad - per group
+// of four steps the four columns (as byte offsets) and 4 x 4 weights - is spread over the quad's four lanes (lane k holds
+// the column of step k and the four weights of output k) and handed round by DPP quad permutations inside the address
+// add and the multiply-adds that use them; the groups are requested two ahead of the arithmetic, the first two of the
+// next layer before this layer's barrier.
+template <int K> __device__ __forceinline__ uint32_t quad_lane(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, K * 0x55, 0xf, 0xf, true);
+}
+// One step of a quad: acc[o][q] += x[q] * (the weight held by lane o of this lane's quad), o, q = 0..3.  The weights
+// are brought over by four DPP moves and the sixteen multiply-adds take register operands only: such a v_fmac_f32
+// issues at twice the rate of one with a DPP or a scalar operand (measured: 0.95 against 1.75 ns per wave instruction
+// and SIMD), so the moves cost less than they save.  Ends with a barrier to the compiler's reordering of memory
+// accesses: the LDS reads of later steps are issued before the step's arithmetic and stay there.
+template <int WMODE> __device__ __forceinline__ void quad_step(float (&acc)[4][4], const float4& x, float w) {
+    const uint32_t wb = __float_as_uint(w);
+    const float wo[4] = {__uint_as_float(quad_lane<0>(wb)), __uint_as_float(quad_lane<1>(wb)), __uint_as_float(quad_lane<2>(wb)),
+                         __uint_as_float(quad_lane<3>(wb))};
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+        acc[o][0] = mac<WMODE>(acc[o][0], x.x, wo[o]);
+        acc[o][1] = mac<WMODE>(acc[o][1], x.y, wo[o]);
+        acc[o][2] = mac<WMODE>(acc[o][2], x.z, wo[o]);
+        acc[o][3] = mac<WMODE>(acc[o][3], x.w, wo[o]);
+    }
+#pragma unroll
+    for (int o = 0; o < 4; ++o)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) asm volatile("" : "+v"(acc[o][q]) : : "memory");
+}
+// the value lane k of this lane's quad holds (k a constant after unrolling)
+__device__ __forceinline__ uint32_t quad_lane_of(uint32_t v, int k) {
+    switch (k & 3) {
+        case 0: return quad_lane<0>(v);
+        case 1: return quad_lane<1>(v);
+        case 2: return quad_lane<2>(v);
+        default: return quad_lane<3>(v);
+    }
+}
+template <int NG, int WMODE>   // NG: groups of four steps per quad (9: bands of 32 entries), 0: as the launch says
+__global__ __launch_bounds__(1024) void band_resident_kernel(ResidentArgs a) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int sh_alive[3];
+    __shared__ int sh_last[16];
+    constexpr int R = 16, PARTS = 4;
+    using GU = const __attribute__((address_space(1))) uint32_t*;
+    using GW = const __attribute__((address_space(1))) f32x4_t*;
+    using GI = const __attribute__((address_space(1))) int32_t*;
+    publish_counts(a.pub);
+    const int t = (int)threadIdx.x, lane = t & 63, nthr = a.N;   // (launched with N threads)
+    const int RB = 64 * a.rl;
+    const unsigned nwg = gridDim.x;
+    const unsigned wg = (nwg % 8u) == 0u ? (blockIdx.x % 8u) * (nwg / 8u) + blockIdx.x / 8u : blockIdx.x;
+    const size_t row0 = (size_t)wg * R;
+    const int rb = (int)(row0 / (size_t)RB), rin = (int)(row0 - (size_t)rb * RB);
+    if (a.check_dead && a.prev_stamp != 0) {   // a row block without an active row is skipped, as by the per-layer kernels
+        int alive = 0;
+        for (int i = t; i < RB; i += nthr) alive |= (a.active[(size_t)rb * RB + i] == a.prev_stamp) ? 1 : 0;
+        if (__syncthreads_or(alive) == 0) return;
+    }
+    const size_t blkf = (size_t)a.N * RB;
+    const uint32_t buf_bytes = (uint32_t)a.N * R * 4;
+    const int total = a.N * PARTS;
+    {
+        const float* __restrict__ gin = ((rb & 1) ? a.first_in.half[1] : a.first_in.half[0]) + (size_t)(rb >> 1) * blkf + rin;
+        // N * 4 pieces (a column's rows in four parts) over N threads: four loads each, all in flight together
+        float4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int idx = t + u * nthr;
+            const int col = idx / PARTS, part = idx - col * PARTS;
+            v[u] = *reinterpret_cast<const float4*>(gin + (size_t)col * RB + part * 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) *reinterpret_cast<float4*>(smem + (size_t)(t + u * nthr) * 16) = v[u];
+    }
+    if (t < 3) sh_alive[t] = 0;
+    if (t < R) sh_last[t] = -1;
+    const int rq = t & 3;
+    const uint32_t lane_off = (uint32_t)rq * 16u;
+    const int ng = NG ? NG : a.ngroups;
+    // this lane's place in a quad's plan stream: group gi lies 4 lanes further on
+    const size_t qoff = (size_t)(t >> 2) * (size_t)ng * 4 + (size_t)rq;
+    uint32_t c_first[2], d_first;
+    f32x4_t w_first[2];
+    // (no layer table here: a table entry read at the top of a layer - a scalar load, then the loads that need its
+    // pointers - would be waited for by every wave of the workgroup at once, right behind the barrier: 2.8 us of a 7 us layer)
+    using GB = const __attribute__((address_space(1))) unsigned char*;
+    const GB col_base = (GB)a.quad_col + qoff * 4, w_base = (GB)a.quad_w + qoff * 16, dst_base = (GB)a.quad_dst + (size_t)t * 4;
+    auto request_first = [&](int j) {
+        const GU colp = (GU)(col_base + (long long)j * a.quad_stride);
+        const GW wp = (GW)(w_base + (long long)j * a.quad_stride);
+        c_first[0] = colp[0];
+        w_first[0] = wp[0];
+        c_first[1] = colp[ng > 1 ? 4 : 0];
+        w_first[1] = wp[ng > 1 ? 4 : 0];
+        d_first = (uint32_t)(*(GI)(dst_base + (long long)j * a.quad_stride));   // (used as it comes: arithmetic on it here would wait for the load)
+    };
+    request_first(0);
+    int last_nz[4] = {-1, -1, -1, -1};
+    bool all_dead = false;
+    int done_layers = 0;
+    __syncthreads();
+    for (int j = 0; j < a.nlayers; ++j) {
+        const unsigned char* const in = smem + ((j & 1) ? buf_bytes : 0u);
+        unsigned char* const out = smem + ((j & 1) ? 0u : buf_bytes);
+        const GU colp = (GU)(col_base + (long long)j * a.quad_stride);
+        const GW wp = (GW)(w_base + (long long)j * a.quad_stride);
+        uint32_t cr[3];
+        f32x4_t wr[3];
+        cr[0] = c_first[0]; cr[1] = c_first[1];
+        wr[0] = w_first[0]; wr[1] = w_first[1];
+        const uint32_t dcol = d_first * (uint32_t)(R * 4);
+        if (j + 1 < a.nlayers) request_first(j + 1);   // in flight under this layer's arithmetic
+        float acc[4][4];
+#pragma unroll
+        for (int o = 0; o < 4; ++o)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[o][q] = 0.0f;
+        // step e = 4 gi + k: the LDS read of step e + 3 is issued before the arithmetic of step e (the waves of a workgroup
+        // leave the barrier together: a wave that waited for each read right after issuing it would wait when all others do)
+        const int nsteps = 4 * ng;
+        float4 xb[4];
+        xb[0] = *reinterpret_cast<const float4*>(in + (quad_lane<0>(cr[0]) + lane_off));
+        xb[1] = *reinterpret_cast<const float4*>(in + (quad_lane<1>(cr[0]) + lane_off));
+        xb[2] = *reinterpret_cast<const float4*>(in + (quad_lane<2>(cr[0]) + lane_off));
+#pragma unroll
+        for (int e = 0; e < 36; ++e) {
+            if (e < nsteps) {
+                const int gi = e >> 2;
+                if ((e & 3) == 0 && e + 8 < 36 && e + 8 < nsteps) {   // the plan stream: two groups ahead
+                    cr[(gi + 2) % 3] = colp[(gi + 2) * 4];
+                    wr[(gi + 2) % 3] = wp[(gi + 2) * 4];
+                }
+                if (e + 3 < 36 && e + 3 < nsteps)
+                    xb[(e + 3) % 4] = *reinterpret_cast<const float4*>(in + (quad_lane_of(cr[((e + 3) >> 2) % 3], e + 3) + lane_off));
+                const f32x4_t wg4 = wr[gi % 3];
+                const float wk = (e & 3) == 0 ? wg4.x : (e & 3) == 1 ? wg4.y : (e & 3) == 2 ? wg4.z : wg4.w;
+                quad_step<WMODE>(acc, xb[e % 4], wk);
+            }
+        }
+        // (outputs are clamped to [0, clamp]: the largest of a row's four is positive exactly when one of them is nonzero)
+        float y[4][4];
+#pragma unroll
+        for (int o = 0; o < 4; ++o) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) y[o][q] = relu_clamp(acc[o][q] + a.bias, a.clampv);
+        }
+        *reinterpret_cast<float4*>(out + (quad_lane<0>(dcol) + lane_off)) = float4{y[0][0], y[0][1], y[0][2], y[0][3]};
+        *reinterpret_cast<float4*>(out + (quad_lane<1>(dcol) + lane_off)) = float4{y[1][0], y[1][1], y[1][2], y[1][3]};
+        *reinterpret_cast<float4*>(out + (quad_lane<2>(dcol) + lane_off)) = float4{y[2][0], y[2][1], y[2][2], y[2][3]};
+        *reinterpret_cast<float4*>(out + (quad_lane<3>(dcol) + lane_off)) = float4{y[3][0], y[3][1], y[3][2], y[3][3]};
+        float top = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float m = __builtin_fmaxf(__builtin_fmaxf(__builtin_fmaxf(y[0][q], y[1][q]), y[2][q]), y[3][q]);
+            if (m > 0.0f) last_nz[q] = j;   // this lane's outputs left row 4 rq + q nonzero
+            top = __builtin_fmaxf(top, m);
+        }
+        // the workgroup goes on while one of its rows is nonzero: a flag per layer, the rows' own last layers are put
+        // together once, behind the loop
+        if (__ballot(top > 0.0f ? 1 : 0) != 0ull && lane == 0) sh_alive[j % 3] = 1;
+        __syncthreads();
+        const int some = sh_alive[j % 3];
+        if (t == 0) sh_alive[(j + 2) % 3] = 0;
+        done_layers = j + 1;
+        if (some == 0 && a.bias <= 0.0f) { all_dead = true; break; }   // zero rows stay zero
+    }
+    // the last layer that left each of the 16 rows nonzero: the largest over the lanes that hold the row's outputs
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        int v = last_nz[q];
+#pragma unroll
+        for (int sft = 4; sft < 64; sft <<= 1) v = max(v, __shfl_xor(v, sft, 64));
+        if (lane < 4 && v >= 0) atomicMax(&sh_last[lane * 4 + q], v);
+    }
+    __syncthreads();
+    const int last_alive = t < R ? sh_last[t] : -1;
+    // the launch's last layer writes the work buffer the layer before it did not (layer 0: the one it did not read)
+    const bool in_a = a.first_in.half[0] == a.buf_a.half[0];
+    const bool to_c = in_a == ((a.nlayers & 1) != 0);
+    float* const o_h0 = to_c ? a.buf_c.half[0] : a.buf_a.half[0];
+    float* const o_h1 = to_c ? a.buf_c.half[1] : a.buf_a.half[1];
+    float* __restrict__ gout = ((rb & 1) ? o_h1 : o_h0) + (size_t)(rb >> 1) * blkf + rin;
+    const unsigned char* const fin = smem + ((done_layers & 1) ? buf_bytes : 0u);
+    for (int idx = t; idx < total; idx += nthr) {
         const int col = idx / PARTS, part = idx - col * PARTS;
         float4 v;
         if (all_dead) v = float4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -2761,6 +2967,40 @@ hipError_t launch_rowtile_resident(const ResidentLaunch& a, int wmode, hipStream
         case 8: return launch_rowtile_resident_r<8>(a, wmode, s);
         default: return launch_rowtile_resident_r<4>(a, wmode, s);
     }
+}
+
+int band_resident_rows(int N) {
+    // N threads (a quad of band positions x four of the 16 rows each), two buffers of N x 16 floats
+    return (N >= 256 && N <= 1024 && (N % 256) == 0) ? 16 : 0;
+}
+
+hipError_t launch_band_resident(const ResidentLaunch& a, int wmode, hipStream_t s) {
+    // host-side shape checks: what the kernel's two LDS buffers, its thread numbering and its plan stream assume
+    if (a.nlayers < 1 || !a.quad_col || !a.quad_w || !a.quad_dst || (a.quad_stride % 16) != 0 || !a.first_in || !a.buf_a || !a.buf_c ||
+        a.buf_a == a.buf_c || !a.active || a.rows <= 0 || (a.rl != 1 && a.rl != 2 && a.rl != 4) || (a.rows % (64 * a.rl)) != 0 ||
+        band_resident_rows(a.N) != 16 || a.ngroups < 1 || a.ngroups > 9)
+        return hipErrorInvalidValue;
+    ResidentArgs k{};
+    k.table = a.table; k.nlayers = a.nlayers; k.first_in = a.first_in; k.buf_a = a.buf_a; k.buf_c = a.buf_c; k.active = a.active;
+    k.N = a.N; k.ngroups = a.ngroups; k.rl = a.rl; k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
+    k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
+    k.quad_col = a.quad_col; k.quad_w = a.quad_w; k.quad_dst = a.quad_dst; k.quad_stride = a.quad_stride;
+    const size_t lds = (size_t)a.N * 16 * 8;
+    dim3 grid((unsigned)(a.rows / 16)), block((unsigned)a.N);
+#define SPDNN_BAND_RESIDENT(NG, WM)                                                                                         \
+    do {                                                                                                                    \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(band_resident_kernel<NG, WM>),     \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);        \
+        if (attr != hipSuccess) return attr;                                                                                \
+        hipLaunchKernelGGL((band_resident_kernel<NG, WM>), grid, block, lds, s, k);                                         \
+    } while (0)
+    if (wmode != 2) {
+        if (a.ngroups == 9) SPDNN_BAND_RESIDENT(9, 1); else SPDNN_BAND_RESIDENT(0, 1);
+    } else {
+        if (a.ngroups == 9) SPDNN_BAND_RESIDENT(9, 2); else SPDNN_BAND_RESIDENT(0, 2);
+    }
+#undef SPDNN_BAND_RESIDENT
+    return hipGetLastError();
 }
 
 hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,

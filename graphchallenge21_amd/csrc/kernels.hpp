@@ -189,7 +189,10 @@ struct LayerDesc {           // one entry of the device-side layer table
     const int32_t* rt_len;
     const int32_t* rt_dst;
     int rt_kpad;
-    int pad_;
+    // QUAD form (BAND layers up to 1024 neurons wide)
+    int quad_groups;
+    const uint32_t* quad_col;
+    const float* quad_w;
 };
 
 struct PersistCtl {          // device words of one persistent launch (zero before the launch)
@@ -245,6 +248,13 @@ struct ResidentLaunch {
     int stamp0, prev_stamp, check_dead;
     float bias, clampv;
     Publish publish;
+    // launch_band_resident only: the QUAD form of the launch's first layer (its steps' columns, their weights, the band's
+    // dst); the arrays of layer j lie j * quad_stride bytes further on (the plans of consecutive layers of one structure
+    // are laid out at equal distances).  It reads no layer table.
+    const uint32_t* quad_col;
+    const float* quad_w;
+    const int32_t* quad_dst;
+    long long quad_stride;
 };
 // The same for TILED layers in their ROWTILE form (any sparsity pattern): `nlayers` consecutive such layers of one
 // weight mode, the R rows of a workgroup in LDS from the first layer to the last, every thread computing whole outputs
@@ -252,6 +262,13 @@ struct ResidentLaunch {
 hipError_t launch_rowtile_resident(const ResidentLaunch& a, int wmode, hipStream_t s);
 // rows such a workgroup keeps (16, 8 or 4 for up to 1024, 2048, 4096 neurons: two buffers of N x R floats), 0 = too wide
 int rowtile_resident_rows(int N);
+
+// The same for BAND layers in their QUAD form (up to 1024 neurons, any weights): 16 rows of a workgroup in LDS, a
+// thread computes the four outputs of a quad of band positions for four of the rows (band_resident_kernel).  ngroups:
+// groups of four steps per quad, the same for every layer of the launch; full is not used.
+hipError_t launch_band_resident(const ResidentLaunch& a, int wmode, hipStream_t s);
+// rows such a workgroup keeps (16), 0 = the shape does not fit
+int band_resident_rows(int N);
 
 // rows a workgroup keeps (16 or 4), 0 if the shape does not fit: two buffers of (N + 1) x R floats in LDS
 // (N <= 1024: 16 rows, N <= 4096: 4) and one (group, row) item per thread of 1024

@@ -183,12 +183,14 @@ struct DevLayer {
     int32_t* alt_dst = nullptr;
     float* alt_wv = nullptr;       // (with alt_cols / alt_cnt / alt_dst: the GATHER form of a TILED layer)
     uint32_t* rt_ent = nullptr;    // (with alt_cnt / alt_dst: its ROWTILE form)
+    uint32_t* quad_col = nullptr;  // the QUAD form of a BAND layer (with dst)
+    float* quad_w = nullptr;
 };
 
 // Where the arrays of one layer's plan lie inside its block of device memory (and inside the
 // pinned host copy of that block when plans are streamed): pairs, ell, rowlen, wv, dst, blk_cols,
-// blk_cnt, alt_cols, alt_cnt, alt_dst, alt_wv, rt_ent, each aligned to 256 bytes.
-constexpr int kPlanArrays = 12;
+// blk_cnt, alt_cols, alt_cnt, alt_dst, alt_wv, rt_ent, quad_col, quad_w, each aligned to 256 bytes.
+constexpr int kPlanArrays = 14;
 struct PlanLayout {
     size_t off[kPlanArrays] = {};
     size_t len[kPlanArrays] = {};
@@ -299,6 +301,8 @@ struct spdnn_net {
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     int64_t tiled_min_rows = 8192;                    // see use_gather_form (SPDNN_TILED_MIN_ROWS)
     int rowtile_mode = 1;                             // TILED layers up to 8192 neurons wide run their ROWTILE form (SPDNN_ROWTILE=0: the tiles)
+    int band_resident_mode = 1;                       // BAND layers up to 1024 neurons wide join resident launches (SPDNN_BAND_RESIDENT=0: never)
+    int band_resident_min_layers = 0;                 // ... of at least this many layers (SPDNN_BAND_RESIDENT_MIN_LAYERS; 0: 6, from 16384 rows up 16)
     long long stream_min_bytes = 96ll << 20;          // see BandLaunch (SPDNN_STREAM_MIN_BYTES, read at creation)
     long long count_timeout_ms = 60000;               // longest wait for one layer's counts (SPDNN_COUNT_TIMEOUT_MS)
     LayerDesc* d_table = nullptr;   // one entry per layer (resident plans only)
@@ -576,7 +580,7 @@ PlanLayout plan_layout(const LayerPlan& p) {
     const size_t len[kPlanArrays] = {p.pairs.size() * 4,    p.ell_col.size() * 4,  p.rowlen.size() * 4,   p.wv.size() * 4,
                                      p.dst.size() * 4,      p.blk_cols.size() * 4, p.blk_cnt.size() * 4,  p.alt_cols.size() * 4,
                                      p.alt_cnt.size() * 4,  p.alt_dst.size() * 4,  p.alt_wv.size() * 4,
-                                     p.rt_ent.size() * 4};
+                                     p.rt_ent.size() * 4,   p.quad_col.size() * 4, p.quad_w.size() * 4};
     for (int k = 0; k < kPlanArrays; ++k) {
         y.off[k] = y.bytes;
         y.len[k] = len[k];
@@ -588,7 +592,7 @@ PlanLayout plan_layout(const LayerPlan& p) {
 void pack_plan(const LayerPlan& p, const PlanLayout& y, char* dst) {
     const void* src[kPlanArrays] = {p.pairs.data(),   p.ell_col.data(),  p.rowlen.data(),  p.wv.data(),      p.dst.data(),
                                     p.blk_cols.data(), p.blk_cnt.data(), p.alt_cols.data(), p.alt_cnt.data(), p.alt_dst.data(),
-                                    p.alt_wv.data(),   p.rt_ent.data()};
+                                    p.alt_wv.data(),   p.rt_ent.data(),   p.quad_col.data(), p.quad_w.data()};
     for (int k = 0; k < kPlanArrays; ++k)
         if (y.len[k]) memcpy(dst + y.off[k], src[k], y.len[k]);
 }
@@ -608,6 +612,8 @@ DevLayer plan_at(const PlanLayout& y, char* base) {
     d.alt_dst = (int32_t*)at(9);
     d.alt_wv = (float*)at(10);
     d.rt_ent = (uint32_t*)at(11);
+    d.quad_col = (uint32_t*)at(12);
+    d.quad_w = (float*)at(13);
     return d;
 }
 
@@ -645,6 +651,9 @@ int upload_plans(spdnn_net* n) {
                 t.dst = n->dl[l].dst;
                 t.steps = p.pair_steps;
                 t.halo = p.info.band_halo;
+                t.quad_groups = p.quad_groups;   // its QUAD form
+                t.quad_col = n->dl[l].quad_col;
+                t.quad_w = n->dl[l].quad_w;
                 if (p.alt_ngroups > 0) {   // its BLOCK form
                     t.ngroups = p.alt_ngroups;
                     t.blk_cols = n->dl[l].alt_cols;
@@ -916,6 +925,8 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
     if (const char* e = getenv("SPDNN_TILED_MIN_ROWS")) n->tiled_min_rows = atoll(e);
     if (const char* e = getenv("SPDNN_ROWTILE")) n->rowtile_mode = atoi(e) != 0 ? 1 : 0;
+    if (const char* e = getenv("SPDNN_BAND_RESIDENT")) n->band_resident_mode = atoi(e) != 0 ? 1 : 0;
+    if (const char* e = getenv("SPDNN_BAND_RESIDENT_MIN_LAYERS")) n->band_resident_min_layers = std::max(0, atoi(e));
     if (const char* e = getenv("SPDNN_STREAM_MIN_BYTES")) n->stream_min_bytes = atoll(e);
     if (const char* e = getenv("SPDNN_COUNT_TIMEOUT_MS")) n->count_timeout_ms = std::max(1ll, atoll(e));
     if (const char* e = getenv("SPDNN_PLAN_WINDOW")) {
@@ -1635,7 +1646,7 @@ static LayerSig layer_sig(const spdnn_net* n, int l, int nblk) {
 // BLOCK form with one exact weight - a BLOCK layer of weight mode 0, or a run-chain BAND layer that carries its
 // BLOCK form - or the ROWTILE form of a TILED layer; and a shape the kernel's LDS buffers and numbering hold.
 struct ResidentSig {
-    int ok = 0;      // 0 no resident form; 1 BLOCK form of one exact weight; 2 ROWTILE form (TILED layers)
+    int ok = 0;      // 0 no resident form; 1 BLOCK form of one exact weight; 2 ROWTILE form (TILED layers); 3 QUAD form (BAND layers)
     int full = 0, ngroups = 0, wmode = 0;
     int rows = 0;    // rows a workgroup keeps
     bool operator==(const ResidentSig& o) const { return ok == o.ok && full == o.full && ngroups == o.ngroups && wmode == o.wmode; }
@@ -1646,11 +1657,25 @@ static ResidentSig resident_sig(const spdnn_net* n, int l) {
     if (p.kernel == SPDNN_KERNEL_BAND && p.alt_ngroups > 0) { g.ok = 1; g.full = p.alt_full ? 1 : 0; g.ngroups = p.alt_ngroups; }
     else if (p.kernel == SPDNN_KERNEL_BLOCK && p.wmode == 0) { g.ok = 1; g.full = p.blk_full ? 1 : 0; g.ngroups = p.ngroups; }
     else if (p.kernel == SPDNN_KERNEL_TILED && !p.rt_ent.empty() && n->rowtile_mode) { g.ok = 2; g.wmode = p.wmode; }
+    else if (p.kernel == SPDNN_KERNEL_BAND && p.quad_groups > 0 && n->band_resident_mode) { g.ok = 3; g.ngroups = p.quad_groups; g.wmode = p.wmode == 2 ? 2 : 1; }
     if (g.ok) {
-        g.rows = g.ok == 1 ? resident_rows_per_workgroup(n->N, g.ngroups) : rowtile_resident_rows(n->N);
+        g.rows = g.ok == 1 ? resident_rows_per_workgroup(n->N, g.ngroups) : g.ok == 2 ? rowtile_resident_rows(n->N) : band_resident_rows(n->N);
         if (g.rows == 0 || n->RB % g.rows != 0) g.ok = 0;
     }
     return g;
+}
+
+// The band resident kernel finds the QUAD form of its j-th layer j strides behind that of its first: whether layer k's
+// arrays lie where that rule, set by layers l0 and l0 + 1, puts them.
+static bool quad_plans_equidistant(const spdnn_net* n, int l0, int k) {
+    const DevLayer& a = n->dl[(size_t)l0];
+    const DevLayer& b = n->dl[(size_t)l0 + 1];
+    const DevLayer& c = n->dl[(size_t)k];
+    const long long stride = (const char*)b.quad_col - (const char*)a.quad_col;
+    const long long j = k - l0;
+    return (stride % 16) == 0 && (const char*)b.quad_w - (const char*)a.quad_w == stride && (const char*)b.dst - (const char*)a.dst == stride &&
+           (const char*)c.quad_col - (const char*)a.quad_col == j * stride && (const char*)c.quad_w - (const char*)a.quad_w == j * stride &&
+           (const char*)c.dst - (const char*)a.dst == j * stride;
 }
 
 static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_run_result* res) {
@@ -1860,17 +1885,23 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
             ResidentSig rsig;
             int cmax = std::min(persist_cmax, last - l + 1);
             if (opt.prune && !persist_asked) cmax = std::min(cmax, st.c_prune);   // short launches while the counts still move
+            // (with at most 16 rows known alive - the rows of one workgroup of a resident launch - the run is about to end:
+            // layer by layer, so that the host sees the end when it comes instead of queueing launches of many layers)
+            if (opt.prune && !persist_asked && st.newest_count >= 0 && st.newest_count <= 16) cmax = 1;
             if (!fb && persist_on && n->resident_mode && n->d_table && (rsig = resident_sig(n, l)).ok) {
                 // Bringing the rows in and out costs such a launch as much as two layers save it with 16 rows per workgroup
                 // (64-byte pieces of a column) and as much as eight save it with 4 rows (16-byte pieces): measured
                 // at 2048 and at 60000 rows.  So left to the library: from 2 layers (even while the counts still move -
                 // workgroups whose rows have all died leave early) and from 8; a caller that asks for launches of a
                 // given length gets them.
-                const bool wide_rows = rsig.rows >= 16;
-                const int rmin = (persist_asked || wide_rows) ? 2 : 8;
+                const bool wide_rows = rsig.rows >= 16 && rsig.ok != 3;
+                // (band quads: a layer inside the launch takes 0.88 of its time alone at 60000 rows, 0.76 at 6000, and rows in
+                // and out cost the launch what 1.5 layers take at either size: worth it from 16 and from 6 layers)
+                const int band_rmin = n->band_resident_min_layers >= 2 ? n->band_resident_min_layers : (n->carried >= 16384 ? 16 : 6);
+                const int rmin = (persist_asked || wide_rows) ? 2 : rsig.ok == 3 ? band_rmin : 8;
                 const int rmax = std::min(wide_rows ? std::max(cmax, 2) : cmax, last - l + 1);
                 int k = 1;
-                while (k < rmax && resident_sig(n, l + k) == rsig) ++k;
+                while (k < rmax && resident_sig(n, l + k) == rsig && (rsig.ok != 3 || quad_plans_equidistant(n, l, l + k))) ++k;
                 // (entry lists for 8 or 4 rows at a time: on large launches the per-layer kernel, which reads them for 16, is the
                 // faster one - measured per layer at batch 60000: N=2048 376 against 337 us, N=4096 1232 against 948; at 2048
                 // rows 13 against 38 and 42 against 57)
@@ -1981,10 +2012,16 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 rl.N = n->N; rl.ngroups = rsig.ngroups; rl.rows = n->carried; rl.rl = n->rl; rl.full = rsig.full;
                 rl.stamp0 = stamp0; rl.prev_stamp = prev_stamp; rl.check_dead = check_dead; rl.bias = n->bias; rl.clampv = n->clampv;
                 rl.publish = st.pub;
-                HIPCHK(rsig.ok == 1 ? launch_block_resident(rl, n->stream) : launch_rowtile_resident(rl, rsig.wmode, n->stream));
+                if (rsig.ok == 3) {
+                    const DevLayer& d0 = n->dl[(size_t)l];
+                    rl.quad_col = d0.quad_col; rl.quad_w = d0.quad_w; rl.quad_dst = d0.dst;
+                    rl.quad_stride = c > 1 ? (long long)((const char*)n->dl[(size_t)l + 1].quad_col - (const char*)d0.quad_col) : 0;
+                }
+                HIPCHK(rsig.ok == 1 ? launch_block_resident(rl, n->stream)
+                       : rsig.ok == 2 ? launch_rowtile_resident(rl, rsig.wmode, n->stream) : launch_band_resident(rl, rsig.wmode, n->stream));
                 if (n->run_verbose)
                     fprintf(stderr, "spdnn: resident launch (%s): layers %d..%d, %d rows, %d rows per workgroup\n",
-                            rsig.ok == 1 ? "groups" : "entry lists", l, l + c - 1, n->carried, rsig.rows);
+                            rsig.ok == 1 ? "groups" : rsig.ok == 2 ? "entry lists" : "band quads", l, l + c - 1, n->carried, rsig.rows);
                 for (int j = 1; j < c; ++j) out = (out == n->A) ? n->C : n->A;  // where the last layer wrote
                 st.r.resident_launches += 1;
             } else if (fb) {

@@ -472,6 +472,7 @@ def test_persistent_launches(gc, orc, fuse, prune, mode, monkeypatch):
     with device-scope fences or the hand-over inside one XCD's L2."""
     for k, v in PERSIST_MODES[mode].items():
         monkeypatch.setenv(k, v)
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", "0")   # (layers this narrow would share resident launches instead)
     N, L, B = 1024, 24, 3000
     print("persistent launches fuse=%d prune=%s %s" % (fuse, prune, mode), flush=True)
     layers = [orc.gen_layer_csr(5, l, N) for l in range(L)]
@@ -503,14 +504,18 @@ def test_persistent_launches(gc, orc, fuse, prune, mode, monkeypatch):
         assert same_floats(net.activations(cats), ref["y"])
 
 
-@pytest.mark.parametrize("N,L,bias", [(1024, 120, -0.3), (4096, 40, -0.35)])
-def test_persistent_by_default_at_full_batch(gc, orc, N, L, bias):
-    """Batch 60000: left to the library (fuse_layers = 0) the layers of these widths share persistent launches (one unit
-    queue per XCD, the hand-over between layers inside the XCD's L2).  Every activation of every row after the last
-    layer, the per-layer counts and the categories must equal those of one launch per layer bit for bit, on live data
-    (rows that survive every layer), pruned and unpruned; an oracle row sample pins both."""
+@pytest.mark.parametrize("N,L,bias,band_resident", [(1024, 120, -0.3, 1), (1024, 120, -0.3, 0), (4096, 40, -0.35, 1)])
+def test_several_layers_per_launch_by_default_at_full_batch(gc, orc, monkeypatch, N, L, bias, band_resident):
+    """Batch 60000: left to the library (fuse_layers = 0) the band layers of these widths share launches - resident
+    ones up to 1024 neurons (16 rows of a workgroup in LDS through the layers), persistent ones above or when the
+    resident form is switched off (one unit queue per XCD, the hand-over between layers inside the XCD's L2).  Every
+    activation of every row after the last layer, the per-layer counts and the categories must equal those of one
+    launch per layer bit for bit, on live data (rows that survive every layer), pruned and unpruned; an oracle row
+    sample pins both."""
     B, S = 60000, 256
-    print("persistent by default N=%d L=%d" % (N, L), flush=True)
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", str(band_resident))
+    resident = band_resident and N <= 1024
+    print("several layers per launch by default N=%d L=%d resident=%d" % (N, L, resident), flush=True)
     layers = [orc.gen_layer_csr(0, l, N) for l in range(L)]
     ref = orc.infer(orc.gen_features(0, N, 0, S, 0.10, 0.70), layers, bias, prune=False, keep={L - 1})
     rows = np.arange(B, dtype=np.int32)
@@ -529,7 +534,8 @@ def test_persistent_by_default_at_full_batch(gc, orc, N, L, bias):
         assert same_floats(want[0][:S], ref["kept"][L - 1][1])
         for attempt in range(3):
             r = net.run(prune=False, collect_counts=True)
-            assert r.persistent_launches >= 1 and r.persistent_fallbacks == 0 and r.launches < L
+            assert (r.resident_launches if resident else r.persistent_launches) >= 1 and r.persistent_fallbacks == 0 and r.launches < L
+            assert (r.persistent_launches if resident else r.resident_launches) == 0
             got = state()
             assert np.array_equal(got[0], want[0]) and got[1] == want[1] and np.array_equal(got[2], want[2]), attempt
         r = net.run(prune=True, collect_counts=True)
@@ -545,6 +551,7 @@ def test_persistent_launch_that_gives_up(gc, orc, prune, mode, monkeypatch):
     far each row block got and finishes the layers with per-layer launches.  Results must not change."""
     for k, v in PERSIST_MODES[mode].items():
         monkeypatch.setenv(k, v)
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", "0")
     N, L, B = 1024, 20, 2600
     print("persistent launch gives up prune=%s %s" % (prune, mode), flush=True)
     layers = [orc.gen_layer_csr(6, l, N) for l in range(L)]
@@ -673,6 +680,64 @@ def test_resident_launches_of_unstructured_layers(gc, orc, N, B, values):
         assert same_floats(net.activations(cats), ref["y"])
 
 
+@pytest.mark.parametrize("N,B,K,values,rl", [(1024, 1500, 32, "uniform", 4), (1024, 700, 32, "general", 2), (512, 900, 16, "pow2", 4),
+                                             (256, 300, 8, "general", 1), (768, 520, 32, "uniform", 4), (1024, 400, 12, "pow2", 4)])
+def test_resident_launches_of_band_layers(gc, orc, monkeypatch, N, B, K, values, rl):
+    """BAND layers up to 1024 neurons wide run as resident launches in their QUAD form: 16 rows of a workgroup stay in
+    LDS through the layers, a thread computes four neighbouring outputs of the band for four rows from one merged
+    step list.  Per-layer counts, categories and activations against the oracle, pruned and unpruned, whole and cut
+    into calls, the state after every layer, and the same run with one launch per layer."""
+    print("resident launches, band layers N=%d B=%d K=%d %s rl=%d" % (N, B, K, values, rl), flush=True)
+    monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
+    rng = np.random.default_rng(N + B + K)
+    L = 9
+    layers = []
+    for l in range(L):
+        rp, c, v = orc.gen_layer_csr(11, l, N, K)
+        if values == "pow2":
+            v = np.ldexp(1.0, rng.integers(-5, -2, size=len(v)) + (2 if K <= 16 else 0)).astype(np.float32)
+        elif values == "general":
+            v = (rng.uniform(-0.05, 0.2, size=len(v)) * (32.0 / K)).astype(np.float32)
+        else:
+            v = np.full(len(v), 2.0 / K, dtype=np.float32)
+        layers.append((rp, c, v))
+    dens = np.where(rng.random(B) < 0.4, 0.8, 0.05).astype(np.float32)
+    feats = ((rng.random((B, N), dtype=np.float32) < dens[:, None]) * rng.uniform(0.5, 2.0, size=(B, N))).astype(np.float32)
+    bias = -0.3
+    ref = orc.infer(feats, layers, bias, prune=True, keep=set(range(L)))
+    want_counts = [len(a) for a in ref["active_ids"]]
+    assert 0 < want_counts[-1] < B, want_counts
+    with gc.Network(N, B, L, bias=bias) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert all(net.layer_plan(l).kernel == gc.KERNEL_BAND for l in range(L))
+        net.set_features_dense(feats)
+        cats = ref["categories"]
+        for prune in (True, False):
+            for fuse in (0, 4, 1):
+                r = net.run(prune=prune, collect_counts=True, fuse_layers=fuse)
+                assert r.layers_run == L
+                if fuse == 1:
+                    assert r.resident_launches == 0
+                elif fuse == 4 or not prune:
+                    assert r.resident_launches >= 1 and r.persistent_launches == 0
+                assert [net.active_count(l) for l in range(L)] == want_counts
+                assert np.array_equal(net.categories(), cats)
+                assert same_floats(net.activations(cats), ref["y"])
+        for l in range(L):    # the state after layer l, from a resident launch that ends there
+            net.run(prune=True, first_layer=0, n_layers=l + 1, fuse_layers=L)
+            gid, y = ref["kept"][l]
+            assert np.array_equal(net.categories(), ref["active_ids"][l])
+            assert same_floats(net.activations(gid), y)
+        net.run(prune=True, first_layer=0, n_layers=3, fuse_layers=3)
+        r = net.run(prune=False, first_layer=3, n_layers=L - 3, collect_counts=True, fuse_layers=L)
+        assert r.resident_launches == 1
+        assert [net.active_count(l) for l in range(3, L)] == want_counts[3:]
+        assert np.array_equal(net.categories(), cats)
+        assert same_floats(net.activations(cats), ref["y"])
+
+
 def test_resident_launches_full_batch(gc, orc):
     """Batch 60000 of RadiX-Net-like layers, N=1024: every activation of every row, the per-layer counts and the
     categories of the default run (resident launches) equal those of one launch per layer bit for bit, on live
@@ -716,6 +781,7 @@ def test_persistent_launches_on_buffers_that_stay_in_l1(gc, orc, rl, monkeypatch
     three times."""
     monkeypatch.setenv("SPDNN_ROWS_PER_LANE", str(rl))
     monkeypatch.setenv("SPDNN_PERSIST_XCD", "1")
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", "0")
     N, B = 256, 1500
     for seed in range(8):
         rng = np.random.default_rng(9100 + seed)
@@ -777,11 +843,12 @@ def test_persistent_launches_block_kernel(gc, orc, N, B, values, mode, monkeypat
 
 @pytest.mark.parametrize("values", ["uniform", "pow2", "general"])
 @pytest.mark.parametrize("N,B", [(1024, 1500), (4096, 700)])
-def test_fused_pairs_in_lds(gc, orc, N, B, values):
+def test_fused_pairs_in_lds(gc, orc, monkeypatch, N, B, values):
     """Layers that are bands over one common neuron order run two per launch, the activations between
     them kept in LDS (the reference's fused kernel, src/microbenchmark/fuse.cu:16-110): counts of every
     layer - the one inside a pair included -, categories and activations must be the oracle's, with
     and without pruning, and the same as with every layer in its own launch."""
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", "0")   # (bands up to 1024 neurons would share resident launches: the pairs are for wider ones)
     print("fused pairs N=%d B=%d %s" % (N, B, values), flush=True)
     rng = np.random.default_rng(N + B)
     L = 7
@@ -1022,8 +1089,9 @@ def test_pruned_run_with_rows_that_never_die(gc, orc, kind, monkeypatch):
         assert np.array_equal(net.categories(), cats)
 
 
-def test_persistent_launches_when_everything_dies(gc, orc):
+def test_persistent_launches_when_everything_dies(gc, orc, monkeypatch):
     """Literal inputs: all rows die within a few layers; the units of dead row blocks are skipped."""
+    monkeypatch.setenv("SPDNN_BAND_RESIDENT", "0")
     N, L, B = 1024, 40, 2000
     print("persistent launches, all rows die", flush=True)
     layers = [orc.gen_layer_csr(0, l, N) for l in range(12)]
@@ -1488,7 +1556,8 @@ def test_randomized_shapes_and_options(gc, orc, monkeypatch):
         same_nnz = int(rng.choice([4, 16, 32]))
         persist = dict(SPDNN_PERSIST=str(int(rng.integers(0, 2))), SPDNN_PERSIST_XCD=str(int(rng.choice([-1, 0, 1]))),
                        SPDNN_PERSIST_LIGHT_SYNC=str(int(rng.integers(0, 2))), SPDNN_RESIDENT=str(int(rng.choice([1, 1, 0]))),
-                       SPDNN_COMMON_ORDER=str(int(rng.choice([1, 1, 0]))))
+                       SPDNN_COMMON_ORDER=str(int(rng.choice([1, 1, 0]))), SPDNN_BAND_RESIDENT=str(int(rng.choice([1, 0]))),
+                       SPDNN_BAND_RESIDENT_MIN_LAYERS=str(int(rng.choice([2, 6]))))
         common_perm = rng.permutation(N)
         wait_us = int(rng.choice([0, 0, -1]))
         layers, kinds = [], []
