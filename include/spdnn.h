@@ -93,8 +93,10 @@ typedef struct spdnn_run_options {
     float   compact_threshold; /* prune: repack when active <= threshold * carried (0 = default .75) */
     int32_t fuse_layers;       /* launches that hold more than one layer.  1 = every layer its own launch.  0 = default:
                                   - resident launches where consecutive layers have a BLOCK form with one exact weight
-                                    (RadiX-Net layers) or are TILED layers, at most 4096 neurons wide: a workgroup keeps
-                                    16, 8 or 4 rows in LDS through up to 64 layers (SPDNN_RESIDENT=0: never);
+                                    (RadiX-Net layers) or are TILED layers, at most 4096 neurons wide, or are BAND layers
+                                    at most 1024 neurons wide (from 6 layers on, from 16 at 16384 rows and more): a workgroup
+                                    keeps 16, 8 or 4 rows in LDS through up to 64 layers (SPDNN_RESIDENT=0: never;
+                                    SPDNN_BAND_RESIDENT=0: not the BAND layers);
                                   - pairs of layers the inspector marked fuse_next as one launch with the intermediate tile
                                     in LDS, on launches of 2^23 rows x neurons and more (SPDNN_PAIR_MIN_ELEMS);
                                   - persistent launches (up to 64 layers of one kernel form, a dependency per row block
