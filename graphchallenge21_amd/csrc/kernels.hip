@@ -1873,7 +1873,7 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
     constexpr int PARTS = R / VW;
     using V = typename VecOf<VW>::type;
     publish_counts(a.pub);
-    const int t = (int)threadIdx.x, lane = t & 63;
+    const int t = (int)threadIdx.x, lane = t & 63, nthr = (int)blockDim.x;   // (ngroups * R threads, rounded up to whole waves)
     const int RB = 64 * a.rl;
     // Workgroups go to the 8 XCDs round robin by number; a 64-byte piece of a column holds the rows of 16 / R
     // workgroups, which should find it in ONE L2: every XCD takes a contiguous eighth of the rows.
@@ -1883,7 +1883,7 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
     const int rb = (int)(row0 / (size_t)RB), rin = (int)(row0 - (size_t)rb * RB);
     if (a.check_dead && a.prev_stamp != 0) {   // a row block without an active row is skipped, as by the per-layer kernels
         int alive = 0;
-        for (int i = t; i < RB; i += 1024) alive |= (a.active[(size_t)rb * RB + i] == a.prev_stamp) ? 1 : 0;
+        for (int i = t; i < RB; i += nthr) alive |= (a.active[(size_t)rb * RB + i] == a.prev_stamp) ? 1 : 0;
         if (__syncthreads_or(alive) == 0) return;
     }
     const size_t blkf = (size_t)a.N * RB;
@@ -1895,17 +1895,17 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
         // (four loads in flight per thread: a workgroup has nothing else to do while its rows come in)
         const float* __restrict__ gin = block_base(a.first_in, rb, blkf) + rin;
         const int total = a.N * PARTS;
-        for (int base = t; base < total; base += 4096) {
+        for (int base = t; base < total; base += 4 * nthr) {
             V v[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const int idx = base + u * 1024;
+                const int idx = base + u * nthr;
                 const int col = idx / PARTS, part = idx - col * PARTS;
                 if (idx < total) v[u] = *reinterpret_cast<const V*>(gin + (size_t)col * RB + part * VW);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const int idx = base + u * 1024;
+                const int idx = base + u * nthr;
                 const int col = idx / PARTS, part = idx - col * PARTS;
                 if (idx < total) *reinterpret_cast<V*>(buf0 + ((size_t)col * R + part * VW) * 4) = v[u];
             }
@@ -1976,7 +1976,7 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
     float* const o_h1 = to_c ? a.buf_c.half[1] : a.buf_a.half[1];
     float* __restrict__ gout = ((rb & 1) ? o_h1 : o_h0) + (size_t)(rb >> 1) * blkf + rin;
     const unsigned char* const fin = (done_layers & 1) ? buf1 : buf0;
-    for (int idx = t; idx < a.N * PARTS; idx += 1024) {
+    for (int idx = t; idx < a.N * PARTS; idx += nthr) {
         const int col = idx / PARTS, part = idx - col * PARTS;
         V v;
         if (all_dead) v = V{};
@@ -2340,18 +2340,24 @@ __global__ __launch_bounds__(1024) void band_resident_kernel(ResidentArgs a) {
     if (t < R && last_alive >= 0) a.active[row0 + t] = a.stamp0 + last_alive;
 }
 
-// counts[i] = rows whose stamp is at least stamp_lo + i (see launch_count_stamp_range): one workgroup, a
-// histogram in LDS (per wave one atomic per distinct value), then sums from the top
+// counts[i] = rows whose stamp is at least stamp_lo + i (see launch_count_stamp_range).  Every workgroup takes a
+// share of the rows: a histogram in LDS (per wave one atomic per distinct value), sums from the top, and - where the
+// launch has several workgroups - the sums added to `partial` (n words, zero when the launch starts).  The workgroup
+// that finishes last (a ticket in partial[kCountTicket]) hands the totals over and leaves partial zero again.
+constexpr int kCountTicket = 8192;   // words of `partial` in front of the ticket: the largest n
 __global__ __launch_bounds__(1024) void count_stamp_range_kernel(const int32_t* __restrict__ stamps, int rows, int stamp_lo,
                                                                  int n, int32_t* __restrict__ counts_dev,
-                                                                 int32_t* __restrict__ counts_host) {
+                                                                 int32_t* __restrict__ counts_host, int32_t* __restrict__ partial) {
     extern __shared__ int hist[];
+    __shared__ int sh_last;
     for (int i = threadIdx.x; i < n; i += 1024) hist[i] = 0;
     __syncthreads();
     const int lane = threadIdx.x & 63;
-    for (int r0 = 0; r0 < rows; r0 += 1024) {
+    const int per = (((rows + (int)gridDim.x - 1) / (int)gridDim.x) + 1023) & ~1023;   // rows per workgroup: whole trips of 1024
+    const int r_begin = (int)blockIdx.x * per, r_end = min(rows, r_begin + per);
+    for (int r0 = r_begin; r0 < r_end; r0 += 1024) {
         const int r = r0 + (int)threadIdx.x;
-        int d = r < rows ? stamps[r] - stamp_lo : -1;
+        int d = r < r_end ? stamps[r] - stamp_lo : -1;
         if (d >= n) d = n - 1;
         unsigned long long todo = __ballot(d >= 0 ? 1 : 0);
         while (todo) {
@@ -2368,6 +2374,18 @@ __global__ __launch_bounds__(1024) void count_stamp_range_kernel(const int32_t* 
         for (int i = n - 1; i >= 0; --i) { acc += hist[i]; hist[i] = acc; }
     }
     __syncthreads();
+    if (gridDim.x > 1) {
+        for (int i = threadIdx.x; i < n; i += 1024)
+            if (hist[i] != 0) atomicAdd(&partial[i], hist[i]);
+        __threadfence();
+        __syncthreads();
+        if (threadIdx.x == 0) sh_last = atomicAdd(&partial[kCountTicket], 1) == (int)gridDim.x - 1 ? 1 : 0;
+        __syncthreads();
+        if (!sh_last) return;
+        __threadfence();
+        for (int i = threadIdx.x; i < n; i += 1024) hist[i] = atomicExch(&partial[i], 0);
+        if (threadIdx.x == 0) atomicExch(&partial[kCountTicket], 0);
+    }
     for (int i = threadIdx.x; i < n; i += 1024) {
         if (counts_dev) counts_dev[i] = hist[i];
         if (counts_host) __hip_atomic_store(counts_host + i, hist[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -2391,11 +2409,18 @@ __global__ __launch_bounds__(1024) void scan_active_kernel(
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int tile = blockIdx.x;
-    int before = 0;  // survivors among this wave's 64 rows of every earlier tile
+    // survivors among this wave's 64 rows of every earlier tile (eight tiles' loads in flight at a time: one after the
+    // other the loop is as long as 58 round trips to L2)
+    int mine = 0;
+#pragma unroll 8
     for (int t = 0; t < tile; ++t) {
         const int r = t * 1024 + (int)threadIdx.x;  // < rows: an earlier tile is a full one
-        before += (int)__popcll(__ballot((active[r] == stamp && gid[r] >= 0) ? 1 : 0));
+        const int st = active[r], gd = gid[r];   // (both loaded whatever the first says: a load behind a test is a round trip of its own)
+        mine += ((st == stamp) & (gd >= 0)) ? 1 : 0;
     }
+    int before = mine;
+#pragma unroll
+    for (int sft = 1; sft < 64; sft <<= 1) before += __shfl_xor(before, sft, 64);
     const int r = tile * 1024 + (int)threadIdx.x;
     const int g = r < rows ? gid[r] : -1;
     const bool alive = r < rows && g >= 0 && active[r] == stamp;
@@ -2904,7 +2929,7 @@ static hipError_t launch_block_resident_r(const ResidentLaunch& a, hipStream_t s
     k.N = a.N; k.ngroups = a.ngroups; k.rl = a.rl; k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
     k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
     const size_t lds = (size_t)(a.N + 1) * R * 8;
-    dim3 grid((unsigned)(a.rows / R)), block(1024);
+    dim3 grid((unsigned)(a.rows / R)), block((unsigned)((a.ngroups * R + 63) / 64 * 64));
 #define SPDNN_RESIDENT(FULL)                                                                                              \
     do {                                                                                                                  \
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(block_resident_kernel<R, FULL>), \
@@ -3003,11 +3028,15 @@ hipError_t launch_band_resident(const ResidentLaunch& a, int wmode, hipStream_t 
     return hipGetLastError();
 }
 
+int count_stamp_partial_words() { return kCountTicket + 1; }
+
 hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,
-                                    int32_t* counts_host, hipStream_t s) {
-    if (!stamps || rows <= 0 || n < 1 || n > 8192 || (!counts_dev && !counts_host)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(count_stamp_range_kernel, dim3(1), dim3(1024), (size_t)n * 4, s, stamps, rows, stamp_lo, n, counts_dev,
-                       counts_host);
+                                    int32_t* counts_host, int32_t* partial, hipStream_t s) {
+    if (!stamps || rows <= 0 || n < 1 || n > kCountTicket || (!counts_dev && !counts_host)) return hipErrorInvalidValue;
+    // a workgroup per 4096 rows, 32 at most; a single one without the partial sums' buffer
+    const int nwg = partial ? std::max(1, std::min(32, rows / 4096)) : 1;
+    hipLaunchKernelGGL(count_stamp_range_kernel, dim3((unsigned)nwg), dim3(1024), (size_t)n * 4, s, stamps, rows, stamp_lo, n,
+                       counts_dev, counts_host, partial);
     return hipGetLastError();
 }
 
@@ -3199,7 +3228,10 @@ hipError_t launch_repack(const Feat& src, const Feat& dst, const int32_t* count,
                          const int32_t* alive_gid, int32_t* gid_out, int N, int rl, int dst_blocks,
                          hipStream_t s) {
     if (dst_blocks <= 0 || dst_blocks > 65535 || N <= 0) return hipErrorInvalidValue;
-    const int cpw = 64;
+    // 64 columns per workgroup where that still makes a couple of thousand workgroups, fewer columns where few row
+    // blocks survive (N=1024, 8 blocks: 128 workgroups of 64 columns took 55 us)
+    int cpw = 64;
+    while (cpw > 8 && (long long)((N + cpw - 1) / cpw) * dst_blocks < 2048) cpw /= 2;
     dim3 grid((N + cpw - 1) / cpw, dst_blocks);
     switch (rl) {
         case 4: hipLaunchKernelGGL(repack_kernel<4>, grid, dim3(256), 0, s, src, dst, count, alive_src, alive_gid, gid_out, N, cpw); break;

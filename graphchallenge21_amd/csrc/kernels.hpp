@@ -278,8 +278,11 @@ hipError_t launch_block_resident(const ResidentLaunch& a, hipStream_t s);
 // counts[i] = number of rows r < rows with stamps[r] >= stamp_lo + i, for i in [0, n): with bias <= 0 a
 // row that is zero stays zero, so the rows that carry the stamp of layer l or a later one are the rows
 // layer l left active.  Written to counts_dev and (system scope) to counts_host, either may be nullptr.
+// partial: count_stamp_partial_words() words of device memory, zero between the launches that use it (every launch
+// leaves it so) - with it the rows are shared out over several workgroups; nullptr: one workgroup counts them all.
 hipError_t launch_count_stamp_range(const int32_t* stamps, int rows, int stamp_lo, int n, int32_t* counts_dev,
-                                    int32_t* counts_host, hipStream_t s);
+                                    int32_t* counts_host, int32_t* partial, hipStream_t s);
+int count_stamp_partial_words();
 
 // Fused pair: two consecutive BAND layers (32 entries per row, unrolled record form, same weight
 // mode, rows per lane 4) of which the first writes its outputs exactly where the second reads them

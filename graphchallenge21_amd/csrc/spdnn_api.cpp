@@ -241,6 +241,7 @@ struct spdnn_net {
     int feat_paired = 0, feat_candidates = 0;
     int32_t* d_active_mid = nullptr;  // row stamps of the first layer of a fused pair (see PairLaunch)
     int32_t *d_active = nullptr, *d_gid = nullptr, *d_gid_tmp = nullptr, *d_count = nullptr;
+    int32_t* d_count_partial = nullptr;   // see launch_count_stamp_range
     int32_t *d_alive_src = nullptr, *d_alive_gid = nullptr, *d_nonfinite = nullptr;
     int32_t* h_count = nullptr;  // pinned
     int32_t* d_counts = nullptr; // per-layer active-row counters (device)
@@ -328,7 +329,7 @@ namespace {
 void release_device_base(spdnn_net* n) {
     hipFree(n->d_active_mid); n->d_active_mid = nullptr;
     hipFree(n->d_active); hipFree(n->d_gid); hipFree(n->d_gid_tmp);
-    hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_nonfinite);
+    hipFree(n->d_alive_src); hipFree(n->d_alive_gid); hipFree(n->d_count); hipFree(n->d_count_partial); hipFree(n->d_nonfinite);
     hipFree(n->d_counts);
     hipFree(n->d_done); hipFree(n->d_ctl); hipFree(n->d_abort); hipFree(n->d_frontier);
     n->d_done = n->d_abort = n->d_frontier = nullptr;
@@ -338,6 +339,7 @@ void release_device_base(spdnn_net* n) {
     if (n->h_count) hipHostFree(n->h_count);
     if (n->h_counts) hipHostFree(n->h_counts);
     n->d_active = n->d_gid = n->d_gid_tmp = n->d_alive_src = n->d_alive_gid = nullptr;
+    n->d_count_partial = nullptr;
     n->d_count = n->d_nonfinite = n->d_counts = n->h_count = n->h_counts = nullptr;
     for (hipEvent_t e : n->ev_layer) hipEventDestroy(e);
     for (const spdnn_net::Trial& t : n->trials) { hipEventDestroy(t.e0); hipEventDestroy(t.e1); }
@@ -378,6 +380,8 @@ int init_device(spdnn_net* n) {
     HIPCHK(dev_malloc(&n->d_alive_src, rows * 4));
     HIPCHK(dev_malloc(&n->d_alive_gid, rows * 4));
     HIPCHK(dev_malloc(&n->d_count, 64));
+    HIPCHK(dev_malloc(&n->d_count_partial, (size_t)count_stamp_partial_words() * 4));
+    HIPCHK(hipMemset(n->d_count_partial, 0, (size_t)count_stamp_partial_words() * 4));
     HIPCHK(dev_malloc(&n->d_nonfinite, 64));
     // coherent: the layer kernels store counts here and the host reads them while kernels still run
     HIPCHK(hipHostMalloc(&n->h_count, 64, hipHostMallocCoherent | hipHostMallocMapped));
@@ -2085,7 +2089,7 @@ static int spdnn_run_impl(spdnn_net* n, const spdnn_run_options* opt_in, spdnn_r
                 const bool with_prev = st.count_pending && prev_stamp != 0 && prev_stamp == stamp0 - 1;
                 const int lo = with_prev ? l - 1 : l, cnt = c + (with_prev ? 1 : 0);
                 HIPCHK(launch_count_stamp_range(n->d_active, n->carried, with_prev ? prev_stamp : stamp0, cnt, n->d_counts + lo,
-                                                polled ? n->h_counts + lo : nullptr, n->stream));
+                                                polled ? n->h_counts + lo : nullptr, n->d_count_partial, n->stream));
                 if (polled) {
                     if (st.pub.n > 0) recs.push_back({(int)(st.pub.src - n->d_counts), st.pub.n, -1});
                     recs.push_back({lo, cnt, persist ? next_slot - 1 : -1});
