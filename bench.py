@@ -129,6 +129,7 @@ def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
     net.synth_features(seed, B, 0.10, 0.25)
     out["zeros"] = timed(0)
     if out["zeros"]["resident_launches_per_pass"]:
+        out["zeros"]["frac"] = None
         out["zeros"]["note"] = ("resident launches: a workgroup whose 16 rows are all zero leaves at once, so this figure is no "
                                 "measure of the kernels - the live figures are")
     net.synth_features(seed, B, 0.10, 0.70)
@@ -151,8 +152,9 @@ def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
     out["feature_buffers_region_paired_candidates_peak_bytes"] = list(net.feature_placement())
     net.close()
     out["wall_s"] = time.time() - t0
-    log("other config %s: zeros %.4f ms/layer (frac %.3f), live %.4f ms/layer (frac %.3f), %.1f s"
-        % (name, out["zeros"]["ms_per_layer"], out["zeros"]["frac"], out["live"]["ms_per_layer"], out["live"]["frac"], out["wall_s"]))
+    log("other config %s: zeros %.4f ms/layer (frac %s), live %.4f ms/layer (frac %.3f), %.1f s"
+        % (name, out["zeros"]["ms_per_layer"], "%.3f" % out["zeros"]["frac"] if out["zeros"]["frac"] is not None else "-",
+           out["live"]["ms_per_layer"], out["live"]["frac"], out["wall_s"]))
     return out
 
 
