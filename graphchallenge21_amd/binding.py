@@ -82,6 +82,7 @@ def load_library():
         "spdnn_get_band_plan": ([vp, C.c_int, _i32p, _i32p, _u8p], C.c_int),
         "spdnn_get_band_pairs": ([vp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int),
                                  C.POINTER(C.c_int), C.c_void_p, C.c_void_p], C.c_int),
+        "spdnn_get_band_quads": ([vp, C.c_int, C.POINTER(C.c_int), C.c_void_p, C.c_void_p], C.c_int),
         "spdnn_get_layer_dst": ([vp, C.c_int, _i32p], C.c_int),
         "spdnn_get_layer_slots": ([vp, C.c_int, C.POINTER(C.c_int)], C.c_int),
         "spdnn_get_input_labelling": ([vp, C.c_int, _i32p], C.c_int),
@@ -269,6 +270,18 @@ class Network:
         _check(self._lib.spdnn_get_band_pairs(self._h, layer, None, None, None, None, rec.ctypes.data,
                                               None if w is None else w.ctypes.data))
         return steps.value, rec, w
+
+    def band_quads(self, layer):
+        """(groups, columns uint32[neuron/4][groups][4] as byte offsets (column * 64), weights
+        float32[neuron/4][groups][4 outputs][4 steps]); groups = 0: the layer has no QUAD form."""
+        groups = C.c_int()
+        _check(self._lib.spdnn_get_band_quads(self._h, layer, C.byref(groups), None, None))
+        g = groups.value
+        cols = np.empty((self.neuron // 4, g, 4), np.uint32)
+        w = np.empty((self.neuron // 4, g, 4, 4), np.float32)
+        if g:
+            _check(self._lib.spdnn_get_band_quads(self._h, layer, None, cols.ctypes.data, w.ctypes.data))
+        return g, cols, w
 
     def receptive_field(self, first_layer, n_layers, out_neurons):
         """Input neurons of layer first_layer that the given output neurons of layer

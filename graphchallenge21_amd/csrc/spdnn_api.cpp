@@ -1244,6 +1244,18 @@ static int spdnn_get_band_pairs_impl(const spdnn_net* n, int layer, int* steps, 
     return SPDNN_OK;
 }
 
+static int spdnn_get_band_quads_impl(const spdnn_net* n, int layer, int* groups, uint32_t* columns, float* weights) {
+    if (!n) return fail(SPDNN_E_ARG, "net is NULL");
+    if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
+    const_cast<spdnn_net*>(n)->pool->wait_all();
+    const LayerPlan& p = n->layers[(size_t)layer];
+    if (!p.set || p.kernel != SPDNN_KERNEL_BAND) return fail(SPDNN_E_STATE, "not a BAND layer");
+    if (groups) *groups = p.quad_groups;
+    if (columns) std::copy(p.quad_col.begin(), p.quad_col.end(), columns);
+    if (weights) std::copy(p.quad_w.begin(), p.quad_w.end(), weights);
+    return SPDNN_OK;
+}
+
 static int spdnn_get_layer_dst_impl(const spdnn_net* n, int layer, int32_t* dst) {
     if (!n || !dst) return fail(SPDNN_E_ARG, "NULL argument");
     if (layer < 0 || layer >= n->L) return fail(SPDNN_E_ARG, "layer out of range");
@@ -2503,6 +2515,9 @@ int spdnn_get_band_plan(const spdnn_net* n, int layer, int32_t* in_pos, int32_t*
 }
 int spdnn_get_band_pairs(const spdnn_net* n, int layer, int* steps, int* stride, int* padded_steps, int* has_weights, uint32_t* records, float* weights) {
     return guarded([&] { return spdnn_get_band_pairs_impl(n, layer, steps, stride, padded_steps, has_weights, records, weights); });
+}
+int spdnn_get_band_quads(const spdnn_net* n, int layer, int* groups, uint32_t* columns, float* weights) {
+    return guarded([&] { return spdnn_get_band_quads_impl(n, layer, groups, columns, weights); });
 }
 int spdnn_get_layer_dst(const spdnn_net* n, int layer, int32_t* dst) {
     return guarded([&] { return spdnn_get_layer_dst_impl(n, layer, dst); });

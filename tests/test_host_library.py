@@ -150,6 +150,64 @@ def test_band_pair_records_reproduce_oracle(gc, orc, monkeypatch):
             assert np.array_equal(y[:, net.input_labelling(l + 1)], want), l
 
 
+def _emulate_band_quads(net, l, y_phys):
+    """CPU emulation of the resident band launch from the QUAD form it streams: the four outputs at band positions
+    4c .. 4c+3 walk one merged list of steps; a step's column enters every output with the step's weight in that
+    output (0 where the output does not use it), rounded multiply then rounded add as the reference does."""
+    n = net.neuron
+    groups, cols, w = net.band_quads(l)
+    assert groups > 0
+    dst = net.layer_dst(l)
+    out = np.zeros_like(y_phys)
+    assert (cols % 64 == 0).all() and (cols // 64 < n).all()
+    for c in range(n // 4):
+        acc = [np.zeros(y_phys.shape[0], np.float32) for _ in range(4)]
+        for g in range(groups):
+            for k in range(4):
+                x = y_phys[:, int(cols[c, g, k]) // 64]
+                for o in range(4):
+                    acc[o] = acc[o] + x * w[c, g, o, k]
+        for o in range(4):
+            y = acc[o] + np.float32(net.bias)
+            out[:, dst[4 * c + o]] = np.where(y < 0, np.float32(0), np.where(y > 32, np.float32(32), y))
+    return out
+
+
+def test_band_quad_form_reproduces_oracle(gc, orc, monkeypatch):
+    """The merged step lists of output quads that the resident launches of band layers stream (35 steps in 9 groups for
+    32 entries per row, 11 in 3 for 8), for circulant bands with one weight and with general weights and for run
+    chains, emulated on the CPU against the oracle; a layer wider than 1024 neurons carries no such form."""
+    monkeypatch.setenv("SPDNN_RUN_CHAINS_MIN_N", "256")
+    n, b = 512, 5
+    rng = np.random.default_rng(23)
+    band8 = orc.gen_layer_csr(4, 1, n, 8)
+    band32 = orc.gen_layer_csr(4, 2, n)
+    layers = [orc.gen_layer_csr(4, 0, n), band8,
+              (band8[0], band8[1], rng.uniform(-0.1, 0.15, size=len(band8[1])).astype(np.float32)),
+              (band32[0], band32[1], np.ldexp(1.0, rng.integers(-6, -3, size=len(band32[1]))).astype(np.float32)),
+              radix_like_csr(rng, n, 16, "general")]
+    with gc.Network(n, b, len(layers), bias=-0.1) as net:
+        for l, csr in enumerate(layers):
+            net.set_layer_csr(l, *csr)
+        net.inspect()
+        assert [net.layer_plan(l).kernel for l in range(len(layers))] == [gc.KERNEL_BAND] * len(layers)
+        assert [net.band_quads(l)[0] for l in range(len(layers))] == [9, 3, 3, 9, 8]
+        feats = orc.gen_features(4, n, 0, b, 0.2, 0.7) * np.float32(1.7)
+        y = np.zeros_like(feats)
+        y[:, net.input_labelling(0)] = feats
+        want = feats
+        for l, csr in enumerate(layers):
+            y = _emulate_band_quads(net, l, y)
+            want, _ = orc.layer(want, csr, -0.1)
+            assert np.array_equal(y[:, net.input_labelling(l + 1)], want), l
+    wide = 2048
+    with gc.Network(wide, b, 1, bias=-0.1) as net:
+        net.set_layer_csr(0, *orc.gen_layer_csr(4, 0, wide))
+        net.inspect()
+        assert net.layer_plan(0).kernel == gc.KERNEL_BAND and net.band_quads(0)[0] == 0
+
+
+
 @pytest.mark.parametrize("tiled", [1, 0])
 def test_inspector_falls_back_to_the_general_classes(gc, orc, tiled, monkeypatch):
     monkeypatch.setenv("SPDNN_TILED", str(tiled))
