@@ -1915,24 +1915,23 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
     const int g = t >> LOG_R, r = t & (R - 1);
     const bool item = g < a.ngroups;
     const int gq = item ? g : 0;               // (lanes without an item go through the motions of group 0 and store to column N)
-    // byte offsets of the group's input columns and of its outputs' columns inside a buffer, spread over the group's lanes
-    uint32_t cb[NC], db[ND], cb_next[NC], db_next[ND];
-    int cnt = 32, cnt_next = 32;
-    auto load_indices = [&](int j, uint32_t (&c)[NC], uint32_t (&d)[ND], int& n_in) {
+    // the group's input columns and its outputs' columns, spread over the group's lanes: requested a layer ahead and
+    // kept as they come (arithmetic on a requested value would make the wave wait for the load then and there - all 16
+    // waves at once, at the top of every layer); turned into byte offsets inside a buffer when their layer begins
+    int32_t c_next[NC], d_next[ND];
+    int cnt_next = 32;
+    auto request_indices = [&](int j) {
         const LayerDesc lay = load_layer_desc(a.table, j);
         // (the pointers come out of the table: said to be global memory, or the loads become flat ones)
         using GI = const __attribute__((address_space(1))) int32_t*;
         const GI cols = (GI)lay.blk_cols, dsts = (GI)lay.blk_dst, cnts = (GI)lay.blk_cnt;
 #pragma unroll
-        for (int i = 0; i < NC; ++i) c[i] = (uint32_t)cols[(size_t)gq * 32 + i * R + r] * (uint32_t)(R * 4);
+        for (int i = 0; i < NC; ++i) c_next[i] = cols[(size_t)gq * 32 + i * R + r];
 #pragma unroll
-        for (int i = 0; i < ND; ++i) {
-            const int dcol = dsts[(size_t)gq * 16 + i * R + r];
-            d[i] = (uint32_t)((item && dcol >= 0) ? dcol : a.N) * (uint32_t)(R * 4);
-        }
-        if (!FULL) n_in = cnts[gq];
+        for (int i = 0; i < ND; ++i) d_next[i] = dsts[(size_t)gq * 16 + i * R + r];
+        if (!FULL) cnt_next = cnts[gq];
     };
-    load_indices(0, cb, db, cnt);
+    request_indices(0);
     int last_alive = -1;
     bool all_dead = false;
     int done_layers = 0;
@@ -1941,7 +1940,13 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
         const unsigned char* const in = ((j & 1) ? buf1 : buf0) + r * 4;
         unsigned char* const out = ((j & 1) ? buf0 : buf1) + r * 4;
         const float wu = load_layer_desc(a.table, j).wu;
-        if (j + 1 < a.nlayers) load_indices(j + 1, cb_next, db_next, cnt_next);   // in flight under this layer's arithmetic
+        uint32_t cb[NC], db[ND];
+#pragma unroll
+        for (int i = 0; i < NC; ++i) cb[i] = (uint32_t)c_next[i] * (uint32_t)(R * 4);
+#pragma unroll
+        for (int i = 0; i < ND; ++i) db[i] = (uint32_t)((item && d_next[i] >= 0) ? d_next[i] : a.N) * (uint32_t)(R * 4);
+        const int cnt = cnt_next;
+        if (j + 1 < a.nlayers) request_indices(j + 1);   // in flight under this layer's arithmetic
         float x[32];
 #pragma unroll
         for (int k = 0; k < 32; ++k) x[k] = *reinterpret_cast<const float*>(in + group_lane<R, NC>(cb, k));
@@ -1963,11 +1968,6 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
         if (t < R && ((mask >> t) & 1)) last_alive = j;
         done_layers = j + 1;
         if (mask == 0 && a.bias <= 0.0f) { all_dead = true; break; }   // zero rows stay zero
-#pragma unroll
-        for (int i = 0; i < NC; ++i) cb[i] = cb_next[i];
-#pragma unroll
-        for (int i = 0; i < ND; ++i) db[i] = db_next[i];
-        cnt = cnt_next;
     }
     // the launch's last layer writes the work buffer the layer before it did not (layer 0: the one it did not read)
     const bool in_a = a.first_in.half[0] == a.buf_a.half[0];
@@ -2037,6 +2037,24 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
 #pragma unroll
     for (int i = 0; i < PARTS; ++i) poff[i] = (uint32_t)(((i + lane) & (PARTS - 1)) * 16);
     const uint32_t estride = (uint32_t)a.N * 8u;
+    // A slot's length, output column and first two entries are requested one slot ahead - for a layer's first slot:
+    // a layer ahead - and kept as they come: a request made where its value is needed is a round trip to L2 that all 16
+    // waves of the workgroup make at once, right behind the barrier (three of them in a row, a third of a layer).
+    // (Entries 0 and 1 exist for every slot: the lists are padded to four entries and more.)
+    int n_in_next, d_next;
+    u32x2 e0_next, e1_next;
+    auto request_slot = [&](const LayerDesc& lay, int slot0) {
+        const int slot = slot0 + t;
+        const bool have = slot < a.N;
+        const GB entb = (GB)lay.rt_ent;
+        const uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
+        n_in_next = ((GI)lay.rt_len)[have ? slot : 0];
+        d_next = ((GI)lay.rt_dst)[have ? slot : 0];
+        e0_next = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+        e1_next = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
+    };
+    LayerDesc lay_next = load_layer_desc(a.table, 0);
+    request_slot(lay_next, 0);
     int last_alive = -1;
     bool all_dead = false;
     int done_layers = 0;
@@ -2044,14 +2062,18 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
     for (int j = 0; j < a.nlayers; ++j) {
         const unsigned char* const in = smem + ((j & 1) ? buf_bytes : 0u);
         unsigned char* const out = smem + ((j & 1) ? 0u : buf_bytes);
-        const LayerDesc lay = load_layer_desc(a.table, j);
+        const LayerDesc lay = lay_next;
+        if (j + 1 < a.nlayers) lay_next = load_layer_desc(a.table, j + 1);
         const GB entb = (GB)lay.rt_ent;
-        const GI lens = (GI)lay.rt_len, dsts = (GI)lay.rt_dst;
         unsigned bits = 0;   // rows that one of this lane's outputs left nonzero
         for (int slot0 = 0; slot0 < a.N; slot0 += 1024) {
             const int slot = slot0 + t;
             const bool have = slot < a.N;
-            const int n_in = have ? lens[slot] : 0;
+            const int n_in = have ? n_in_next : 0;
+            const int d = have ? d_next : -1;
+            u32x2 e0 = e0_next, e1 = e1_next;
+            if (slot0 + 1024 < a.N) request_slot(lay, slot0 + 1024);
+            else if (j + 1 < a.nlayers) request_slot(lay_next, 0);
             const int n_wave = __builtin_amdgcn_readfirstlane(n_in);   // slots are ordered by length: the wave's first lane has the most
             float acc[R];
 #pragma unroll
@@ -2061,11 +2083,6 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
             // own length: behind a list the array holds (column 0, weight +0), and adding x * (+0) to an accumulator
             // that started at +0 changes nothing (it can never be -0).
             uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
-            u32x2 e0 = {0u, 0u}, e1 = {0u, 0u};
-            if (n_wave > 0) {
-                e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
-                e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
-            }
             for (int k = 0; k < n_wave; k += 2) {
                 const u32x2 c0 = e0, c1 = e1;
                 eoff += 2u * estride;
@@ -2095,7 +2112,6 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
                     acc[i * 4 + 3] = mac<WMODE>(acc[i * 4 + 3], x1[i].w, w1);
                 }
             }
-            const int d = have ? dsts[slot] : -1;
 #pragma unroll
             for (int i = 0; i < PARTS; ++i) {
                 float4 y;
