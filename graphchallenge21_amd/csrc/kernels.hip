@@ -1899,9 +1899,9 @@ __global__ __launch_bounds__(1024) void block_resident_kernel(ResidentArgs a) {
             V v[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const int idx = base + u * nthr;
+                const int idx = min(base + u * nthr, total - 1);   // (a lane past the end reads the last piece again and drops it)
                 const int col = idx / PARTS, part = idx - col * PARTS;
-                if (idx < total) v[u] = *reinterpret_cast<const V*>(gin + (size_t)col * RB + part * VW);
+                v[u] = *reinterpret_cast<const V*>(gin + (size_t)col * RB + part * VW);
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
