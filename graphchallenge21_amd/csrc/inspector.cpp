@@ -881,7 +881,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.pairs.clear();
         // its GATHER form, for launches too small to fill the chip with tiles, and its ROWTILE form; both over
         // the outputs ordered by length, longest first
-        const int kw = std::max(kmax, 1);
+        const int kw = (std::max(kmax, 1) + 3) / 4 * 4;   // (the gather kernel takes four entries per trip: rows padded with column 0, weight +0)
         plan.alt_kmax = kw;
         plan.alt_cols.assign((size_t)N * kw, 0);
         plan.alt_wv.assign((size_t)N * kw, 0.0f);
@@ -915,7 +915,7 @@ void inspect_layer(int N, const std::vector<int32_t>& rowptr, const std::vector<
         plan.out_at.resize((size_t)N);
         std::iota(plan.in_pos.begin(), plan.in_pos.end(), 0);
         std::iota(plan.out_at.begin(), plan.out_at.end(), 0);
-        const int kw = std::max(kmax, 1);
+        const int kw = (std::max(kmax, 1) + 3) / 4 * 4;   // (four entries per trip: rows padded with column 0, weight +0)
         plan.ell_col.assign((size_t)N * kw, 0);
         plan.wv.assign((size_t)N * kw, 0.0f);
         plan.rowlen.resize((size_t)N);

@@ -1031,19 +1031,35 @@ __global__ __launch_bounds__(256) void gather_kernel(
 
     for (int j = j0; j < j1; ++j) {
         const int cnt = rowlen[j];
-        const int32_t* cp = cols + (size_t)j * kmax;
-        const float* wp = wv + (size_t)j * kmax;
+        // Four entries per trip, their four columns requested together (one entry after the other every trip is a
+        // scalar load, then a column load, then the arithmetic, each waiting for the one before).  Rows are padded to a
+        // multiple of four entries with (column 0, weight +0): x * (+0) added to an accumulator that started at +0
+        // changes nothing.  The next trip's entries are requested before this trip's arithmetic.
+        const __attribute__((address_space(4))) uint32_t* cp = (const __attribute__((address_space(4))) uint32_t*)(cols + (size_t)j * kmax);
+        const __attribute__((address_space(4))) float* wp = (const __attribute__((address_space(4))) float*)(wv + (size_t)j * kmax);
         float acc[RL];
 #pragma unroll
         for (int q = 0; q < RL; ++q) acc[q] = 0.0f;
-        for (int m = 0; m < cnt; ++m) {
-            const int c = cp[m];
-            const float w = wp[m];
-            V xv = *reinterpret_cast<const V*>(yin + (size_t)c * RB + loff);
-            float x[RL];
-            vec_to_arr<RL>(xv, x);
+        uint4 c4 = make_uint4(0u, 0u, 0u, 0u);
+        float4 w4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (cnt > 0) { c4 = load_const_u4(cp); w4 = load_const_f4(wp); }
+        for (int m = 0; m < cnt; m += 4) {
+            const uint4 c = c4;
+            const float4 w = w4;
+            V xv[4];
+            xv[0] = *reinterpret_cast<const V*>(yin + (size_t)c.x * RB + loff);
+            xv[1] = *reinterpret_cast<const V*>(yin + (size_t)c.y * RB + loff);
+            xv[2] = *reinterpret_cast<const V*>(yin + (size_t)c.z * RB + loff);
+            xv[3] = *reinterpret_cast<const V*>(yin + (size_t)c.w * RB + loff);
+            if (m + 4 < cnt) { c4 = load_const_u4(cp + m + 4); w4 = load_const_f4(wp + m + 4); }
+            const float ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-            for (int q = 0; q < RL; ++q) acc[q] = mac<WMODE>(acc[q], x[q], w);
+            for (int e = 0; e < 4; ++e) {
+                float x[RL];
+                vec_to_arr<RL>(xv[e], x);
+#pragma unroll
+                for (int q = 0; q < RL; ++q) acc[q] = mac<WMODE>(acc[q], x[q], ws[e]);
+            }
         }
         float y[RL];
 #pragma unroll
@@ -3112,7 +3128,8 @@ hipError_t launch_count_stamped(const int32_t* stamps, int rows, int stamp, int3
 }
 
 hipError_t launch_gather(const GatherLaunch& a, hipStream_t s) {
-    if (a.N <= 0 || a.kmax < 0 || a.nblk <= 0 || !a.yin || !a.yout || !a.cols || !a.rowlen || !a.wv ||
+    // (kmax: the rows' stride in cols and wv, a multiple of four - the kernel takes four entries per trip)
+    if (a.N <= 0 || a.kmax < 0 || (a.kmax % 4) != 0 || a.nblk <= 0 || !a.yin || !a.yout || !a.cols || !a.rowlen || !a.wv ||
         !a.dst || !a.active)
         return hipErrorInvalidValue;
     const int opg = 8;

@@ -301,6 +301,7 @@ struct spdnn_net {
     int64_t pair_min_elems = (int64_t)1 << 23;
     int64_t block_form_max_elems = (int64_t)1 << 26;  // see use_block_form
     int64_t tiled_min_rows = 8192;                    // see use_gather_form (SPDNN_TILED_MIN_ROWS)
+    bool tiled_min_rows_given = false;                // ... set in the environment: also layers with a ROWTILE form follow it
     int rowtile_mode = 1;                             // TILED layers up to 8192 neurons wide run their ROWTILE form (SPDNN_ROWTILE=0: the tiles)
     int band_resident_mode = 1;                       // BAND layers up to 1024 neurons wide join resident launches (SPDNN_BAND_RESIDENT=0: never)
     int band_resident_min_layers = 0;                 // ... of at least this many layers (SPDNN_BAND_RESIDENT_MIN_LAYERS; 0: 6, from 16384 rows up 16)
@@ -927,7 +928,7 @@ static int spdnn_create_impl(int neuron, int max_batch, int layers, float bias, 
     if (const char* e = getenv("SPDNN_PAIR_SEGLEN")) n->pair_seglen = atoi(e);
     if (const char* e = getenv("SPDNN_PAIR_MIN_ELEMS")) n->pair_min_elems = atoll(e);
     if (const char* e = getenv("SPDNN_BLOCK_FORM_MAX_ELEMS")) n->block_form_max_elems = atoll(e);
-    if (const char* e = getenv("SPDNN_TILED_MIN_ROWS")) n->tiled_min_rows = atoll(e);
+    if (const char* e = getenv("SPDNN_TILED_MIN_ROWS")) { n->tiled_min_rows = atoll(e); n->tiled_min_rows_given = true; }
     if (const char* e = getenv("SPDNN_ROWTILE")) n->rowtile_mode = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_BAND_RESIDENT")) n->band_resident_mode = atoi(e) != 0 ? 1 : 0;
     if (const char* e = getenv("SPDNN_BAND_RESIDENT_MIN_LAYERS")) n->band_resident_min_layers = std::max(0, atoi(e));
@@ -1530,9 +1531,16 @@ static bool use_block_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
 // random inputs per output, per layer: N=1024 4096 rows 46 against 31 us, 16384 rows 55 against 77; N=2048 67 against
 // 46 and 162 against 190; N=4096 98 against 79 and 465 against 431 (60000 rows: 1641 against 1900); N <= 512: the
 // tiles are never slower.  So: the gather form below 8192 rows on layers of 1024 neurons and more.
+// That was measured against the tiles.  The ROWTILE form (whole outputs per thread, up to 8192 neurons) is the faster of
+// the two at every size - per layer against the gather form: N=1024 11.5 against 17.5 us at 2048 rows and 71 against 183 at
+// 32768, N=2048 19.0 against 19.2 and 176 against 420, N=4096 25.6 against 29.1 and 396 against 923 - so where a layer has
+// it the gather form is used only if SPDNN_TILED_MIN_ROWS asks for it.
 static bool use_gather_form(const spdnn_net* n, const LayerPlan& p, int nblk) {
-    return p.kernel == SPDNN_KERNEL_TILED && p.alt_kmax > 0 && n->N >= 1024 &&
-           (int64_t)nblk * (int64_t)n->RB < n->tiled_min_rows;
+    if (p.kernel != SPDNN_KERNEL_TILED || p.alt_kmax <= 0 || n->N < 1024) return false;
+    const int rt_rows = rowtile_rows_per_workgroup(n->N);
+    const bool has_rowtile = n->rowtile_mode && !p.rt_ent.empty() && rt_rows > 0 && n->RB % rt_rows == 0;
+    if (has_rowtile && !n->tiled_min_rows_given) return false;
+    return (int64_t)nblk * (int64_t)n->RB < n->tiled_min_rows;
 }
 
 static hipError_t launch_layer(spdnn_net* n, int l, const Feat& in, const Feat& out, int nblk, int stamp,

@@ -75,8 +75,9 @@ typedef struct spdnn_layer_plan {
     int64_t nnz;
     int64_t plan_bytes;      /* device bytes held for this layer                                  */
     int32_t block_form;      /* second form the layer holds for small launches: 1 = a run-chain BAND layer with its
-                                BLOCK form, 2 = a TILED layer with its GATHER form (below 8192 rows on layers of
-                                1024 neurons and more, SPDNN_TILED_MIN_ROWS); 0 = none                  */
+                                BLOCK form, 2 = a TILED layer with its GATHER form (used below 8192 rows on layers of
+                                1024 neurons and more that have no ROWTILE form - wider than 8192 neurons or
+                                SPDNN_ROWTILE=0 - or where SPDNN_TILED_MIN_ROWS asks for it); 0 = none */
     int32_t fuse_next;       /* 1 (after spdnn_inspect): this layer and the next can run as one fused launch, the
                                 activations between them kept in LDS (see spdnn_run_options.fuse_layers)  */
     int32_t common_order;    /* run chains, after spdnn_inspect: 0 = the layer has a labelling of its own; 1 or 2 = it is
