@@ -1371,6 +1371,25 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
         if (a.check_dead && __builtin_amdgcn_readfirstlane(__syncthreads_or(alive ? 1 : 0)) == 0) return;
     }
     const size_t blkf = (size_t)a.N * RB;
+    // A slot's length, output column and first entries are requested ahead - for the first slot before the rows come
+    // in, for a later one under the slot before it - and kept as they come: requested where they are needed they are
+    // two round trips to L2 in a row that the whole workgroup waits for.  (Entries 0 and 1 exist for every slot: the
+    // lists are padded to four entries and more.)
+    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+    using GB = const __attribute__((address_space(1))) unsigned char*;
+    const GB entb = (GB)a.ent;
+    const uint32_t estride = (uint32_t)a.N * 8u;   // bytes from a slot's entry k to its entry k + 1
+    int n_in_next, d_next;
+    u32x2 e0_next, e1_next;
+    auto request_slot = [&](int slot0) {
+        const int slot = slot0 + t;
+        const int sq = slot < a.N ? slot : 0;
+        n_in_next = a.len[sq];
+        d_next = a.dst[sq];
+        e0_next = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (uint32_t)sq * 8u);
+        e1_next = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + ((uint32_t)sq * 8u + estride));
+    };
+    request_slot(0);
     {
         // (half by half: indexing the halves of a Feat inside the argument struct would put the struct into scratch memory)
         const float* __restrict__ gin = ((rb & 1) ? a.yin.half[1] : a.yin.half[0]) + (size_t)(rb >> 1) * blkf + rin;
@@ -1393,10 +1412,6 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
     if (t == 0) sh_alive = 0;
     __syncthreads();
     float* __restrict__ gout = ((rb & 1) ? a.yout.half[1] : a.yout.half[0]) + (size_t)(rb >> 1) * blkf + rin;
-    typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-    using GB = const __attribute__((address_space(1))) unsigned char*;
-    const GB entb = (GB)a.ent;
-    const uint32_t estride = (uint32_t)a.N * 8u;   // bytes from a slot's entry k to its entry k + 1
     // this lane's order of the four-row parts of a column, as byte offsets
     uint32_t poff[PARTS];
 #pragma unroll
@@ -1405,7 +1420,10 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
     for (int slot0 = 0; slot0 < a.N; slot0 += 1024) {
         const int slot = slot0 + t;
         const bool have = slot < a.N;
-        const int n_in = have ? a.len[slot] : 0;
+        const int n_in = have ? n_in_next : 0;
+        const int d = have ? d_next : -1;
+        const u32x2 e0_first = e0_next, e1_first = e1_next;
+        if (slot0 + 1024 < a.N) request_slot(slot0 + 1024);
         // the slots are ordered by length, longest first: the wave's first lane has the most entries
         const int n_wave = __builtin_amdgcn_readfirstlane(n_in);
         float acc[R];
@@ -1415,8 +1433,7 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
             // (one entry at a time where two workgroups fit a CU - 16 rows of up to 1280 neurons: with two entries the
             // sixteen more registers for the second column leave it one - N=1024, batch 60000: 170 against 156 us per layer)
             uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
-            u32x2 e = {0u, 0u};
-            if (n_wave > 0) e = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
+            u32x2 e = e0_first;
             for (int k = 0; k < n_wave; ++k) {
                 const u32x2 cur = e;
                 eoff += estride;
@@ -1440,11 +1457,7 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
             // length: behind a list the array holds (column 0, weight +0), and adding x * (+0) to an accumulator that
             // started at +0 changes nothing (it can never be -0).
             uint32_t eoff = (uint32_t)(have ? slot : 0) * 8u;
-            u32x2 e0 = {0u, 0u}, e1 = {0u, 0u};
-            if (n_wave > 0) {
-                e0 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + eoff);
-                e1 = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(entb + (eoff + estride));
-            }
+            u32x2 e0 = e0_first, e1 = e1_first;
             for (int k = 0; k < n_wave; k += 2) {
                 const u32x2 c0 = e0, c1 = e1;
                 eoff += 2u * estride;
@@ -1475,7 +1488,6 @@ __global__ __launch_bounds__(1024) void rowtile_kernel(RowtileArgs a) {
                 }
             }
         }
-        const int d = have ? a.dst[slot] : -1;
         float4 y[PARTS];
 #pragma unroll
         for (int i = 0; i < PARTS; ++i) {
