@@ -158,6 +158,43 @@ def sustained_block(gc, name, seed, log, per_layer_too, with_cpu=True):
     return out
 
 
+def structure_block(gc, structure, N, L, B, bias, log):
+    """The other layer classes at a BASELINE shape, sustained on live data (feature densities U[0.10, 0.70], pruning off,
+    two timed passes after a warm-up): RadiX-Net-like layers (BLOCK class: strides 16 .. N/2 in turn behind random
+    relabellings, 32 nnz/row of 0.0625) or layers without structure (TILED class: 1..24 random inputs per output, random
+    weights; bias +0.01 so that rows stay alive), left to the library and with one launch per layer."""
+    rng = np.random.default_rng(N)
+    t0 = time.time()
+    if structure == "radix":
+        kinds = [radix_layer(rng, N, 16 << k) for k in range(int(np.log2(N // 16)))]
+    else:
+        kinds = [irregular_layer(rng, N) for _ in range(4)]
+        bias = 0.01
+    net = gc.Network(N, B, L, bias=bias)
+    for l in range(L):
+        net.set_layer_csr(l, *kinds[l % len(kinds)])
+    net.inspect()
+    net.synth_features(1, B, 0.10, 0.70)
+    alg = 8.0 * B * N
+    out = {"structure": structure, "neuron": N, "layers": L, "batch": B, "bias": bias,
+           "kernel_classes": sorted({int(net.layer_plan(l).kernel) for l in range(L)})}
+    for key, fuse in (("default", 0), ("one_launch_per_layer", 1)):
+        net.run(prune=False, fuse_layers=fuse)
+        best, r = None, None
+        for _ in range(2):
+            r = net.run(prune=False, fuse_layers=fuse)
+            best = r.ms_total if best is None else min(best, r.ms_total)
+        ms = best / L
+        out[key] = {"ms_per_layer": ms, "algorithmic_bytes_over_time_frac": alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                    "launches_per_pass": int(r.launches), "resident_launches_per_pass": int(r.resident_launches),
+                    "rows_nonzero_at_end": int(r.active_rows)}
+    net.close()
+    out["wall_s"] = time.time() - t0
+    log("structure %s N=%d: default %.4f ms/layer, one launch per layer %.4f ms/layer, %.1f s"
+        % (structure, N, out["default"]["ms_per_layer"], out["one_launch_per_layer"]["ms_per_layer"], out["wall_s"]))
+    return out
+
+
 def challenge_like_block(gc, N, L, B, bias, log):
     """A run shaped like the challenge's own (the official files are not available offline): RadiX-Net-like layers of
     strides 16, 32, ... N/2 in turn behind random relabellings, batch B of which 3 % are dense rows that survive every
@@ -454,8 +491,11 @@ def main():
     net.close()
 
     # ---- beside the headline run: the other BASELINE configurations and challenge-like pruned runs -----------
-    other, challenge = None, None
+    other, challenge, structures = None, None, None
     if not args.no_extras and args.structure == "circulant":
+        structures = [structure_block(gc, st_, n_, l_, 60000, b_, log)
+                      for st_, n_, l_, b_ in (("radix", 1024, 120, -0.30), ("radix", 4096, 128, -0.35), ("irregular", 1024, 64, 0.01),
+                                              ("irregular", 4096, 16, 0.01))]
         other = {name: sustained_block(gc, name, seed, log, per_layer_too=name in ("cfg0", "cfg1", "cfg2"), with_cpu=not args.no_cpu)
                  for name in ("cfg0", "cfg1", "cfg2", "cfg3") if name != args.config}
         challenge = {"workload": "RadiX-Net-like layers (strides 16 .. N/2 in turn, random relabellings), batch 60000 with 3 % "
@@ -525,6 +565,7 @@ def main():
         "events_ms_per_step": ms_events / args.steps,
         "other_configs": other,
         "challenge_like": challenge,
+        "other_structures": structures,
     }
     print(json.dumps(out))
     return 0
