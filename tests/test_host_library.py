@@ -634,6 +634,12 @@ def test_argument_and_state_errors(gc, orc):
         with pytest.raises(gc.SpdnnError) as e:
             net.layer_plan(1)
         assert e.value.code == E_STATE
+        with pytest.raises(gc.SpdnnError) as e:
+            net.band_quads(1)                       # no such layer yet
+        assert e.value.code == E_STATE
+        with pytest.raises(gc.SpdnnError) as e:
+            net.band_quads(7)
+        assert e.value.code == E_ARG
         with pytest.raises(gc.SpdnnError) as e:     # features need the inspected network
             net.set_features_dense(np.zeros((4, n), np.float32))
         assert e.value.code == E_STATE
