@@ -2192,17 +2192,19 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
 // circulant band of K entries): per step ONE 16-byte LDS read - the column's four rows - feeds 16 multiply-adds, a
 // step an output does not use entering it with weight 0 (an exact zero added).  The plan stream of a quad - per group
 // of four steps the four columns (as byte offsets) and 4 x 4 weights - is spread over the quad's four lanes (lane k holds
-// the column of step k and the four weights of output k) and handed round by DPP quad permutations inside the address
-// add and the multiply-adds that use them; the groups are requested two ahead of the arithmetic, the first two of the
-// next layer before this layer's barrier.
+// the column of step k and the four weights of output k) and handed round by DPP quad permutations (the columns inside
+// the address adds, the weights by moves in front of the multiply-adds); the groups are requested two ahead of the
+// arithmetic, the first two of the next layer before this layer's barrier.
 template <int K> __device__ __forceinline__ uint32_t quad_lane(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, K * 0x55, 0xf, 0xf, true);
 }
 // One step of a quad: acc[o][q] += x[q] * (the weight held by lane o of this lane's quad), o, q = 0..3.  The weights
-// are brought over by four DPP moves and the sixteen multiply-adds take register operands only: such a v_fmac_f32
-// issues at twice the rate of one with a DPP or a scalar operand (measured: 0.95 against 1.75 ns per wave instruction
-// and SIMD), so the moves cost less than they save.  Ends with a barrier to the compiler's reordering of memory
-// accesses: the LDS reads of later steps are issued before the step's arithmetic and stay there.
+// are brought over by four DPP moves and the sixteen multiply-adds take register operands only.  Measured (register-
+// only loops, 4 waves per SIMD, per wave instruction and SIMD): such a v_fmac_f32 0.95 - 1.1 ns, one with a DPP or a
+// scalar operand 1.75 ns, a DPP move in front of multiply-adds that depend on it 2.7 ns - so this form and sixteen
+// DPP multiply-adds cost the same 28 ns per step; this is the one the compiler makes of the plain source.  Ends with a
+// barrier to the compiler's reordering of memory accesses: the LDS reads of later steps are issued before the step's
+// arithmetic and stay there.
 template <int WMODE> __device__ __forceinline__ void quad_step(float (&acc)[4][4], const float4& x, float w) {
     const uint32_t wb = __float_as_uint(w);
     const float wo[4] = {__uint_as_float(quad_lane<0>(wb)), __uint_as_float(quad_lane<1>(wb)), __uint_as_float(quad_lane<2>(wb)),
