@@ -668,7 +668,7 @@ static void build_quad_form(int N, const std::vector<int32_t>& rowptr, const std
             for (int j = 0; j < 4; ++j) {
                 const int row = plan.out_at[(size_t)4 * c + j];
                 if (at[j] < rowptr[row + 1] && col[at[j]] == in) {
-                    plan.quad_w[(grp * 4 + (size_t)j) * 4 + (size_t)(m & 3)] = val[at[j]];
+                    plan.quad_w[(grp * 4 + (size_t)(m & 3)) * 4 + (size_t)j] = val[at[j]];
                     ++at[j];
                 }
             }

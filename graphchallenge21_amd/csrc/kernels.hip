@@ -2198,17 +2198,12 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
 template <int K> __device__ __forceinline__ uint32_t quad_lane(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, K * 0x55, 0xf, 0xf, true);
 }
-// One step of a quad: acc[o][q] += x[q] * (the weight held by lane o of this lane's quad), o, q = 0..3.  The weights
-// are brought over by four DPP moves and the sixteen multiply-adds take register operands only.  Measured (register-
-// only loops, 4 waves per SIMD, per wave instruction and SIMD): such a v_fmac_f32 0.95 - 1.1 ns, one with a DPP or a
-// scalar operand 1.75 ns, a DPP move in front of multiply-adds that depend on it 2.7 ns - so this form and sixteen
-// DPP multiply-adds cost the same 28 ns per step; this is the one the compiler makes of the plain source.  Ends with a
-// barrier to the compiler's reordering of memory accesses: the LDS reads of later steps are issued before the step's
-// arithmetic and stay there.
-template <int WMODE> __device__ __forceinline__ void quad_step(float (&acc)[4][4], const float4& x, float w) {
-    const uint32_t wb = __float_as_uint(w);
-    const float wo[4] = {__uint_as_float(quad_lane<0>(wb)), __uint_as_float(quad_lane<1>(wb)), __uint_as_float(quad_lane<2>(wb)),
-                         __uint_as_float(quad_lane<3>(wb))};
+// One step of a quad: acc[o][q] += x[q] * w[o], o, q = 0..3, all operands registers of the lane itself (a v_fmac_f32 on
+// three vector registers issues in 0.95 - 1.1 ns per wave and SIMD, one with a DPP or scalar operand in 1.75 ns).  Ends
+// with a barrier to the compiler's reordering of memory accesses: the LDS reads of later steps are issued before the
+// step's arithmetic and stay there.
+template <int WMODE> __device__ __forceinline__ void quad_step(float (&acc)[4][4], const float4& x, const float4& w) {
+    const float wo[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int o = 0; o < 4; ++o) {
         acc[o][0] = mac<WMODE>(acc[o][0], x.x, wo[o]);
@@ -2271,6 +2266,8 @@ __global__ __launch_bounds__(1024) void band_resident_kernel(ResidentArgs a) {
     if (t < R) sh_last[t] = -1;
     const int rq = t & 3;
     const uint32_t lane_off = (uint32_t)rq * 16u;
+    // the wave's own KiB behind the two row buffers, this lane's quad's 64 bytes of it
+    unsigned char* const wslot = smem + 2u * buf_bytes + (uint32_t)(t >> 6) * 1024u + (uint32_t)((t & 63) >> 2) * 64u;
     const int ng = NG ? NG : a.ngroups;
     // this lane's place in a quad's plan stream: group gi lies 4 lanes further on
     const size_t qoff = (size_t)(t >> 2) * (size_t)ng * 4 + (size_t)rq;
@@ -2311,12 +2308,19 @@ __global__ __launch_bounds__(1024) void band_resident_kernel(ResidentArgs a) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) acc[o][q] = 0.0f;
         // step e = 4 gi + k: the LDS read of step e + 3 is issued before the arithmetic of step e (the waves of a workgroup
-        // leave the barrier together: a wave that waited for each read right after issuing it would wait when all others do)
+        // leave the barrier together: a wave that waited for each read right after issuing it would wait when all others do).
+        // The weights of a group of four steps go through the wave's own 1 KiB of LDS: lane k of a quad has requested the
+        // four outputs' weights of step k, writes them behind the last read of the group before (one wave's LDS
+        // instructions run in order: no barrier), and every lane of the quad reads a step's four weights back, one
+        // step ahead - all sixteen multiply-adds of a step then take their operands from the lane's own registers.
         const int nsteps = 4 * ng;
         float4 xb[4];
+        float4 wq[2];
         xb[0] = *reinterpret_cast<const float4*>(in + (quad_lane<0>(cr[0]) + lane_off));
         xb[1] = *reinterpret_cast<const float4*>(in + (quad_lane<1>(cr[0]) + lane_off));
         xb[2] = *reinterpret_cast<const float4*>(in + (quad_lane<2>(cr[0]) + lane_off));
+        *reinterpret_cast<f32x4_t*>(wslot + lane_off) = wr[0];
+        wq[0] = *reinterpret_cast<const float4*>(wslot);
 #pragma unroll
         for (int e = 0; e < 36; ++e) {
             if (e < nsteps) {
@@ -2327,9 +2331,11 @@ __global__ __launch_bounds__(1024) void band_resident_kernel(ResidentArgs a) {
                 }
                 if (e + 3 < 36 && e + 3 < nsteps)
                     xb[(e + 3) % 4] = *reinterpret_cast<const float4*>(in + (quad_lane_of(cr[((e + 3) >> 2) % 3], e + 3) + lane_off));
-                const f32x4_t wg4 = wr[gi % 3];
-                const float wk = (e & 3) == 0 ? wg4.x : (e & 3) == 1 ? wg4.y : (e & 3) == 2 ? wg4.z : wg4.w;
-                quad_step<WMODE>(acc, xb[e % 4], wk);
+                if (e + 1 < 36 && e + 1 < nsteps) {
+                    if ((e & 3) == 3) *reinterpret_cast<f32x4_t*>(wslot + lane_off) = wr[(gi + 1) % 3];   // the next group's weights
+                    wq[(e + 1) & 1] = *reinterpret_cast<const float4*>(wslot + ((e + 1) & 3) * 16);
+                }
+                quad_step<WMODE>(acc, xb[e % 4], wq[e & 1]);
             }
         }
         // (outputs are clamped to [0, clamp]: the largest of a row's four is positive exactly when one of them is nonzero)
@@ -3056,12 +3062,12 @@ hipError_t launch_band_resident(const ResidentLaunch& a, int wmode, hipStream_t 
     k.N = a.N; k.ngroups = a.ngroups; k.rl = a.rl; k.stamp0 = a.stamp0; k.prev_stamp = a.prev_stamp; k.check_dead = a.check_dead;
     k.bias = a.bias; k.clampv = a.clampv; k.pub = a.publish;
     k.quad_col = a.quad_col; k.quad_w = a.quad_w; k.quad_dst = a.quad_dst; k.quad_stride = a.quad_stride;
-    const size_t lds = (size_t)a.N * 16 * 8;
+    const size_t lds = (size_t)a.N * 16 * 8 + (size_t)(a.N / 64) * 1024;   // two row buffers, then a KiB per wave for the weights
     dim3 grid((unsigned)(a.rows / 16)), block((unsigned)a.N);
 #define SPDNN_BAND_RESIDENT(NG, WM)                                                                                         \
     do {                                                                                                                    \
         static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(band_resident_kernel<NG, WM>),     \
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);        \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024);        \
         if (attr != hipSuccess) return attr;                                                                                \
         hipLaunchKernelGGL((band_resident_kernel<NG, WM>), grid, block, lds, s, k);                                         \
     } while (0)

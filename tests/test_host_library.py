@@ -166,7 +166,7 @@ def _emulate_band_quads(net, l, y_phys):
             for k in range(4):
                 x = y_phys[:, int(cols[c, g, k]) // 64]
                 for o in range(4):
-                    acc[o] = acc[o] + x * w[c, g, o, k]
+                    acc[o] = acc[o] + x * w[c, g, k, o]
         for o in range(4):
             y = acc[o] + np.float32(net.bias)
             out[:, dst[4 * c + o]] = np.where(y < 0, np.float32(0), np.where(y > 32, np.float32(32), y))
