@@ -273,7 +273,7 @@ class Network:
 
     def band_quads(self, layer):
         """(groups, columns uint32[neuron/4][groups][4] as byte offsets (column * 64), weights
-        float32[neuron/4][groups][4 outputs][4 steps]); groups = 0: the layer has no QUAD form."""
+        float32[neuron/4][groups][4 steps][4 outputs]); groups = 0: the layer has no QUAD form."""
         groups = C.c_int()
         _check(self._lib.spdnn_get_band_quads(self._h, layer, C.byref(groups), None, None))
         g = groups.value

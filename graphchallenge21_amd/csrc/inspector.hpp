@@ -71,8 +71,8 @@ struct LayerPlan {
     // LDS through the layers: the four outputs at band positions 4c .. 4c+3 add their inputs in ascending input index,
     // so their lists merge into one list of steps (K + 3 for a circulant band), padded to quad_groups groups of four.
     // quad_col [N/4][quad_groups][4] = input column of each step, as the byte offset of the column in a buffer of 16 rows per
-    // column; quad_w [N/4][quad_groups][4 outputs][4 steps] = the
-    // weight of the step in each output, 0 where the output does not use it (padding steps repeat the last column).
+    // column; quad_w [N/4][quad_groups][4 steps][4 outputs] = the weight of the step in each output, 0 where the output
+    // does not use it (padding steps repeat the last column): the 16 bytes a lane of the quad loads are one step's.
     std::vector<uint32_t> quad_col;
     std::vector<float> quad_w;
     int quad_groups = 0;

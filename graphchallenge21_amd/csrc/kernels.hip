@@ -2191,10 +2191,15 @@ __global__ __launch_bounds__(1024) void rowtile_resident_kernel(ResidentArgs a) 
 // outputs add their inputs in ascending input index, so their lists are one merged list of steps (K + 3 for a
 // circulant band of K entries): per step ONE 16-byte LDS read - the column's four rows - feeds 16 multiply-adds, a
 // step an output does not use entering it with weight 0 (an exact zero added).  The plan stream of a quad - per group
-// of four steps the four columns (as byte offsets) and 4 x 4 weights - is spread over the quad's four lanes (lane k holds
-// the column of step k and the four weights of output k) and handed round by DPP quad permutations (the columns inside
-// the address adds, the weights by moves in front of the multiply-adds); the groups are requested two ahead of the
-// arithmetic, the first two of the next layer before this layer's barrier.
+// of four steps the four columns (as byte offsets) and 4 x 4 weights - is spread over the quad's four lanes: lane k holds
+// the column of step k and the four outputs' weights of step k.  The columns are handed round by DPP quad permutations
+// inside the address adds.  The weights go through LDS: each wave owns a KiB behind the two row buffers, 64 bytes per
+// quad; lane k writes its 16 bytes there behind the last read of the group before (the LDS operations of one wave run
+// in order, so no barrier is needed) and every lane of the quad reads a step's 16 bytes back, one step ahead of its
+// use - a broadcast - so that the 16 multiply-adds of a step have all three operands in the lane's own registers.
+// (Handing the weights round by DPP instead costs 4 moves per step in front of dependent multiply-adds, a tenth of the
+// layer's time more.)  The groups are requested two ahead of the arithmetic, the first two of the next layer before
+// this layer's barrier.
 template <int K> __device__ __forceinline__ uint32_t quad_lane(uint32_t v) {
     return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, K * 0x55, 0xf, 0xf, true);
 }

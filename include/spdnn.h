@@ -247,7 +247,7 @@ int spdnn_get_band_pairs(const spdnn_net* net, int layer, int* steps, int* strid
 /* The QUAD form a BAND layer of up to 1024 neurons also carries, for resident launches (16 rows of a workgroup kept in
  * LDS through the layers): the four outputs at band positions 4c .. 4c+3 share one merged list of steps, in *groups
  * groups of four.  columns (neuron/4 * *groups * 4 words): the input column of every step as its byte offset in a buffer
- * of 16 rows per column (column * 64); weights (neuron/4 * *groups * 4 * 4 floats: [quad][group][output][step]): the
+ * of 16 rows per column (column * 64); weights (neuron/4 * *groups * 4 * 4 floats: [quad][group][step][output]): the
  * step's weight in each of the four outputs, 0 where the output does not use it.  *groups = 0: the layer has no such
  * form.  No counterpart in the reference (its kernels keep a layer's outputs in shared memory for one layer only);
  * inspection interface like spdnn_get_band_pairs. */
