@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstdint>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -34,7 +35,9 @@ bool read_triples(const std::string& path, std::vector<Triple>& out, std::string
         const float v = strtof(p, &q);
         if (q == p) { err = "malformed line in " + path; return false; }
         p = q;
-        out.push_back(Triple{(int32_t)a, (int32_t)b, v});
+        // an index beyond 32 bits stays out of range for every width instead of wrapping into it
+        const long lo = INT32_MIN, hi = INT32_MAX;
+        out.push_back(Triple{(int32_t)std::min(std::max(a, lo), hi), (int32_t)std::min(std::max(b, lo), hi), v});
     }
     return true;
 }

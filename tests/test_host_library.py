@@ -442,6 +442,13 @@ def test_tsv_layer_through_the_library(gc, orc, tmp_path):
         with pytest.raises(gc.SpdnnError) as e:
             a.load_layer_tsv(0, str(tmp_path / "missing.tsv"))
         assert e.value.code == 3 and "does not exists" in e.value.message
+        # an index that does not fit 32 bits is out of range, not the neuron it would wrap round to
+        for bad in ("4294967297\t1\t0.5\n", "1\t4294967297\t0.5\n", "-4294967295\t1\t0.5\n", "0\t1\t0.5\n"):
+            q = tmp_path / "wrap.tsv"
+            q.write_text("".join(lines[:5]) + bad)
+            with pytest.raises(gc.SpdnnError) as e:
+                a.load_layer_tsv(0, str(q))
+            assert e.value.code == 3 and "out of range" in e.value.message
     # the committed fixture layers are plain (non-band) layers of width 64
     with gc.Network(64, 12, 2, bias=-0.3) as net:
         net.load_layer_tsv(0, os.path.join(GOLD, "tiny_n64-l1.tsv"))
